@@ -1,0 +1,224 @@
+"""CPU oracle for the DAX dynamic W8A8 linear (INT8 and FP8-e4m3fn).
+
+TEST INFRASTRUCTURE ONLY.  This file is the checker that the HIP kernels are
+compared against; nothing in the shipped package may import or call it.  It is
+used by ``tests/``, by ``__graft_entry__.smoke()`` and by the ``cpu_baseline``
+leg of ``bench.py``.
+
+Every function restates, with plain PyTorch CPU ops and the same dtype chain as
+the reference's *eager* execution, the reference lines cited in its docstring
+(paths are relative to the reference checkout).  The reference package itself is
+never imported: it raises at import time on a non-CUDA torch
+(dax/quant/nn/quantized/linear.py:21-25).
+
+How each function is pinned (see tests/test_oracle_*.py):
+
+* act_scale                exhaustive over every finite bf16 amax against the
+                           bit-level C closed form (oracle/daxq_oracle_c.c)
+* quantize_to_int8         C closed form on every bf16 x for sampled reachable
+                           scales + special rows (zero row, +-amax -> +-127)
+* quantize_to_fp8          torch's f32->e4m3fn cast against the bit-level C
+                           encoder on all 2^16 bf16 inputs x many scales and on
+                           a dense sweep of f32 bit patterns; tie / saturation
+                           / subnormal known answers
+* weight_scale / quant     C closed form, brute force on small matrices
+* int_mm                   numpy int64 brute force, adversarial +-127 / -128
+* linear_int8 epilogue     C closed form bf16(bf16(f32(acc)*sx*sw)+bias)
+* linear_fp8               accumulation order is not fixed by the reference
+                           (cuBLASLt fast-accum): "parity unpinned" at bit
+                           level, tolerance 2e-2 relative L2; the per-tensor
+                           special case is checked against torch._scaled_mm CPU
+"""
+
+from __future__ import annotations
+
+from typing import Dict, Optional, Tuple
+
+import torch
+
+INT8_QMAX = 127  # torch.iinfo(torch.int8).max      dynamic/functional.py:199
+E4M3_QMAX = 448.0  # torch.finfo(torch.float8_e4m3fn).max   dynamic/functional.py:170
+EPS = torch.finfo(torch.float32).eps  # 2**-23     dynamic/functional.py:171,200
+
+
+# --------------------------------------------------------------------------- #
+# host-side shape helpers
+# --------------------------------------------------------------------------- #
+def get_block_size(shape: Tuple[int, ...], qscheme: str) -> Tuple[int, ...]:
+    """dax/quant/qscheme.py:10-26."""
+    kind = qscheme.rsplit(".", 1)[-1]
+    if kind == "per_tensor_symmetric":
+        return tuple(shape)
+    if kind == "per_token_symmetric":
+        return (1,) * (len(shape) - 1) + (shape[-1],)
+    if kind == "per_channel_symmetric":
+        return tuple(shape[:-1]) + (1,)
+    raise ValueError(f"Unsupported QScheme: {qscheme}")
+
+
+# --------------------------------------------------------------------------- #
+# activation quantisation (per token)
+# --------------------------------------------------------------------------- #
+def act_scale(x: torch.Tensor, qmax: float) -> torch.Tensor:
+    """Per-token scale, eager dtype chain.  dax/quant/nn/dynamic/functional.py:124-135.
+
+    ``x`` is [M, K] in its original dtype (bf16 on the hot path).  The division
+    and the clamp happen in x's dtype; only then is the scale widened to fp32.
+    Returns fp32 [M, 1].
+    """
+    amax = x.abs().amax(dim=-1, keepdim=False)  # :124
+    scale = amax / float(qmax)  # :126
+    scale = torch.clamp(scale, min=EPS)  # :127
+    if scale.dtype != torch.float32:  # :128-129
+        scale = scale.to(torch.float32)
+    return scale.view(-1, 1)  # :131-135
+
+
+def quantize_to_int8(x: torch.Tensor, scale: torch.Tensor) -> torch.Tensor:
+    """dax/quant/nn/quantized/functional.py:17-20 (reciprocal-multiply, RNE, clamp)."""
+    return torch.clamp(torch.round(x * (1.0 / scale)), -128, 127).to(torch.int8)
+
+
+def quantize_to_fp8(x: torch.Tensor, scale: torch.Tensor) -> torch.Tensor:
+    """dax/quant/nn/quantized/functional.py:11-13 (true division, clamp, RNE cast)."""
+    return (x / scale).clamp(-E4M3_QMAX, E4M3_QMAX).to(torch.float8_e4m3fn)
+
+
+def act_quant_int8(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """dynamic_quantize_to_int8, per-token.  dynamic/functional.py:181-206, :54-148."""
+    x2 = x.reshape(-1, x.shape[-1])
+    s = act_scale(x2, INT8_QMAX)
+    return quantize_to_int8(x2, s), s
+
+
+def act_quant_e4m3(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """dynamic_quantize_to_fp8, per-token, e4m3fn.  dynamic/functional.py:152-177."""
+    x2 = x.reshape(-1, x.shape[-1])
+    s = act_scale(x2, E4M3_QMAX)
+    return quantize_to_fp8(x2, s), s
+
+
+# --------------------------------------------------------------------------- #
+# weight quantisation (per output channel, one time)
+# --------------------------------------------------------------------------- #
+def weight_scale(w: torch.Tensor, qmax: float) -> torch.Tensor:
+    """PerChannelMinMaxObserver + _calculate_qparams.
+
+    dax/quant/quantization/observer.py:284-312 (fp32 row min/max) and :97-134
+    (amax / qmax, floor at eps) -- all in fp32, no bf16 rounding.  Returns fp32 [N].
+    """
+    y = w.detach().to(torch.float32).flatten(1)  # :298-299
+    lo, hi = torch.aminmax(y, dim=1)  # :301
+    amax = torch.max(-lo, hi)  # :123
+    scale = amax / float(qmax)  # :125
+    return torch.max(scale, torch.tensor([EPS], dtype=torch.float32))  # :126
+
+
+def weight_quant_int8(w: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """dax/quant/nn/dynamic/linear.py:276-299 with the int8 leaf quantiser."""
+    s = weight_scale(w, INT8_QMAX)
+    return quantize_to_int8(w, s.view(-1, 1)), s.view(1, -1)
+
+
+def weight_quant_e4m3(w: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """dax/quant/nn/dynamic/linear.py:276-299 with the fp8 leaf quantiser."""
+    s = weight_scale(w, E4M3_QMAX)
+    return quantize_to_fp8(w, s.view(-1, 1)), s.view(1, -1)
+
+
+def dequant_weight(qweight: torch.Tensor, wscale: torch.Tensor, out_dtype=torch.bfloat16) -> torch.Tensor:
+    """Linear.weight property.  dax/quant/nn/dynamic/linear.py:139-141."""
+    return qweight.to(out_dtype) * wscale.T.to(out_dtype)
+
+
+# --------------------------------------------------------------------------- #
+# GEMM + epilogue
+# --------------------------------------------------------------------------- #
+def int_mm(xq: torch.Tensor, wq: torch.Tensor) -> torch.Tensor:
+    """int8 [M,K] x int8 [N,K]^T -> int32 [M,N], exact.
+
+    dax/quant/nn/dynamic/linear.py:218-220 (out_dtype(aten.mm, int32, ...)).
+    torch._int_mm is the library routine BASELINE names for the CPU path; it is
+    exact integer arithmetic, so any summation order gives the same bits.
+    """
+    return torch._int_mm(xq.contiguous(), wq.t())
+
+
+def epilogue_int8(acc: torch.Tensor, sx: torch.Tensor, sw: torch.Tensor,
+                  bias: Optional[torch.Tensor], out_dtype=torch.bfloat16) -> torch.Tensor:
+    """dax/quant/nn/dynamic/linear.py:214,221-228.
+
+    int32 * fp32 -> fp32 (acc converted RNE), * weight_scale fp32, cast to
+    out_dtype, then a second rounding when the bf16 bias is added.
+    """
+    m, n = acc.shape
+    out = acc * sx.reshape(-1, 1).expand(m, n)  # :214,:221
+    out = out * sw.reshape(1, -1)  # :222
+    if out.dtype != out_dtype:  # :225-226
+        out = out.to(out_dtype)
+    if bias is not None:  # :227-228
+        out = out + bias
+    return out
+
+
+def linear_int8(x: torch.Tensor, qweight: torch.Tensor, wscale: torch.Tensor,
+                bias: Optional[torch.Tensor], row_chunk: int = 8192,
+                keep_acc: bool = True) -> Dict[str, torch.Tensor]:
+    """Whole INT8 forward.  dax/quant/nn/dynamic/linear.py:180-228.
+
+    Processes rows in chunks so that the int32 accumulator of the big shapes is
+    never resident in full unless ``keep_acc``.  Returns xq, sx, (acc), out.
+    """
+    prev = x.shape[:-1]
+    x2 = x.reshape(-1, x.shape[-1])
+    xq, sx = act_quant_int8(x2)
+    outs, accs = [], []
+    for r0 in range(0, x2.shape[0], row_chunk):
+        acc = int_mm(xq[r0:r0 + row_chunk], qweight)
+        outs.append(epilogue_int8(acc, sx[r0:r0 + row_chunk], wscale, bias, x.dtype))
+        if keep_acc:
+            accs.append(acc)
+    out = torch.cat(outs, 0).view(*prev, qweight.shape[0])
+    res = {"xq": xq, "sx": sx, "out": out}
+    if keep_acc:
+        res["acc"] = torch.cat(accs, 0)
+    return res
+
+
+def linear_e4m3(x: torch.Tensor, qweight: torch.Tensor, wscale: torch.Tensor,
+                bias: Optional[torch.Tensor], row_chunk: int = 8192) -> Dict[str, torch.Tensor]:
+    """Whole FP8 forward.  dax/quant/nn/dynamic/linear.py:145-178.
+
+    torch._scaled_mm with row-wise scales is CUDA-only, so the matmul is
+    emulated in fp32: bf16( (Xq . Wq^T in fp32) * sx * sw + bias ), one rounding.
+    The summation order of the reference (cuBLASLt, use_fast_accum=True) is not
+    specified; comparisons against this function use a tolerance.
+    """
+    prev = x.shape[:-1]
+    x2 = x.reshape(-1, x.shape[-1])
+    xq, sx = act_quant_e4m3(x2)
+    wf = qweight.to(torch.float32)
+    outs = []
+    for r0 in range(0, x2.shape[0], row_chunk):
+        acc = xq[r0:r0 + row_chunk].to(torch.float32) @ wf.t()
+        o = acc * sx[r0:r0 + row_chunk] * wscale.reshape(1, -1)
+        if bias is not None:
+            o = o + bias.to(torch.float32)
+        outs.append(o.to(torch.bfloat16))
+    out = torch.cat(outs, 0).view(*prev, qweight.shape[0])
+    return {"xq": xq, "sx": sx, "out": out}
+
+
+# --------------------------------------------------------------------------- #
+# synthetic workload of the benchmark configs (shared by tests and bench.py)
+# --------------------------------------------------------------------------- #
+def make_inputs(m: int, k: int, n: int, seed: int = 0):
+    """Seeded synthetic X, W, bias with 1 % outlier channels (x20), all bf16, on CPU."""
+    g = torch.Generator("cpu").manual_seed(seed)
+    x = torch.randn(m, k, generator=g)
+    idx = torch.randperm(k, generator=g)[: max(1, round(0.01 * k))]
+    x[:, idx] *= 20
+    x = x.bfloat16()
+    w = (torch.randn(n, k, generator=g) * 0.02).bfloat16()
+    b = (torch.randn(n, generator=g) * 0.01).bfloat16()
+    return x, w, b
