@@ -1,0 +1,172 @@
+"""W8A8 linear throughput at the Wan2.1-14B 720p shapes on one MI355X.
+
+One step = one pass of the quantised-linear hot path over the four linears of a DiT block
+at M = 75600 tokens (QKV 5120->15360, out-proj 5120->5120, FFN 5120->13824, FFN 13824->5120):
+per linear, the per-token activation quantiser and the MFMA GEMM with the fused epilogue.
+Inputs (bf16 activations, pre-quantised weights, scales, bias) are resident in HBM before the
+timed region.  Prints one JSON line.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--dtype int8|fp8] [--no-cpu-baseline]
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+M_TOKENS = 75600
+SHAPES = [("qkv", 5120, 15360), ("out", 5120, 5120), ("ffn_up", 5120, 13824), ("ffn_down", 13824, 5120)]
+PEAK_TOPS = {"int8": 5000.0, "fp8": 5000.0}  # MI355X dense 8-bit MFMA peak
+
+
+def cpu_baseline(dtype: str, rows: int):
+    """The reference's CPU path (oracle: eager quantiser + torch._int_mm / fp32-emulated fp8
+    matmul + epilogue) on a bounded sample of `rows` tokens of the same four shapes."""
+    import torch
+
+    from oracle import daxq_oracle as O
+
+    ops_done, t_total = 0.0, 0.0
+    for i, (_, k, n) in enumerate(SHAPES):
+        x, w, b = O.make_inputs(rows, k, n, seed=i)
+        if dtype == "int8":
+            qw, sw = O.weight_quant_int8(w)
+            t0 = time.perf_counter()
+            O.linear_int8(x, qw, sw, b, keep_acc=False)
+        else:
+            qw, sw = O.weight_quant_e4m3(w)
+            t0 = time.perf_counter()
+            O.linear_e4m3(x, qw, sw, b)
+        t_total += time.perf_counter() - t0
+        ops_done += 2.0 * rows * n * k
+    return {"value": ops_done / t_total / 1e12, "unit": "TOPS", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"first {rows} of {M_TOKENS} tokens of each of the 4 shapes, {t_total:.1f} s, "
+                      f"os.cpu_count()={os.cpu_count()}"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--dtype", choices=["int8", "fp8"], default="int8")
+    ap.add_argument("--variant", type=int, default=0)
+    ap.add_argument("--m", type=int, default=M_TOKENS)
+    ap.add_argument("--cpu-rows", type=int, default=4096)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build measures one GPU; --gpus must be 1 (the path shards by token rows, "
+                 "no multi-GPU figure is produced)")
+
+    import torch
+
+    import dax_amd.ops as ops
+    from dax_amd import _capi
+
+    assert torch.cuda.is_available(), "bench.py needs an MI355X"
+    _capi.require_gfx950(0)
+    _capi.set_gemm_variant(args.variant)
+    dev = torch.device("cuda:0")
+    fp8 = args.dtype == "fp8"
+    m = args.m
+
+    # ---- synthetic inputs, resident in HBM
+    g = torch.Generator(device="cpu").manual_seed(0)
+    layers = []
+    xs = {}
+    for i, (name, k, n) in enumerate(SHAPES):
+        if k not in xs:
+            x = torch.randn(m, k, device=dev, dtype=torch.bfloat16)
+            idx = torch.randperm(k, generator=g)[: max(1, round(0.01 * k))].to(dev)
+            x[:, idx] *= 20
+            xs[k] = x
+        w = (torch.randn(n, k, device=dev) * 0.02).bfloat16()
+        b = (torch.randn(n, device=dev) * 0.01).bfloat16()
+        lo, hi = ops.row_minmax(w)
+        sw = ops.scale_from_minmax(lo, hi, 448.0 if fp8 else 127.0)
+        qw = (ops.quantize_rows_e4m3 if fp8 else ops.quantize_rows_i8)(w, sw, True)
+        layers.append((name, k, n, xs[k], qw, sw, b))
+        del w
+    act_quant = ops.act_quant_e4m3 if fp8 else ops.act_quant_i8
+    linear = ops.linear_e4m3 if fp8 else ops.linear_i8
+
+    def step(ev=None):
+        for li, (name, k, n, x, qw, sw, b) in enumerate(layers):
+            if ev is not None:
+                ev[li][0].record()
+            xq, sx = act_quant(x)
+            if ev is not None:
+                ev[li][1].record()
+            out = linear(xq, sx, qw, sw, b)
+            if ev is not None:
+                ev[li][2].record()
+        return out
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    evs = [[[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in layers] for _ in range(args.steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for s in range(args.steps):
+        step(evs[s])
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+
+    ms_per_step = (t1 - t0) * 1e3 / args.steps
+    total_ops = sum(2.0 * m * n * k for _, k, n in SHAPES)
+    value = total_ops / (ms_per_step * 1e-3) / 1e12
+
+    # ---- per-kernel durations from the events recorded on the launch stream inside the timed region
+    per_layer = {}
+    gemm_ms_sum, quant_ms_sum = 0.0, 0.0
+    for li, (name, k, n, *_rest) in enumerate(layers):
+        q_ms = sum(evs[s][li][0].elapsed_time(evs[s][li][1]) for s in range(args.steps)) / args.steps
+        g_ms = sum(evs[s][li][1].elapsed_time(evs[s][li][2]) for s in range(args.steps)) / args.steps
+        ops_l = 2.0 * m * n * k
+        per_layer[name] = {"k": k, "n": n, "quant_ms": round(q_ms, 4), "gemm_ms": round(g_ms, 4),
+                           "gemm_tops": round(ops_l / (g_ms * 1e-3) / 1e12, 1),
+                           "quant_gbps": round((3.0 * m * k + 4.0 * m) / (q_ms * 1e-3) / 1e9, 1)}
+        gemm_ms_sum += g_ms
+        quant_ms_sum += q_ms
+    achieved = total_ops / (gemm_ms_sum * 1e-3) / 1e12
+    peak = PEAK_TOPS[args.dtype]
+
+    info = _capi.device_info(0)
+    res = {
+        "metric": f"w8a8_linear_tops_wan2.1_14b_720p_{args.dtype}",
+        "value": round(value, 2),
+        "unit": "TOPS",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "int8" if not fp8 else "fp8_e4m3fn",
+        "data": "synthetic",
+        "config": {"workload": f"Wan2.1-14B 720p linear set, {args.dtype.upper()} W8A8, M={m} tokens: "
+                               "QKV 5120->15360, out 5120->5120, FFN 5120->13824, FFN 13824->5120; "
+                               "per linear: per-token act quant + MFMA GEMM + fused scale/bias/bf16 epilogue",
+                   "gemm_variant": args.variant},
+        "pct_of_mfma_peak": round(100.0 * value / peak, 2),
+        "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": peak, "unit": "TFLOP/s",
+                     "frac": round(achieved / peak, 4), "traffic": None,
+                     "kernel": "gemm_w8a8_kernel (all four shapes; 8-bit ops counted as 2*M*N*K)",
+                     "gemm_ms_per_step": round(gemm_ms_sum, 4), "quant_ms_per_step": round(quant_ms_sum, 4)},
+        "per_linear": per_layer,
+        "device": {"arch": info["arch"], "cu_count": info["cu_count"], "max_clock_mhz": info["clock_khz"] / 1000.0},
+    }
+    if not args.no_cpu_baseline:
+        res["cpu_baseline"] = cpu_baseline(args.dtype, args.cpu_rows)
+    print(json.dumps(res), flush=True)
+
+
+if __name__ == "__main__":
+    main()

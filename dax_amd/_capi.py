@@ -1,0 +1,93 @@
+"""ctypes binding of the C ABI in include/daxq.h (dax_amd/lib/libdaxq.so).
+
+Loading is lazy and loud: a missing library or a non-gfx950 device raises RuntimeError;
+nothing here falls back to another implementation.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+import threading
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libdaxq.so")
+ABI_VERSION = 1
+
+_lock = threading.Lock()
+_lib = None
+_checked_devices = set()
+
+_P, _I64, _F32, _INT = C.c_void_p, C.c_int64, C.c_float, C.c_int
+
+# name -> argtypes; every entry point declared in include/daxq.h
+SIGNATURES = {
+    "daxq_abi_version": [],
+    "daxq_last_error": [],
+    "daxq_device_info": [_INT, C.POINTER(_INT), C.POINTER(_INT), C.POINTER(_INT), C.c_char_p, _INT],
+    "daxq_act_quant_i8": [_P, _I64, _I64, _I64, _P, _I64, _P, _P],
+    "daxq_act_quant_e4m3": [_P, _I64, _I64, _I64, _P, _I64, _P, _P],
+    "daxq_quantize_rows_i8": [_P, _I64, _I64, _I64, _P, _P, _I64, _P],
+    "daxq_quantize_rows_e4m3": [_P, _I64, _I64, _I64, _P, _P, _I64, _P],
+    "daxq_row_minmax": [_P, _I64, _I64, _I64, _P, _P, _P],
+    "daxq_scale_from_minmax": [_P, _P, _I64, _F32, _P, _P],
+    "daxq_linear_i8": [_P, _I64, _P, _P, _I64, _P, _P, _P, _I64, _P, _I64, _I64, _I64, _I64, _P],
+    "daxq_linear_e4m3": [_P, _I64, _P, _P, _I64, _P, _P, _P, _I64, _P, _I64, _I64, _I64, _I64, _P],
+    "daxq_set_gemm_variant": [_INT],
+}
+
+
+class DaxqError(RuntimeError):
+    """A daxq entry point returned a negative status."""
+
+
+def lib() -> C.CDLL:
+    global _lib
+    if _lib is None:
+        with _lock:
+            if _lib is None:
+                if not os.path.exists(LIB_PATH):
+                    raise RuntimeError(
+                        f"{LIB_PATH} is not built; run `python -c 'import __graft_entry__ as g; g.build()'` "
+                        "(hipcc, gfx950). dax_amd has no other implementation to fall back to.")
+                L = C.CDLL(LIB_PATH)
+                for name, args in SIGNATURES.items():
+                    fn = getattr(L, name)
+                    fn.argtypes = args
+                    fn.restype = C.c_char_p if name == "daxq_last_error" else _INT
+                got = L.daxq_abi_version()
+                if got != ABI_VERSION:
+                    raise RuntimeError(f"libdaxq ABI {got} != expected {ABI_VERSION}; rebuild the library")
+                _lib = L
+    return _lib
+
+
+def last_error() -> str:
+    msg = lib().daxq_last_error()
+    return msg.decode() if msg else ""
+
+
+def check(status: int, what: str) -> None:
+    if status != 0:
+        raise DaxqError(f"{what} failed with status {status}: {last_error()}")
+
+
+def device_info(device: int = 0) -> dict:
+    cu, clk, lds = _INT(0), _INT(0), _INT(0)
+    arch = C.create_string_buffer(64)
+    st = lib().daxq_device_info(device, C.byref(cu), C.byref(clk), C.byref(lds), arch, 64)
+    return {"status": st, "cu_count": cu.value, "clock_khz": clk.value, "lds_bytes": lds.value,
+            "arch": arch.value.decode()}
+
+
+def require_gfx950(device: int) -> None:
+    """Raises unless `device` is a gfx950 (checked once per device)."""
+    if device in _checked_devices:
+        return
+    info = device_info(device)
+    if info["status"] != 0:
+        raise RuntimeError(f"daxq needs an MI355X (gfx950) device: {last_error()}")
+    _checked_devices.add(device)
+
+
+def set_gemm_variant(v: int) -> None:
+    check(lib().daxq_set_gemm_variant(int(v)), "daxq_set_gemm_variant")

@@ -1,0 +1,217 @@
+"""``torch.ops.daxq.*``: the HIP kernels of libdaxq as PyTorch custom ops.
+
+Each op allocates its outputs with torch (device memory is torch's), passes raw device
+pointers and the current HIP stream through the C ABI, and has a fake (meta) kernel so a
+surrounding ``torch.compile`` graph can trace through it.  No op has a CPU kernel.
+"""
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import torch
+
+from . import _capi
+
+K_ALIGN = 128  # DAXQ_K_ALIGN
+
+
+def pad_k(k: int) -> int:
+    return (k + K_ALIGN - 1) // K_ALIGN * K_ALIGN
+
+
+def _stream(t: torch.Tensor) -> int:
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _need_gpu(t: torch.Tensor, what: str) -> None:
+    if t.device.type != "cuda":
+        raise RuntimeError(f"daxq::{what}: tensor is on {t.device}; the daxq kernels only run on an MI355X "
+                           "(there is no CPU implementation)")
+    _capi.require_gfx950(t.device.index if t.device.index is not None else torch.cuda.current_device())
+
+
+def _rows_bf16(x: torch.Tensor, what: str) -> None:
+    _need_gpu(x, what)
+    if x.dtype != torch.bfloat16:
+        raise NotImplementedError(f"daxq::{what}: only bfloat16 inputs are implemented, got {x.dtype}")
+    if x.dim() != 2 or x.stride(1) != 1:
+        raise ValueError(f"daxq::{what}: expected a 2-d tensor with contiguous rows, got shape {tuple(x.shape)} "
+                         f"strides {x.stride()}")
+
+
+# ----------------------------------------------------------------------------- act quant
+def _act_quant(x: torch.Tensor, fp8: bool) -> Tuple[torch.Tensor, torch.Tensor]:
+    name = "act_quant_e4m3" if fp8 else "act_quant_i8"
+    _rows_bf16(x, name)
+    m, k = x.shape
+    kp = pad_k(k)
+    with torch.cuda.device(x.device):
+        q = torch.empty((m, kp), dtype=torch.uint8 if fp8 else torch.int8, device=x.device)
+        s = torch.empty((m,), dtype=torch.float32, device=x.device)
+        if m:
+            fn = _capi.lib().daxq_act_quant_e4m3 if fp8 else _capi.lib().daxq_act_quant_i8
+            ld_x = x.stride(0) if m > 1 else k
+            _capi.check(fn(x.data_ptr(), m, k, ld_x, q.data_ptr(), kp, s.data_ptr(), _stream(x)), name)
+    return q, s
+
+
+@torch.library.custom_op("daxq::act_quant_i8", mutates_args=(), device_types="cuda")
+def act_quant_i8(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """bf16 [M,K] -> (int8 [M, pad128(K)] zero padded, fp32 [M] per-token scale)."""
+    return _act_quant(x, False)
+
+
+@torch.library.custom_op("daxq::act_quant_e4m3", mutates_args=(), device_types="cuda")
+def act_quant_e4m3(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """bf16 [M,K] -> (e4m3fn bytes as uint8 [M, pad128(K)], fp32 [M] per-token scale)."""
+    return _act_quant(x, True)
+
+
+def _act_quant_fake(x, dtype):
+    return x.new_empty((x.shape[0], pad_k(x.shape[1])), dtype=dtype), x.new_empty((x.shape[0],), dtype=torch.float32)
+
+
+act_quant_i8.register_fake(lambda x: _act_quant_fake(x, torch.int8))
+act_quant_e4m3.register_fake(lambda x: _act_quant_fake(x, torch.uint8))
+
+
+# ----------------------------------------------------------------------------- leaf quantisers
+def _quantize_rows(x: torch.Tensor, scale: torch.Tensor, fp8: bool, padded: bool) -> torch.Tensor:
+    name = "quantize_rows_e4m3" if fp8 else "quantize_rows_i8"
+    _rows_bf16(x, name)
+    m, k = x.shape
+    if scale.dtype != torch.float32 or scale.numel() != m or scale.device != x.device:
+        raise ValueError(f"daxq::{name}: scale must be fp32 with one value per row on {x.device}")
+    scale = scale.reshape(-1).contiguous()
+    ld_q = pad_k(k) if padded else k
+    with torch.cuda.device(x.device):
+        q = torch.empty((m, ld_q), dtype=torch.uint8 if fp8 else torch.int8, device=x.device)
+        if m:
+            fn = _capi.lib().daxq_quantize_rows_e4m3 if fp8 else _capi.lib().daxq_quantize_rows_i8
+            ld_x = x.stride(0) if m > 1 else k
+            _capi.check(fn(x.data_ptr(), m, k, ld_x, scale.data_ptr(), q.data_ptr(), ld_q, _stream(x)), name)
+    return q
+
+
+@torch.library.custom_op("daxq::quantize_rows_i8", mutates_args=(), device_types="cuda")
+def quantize_rows_i8(x: torch.Tensor, scale: torch.Tensor, padded: bool = False) -> torch.Tensor:
+    return _quantize_rows(x, scale, False, padded)
+
+
+@torch.library.custom_op("daxq::quantize_rows_e4m3", mutates_args=(), device_types="cuda")
+def quantize_rows_e4m3(x: torch.Tensor, scale: torch.Tensor, padded: bool = False) -> torch.Tensor:
+    return _quantize_rows(x, scale, True, padded)
+
+
+quantize_rows_i8.register_fake(
+    lambda x, scale, padded=False: x.new_empty((x.shape[0], pad_k(x.shape[1]) if padded else x.shape[1]), dtype=torch.int8))
+quantize_rows_e4m3.register_fake(
+    lambda x, scale, padded=False: x.new_empty((x.shape[0], pad_k(x.shape[1]) if padded else x.shape[1]), dtype=torch.uint8))
+
+
+# ----------------------------------------------------------------------------- weight observer statistics
+@torch.library.custom_op("daxq::row_minmax", mutates_args=(), device_types="cuda")
+def row_minmax(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Per-row (min, max) of a bf16 matrix in fp32."""
+    _rows_bf16(x, "row_minmax")
+    m, k = x.shape
+    with torch.cuda.device(x.device):
+        lo = torch.empty((m,), dtype=torch.float32, device=x.device)
+        hi = torch.empty((m,), dtype=torch.float32, device=x.device)
+        if m:
+            ld_x = x.stride(0) if m > 1 else k
+            _capi.check(_capi.lib().daxq_row_minmax(x.data_ptr(), m, k, ld_x, lo.data_ptr(), hi.data_ptr(), _stream(x)),
+                        "row_minmax")
+    return lo, hi
+
+
+row_minmax.register_fake(lambda x: (x.new_empty((x.shape[0],), dtype=torch.float32),
+                                    x.new_empty((x.shape[0],), dtype=torch.float32)))
+
+
+@torch.library.custom_op("daxq::scale_from_minmax", mutates_args=(), device_types="cuda")
+def scale_from_minmax(min_val: torch.Tensor, max_val: torch.Tensor, qmax: float) -> torch.Tensor:
+    """max(max(-min, max) / qmax, 2^-23) element-wise in fp32."""
+    _need_gpu(min_val, "scale_from_minmax")
+    if min_val.dtype != torch.float32 or max_val.dtype != torch.float32 or min_val.shape != max_val.shape:
+        raise ValueError("daxq::scale_from_minmax: min/max must be fp32 tensors of one shape")
+    lo, hi = min_val.contiguous(), max_val.contiguous()
+    with torch.cuda.device(lo.device):
+        s = torch.empty_like(lo)
+        _capi.check(_capi.lib().daxq_scale_from_minmax(lo.data_ptr(), hi.data_ptr(), lo.numel(), float(qmax),
+                                                       s.data_ptr(), _stream(lo)), "scale_from_minmax")
+    return s
+
+
+scale_from_minmax.register_fake(lambda min_val, max_val, qmax: torch.empty_like(min_val))
+
+
+# ----------------------------------------------------------------------------- GEMM + epilogue
+def _linear(xq, sx, wq, sw, bias, fp8: bool, want_acc: bool):
+    name = "linear_e4m3" if fp8 else "linear_i8"
+    _need_gpu(xq, name)
+    qdt = torch.uint8 if fp8 else torch.int8
+    if xq.dtype != qdt or wq.dtype != qdt:
+        raise ValueError(f"daxq::{name}: operands must be {qdt}")
+    if xq.dim() != 2 or wq.dim() != 2 or xq.stride(1) != 1 or wq.stride(1) != 1 or xq.shape[1] != wq.shape[1]:
+        raise ValueError(f"daxq::{name}: expected xq [M,Kp] and wq [N,Kp] with contiguous rows, got "
+                         f"{tuple(xq.shape)} and {tuple(wq.shape)}")
+    m, k = xq.shape
+    n = wq.shape[0]
+    if sx.dtype != torch.float32 or sw.dtype != torch.float32 or sx.numel() != m or sw.numel() != n:
+        raise ValueError(f"daxq::{name}: sx must be fp32 [M] and sw fp32 [N]")
+    if bias is not None and (bias.dtype != torch.bfloat16 or bias.numel() != n):
+        raise ValueError(f"daxq::{name}: bias must be bf16 [N]")
+    sx = sx.reshape(-1).contiguous()
+    sw = sw.reshape(-1).contiguous()
+    bias_c = bias.contiguous() if bias is not None else None
+    with torch.cuda.device(xq.device):
+        out = torch.empty((m, n), dtype=torch.bfloat16, device=xq.device)
+        acc = torch.empty((m, n), dtype=torch.float32 if fp8 else torch.int32, device=xq.device) if want_acc else None
+        if m and n:
+            fn = _capi.lib().daxq_linear_e4m3 if fp8 else _capi.lib().daxq_linear_i8
+            ld_x = xq.stride(0) if m > 1 else k
+            ld_w = wq.stride(0) if n > 1 else k
+            _capi.check(fn(xq.data_ptr(), ld_x, sx.data_ptr(), wq.data_ptr(), ld_w, sw.data_ptr(),
+                           bias_c.data_ptr() if bias_c is not None else None, out.data_ptr(), n,
+                           acc.data_ptr() if acc is not None else None, n, m, n, k, _stream(xq)), name)
+    return out, acc
+
+
+@torch.library.custom_op("daxq::linear_i8", mutates_args=(), device_types="cuda")
+def linear_i8(xq: torch.Tensor, sx: torch.Tensor, wq: torch.Tensor, sw: torch.Tensor,
+              bias: Optional[torch.Tensor]) -> torch.Tensor:
+    """int8 [M,Kp] x int8 [N,Kp]^T with the fused per-token / per-channel scale, bias and bf16 cast."""
+    return _linear(xq, sx, wq, sw, bias, False, False)[0]
+
+
+@torch.library.custom_op("daxq::linear_i8_acc", mutates_args=(), device_types="cuda")
+def linear_i8_acc(xq: torch.Tensor, sx: torch.Tensor, wq: torch.Tensor, sw: torch.Tensor,
+                  bias: Optional[torch.Tensor]) -> Tuple[torch.Tensor, torch.Tensor]:
+    """As linear_i8, also returning the exact int32 accumulators [M,N]."""
+    return _linear(xq, sx, wq, sw, bias, False, True)
+
+
+@torch.library.custom_op("daxq::linear_e4m3", mutates_args=(), device_types="cuda")
+def linear_e4m3(xq: torch.Tensor, sx: torch.Tensor, wq: torch.Tensor, sw: torch.Tensor,
+                bias: Optional[torch.Tensor]) -> torch.Tensor:
+    """e4m3fn [M,Kp] x e4m3fn [N,Kp]^T (bytes as uint8), fp32 accumulate, fused scales + bias + bf16."""
+    return _linear(xq, sx, wq, sw, bias, True, False)[0]
+
+
+@torch.library.custom_op("daxq::linear_e4m3_acc", mutates_args=(), device_types="cuda")
+def linear_e4m3_acc(xq: torch.Tensor, sx: torch.Tensor, wq: torch.Tensor, sw: torch.Tensor,
+                    bias: Optional[torch.Tensor]) -> Tuple[torch.Tensor, torch.Tensor]:
+    return _linear(xq, sx, wq, sw, bias, True, True)
+
+
+def _lin_fake(xq, sx, wq, sw, bias):
+    return xq.new_empty((xq.shape[0], wq.shape[0]), dtype=torch.bfloat16)
+
+
+linear_i8.register_fake(_lin_fake)
+linear_e4m3.register_fake(_lin_fake)
+linear_i8_acc.register_fake(lambda xq, sx, wq, sw, bias: (
+    _lin_fake(xq, sx, wq, sw, bias), xq.new_empty((xq.shape[0], wq.shape[0]), dtype=torch.int32)))
+linear_e4m3_acc.register_fake(lambda xq, sx, wq, sw, bias: (
+    _lin_fake(xq, sx, wq, sw, bias), xq.new_empty((xq.shape[0], wq.shape[0]), dtype=torch.float32)))

@@ -1,0 +1,213 @@
+"""Dynamic W8A8 ``Linear``: the module that takes the place of ``nn.Linear`` inside the DiT.
+
+Drop-in for dax/quant/nn/dynamic/linear.py:27-341: same constructor signature, the same
+persistent state (``qweight`` [N,K] int8 / float8_e4m3fn, ``weight_scale`` fp32 [1,N],
+``bias``), the same ``from_float`` / ``get_qlinear`` / ``weight`` / ``extra_repr`` surface
+and the same exceptions for invalid dtype / qscheme combinations.
+
+What differs is where the arithmetic runs: ``forward`` is two HIP launches -- the fused
+per-token quantiser and the MFMA GEMM with the scale / bias / bf16 epilogue -- and the
+conversion in ``get_qlinear`` uses the HIP observer and leaf-quantiser kernels.  Numerics are
+those of the reference's eager op sequence (:180-228 for INT8, :145-178 for FP8).  The
+reference's eager-only escape to a float matmul for M <= 16 or misaligned K/N (:186-202,
+never taken under its own ``torch.compile`` decorator) does not exist here: every shape goes
+through the quantised kernels.
+"""
+from __future__ import annotations
+
+import logging
+
+import torch
+from torch import Tensor, nn
+
+from .... import ops
+from ...qscheme import per_channel_symmetric, per_tensor_symmetric, per_token_symmetric
+from .functional import FP8_ALLOWED_DTYPES
+
+logger = logging.getLogger(__name__)
+
+
+class Linear(nn.Module):
+    _FLOAT_MODULE = nn.Linear
+
+    def __init__(
+        self,
+        in_features: int,
+        out_features: int,
+        bias: bool = True,
+        device=None,
+        weight_dtype=None,
+        input_dtype=None,
+        out_dtype=None,
+        weight_qscheme=None,
+        input_qscheme=None,
+    ) -> None:
+        # --- which arithmetic: same acceptance rules as the reference constructor (:42-89)
+        if weight_dtype in FP8_ALLOWED_DTYPES and input_dtype in FP8_ALLOWED_DTYPES:
+            token_channel = input_qscheme == per_token_symmetric and weight_qscheme == per_channel_symmetric
+            tensor_tensor = input_qscheme == per_tensor_symmetric and weight_qscheme == per_tensor_symmetric
+            if not (token_channel or tensor_tensor):
+                raise ValueError(
+                    f"Invalid qscheme combination! input_qscheme: {input_qscheme}, weight_qscheme: {weight_qscheme}")
+            compute_dtype = "FP8"
+        elif weight_dtype == torch.int8 and input_dtype == torch.int8:
+            compute_dtype = "INT8"
+        else:
+            raise ValueError(f"Unsupported dtype combination! weight_dtype: {weight_dtype}, input_dtype: {input_dtype}")
+
+        # --- what the gfx950 kernels cover; anything else is reported as not implemented so
+        #     that get_qlinear keeps the float module, as the reference does on NotImplementedError
+        if not (input_qscheme == per_token_symmetric and weight_qscheme == per_channel_symmetric):
+            raise NotImplementedError(
+                "daxq implements per-token activations with per-channel weights; "
+                f"got input_qscheme={input_qscheme}, weight_qscheme={weight_qscheme}")
+        if compute_dtype == "FP8" and not (weight_dtype == input_dtype == torch.float8_e4m3fn):
+            raise NotImplementedError(
+                f"daxq implements float8_e4m3fn x float8_e4m3fn; got weight {weight_dtype}, input {input_dtype} "
+                "(pass activation_dtype=torch.float8_e4m3fn to the fp8 qconfig factory)")
+        if out_dtype not in (None, torch.bfloat16):
+            raise NotImplementedError(f"daxq kernels produce bfloat16 outputs, got out_dtype={out_dtype}")
+
+        super().__init__()
+        self.in_features = in_features
+        self.out_features = out_features
+
+        self.register_buffer(
+            "qweight", torch.empty((out_features, in_features), device=device, dtype=weight_dtype), persistent=True)
+        if bias:
+            # bf16 either way: FP8 row-wise needs it (:111-116), and out_dtype is bf16 here
+            self.bias = nn.Parameter(torch.empty(out_features, device=device, dtype=torch.bfloat16))
+        else:
+            self.register_parameter("bias", None)
+        self.register_buffer(
+            "weight_scale", torch.ones((1, out_features), device=device, dtype=torch.float32), persistent=True)
+
+        self.out_dtype = out_dtype if out_dtype is not None else torch.bfloat16
+        self.weight_dtype = weight_dtype
+        self.input_dtype = input_dtype
+        self.compute_dtype = compute_dtype
+        self.weight_qscheme = weight_qscheme
+        self.input_qscheme = input_qscheme
+        # derived, never saved: (key, K-padded byte view of qweight) for the GEMM
+        self._packed = None
+
+    # ------------------------------------------------------------------ derived views
+    @property
+    def weight(self):
+        """De-quantised weight in out_dtype, [N,K] (:139-141)."""
+        return self.qweight.to(self.out_dtype) * self.weight_scale.T.to(self.out_dtype)
+
+    def _gemm_weight(self) -> Tensor:
+        """qweight as the byte matrix [N, pad128(K)] the GEMM reads; a zero-padded copy is
+        kept only when K is not a multiple of 128, and rebuilt when qweight changes."""
+        qw = self.qweight
+        if qw.dtype == torch.float8_e4m3fn:
+            qw = qw.view(torch.uint8)
+        k = qw.shape[1]
+        kp = ops.pad_k(k)
+        if kp == k and qw.is_contiguous():
+            return qw
+        key = (self.qweight.data_ptr(), self.qweight._version, str(qw.device))
+        if self._packed is None or self._packed[0] != key:
+            buf = torch.zeros((qw.shape[0], kp), dtype=qw.dtype, device=qw.device)
+            buf[:, :k] = qw
+            self._packed = (key, buf)
+        return self._packed[1]
+
+    # ------------------------------------------------------------------ forward
+    def forward(self, input: Tensor) -> Tensor:
+        prev_dims = input.shape[:-1]
+        flat = input.view(-1, self.in_features)
+        wq = self._gemm_weight()
+        sw = self.weight_scale.view(-1)
+        if self.compute_dtype == "FP8":
+            xq, sx = ops.act_quant_e4m3(flat)
+            out = ops.linear_e4m3(xq, sx, wq, sw, self.bias)
+        else:
+            xq, sx = ops.act_quant_i8(flat)
+            out = ops.linear_i8(xq, sx, wq, sw, self.bias)
+        out = out.view(*prev_dims, self.out_features)
+        if out.dtype != self.out_dtype:
+            out = out.to(self.out_dtype)
+        return out
+
+    def extra_repr(self) -> str:
+        s = f"in_features={self.in_features}, out_features={self.out_features}"
+        if self.bias is None:
+            s += ", bias=False"
+        s += f", weight_scale={self.weight_scale}"
+        return s
+
+    # ------------------------------------------------------------------ conversion
+    @classmethod
+    @torch.no_grad()
+    def get_qlinear(cls, mod, activation_post_process, weight_post_process, reserve_float_weight):
+        """Builds the quantised module from a float ``nn.Linear`` (:240-309).
+
+        The weight statistics, the per-channel scale and the quantised weight are computed by
+        HIP kernels; a module that still lives on the CPU is staged through the current
+        ROCm device and the results are moved back to where the module was.
+        """
+        if activation_post_process is None or activation_post_process.dtype == torch.float:
+            raise ValueError("Input must be quantized!")
+        try:
+            qlinear = cls(
+                mod.in_features,
+                mod.out_features,
+                mod.bias is not None,
+                mod.weight.device,
+                weight_post_process.dtype,
+                activation_post_process.dtype,
+                mod.weight.dtype,
+                weight_post_process.qscheme,
+                activation_post_process.qscheme,
+            )
+        except NotImplementedError as e:
+            logger.warning("Quantized linear is not supported for this combination of arguments. "
+                           "Falling back to float module. Message: %s", e)
+            return mod
+
+        home = mod.weight.device
+        w = mod.weight.detach()
+        if home.type != "cuda":
+            if not torch.cuda.is_available():
+                raise RuntimeError("daxq converts weights with HIP kernels and found no ROCm device "
+                                   f"(module is on {home}); there is no CPU implementation")
+            w = w.to(torch.device("cuda", torch.cuda.current_device()))
+
+        weight_post_process.to(w.device)
+        weight_post_process(w)
+        if weight_post_process.dtype in FP8_ALLOWED_DTYPES:
+            from ..quantized.functional import quantize_to_fp8 as quantize_func
+        elif weight_post_process.dtype == torch.int8:
+            from ..quantized.functional import quantize_to_int8 as quantize_func
+        else:
+            raise NotImplementedError(f"Unsupported dtype {weight_post_process.dtype}")
+
+        weight_scale = weight_post_process.calculate_qparams()
+        if weight_scale is not None:
+            assert mod.weight.shape[0] == weight_scale.numel()
+            qweight = quantize_func(w, scale=weight_scale.reshape(-1, 1), dtype=weight_post_process.dtype)
+            qlinear.qweight = qweight.to(home)
+            qlinear.weight_scale.copy_(weight_scale.reshape(qlinear.weight_scale.shape))
+        if qlinear.bias is not None:
+            qlinear.bias.copy_(mod.bias)
+
+        if not reserve_float_weight:  # release the float parameters' memory
+            del mod.weight
+            del mod.bias
+        return qlinear
+
+    @classmethod
+    def from_float(cls, mod, reserve_float_weight=False):
+        if hasattr(mod, "weight_fake_quant"):  # QAT module carrying its own observers
+            assert hasattr(mod, "activation_post_process"), "Input QAT module must have observer attached"
+            weight_post_process = mod.weight_fake_quant
+            activation_post_process = mod.activation_post_process
+        else:
+            assert type(mod) == cls._FLOAT_MODULE, (
+                f" nnq.{cls.__name__}.from_float only works for {cls._FLOAT_MODULE.__name__} but got:{type(mod)}")
+            assert hasattr(mod, "qconfig"), "Input float module must have qconfig defined."
+            activation_post_process = mod.qconfig.activation()
+            weight_post_process = mod.qconfig.weight()
+        return cls.get_qlinear(mod, activation_post_process, weight_post_process, reserve_float_weight)

@@ -1,0 +1,133 @@
+/*
+ * daxq -- C ABI of the MI355X (gfx950) W8A8 linear that replaces the DAX dynamic
+ * quantized Linear (INT8 and FP8 OCP e4m3fn).
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer unless stated; the caller owns and
+ *     allocates all buffers, the library never allocates, never synchronises the
+ *     device and only uses the stream it is given (a hipStream_t passed as void*;
+ *     NULL is the null stream);
+ *   - matrices are row-major with an explicit leading dimension in ELEMENTS;
+ *   - return value 0 on success, a negative DAXQ_ERR_* otherwise; the text of
+ *     the last error on the calling thread is returned by daxq_last_error();
+ *   - calls on different streams may run concurrently.
+ *
+ * Reference paths cited below are relative to the DAX checkout.
+ */
+#ifndef DAXQ_H
+#define DAXQ_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define DAXQ_ABI_VERSION 1
+
+#define DAXQ_OK 0
+#define DAXQ_ERR_ARG (-1)    /* null pointer, negative size, bad enum */
+#define DAXQ_ERR_ALIGN (-2)  /* pointer / leading dimension / K not aligned as required */
+#define DAXQ_ERR_DEVICE (-3) /* current device is not gfx950 */
+#define DAXQ_ERR_LAUNCH (-4) /* the HIP runtime refused the launch */
+
+/* K granularity of the GEMM entry points: operands whose logical K is not a
+ * multiple of this are zero-padded by the producer (the quantisers below pad
+ * columns [k, ld_q) with zeros). */
+#define DAXQ_K_ALIGN 128
+
+typedef void* daxq_stream_t;
+
+int daxq_abi_version(void);
+const char* daxq_last_error(void);
+
+/* Fills in facts about `device` (CU count, max engine clock in kHz, LDS bytes per
+ * workgroup, gcnArchName) and returns DAXQ_ERR_DEVICE when it is not a gfx950.
+ * Replaces the CUDA-version guards of dax/quant/nn/dynamic/linear.py:44-57. */
+int daxq_device_info(int device, int* cu_count, int* clock_khz, int* lds_bytes, char* arch, int arch_len);
+
+/*
+ * Dynamic per-token symmetric activation quantisation, INT8.
+ * Replaces dynamic_quantize_to_int8 / _dynamic_quantize_func / quantize_to_int8
+ *   dax/quant/nn/dynamic/functional.py:181-206, :54-148
+ *   dax/quant/nn/quantized/functional.py:17-20
+ * x      bf16 [m, k], leading dimension ld_x
+ * q      int8 [m, ld_q]; columns [k, ld_q) are written as zeros
+ * scale  fp32 [m]   = f32( max( bf16_rne( f32(rowamax) / 127 ), 2^-23 ) )
+ * q[r,c] = clamp( rint( f32(x[r,c]) * (1.0f / scale[r]) ), -128, 127 )
+ */
+int daxq_act_quant_i8(const void* x, int64_t m, int64_t k, int64_t ld_x,
+                      int8_t* q, int64_t ld_q, float* scale, daxq_stream_t stream);
+
+/*
+ * Dynamic per-token symmetric activation quantisation, FP8 OCP e4m3fn.
+ * Replaces dynamic_quantize_to_fp8 / quantize_to_fp8
+ *   dax/quant/nn/dynamic/functional.py:152-177, dax/quant/nn/quantized/functional.py:11-13
+ * scale as above with 448; q = e4m3fn_rne( clamp( f32(x) / scale, -448, 448 ) ), one byte each.
+ */
+int daxq_act_quant_e4m3(const void* x, int64_t m, int64_t k, int64_t ld_x,
+                        uint8_t* q, int64_t ld_q, float* scale, daxq_stream_t stream);
+
+/*
+ * Leaf quantisers with a caller-supplied per-row scale (used once per weight at conversion).
+ * Replace quantize_to_int8 / quantize_to_fp8 with a [rows,1] scale
+ *   dax/quant/nn/quantized/functional.py:11-20, called from dax/quant/nn/dynamic/linear.py:292-296
+ * x bf16 [m, k]; scale fp32 [m]; q [m, ld_q] with columns [k, ld_q) zero.
+ */
+int daxq_quantize_rows_i8(const void* x, int64_t m, int64_t k, int64_t ld_x, const float* scale,
+                          int8_t* q, int64_t ld_q, daxq_stream_t stream);
+int daxq_quantize_rows_e4m3(const void* x, int64_t m, int64_t k, int64_t ld_x, const float* scale,
+                            uint8_t* q, int64_t ld_q, daxq_stream_t stream);
+
+/*
+ * Per-row min and max of a bf16 matrix, in fp32: the statistics of the per-channel weight observer.
+ * Replaces PerChannelMinMaxObserver.forward   dax/quant/quantization/observer.py:284-312
+ */
+int daxq_row_minmax(const void* x, int64_t m, int64_t k, int64_t ld_x,
+                    float* min_out, float* max_out, daxq_stream_t stream);
+
+/*
+ * scale[i] = max( max(-min[i], max[i]) / qmax, 2^-23 ) in fp32 (no bf16 rounding).
+ * Replaces UniformQuantizationObserverBase._calculate_qparams   dax/quant/quantization/observer.py:97-134
+ */
+int daxq_scale_from_minmax(const float* min_in, const float* max_in, int64_t n, float qmax,
+                           float* scale, daxq_stream_t stream);
+
+/*
+ * INT8 GEMM on MFMA with the fused epilogue.
+ * Replaces out_dtype(aten.mm, int32, Xq, Wq^T) and the scale / cast / bias tail
+ *   dax/quant/nn/dynamic/linear.py:214-228
+ * xq   int8 [m, k] (ld_xq), sx fp32 [m]; wq int8 [n, k] (ld_wq), sw fp32 [n];
+ * bias bf16 [n] or NULL; out bf16 [m, n] (ld_out).
+ * acc  optional int32 [m, n] (ld_acc) dump of the exact accumulators, or NULL.
+ * k must be a multiple of DAXQ_K_ALIGN; xq, wq 16-byte aligned with ld % 16 == 0.
+ *   acc[i,j] = sum_k xq[i,k] * wq[j,k]                         (exact)
+ *   out[i,j] = bf16( f32( bf16( f32_rne(acc) * sx[i] * sw[j] ) ) + f32(bias[j]) )
+ */
+int daxq_linear_i8(const int8_t* xq, int64_t ld_xq, const float* sx,
+                   const int8_t* wq, int64_t ld_wq, const float* sw,
+                   const void* bias, void* out, int64_t ld_out,
+                   int32_t* acc, int64_t ld_acc,
+                   int64_t m, int64_t n, int64_t k, daxq_stream_t stream);
+
+/*
+ * FP8 e4m3fn GEMM on MFMA (fp32 accumulate) with the fused epilogue.
+ * Replaces torch._scaled_mm(Xq, Wq^T, scale_a, scale_b, bias, out_dtype=bf16)
+ *   dax/quant/nn/dynamic/linear.py:155-173
+ *   out[i,j] = bf16( (sum_k f32(xq[i,k]) * f32(wq[j,k])) * sx[i] * sw[j] + f32(bias[j]) )
+ * acc is an optional fp32 [m, n] dump of the raw accumulators, or NULL.
+ */
+int daxq_linear_e4m3(const uint8_t* xq, int64_t ld_xq, const float* sx,
+                     const uint8_t* wq, int64_t ld_wq, const float* sw,
+                     const void* bias, void* out, int64_t ld_out,
+                     float* acc, int64_t ld_acc,
+                     int64_t m, int64_t n, int64_t k, daxq_stream_t stream);
+
+/* Selects a GEMM kernel variant for tuning and tests (0 = library default).
+ * Process-wide; not part of the reference interface. */
+int daxq_set_gemm_variant(int variant);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DAXQ_H */

@@ -1,0 +1,279 @@
+"""GPU parity of the MFMA GEMM + epilogue and of the swapped module against the oracle.
+
+INT8: quantised activations, int32 accumulators and bf16 outputs are compared bit for bit.
+FP8 : quantised activations bit for bit; outputs within 2e-2 relative L2 (the bound the task
+      states; the reference's own accumulation order is unspecified), and in practice ~1e-3.
+"""
+import numpy as np
+import pytest
+import torch
+from torch import nn
+
+from oracle import daxq_oracle as O
+from tests.util import bf16_bits, rel_l2
+
+pytestmark = pytest.mark.gpu
+
+VARIANTS = [1, 2, 4, 5]
+FP8_TOL = 2e-2
+
+
+@pytest.fixture(scope="module")
+def ops():
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    import dax_amd.ops as ops
+
+    return ops
+
+
+@pytest.fixture(autouse=True)
+def _default_variant():
+    yield
+    from dax_amd import _capi
+
+    _capi.set_gemm_variant(0)
+
+
+def dev(t):
+    return t.to("cuda") if t is not None else None
+
+
+GEMM_SHAPES = [(256, 256, 128), (300, 520, 256), (1, 8, 128), (17, 24, 384), (512, 1536, 1536), (1000, 72, 640),
+               (257, 257, 128), (4096, 1536, 1536)]
+
+
+@pytest.mark.parametrize("variant", VARIANTS)
+@pytest.mark.parametrize("m,n,k", GEMM_SHAPES)
+def test_linear_i8_bit_exact(ops, variant, m, n, k):
+    from dax_amd import _capi
+
+    _capi.set_gemm_variant(variant)
+    x, w, b = O.make_inputs(m, k, n, seed=m + n + k)
+    qw, sw = O.weight_quant_int8(w)
+    ref = O.linear_int8(x, qw, sw, b)
+    xq, sx = ops.act_quant_i8(dev(x))
+    out, acc = ops.linear_i8_acc(xq, sx, dev(qw), dev(sw.view(-1)), dev(b))
+    torch.cuda.synchronize()
+    assert torch.equal(xq[:, :k].cpu(), ref["xq"])
+    assert torch.equal(acc.cpu(), ref["acc"]), f"{(acc.cpu() != ref['acc']).sum().item()} accumulator mismatches"
+    np.testing.assert_array_equal(bf16_bits(out), bf16_bits(ref["out"]))
+    out2 = ops.linear_i8(xq, sx, dev(qw), dev(sw.view(-1)), None)
+    ref2 = O.epilogue_int8(ref["acc"], ref["sx"], sw, None)
+    np.testing.assert_array_equal(bf16_bits(out2), bf16_bits(ref2))
+
+
+@pytest.mark.parametrize("variant", VARIANTS)
+def test_linear_i8_adversarial_extremes(ops, variant):
+    from dax_amd import _capi
+
+    _capi.set_gemm_variant(variant)
+    m, n, k = 130, 264, 13824
+    xq = torch.full((m, k), -128, dtype=torch.int8)
+    xq[1::2] = 127
+    wq = torch.full((n, k), -128, dtype=torch.int8)
+    wq[::3] = 127
+    wq[5, ::2] = 1
+    sx = torch.full((m,), 2.0 ** -10)
+    sw = torch.full((n,), 2.0 ** -12)
+    out, acc = ops.linear_i8_acc(dev(xq), dev(sx), dev(wq), dev(sw), None)
+    want = O.int_mm(xq, wq)
+    assert torch.equal(acc.cpu(), want)
+    assert int(want.max()) == 128 * 128 * k
+    np.testing.assert_array_equal(bf16_bits(out), bf16_bits(O.epilogue_int8(want, sx.view(-1, 1), sw.view(1, -1), None)))
+
+
+def test_linear_i8_one_hot_layout(ops):
+    # a single non-zero in each operand lands in exactly one accumulator: catches any
+    # row/column or operand transposition inside the MFMA tiling
+    m, n, k = 300, 300, 256
+    rng = np.random.default_rng(0)
+    for _ in range(6):
+        i, j, kk = int(rng.integers(m)), int(rng.integers(n)), int(rng.integers(k))
+        xq = torch.zeros(m, k, dtype=torch.int8)
+        wq = torch.zeros(n, k, dtype=torch.int8)
+        xq[i, kk] = 3
+        wq[j, kk] = -5
+        _, acc = ops.linear_i8_acc(dev(xq), dev(torch.ones(m)), dev(wq), dev(torch.ones(n)), None)
+        acc = acc.cpu()
+        assert acc[i, j] == -15 and acc.abs().sum() == 15, (i, j, kk)
+
+
+@pytest.mark.parametrize("variant", VARIANTS)
+@pytest.mark.parametrize("m,n,k", [(256, 256, 128), (300, 520, 256), (17, 24, 384), (512, 1536, 1536)])
+def test_linear_e4m3_within_tolerance(ops, variant, m, n, k):
+    from dax_amd import _capi
+
+    _capi.set_gemm_variant(variant)
+    x, w, b = O.make_inputs(m, k, n, seed=m + n + k + 1)
+    qw, sw = O.weight_quant_e4m3(w)
+    ref = O.linear_e4m3(x, qw, sw, b)
+    xq, sx = ops.act_quant_e4m3(dev(x))
+    assert torch.equal(xq[:, :k].cpu(), ref["xq"].view(torch.uint8))
+    out, acc = ops.linear_e4m3_acc(xq, sx, dev(qw.view(torch.uint8)), dev(sw.view(-1)), dev(b))
+    acc_ref = ref["xq"].float() @ qw.float().t()
+    assert rel_l2(acc, acc_ref) < 1e-5          # fp32 accumulation, only the order differs
+    r = rel_l2(out, ref["out"])
+    assert r < FP8_TOL, r
+    assert r < 3e-3, r                          # what fp32 accumulation actually delivers
+
+
+def test_linear_rejects_unaligned_k(ops):
+    from dax_amd._capi import DaxqError
+
+    xq = torch.zeros(8, 64, dtype=torch.int8, device="cuda")
+    wq = torch.zeros(8, 64, dtype=torch.int8, device="cuda")
+    with pytest.raises(DaxqError, match="multiple of 128"):
+        ops.linear_i8(xq, torch.ones(8, device="cuda"), wq, torch.ones(8, device="cuda"), None)
+
+
+# --------------------------------------------------------------------------- the swapped module
+class ToyBlock(nn.Module):
+    def __init__(self, d=256, f=520):
+        super().__init__()
+        self.to_q = nn.Linear(d, d)
+        self.ffn = nn.Sequential(nn.Linear(d, f), nn.GELU(approximate="tanh"), nn.Linear(f, d, bias=False))
+        self.proj_out = nn.Linear(d, 64)
+
+    def forward(self, x):
+        return self.proj_out(self.ffn(self.to_q(x)))
+
+
+def _toy(seed=0):
+    torch.manual_seed(seed)
+    m = ToyBlock().bfloat16()
+    with torch.no_grad():
+        for p in m.parameters():
+            p.mul_(0.5)
+    return m
+
+
+@pytest.mark.parametrize("home", ["cuda", "cpu"])
+def test_quantize_dynamic_int8_module_matches_oracle(home):
+    from dax_amd.quant.nn.dynamic import Linear as QLinear
+    from dax_amd.quant.quantization import quantize_dynamic
+    from dax_amd.quant.quantization.qconfig import get_dynamic_int8_per_token_act_per_channel_weight_qconfig as cfg
+
+    model = _toy().to(home)
+    w = model.to_q.weight.detach().cpu().clone()
+    b = model.to_q.bias.detach().cpu().clone()
+    quantize_dynamic(model, {"": cfg(), "proj_out": None})
+    assert isinstance(model.to_q, QLinear) and isinstance(model.ffn[0], QLinear) and isinstance(model.ffn[2], QLinear)
+    assert type(model.proj_out) is nn.Linear
+    assert model.to_q.qweight.device.type == home
+    qw, sw = O.weight_quant_int8(w)
+    assert torch.equal(model.to_q.qweight.cpu(), qw)
+    assert torch.equal(model.to_q.weight_scale.cpu(), sw)
+    assert model.to_q.weight_scale.shape == (1, 256) and model.to_q.weight_scale.dtype == torch.float32
+    assert set(model.to_q.state_dict().keys()) == {"qweight", "weight_scale", "bias"}
+    assert model.ffn[2].bias is None
+    model = model.to("cuda")
+    x, _, _ = O.make_inputs(2 * 75, 256, 8, seed=2)
+    y = model.to_q(x.view(2, 75, 256).to("cuda"))
+    assert y.shape == (2, 75, 256) and y.dtype == torch.bfloat16
+    ref = O.linear_int8(x, qw, sw, b)["out"]
+    np.testing.assert_array_equal(bf16_bits(y.view(-1, 256)), bf16_bits(ref))
+    # dequantised weight property
+    assert torch.equal(model.to_q.weight.cpu(), O.dequant_weight(qw, sw))
+    # whole block runs (K=520 is not a multiple of 128: padded operands)
+    z = model(x.view(2, 75, 256).to("cuda"))
+    h = O.linear_int8(x, qw, sw, b)["out"]
+    qw1, sw1 = model.ffn[0].qweight.cpu(), model.ffn[0].weight_scale.cpu()
+    h = O.linear_int8(h, qw1, sw1, model.ffn[0].bias.detach().cpu())["out"]
+    h = torch.nn.functional.gelu(h.to("cuda"), approximate="tanh").cpu()
+    h = O.linear_int8(h, model.ffn[2].qweight.cpu(), model.ffn[2].weight_scale.cpu(), None)["out"]
+    h = torch.nn.functional.linear(h.to("cuda"), model.proj_out.weight, model.proj_out.bias)
+    np.testing.assert_array_equal(bf16_bits(z.view(-1, 64)), bf16_bits(h))
+
+
+def test_quantize_dynamic_fp8_module_matches_oracle():
+    from dax_amd.quant.nn.dynamic import Linear as QLinear
+    from dax_amd.quant.quantization import quantize_dynamic
+    from dax_amd.quant.quantization.qconfig import get_dynamic_fp8_per_token_act_per_channel_weight_qconfig as cfg
+
+    model = _toy(1).to("cuda")
+    w = model.to_q.weight.detach().cpu().clone()
+    b = model.to_q.bias.detach().cpu().clone()
+    quantize_dynamic(model, {"": cfg(activation_dtype=torch.float8_e4m3fn), "proj_out": None})
+    assert isinstance(model.to_q, QLinear) and model.to_q.compute_dtype == "FP8"
+    assert model.to_q.qweight.dtype == torch.float8_e4m3fn
+    qw, sw = O.weight_quant_e4m3(w)
+    assert torch.equal(model.to_q.qweight.cpu().view(torch.uint8), qw.view(torch.uint8))
+    assert torch.equal(model.to_q.weight_scale.cpu(), sw)
+    x, _, _ = O.make_inputs(150, 256, 8, seed=3)
+    y = model.to_q(x.to("cuda"))
+    ref = O.linear_e4m3(x, qw, sw, b)["out"]
+    assert rel_l2(y, ref) < FP8_TOL
+
+
+def test_fp8_default_e5m2_activation_keeps_float_module():
+    from dax_amd.quant.quantization import quantize_dynamic
+    from dax_amd.quant.quantization.qconfig import get_dynamic_fp8_per_token_act_per_channel_weight_qconfig as cfg
+
+    model = _toy(2).to("cuda")
+    quantize_dynamic(model, {"": cfg()})       # reference default: e5m2 activations, not built
+    assert type(model.to_q) is nn.Linear
+
+
+def test_state_dict_round_trip_and_hooks():
+    from dax_amd.quant.nn.dynamic import Linear as QLinear
+    from dax_amd.quant.qscheme import per_channel_symmetric, per_token_symmetric
+    from dax_amd.quant.quantization import quantize_dynamic
+    from dax_amd.quant.quantization.qconfig import get_dynamic_int8_per_token_act_per_channel_weight_qconfig as cfg
+
+    model = _toy(3).to("cuda")
+    calls = []
+    model.to_q.register_forward_hook(lambda mod, inp, out: calls.append("post"))
+    model.to_q.register_forward_pre_hook(lambda mod, inp: calls.append("pre"))
+    quantize_dynamic(model, {"": cfg()})
+    x = torch.randn(20, 256, device="cuda").bfloat16()
+    y = model.to_q(x)
+    assert calls == ["pre", "post"]
+    fresh = QLinear(256, 256, True, None, torch.int8, torch.int8, torch.bfloat16, per_channel_symmetric,
+                    per_token_symmetric)
+    fresh.load_state_dict(model.to_q.state_dict())
+    fresh = fresh.to("cuda")
+    assert torch.equal(fresh(x), y)
+
+
+# --------------------------------------------------------------------------- full-size properties
+@pytest.mark.parametrize("fp8", [False, True])
+def test_full_size_14b_out_proj_rows_and_checksum(ops, fp8):
+    """M=75600, K=5120, N=5120 (Wan2.1-14B 720p out-projection).  Rows are independent, so a
+    sample of rows (incl. the first / last rows of the first / last tiles) is checked against
+    the oracle exactly; the whole accumulator matrix is checked through the identity
+    sum_ij acc[i,j] = sum_k (sum_i xq[i,k]) * (sum_j wq[j,k])."""
+    m, k, n = 75600, 5120, 5120
+    x, w, b = O.make_inputs(m, k, n, seed=2)
+    xd = dev(x)
+    rows = torch.cat([torch.arange(0, 3), torch.arange(255, 258), torch.arange(m - 82, m - 78), torch.arange(m - 3, m),
+                      torch.randint(0, m, (180,), generator=torch.Generator().manual_seed(0))]).unique()
+    if fp8:
+        qw, sw = O.weight_quant_e4m3(w)
+        xq, sx = ops.act_quant_e4m3(xd)
+        out, acc = ops.linear_e4m3_acc(xq, sx, dev(qw.view(torch.uint8)), dev(sw.view(-1)), dev(b))
+        ref = O.linear_e4m3(x[rows], qw, sw, b)
+        assert torch.equal(xq[rows.to("cuda")][:, :k].cpu(), ref["xq"].view(torch.uint8))
+        assert rel_l2(out[rows.to("cuda")], ref["out"]) < FP8_TOL
+        # linearity of the fp32 accumulation in the row sums (tolerance: fp32 summation)
+        tot = acc.double().sum().item()
+        xs = xq[:, :k].view(torch.float8_e4m3fn).float().sum(0).double()
+        ws = dev(qw).float().sum(0).double()
+        want = float((xs * ws).sum().item())
+        assert abs(tot - want) <= 1e-4 * max(1.0, abs(want))
+    else:
+        qw, sw = O.weight_quant_int8(w)
+        xq, sx = ops.act_quant_i8(xd)
+        out, acc = ops.linear_i8_acc(xq, sx, dev(qw), dev(sw.view(-1)), dev(b))
+        ref = O.linear_int8(x[rows], qw, sw, b)
+        rd = rows.to("cuda")
+        assert torch.equal(xq[rd][:, :k].cpu(), ref["xq"])
+        assert torch.equal(sx[rd].cpu(), ref["sx"].view(-1))
+        assert torch.equal(acc[rd].cpu(), ref["acc"])
+        np.testing.assert_array_equal(bf16_bits(out[rd]), bf16_bits(ref["out"]))
+        tot = int(acc.sum(dtype=torch.int64).item())
+        xs = xq[:, :k].sum(0, dtype=torch.int64)
+        ws = dev(qw).sum(0, dtype=torch.int64)
+        assert tot == int((xs * ws).sum().item())
+        # idempotence: a second launch over the same operands gives the same bits
+        out2 = ops.linear_i8(xq, sx, dev(qw), dev(sw.view(-1)), dev(b))
+        assert torch.equal(out2, out)

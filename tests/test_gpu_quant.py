@@ -1,0 +1,139 @@
+"""GPU parity of the HIP quantisers against the oracle, through torch.ops.daxq -> C ABI.
+
+Integer / byte outputs and scales are compared bit for bit.
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import daxq_oracle as O
+from tests.util import ALL_POS_FINITE, FINITE_BF16, bf16_bits, from_bits
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ops():
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    import dax_amd.ops as ops
+
+    return ops
+
+
+def dev(t):
+    return t.to("cuda")
+
+
+def test_device_is_gfx950():
+    from dax_amd import _capi
+
+    info = _capi.device_info(0)
+    assert info["status"] == 0 and info["arch"].startswith("gfx950"), info
+    print("device:", info)
+
+
+SHAPES = [(64, 384), (130, 1536), (33, 5120), (17, 13824), (5, 8960), (7, 200), (3, 100), (1, 8), (2, 7),
+          (9, 18432), (4, 20480), (300, 128)]
+
+
+@pytest.mark.parametrize("m,k", SHAPES)
+def test_act_quant_i8_matches_oracle(ops, m, k):
+    x, _, _ = O.make_inputs(m, k, 8, seed=m * 7 + k)
+    if m > 2:
+        x[1] = 0                      # zero row -> scale 2^-23, all zeros
+        x[2] = 0
+        x[2, k // 2] = -3e-30         # below the eps floor
+    q, s = ops.act_quant_i8(dev(x))
+    torch.cuda.synchronize()
+    qo, so = O.act_quant_int8(x)
+    kp = ops.pad_k(k)
+    assert q.shape == (m, kp) and q.dtype == torch.int8 and s.shape == (m,)
+    np.testing.assert_array_equal(s.cpu().numpy().view(np.uint32), so.view(-1).numpy().view(np.uint32))
+    np.testing.assert_array_equal(q[:, :k].cpu().numpy(), qo.numpy())
+    assert not q[:, k:].any()         # K padding is zero
+
+
+@pytest.mark.parametrize("m,k", SHAPES)
+def test_act_quant_e4m3_matches_oracle(ops, m, k):
+    x, _, _ = O.make_inputs(m, k, 8, seed=m * 11 + k)
+    if m > 2:
+        x[1] = 0
+    q, s = ops.act_quant_e4m3(dev(x))
+    torch.cuda.synchronize()
+    qo, so = O.act_quant_e4m3(x)
+    np.testing.assert_array_equal(s.cpu().numpy().view(np.uint32), so.view(-1).numpy().view(np.uint32))
+    np.testing.assert_array_equal(q[:, :k].cpu().numpy(), qo.view(torch.uint8).numpy())
+    assert not q[:, k:].any()
+
+
+def test_act_quant_strided_rows(ops):
+    x, _, _ = O.make_inputs(40, 512, 8, seed=5)
+    big = torch.zeros(40, 640, dtype=torch.bfloat16)
+    big[:, :512] = x
+    xs = dev(big)[:, :512]            # row stride 640
+    q, s = ops.act_quant_i8(xs)
+    qo, so = O.act_quant_int8(x)
+    np.testing.assert_array_equal(q[:, :512].cpu().numpy(), qo.numpy())
+    np.testing.assert_array_equal(s.cpu().numpy(), so.view(-1).numpy())
+
+
+@pytest.mark.parametrize("fp8", [False, True])
+def test_act_scale_exhaustive_every_bf16_amax(ops, fp8):
+    # one row per amax value; the amax sits in a different column each row, negative on odd rows
+    n = ALL_POS_FINITE.size
+    x = torch.zeros(n, 64, dtype=torch.bfloat16)
+    vals = from_bits(ALL_POS_FINITE)
+    cols = torch.arange(n) % 64
+    sign = torch.where(torch.arange(n) % 2 == 1, -1.0, 1.0).bfloat16()
+    x[torch.arange(n), cols] = vals * sign
+    q, s = (ops.act_quant_e4m3 if fp8 else ops.act_quant_i8)(dev(x))
+    qo, so = (O.act_quant_e4m3 if fp8 else O.act_quant_int8)(x)
+    np.testing.assert_array_equal(s.cpu().numpy().view(np.uint32), so.view(-1).numpy().view(np.uint32))
+    qo_b = qo.view(torch.uint8).numpy() if fp8 else qo.numpy()
+    np.testing.assert_array_equal(q[:, :64].cpu().numpy(), qo_b)
+
+
+def _sampled_scales(qmax, n_act, n_f32, seed):
+    x = from_bits(ALL_POS_FINITE).view(-1, 1)
+    reach = np.unique(O.act_scale(x, qmax).view(-1).numpy())
+    rng = np.random.default_rng(seed)
+    act = np.concatenate([reach[:3], reach[-3:], rng.choice(reach, n_act, replace=False)])
+    # un-rounded fp32 scales as the weight path produces them
+    f32 = np.exp(rng.uniform(np.log(1e-6), np.log(10.0), n_f32)).astype(np.float32)
+    return np.concatenate([act, f32]).astype(np.float32)
+
+
+@pytest.mark.parametrize("fp8", [False, True])
+def test_leaf_quantiser_every_bf16_x_many_scales(ops, fp8):
+    # rows = scales, columns = every finite bf16 value: 65280 x 384 = 25 M (x, scale) pairs
+    scales = _sampled_scales(448.0 if fp8 else 127.0, 250, 128, seed=3)
+    xrow = from_bits(FINITE_BF16)
+    x = xrow.view(1, -1).expand(scales.size, -1).contiguous()
+    st = torch.from_numpy(scales)
+    fn = ops.quantize_rows_e4m3 if fp8 else ops.quantize_rows_i8
+    q = fn(dev(x), dev(st)).cpu()
+    if fp8:
+        want = O.quantize_to_fp8(x, st.view(-1, 1)).view(torch.uint8)
+    else:
+        want = O.quantize_to_int8(x, st.view(-1, 1))
+    assert torch.equal(q, want), f"{(q != want).sum().item()} mismatches"
+
+
+@pytest.mark.parametrize("qmax", [127.0, 448.0])
+def test_weight_observer_kernels(ops, qmax):
+    _, w, _ = O.make_inputs(4, 1000, 300, seed=8)
+    w[3] = 0
+    w[4, 0] = -2.0
+    w[5] = w[5].abs()                 # all-positive row: -min < 0
+    w[6] = -w[6].abs() - 0.01         # all-negative row
+    lo, hi = ops.row_minmax(dev(w))
+    lo_o, hi_o = torch.aminmax(w.float(), dim=1)
+    assert torch.equal(lo.cpu(), lo_o) and torch.equal(hi.cpu(), hi_o)
+    s = ops.scale_from_minmax(lo, hi, qmax).cpu()
+    so = O.weight_scale(w, qmax)
+    np.testing.assert_array_equal(s.numpy().view(np.uint32), so.numpy().view(np.uint32))
+
+
+def test_cpu_tensor_is_rejected_loudly(ops):
+    with pytest.raises((RuntimeError, NotImplementedError)):
+        ops.act_quant_i8(torch.zeros(4, 128, dtype=torch.bfloat16))
