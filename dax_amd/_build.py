@@ -14,7 +14,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 LIB = os.path.join(LIBDIR, "libdaxq.so")
-SOURCES = ["capi.hip", "quant_rows.hip", "gemm_w8a8.hip"]
+SOURCES = ["capi.hip", "quant_rows.hip", "gemm_w8a8.hip", "gemm_tile256.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-fast-math",

@@ -1,0 +1,62 @@
+// Types and helpers shared by the W8A8 GEMM kernels (gfx950).
+#pragma once
+
+#include "daxq_common.h"
+
+namespace daxq {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef unsigned v2u __attribute__((ext_vector_type(2)));
+
+#define DAXQ_LDS __attribute__((address_space(3)))
+#define DAXQ_GLOBAL __attribute__((address_space(1)))
+
+template <bool FP8>
+struct AccT {
+    typedef v16i type;
+};
+template <>
+struct AccT<true> {
+    typedef v16f type;
+};
+
+struct GemmArgs {
+    const uint8_t* a;  // xq [m, k]
+    const uint8_t* b;  // wq [n, k]
+    const float* sx;   // [m]
+    const float* sw;   // [n]
+    const uint16_t* bias;  // bf16 [n] or null
+    uint16_t* out;     // bf16 [m, n]
+    void* acc;         // int32 / fp32 [m, n] dump or null
+    int64_t lda, ldb, ldo, ldacc;
+    int m, n, k;
+    int tiles_m, tiles_n;
+};
+
+// s_waitcnt immediate that waits for vmcnt <= n only (gfx9 encoding: vmcnt in bits 3:0 and 15:14,
+// expcnt 6:4 and lgkmcnt 11:8 left at their maxima)
+constexpr int vmcnt_imm(int n) { return (n & 15) | ((n >> 4) << 14) | 0x0070 | 0x0f00; }
+
+__device__ __forceinline__ int swz(int row) { return (row & 7) ^ ((row >> 3) & 1); }
+
+// Maps the flat workgroup id to an output tile.  Hardware deals consecutive ids round-robin
+// over the 8 XCDs; give each XCD one contiguous range of the tile sequence, and order the
+// sequence in groups of GM tile rows so a range covers a near-square patch.
+template <int GM>
+__device__ __forceinline__ void tile_of_block(int pid, int tiles_m, int tiles_n, int& tm, int& tn) {
+    const int nt = tiles_m * tiles_n;
+    const int xcd = pid & 7, q = nt >> 3, r = nt & 7;
+    const int id = xcd * q + (xcd < r ? xcd : r) + (pid >> 3);
+    const int per_group = GM * tiles_n;
+    const int g = id / per_group;
+    const int first = g * GM;
+    const int gsz = (tiles_m - first) < GM ? (tiles_m - first) : GM;
+    const int in_g = id - g * per_group;
+    tm = first + in_g % gsz;
+    tn = in_g / gsz;
+}
+
+}  // namespace daxq

@@ -1,0 +1,331 @@
+// 256x256-tile W8A8 GEMM for gfx950: the kernel the large DiT shapes run on.
+//
+// Work decomposition
+//   workgroup  256 x 256 outputs, 4 wavefronts (one per SIMD) in a 2 x 2 grid
+//   wavefront  128 x 128 outputs = 4 x 4 MFMA 32x32 blocks, 256 accumulator registers
+//   K          128-byte slices, two LDS stages of 64 KB (A 32 KB + B 32 KB)
+// A 2 x 2 wave grid is what minimises LDS reads per MFMA for a square tile: each K slice is
+// read (2 + 2) * 256 * 128 B = 128 KB per workgroup against 128 MFMAs of 32 cycles per wave.
+//
+// Data movement
+//   HBM/L2 -> LDS   global_load_lds_dwordx4: 16 instructions per thread and slice, no VGPR
+//                   staging; the 16-byte chunk swizzle is applied to the global address
+//   LDS -> VGPR     ds_read_b128, bank-conflict free thanks to the swizzle, software
+//                   pipelined one MFMA step ahead in a second set of fragment registers
+//   one s_barrier per K slice, placed before the last MFMA step of the slice so that the
+//   MFMAs of that step cover the barrier and the first fragment reads of the next slice.
+//
+// Tiles at the M / N edge are shifted inwards (origin min(tile*256, dim-256)) instead of being
+// predicated: the overlap rows are computed twice with identical results.  Shapes with
+// M < 256 or N < 256 take the generic kernel in gemm_w8a8.hip.
+#include "gemm_common.h"
+
+namespace daxq {
+
+namespace t256 {
+constexpr int BM = 256, BN = 256, BK = 128, T = 256;
+constexpr int A_BYTES = BM * BK, STAGE = (BM + BN) * BK;
+constexpr int LOADS = (BM + BN) * BK / 16 / T;  // 16 per thread per slice
+}  // namespace t256
+
+template <bool FP8>
+struct Frag {
+    typedef v4i type;
+};
+template <>
+struct Frag<true> {
+    typedef v8i type;
+};
+
+struct Yes {
+    static constexpr bool value = true;
+};
+struct No {
+    static constexpr bool value = false;
+};
+
+// sched_group_barrier masks
+#define DAXQ_SG_MFMA 0x008
+#define DAXQ_SG_VMEM_RD 0x020
+#define DAXQ_SG_DS_RD 0x100
+
+// DUMP: also write the raw accumulators to p.acc (tests); a separate instantiation so that the
+// production kernel carries none of that code.
+template <bool FP8, bool DUMP>
+__global__ __launch_bounds__(256) void gemm_tile256_kernel(const GemmArgs p) {
+    using namespace t256;
+    typedef typename AccT<FP8>::type acc_t;
+    typedef typename Frag<FP8>::type frag_t;
+
+    extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    int tm, tn;
+    tile_of_block<8>(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn);
+    int m0 = tm * BM, n0 = tn * BN;
+    m0 = m0 + BM <= p.m ? m0 : p.m - BM;
+    n0 = n0 + BN <= p.n ? n0 : p.n - BN;
+
+    // ---- HBM -> LDS: load instruction j of a thread covers tile row j*32 + t/8, LDS chunk slot t%8.
+    //      Global address = uniform row-block base (SGPR pair) + per-lane 32-bit offset (one VGPR per
+    //      operand, advanced by 128 per slice); LDS address = uniform (M0), 64 lanes x 16 B in a row.
+    const int r8 = t >> 3, slot = t & 7;
+    const uint32_t chunk = (uint32_t)((slot ^ swz(r8)) << 4);
+    uint32_t voff_a = (uint32_t)r8 * (uint32_t)p.lda + chunk;
+    uint32_t voff_b = (uint32_t)r8 * (uint32_t)p.ldb + chunk;
+    const uint8_t* abase = p.a + (int64_t)m0 * p.lda;
+    const uint8_t* bbase = p.b + (int64_t)n0 * p.ldb;
+    const int64_t a_step = 32 * p.lda, b_step = 32 * p.ldb;
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(DAXQ_LDS uint8_t*)smem;
+    const uint32_t wave_lds = lds0 + (uint32_t)__builtin_amdgcn_readfirstlane(wave * 1024);
+
+    auto issue_a = [&](int stage, int j) {
+        __builtin_amdgcn_global_load_lds((const DAXQ_GLOBAL void*)(abase + j * a_step + voff_a),
+                                         (DAXQ_LDS void*)(uintptr_t)(wave_lds + stage * STAGE + j * 4096), 16, 0, 0);
+    };
+    auto issue_b = [&](int stage, int j) {
+        __builtin_amdgcn_global_load_lds((const DAXQ_GLOBAL void*)(bbase + j * b_step + voff_b),
+                                         (DAXQ_LDS void*)(uintptr_t)(wave_lds + stage * STAGE + A_BYTES + j * 4096), 16, 0, 0);
+    };
+    auto issue = [&](int stage) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) issue_a(stage, j);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) issue_b(stage, j);
+        voff_a += BK;
+        voff_b += BK;
+    };
+
+    // ---- LDS -> MFMA operands: lane l reads K half l/32 of row l%32 of each 32-row block
+    const int l31 = lane & 31, hi = lane >> 5;
+    const int fl = swz(l31);
+    const uint8_t* a_rd = smem + (wm * 128 + l31) * BK;
+    const uint8_t* b_rd = smem + A_BYTES + (wn * 128 + l31) * BK;
+
+    auto load_frags = [&](int stage, int ks, frag_t (&af)[4], frag_t (&bf)[4]) {
+        const uint8_t* pa = a_rd + stage * STAGE;
+        const uint8_t* pb = b_rd + stage * STAGE;
+        if constexpr (!FP8) {
+            const int xo = ((ks * 2 + hi) ^ fl) << 4;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) af[i] = *reinterpret_cast<const v4i*>(pa + i * 32 * BK + xo);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) bf[j] = *reinterpret_cast<const v4i*>(pb + j * 32 * BK + xo);
+        } else {
+            const int xo0 = ((ks * 4 + hi * 2) ^ fl) << 4, xo1 = ((ks * 4 + hi * 2 + 1) ^ fl) << 4;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                v4i lo = *reinterpret_cast<const v4i*>(pa + i * 32 * BK + xo0);
+                v4i up = *reinterpret_cast<const v4i*>(pa + i * 32 * BK + xo1);
+                af[i] = __builtin_shufflevector(lo, up, 0, 1, 2, 3, 4, 5, 6, 7);
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                v4i lo = *reinterpret_cast<const v4i*>(pb + j * 32 * BK + xo0);
+                v4i up = *reinterpret_cast<const v4i*>(pb + j * 32 * BK + xo1);
+                bf[j] = __builtin_shufflevector(lo, up, 0, 1, 2, 3, 4, 5, 6, 7);
+            }
+        }
+    };
+
+    // acc[j][i]: 32x32 block with rows = n (W rows, MFMA "A" operand) and columns = m (X rows, "B"
+    // operand), so that a lane ends up owning one output row m and runs of 4 consecutive n.
+    acc_t acc[4][4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[j][i][v] = 0;
+
+    auto mfma_step = [&](const frag_t (&af)[4], const frag_t (&bf)[4]) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                if constexpr (!FP8)
+                    acc[j][i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[j], af[i], acc[j][i], 0, 0, 0);
+                else
+                    acc[j][i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bf[j], af[i], acc[j][i], 0, 0, 0, 0, 0, 0);
+            }
+    };
+
+    const int KT = p.k / BK;
+    frag_t fa0[4], fb0[4], fa1[4], fb1[4];
+
+    // One K slice.  ISSUE: start the loads of slice kt+2 into the buffer slice kt leaves;
+    // NEXT: prefetch the first fragments of slice kt+1.  Both are compile-time so that the body is a
+    // single basic block the scheduler can interleave.
+    auto slice = [&](int cur, auto ISSUE, auto NEXT) {
+        if constexpr (!FP8) {
+            load_frags(cur, 1, fa1, fb1);
+            mfma_step(fa0, fb0);
+#pragma unroll
+            for (int g = 0; g < 8; ++g) {
+                __builtin_amdgcn_sched_group_barrier(DAXQ_SG_DS_RD, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(DAXQ_SG_MFMA, 2, 0);
+            }
+            load_frags(cur, 2, fa0, fb0);
+            mfma_step(fa1, fb1);
+#pragma unroll
+            for (int g = 0; g < 8; ++g) {
+                __builtin_amdgcn_sched_group_barrier(DAXQ_SG_DS_RD, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(DAXQ_SG_MFMA, 2, 0);
+            }
+            load_frags(cur, 3, fa1, fb1);
+            mfma_step(fa0, fb0);
+#pragma unroll
+            for (int g = 0; g < 8; ++g) {
+                __builtin_amdgcn_sched_group_barrier(DAXQ_SG_DS_RD, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(DAXQ_SG_MFMA, 2, 0);
+            }
+        } else {
+            load_frags(cur, 1, fa1, fb1);
+            mfma_step(fa0, fb0);
+#pragma unroll
+            for (int g = 0; g < 16; ++g) {
+                __builtin_amdgcn_sched_group_barrier(DAXQ_SG_DS_RD, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(DAXQ_SG_MFMA, 1, 0);
+            }
+        }
+        // slice kt+1 must have landed for every wave, and every wave must be done reading slice kt
+        __syncthreads();
+        if constexpr (ISSUE.value) issue(cur);
+        if constexpr (NEXT.value) load_frags(cur ^ 1, 0, fa0, fb0);
+        mfma_step(fa1, fb1);
+        if constexpr (ISSUE.value && NEXT.value) {
+#pragma unroll
+            for (int g = 0; g < 16; ++g) {
+                __builtin_amdgcn_sched_group_barrier(DAXQ_SG_MFMA, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(DAXQ_SG_VMEM_RD, 1, 0);
+                if (FP8 || g < 8) __builtin_amdgcn_sched_group_barrier(DAXQ_SG_DS_RD, 1, 0);
+            }
+        }
+    };
+
+    issue(0);
+    if (KT > 1) {
+        issue(1);
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm(LOADS));  // slice 0 has landed, slice 1 may be in flight
+    } else {
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+    }
+    __builtin_amdgcn_s_barrier();
+    load_frags(0, 0, fa0, fb0);
+
+    int kt = 0;
+    for (; kt + 2 < KT; ++kt) slice(kt & 1, Yes{}, Yes{});
+    if (kt + 1 < KT) {
+        slice(kt & 1, No{}, Yes{});
+        ++kt;
+    }
+    slice(kt & 1, No{}, No{});
+
+    // ---- epilogue.  In a 32x32 block a lane owns output row m = l%32 and, in registers 4q..4q+3,
+    //      the columns n = 8q + 4*(l/32) + {0..3}.  Two v_permlane32_swap per pair of q give each
+    //      lane 8 consecutive columns, stored as one 16-byte write.
+    float* s_sx = reinterpret_cast<float*>(smem);
+    float* s_sw = s_sx + 256;
+    float* s_bias = s_sw + 256;
+    s_sx[t] = p.sx[m0 + t];
+    s_sw[t] = p.sw[n0 + t];
+    s_bias[t] = p.bias ? bf16_bits_to_f32(p.bias[n0 + t]) : -0.0f;  // x + (-0.0) == x bit for bit
+    __syncthreads();
+
+    if constexpr (DUMP) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int64_t m = m0 + wm * 128 + i * 32 + l31;
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const int n = n0 + wn * 128 + j * 32 + 8 * (v >> 2) + 4 * hi + (v & 3);
+                    if constexpr (!FP8)
+                        static_cast<int32_t*>(p.acc)[m * p.ldacc + n] = acc[j][i][v];
+                    else
+                        static_cast<float*>(p.acc)[m * p.ldacc + n] = acc[j][i][v];
+                }
+            }
+    }
+
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int ml = wm * 128 + i * 32 + l31;
+        const float sxv = s_sx[ml];
+        uint16_t* orow = p.out + (int64_t)(m0 + ml) * p.ldo + n0 + wn * 128 + 8 * hi;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            uint32_t pk[4][2];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int nl = wn * 128 + j * 32 + 8 * q + 4 * hi;
+                const float4 sw4 = *reinterpret_cast<const float4*>(s_sw + nl);
+                const float4 b4 = *reinterpret_cast<const float4*>(s_bias + nl);
+                const float sws[4] = {sw4.x, sw4.y, sw4.z, sw4.w};
+                const float bs[4] = {b4.x, b4.y, b4.z, b4.w};
+                uint32_t o[4];
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    if constexpr (!FP8) {
+                        float y = (float)acc[j][i][q * 4 + r];  // v_cvt_f32_i32, round to nearest even
+                        y = y * sxv;
+                        y = y * sws[r];
+                        const uint32_t o1 = f32_to_bf16_bits(y);
+                        o[r] = f32_to_bf16_bits(bf16_bits_to_f32(o1) + bs[r]);
+                    } else {
+                        o[r] = f32_to_bf16_bits(acc[j][i][q * 4 + r] * sxv * sws[r] + bs[r]);
+                    }
+                }
+                pk[q][0] = o[0] | (o[1] << 16);
+                pk[q][1] = o[2] | (o[3] << 16);
+            }
+#pragma unroll
+            for (int qp = 0; qp < 2; ++qp) {
+                // lanes 0-31 keep their half of q=2qp and receive the upper lanes' half of it;
+                // lanes 32-63 receive the lower lanes' half of q=2qp+1 and keep their own
+                v2u s0 = __builtin_amdgcn_permlane32_swap(pk[2 * qp][0], pk[2 * qp + 1][0], false, false);
+                v2u s1 = __builtin_amdgcn_permlane32_swap(pk[2 * qp][1], pk[2 * qp + 1][1], false, false);
+                // lower lanes: (own q0 n0..3) then (upper's q0 n4..7); upper lanes: (lower's q1 n0..3) then (own q1 n4..7)
+                *reinterpret_cast<uint4*>(orow + j * 32 + 16 * qp) = make_uint4(s0.x, s1.x, s0.y, s1.y);
+            }
+        }
+    }
+}
+
+template <bool FP8, bool DUMP>
+static int launch_tile256_impl(const GemmArgs& a, hipStream_t st) {
+    using namespace t256;
+    constexpr int smem = 2 * STAGE;
+    auto kern = gemm_tile256_kernel<FP8, DUMP>;
+    static bool attr_done = false;
+    if (!attr_done) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+        if (e != hipSuccess) return fail(DAXQ_ERR_LAUNCH, "hipFuncSetAttribute(%d bytes LDS): %s", smem, hipGetErrorString(e));
+        attr_done = true;
+    }
+    const int64_t nt = (int64_t)a.tiles_m * a.tiles_n;
+    if (nt > 0x7fffffff) return fail(DAXQ_ERR_ARG, "gemm: too many tiles");
+    hipLaunchKernelGGL(kern, dim3((unsigned)nt), dim3(T), smem, st, a);
+    return check_launch("gemm_tile256");
+}
+
+template <bool FP8>
+int launch_tile256(const GemmArgs& a0, hipStream_t st) {
+    using namespace t256;
+    GemmArgs a = a0;
+    a.tiles_m = (a.m + BM - 1) / BM;
+    a.tiles_n = (a.n + BN - 1) / BN;
+    return a.acc ? launch_tile256_impl<FP8, true>(a, st) : launch_tile256_impl<FP8, false>(a, st);
+}
+
+// the kernel applies: both dimensions hold a whole tile and the 32-bit row offsets cannot overflow
+bool tile256_applies(const GemmArgs& a) {
+    return a.m >= t256::BM && a.n >= t256::BN && a.lda < (1 << 26) && a.ldb < (1 << 26);
+}
+
+template int launch_tile256<false>(const GemmArgs&, hipStream_t);
+template int launch_tile256<true>(const GemmArgs&, hipStream_t);
+
+}  // namespace daxq

@@ -17,62 +17,9 @@
 // that the ds_read_b128 of 16 consecutive rows at one K offset hits 16 different bank
 // groups.  Workgroup ids are remapped so that the tiles resident on one XCD (ids
 // congruent mod 8) form a compact patch of the output and share A/B panels in that XCD's L2.
-#include "daxq_common.h"
+#include "gemm_common.h"
 
 namespace daxq {
-
-typedef int v4i __attribute__((ext_vector_type(4)));
-typedef int v8i __attribute__((ext_vector_type(8)));
-typedef int v16i __attribute__((ext_vector_type(16)));
-typedef float v16f __attribute__((ext_vector_type(16)));
-
-#define DAXQ_LDS __attribute__((address_space(3)))
-#define DAXQ_GLOBAL __attribute__((address_space(1)))
-
-template <bool FP8>
-struct AccT {
-    typedef v16i type;
-};
-template <>
-struct AccT<true> {
-    typedef v16f type;
-};
-
-struct GemmArgs {
-    const uint8_t* a;  // xq [m, k]
-    const uint8_t* b;  // wq [n, k]
-    const float* sx;   // [m]
-    const float* sw;   // [n]
-    const uint16_t* bias;  // bf16 [n] or null
-    uint16_t* out;     // bf16 [m, n]
-    void* acc;         // int32 / fp32 [m, n] dump or null
-    int64_t lda, ldb, ldo, ldacc;
-    int m, n, k;
-    int tiles_m, tiles_n;
-};
-
-// s_waitcnt immediate that waits for vmcnt <= n only (gfx9 encoding: vmcnt in bits 3:0 and 15:14,
-// expcnt 6:4 and lgkmcnt 11:8 left at their maxima)
-constexpr int vmcnt_imm(int n) { return (n & 15) | ((n >> 4) << 14) | 0x0070 | 0x0f00; }
-
-__device__ __forceinline__ int swz(int row) { return (row & 7) ^ ((row >> 3) & 1); }
-
-// Maps the flat workgroup id to an output tile.  Hardware deals consecutive ids round-robin
-// over the 8 XCDs; give each XCD one contiguous range of the tile sequence, and order the
-// sequence in groups of GM tile rows so a range covers a near-square patch.
-template <int GM>
-__device__ __forceinline__ void tile_of_block(int pid, int tiles_m, int tiles_n, int& tm, int& tn) {
-    const int nt = tiles_m * tiles_n;
-    const int xcd = pid & 7, q = nt >> 3, r = nt & 7;
-    const int id = xcd * q + (xcd < r ? xcd : r) + (pid >> 3);
-    const int per_group = GM * tiles_n;
-    const int g = id / per_group;
-    const int first = g * GM;
-    const int gsz = (tiles_m - first) < GM ? (tiles_m - first) : GM;
-    const int in_g = id - g * per_group;
-    tm = first + in_g % gsz;
-    tn = in_g / gsz;
-}
 
 template <bool FP8, int BM, int BN, int BK, int WM, int WN, bool DIRECT>
 __global__ __launch_bounds__(WM* WN * 64) void gemm_w8a8_kernel(const GemmArgs p) {
@@ -262,6 +209,10 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_w8a8_kernel(const GemmArgs p
 
 static int g_variant = 0;
 
+template <bool FP8>
+int launch_tile256(const GemmArgs& a, hipStream_t st);
+bool tile256_applies(const GemmArgs& a);
+
 template <bool FP8, int BM, int BN, int BK, int WM, int WN, bool DIRECT>
 static int launch_cfg(const GemmArgs& a0, hipStream_t st) {
     GemmArgs a = a0;
@@ -312,12 +263,14 @@ static int launch_gemm(const void* xq, int64_t ld_xq, const float* sx, const voi
     a.k = (int)k;
     a.tiles_m = a.tiles_n = 0;
     switch (g_variant) {
-        case 0:
-        case 1: return launch_cfg<FP8, 256, 256, 128, 2, 4, false>(a, st);
+        case 0:  // library default: the 256x256 kernel when both dimensions hold a tile, else the generic one
+            if (tile256_applies(a)) return launch_tile256<FP8>(a, st);
+            return launch_cfg<FP8, 128, 128, 128, 2, 2, true>(a, st);
         case 2: return launch_cfg<FP8, 256, 256, 128, 2, 4, true>(a, st);
-        case 3: return launch_cfg<FP8, 256, 256, 128, 2, 2, true>(a, st);
-        case 4: return launch_cfg<FP8, 128, 128, 128, 2, 2, false>(a, st);
         case 5: return launch_cfg<FP8, 128, 128, 128, 2, 2, true>(a, st);
+        case 6:
+            if (!tile256_applies(a)) return fail(DAXQ_ERR_ARG, "linear: the 256x256 kernel needs m, n >= 256");
+            return launch_tile256<FP8>(a, st);
         default: return fail(DAXQ_ERR_ARG, "linear: unknown gemm variant %d", g_variant);
     }
 }
@@ -327,7 +280,7 @@ static int launch_gemm(const void* xq, int64_t ld_xq, const float* sx, const voi
 extern "C" {
 
 int daxq_set_gemm_variant(int variant) {
-    if (variant < 0 || variant > 5) return daxq::fail(DAXQ_ERR_ARG, "unknown gemm variant %d", variant);
+    if (variant != 0 && variant != 2 && variant != 5 && variant != 6) return daxq::fail(DAXQ_ERR_ARG, "unknown gemm variant %d", variant);
     daxq::g_variant = variant;
     return DAXQ_OK;
 }

@@ -14,7 +14,7 @@ from tests.util import bf16_bits, rel_l2
 
 pytestmark = pytest.mark.gpu
 
-VARIANTS = [1, 2, 4, 5]
+VARIANTS = [0, 2, 5]
 FP8_TOL = 2e-2
 
 
