@@ -58,6 +58,8 @@ def main():
     ap.add_argument("--m", type=int, default=M_TOKENS)
     ap.add_argument("--cpu-rows", type=int, default=4096)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calib-copy", action="store_true",
+                    help="also run one plain 1 GiB device copy (reference point for HBM traffic counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU; --gpus must be 1 (the path shards by token rows, "
@@ -117,6 +119,12 @@ def main():
         step(evs[s])
     torch.cuda.synchronize()
     t1 = time.perf_counter()
+
+    if args.calib_copy:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
 
     ms_per_step = (t1 - t0) * 1e3 / args.steps
     total_ops = sum(2.0 * m * n * k for _, k, n in SHAPES)

@@ -40,6 +40,9 @@ struct GemmArgs {
 // expcnt 6:4 and lgkmcnt 11:8 left at their maxima)
 constexpr int vmcnt_imm(int n) { return (n & 15) | ((n >> 4) << 14) | 0x0070 | 0x0f00; }
 
+// and-mask that turns an s_waitcnt immediate into one that also waits for lgkmcnt == 0
+constexpr int lgkmcnt0_mask() { return ~0x0f00; }
+
 __device__ __forceinline__ int swz(int row) { return (row & 7) ^ ((row >> 3) & 1); }
 
 // Maps the flat workgroup id to an output tile.  Hardware deals consecutive ids round-robin

@@ -2,18 +2,25 @@
 //
 // Work decomposition
 //   workgroup  256 x 256 outputs, 4 wavefronts (one per SIMD) in a 2 x 2 grid
-//   wavefront  128 x 128 outputs = 4 x 4 MFMA 32x32 blocks, 256 accumulator registers
-//   K          128-byte slices, two LDS stages of 64 KB (A 32 KB + B 32 KB)
+//   wavefront  128 x 128 outputs = 4 x 4 MFMA 32x32 blocks, 256 accumulator registers (AGPRs)
+//   K          128-byte slices; two 64 KB LDS buffers (A 32 KB + B 32 KB each)
 // A 2 x 2 wave grid is what minimises LDS reads per MFMA for a square tile: each K slice is
 // read (2 + 2) * 256 * 128 B = 128 KB per workgroup against 128 MFMAs of 32 cycles per wave.
+// Rows are kept as whole 128-byte lines because L2 serves a 64-byte half line at the price of
+// a full one (measured: 17 TB/s against 33 TB/s device-wide).
 //
 // Data movement
-//   HBM/L2 -> LDS   global_load_lds_dwordx4: 16 instructions per thread and slice, no VGPR
-//                   staging; the 16-byte chunk swizzle is applied to the global address
-//   LDS -> VGPR     ds_read_b128, bank-conflict free thanks to the swizzle, software
-//                   pipelined one MFMA step ahead in a second set of fragment registers
-//   one s_barrier per K slice, placed before the last MFMA step of the slice so that the
-//   MFMAs of that step cover the barrier and the first fragment reads of the next slice.
+//   HBM/L2 -> LDS   global_load_lds_dwordx4 (no VGPR staging): 16 per thread and slice.  The 16-byte
+//                   chunk c of tile row r lands in LDS at chunk slot c ^ f(r); the swizzle is applied
+//                   to the global address because the LDS side of a DMA load is fixed (64 lanes in a row)
+//   LDS -> VGPR     ds_read_b128, bank-conflict free thanks to the swizzle, read one MFMA step
+//                   ahead into a second fragment register set
+//   one s_barrier per K slice, placed before the last MFMA step of the slice; that step is cut into
+//   16 scheduling regions of one MFMA + one DMA load + one fragment read so that the loads of slice
+//   kt+2 and the first fragments of slice kt+1 are spread over its MFMAs.
+// One slice is in flight while one is computed on.  A variant that staged two slices through 128
+// VGPRs to keep two slices in flight moved data faster but could not be register-allocated by the
+// compiler without spilling, and was dropped.
 //
 // Tiles at the M / N edge are shifted inwards (origin min(tile*256, dim-256)) instead of being
 // predicated: the overlap rows are computed twice with identical results.  Shapes with
@@ -26,6 +33,7 @@ namespace t256 {
 constexpr int BM = 256, BN = 256, BK = 128, T = 256;
 constexpr int A_BYTES = BM * BK, STAGE = (BM + BN) * BK;
 constexpr int LOADS = (BM + BN) * BK / 16 / T;  // 16 per thread per slice
+constexpr int SMEM = 2 * STAGE;
 }  // namespace t256
 
 template <bool FP8>
@@ -46,185 +54,94 @@ struct No {
 
 // sched_group_barrier masks
 #define DAXQ_SG_MFMA 0x008
-#define DAXQ_SG_VMEM_RD 0x020
 #define DAXQ_SG_DS_RD 0x100
 
-// DUMP: also write the raw accumulators to p.acc (tests); a separate instantiation so that the
-// production kernel carries none of that code.
-template <bool FP8, bool DUMP>
-__global__ __launch_bounds__(256) void gemm_tile256_kernel(const GemmArgs p) {
+// per-lane constants of the LDS -> MFMA operand reads
+struct FragAddr {
+    const uint8_t* a_rd;  // row (wm*128 + l%32) of the A part of buffer 0
+    const uint8_t* b_rd;  // row (wn*128 + l%32) of the B part of buffer 0
+    int hi, fl;           // K half l/32, swizzle f(l%32)
+};
+
+template <bool FP8>
+__device__ __forceinline__ void load_frags(const FragAddr& fa, int stage, int ks, typename Frag<FP8>::type (&af)[4],
+                                           typename Frag<FP8>::type (&bf)[4]) {
     using namespace t256;
-    typedef typename AccT<FP8>::type acc_t;
-    typedef typename Frag<FP8>::type frag_t;
-
-    extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
-
-    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
-    const int wm = wave >> 1, wn = wave & 1;
-    int tm, tn;
-    tile_of_block<8>(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn);
-    int m0 = tm * BM, n0 = tn * BN;
-    m0 = m0 + BM <= p.m ? m0 : p.m - BM;
-    n0 = n0 + BN <= p.n ? n0 : p.n - BN;
-
-    // ---- HBM -> LDS: load instruction j of a thread covers tile row j*32 + t/8, LDS chunk slot t%8.
-    //      Global address = uniform row-block base (SGPR pair) + per-lane 32-bit offset (one VGPR per
-    //      operand, advanced by 128 per slice); LDS address = uniform (M0), 64 lanes x 16 B in a row.
-    const int r8 = t >> 3, slot = t & 7;
-    const uint32_t chunk = (uint32_t)((slot ^ swz(r8)) << 4);
-    uint32_t voff_a = (uint32_t)r8 * (uint32_t)p.lda + chunk;
-    uint32_t voff_b = (uint32_t)r8 * (uint32_t)p.ldb + chunk;
-    const uint8_t* abase = p.a + (int64_t)m0 * p.lda;
-    const uint8_t* bbase = p.b + (int64_t)n0 * p.ldb;
-    const int64_t a_step = 32 * p.lda, b_step = 32 * p.ldb;
-    const uint32_t lds0 = (uint32_t)(uintptr_t)(DAXQ_LDS uint8_t*)smem;
-    const uint32_t wave_lds = lds0 + (uint32_t)__builtin_amdgcn_readfirstlane(wave * 1024);
-
-    auto issue_a = [&](int stage, int j) {
-        __builtin_amdgcn_global_load_lds((const DAXQ_GLOBAL void*)(abase + j * a_step + voff_a),
-                                         (DAXQ_LDS void*)(uintptr_t)(wave_lds + stage * STAGE + j * 4096), 16, 0, 0);
-    };
-    auto issue_b = [&](int stage, int j) {
-        __builtin_amdgcn_global_load_lds((const DAXQ_GLOBAL void*)(bbase + j * b_step + voff_b),
-                                         (DAXQ_LDS void*)(uintptr_t)(wave_lds + stage * STAGE + A_BYTES + j * 4096), 16, 0, 0);
-    };
-    auto issue = [&](int stage) {
+    const uint8_t* pa = fa.a_rd + stage * STAGE;
+    const uint8_t* pb = fa.b_rd + stage * STAGE;
+    if constexpr (!FP8) {
+        const int xo = ((ks * 2 + fa.hi) ^ fa.fl) << 4;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) issue_a(stage, j);
+        for (int i = 0; i < 4; ++i) af[i] = *reinterpret_cast<const v4i*>(pa + i * 32 * BK + xo);
 #pragma unroll
-        for (int j = 0; j < 8; ++j) issue_b(stage, j);
-        voff_a += BK;
-        voff_b += BK;
-    };
-
-    // ---- LDS -> MFMA operands: lane l reads K half l/32 of row l%32 of each 32-row block
-    const int l31 = lane & 31, hi = lane >> 5;
-    const int fl = swz(l31);
-    const uint8_t* a_rd = smem + (wm * 128 + l31) * BK;
-    const uint8_t* b_rd = smem + A_BYTES + (wn * 128 + l31) * BK;
-
-    auto load_frags = [&](int stage, int ks, frag_t (&af)[4], frag_t (&bf)[4]) {
-        const uint8_t* pa = a_rd + stage * STAGE;
-        const uint8_t* pb = b_rd + stage * STAGE;
-        if constexpr (!FP8) {
-            const int xo = ((ks * 2 + hi) ^ fl) << 4;
+        for (int j = 0; j < 4; ++j) bf[j] = *reinterpret_cast<const v4i*>(pb + j * 32 * BK + xo);
+    } else {
+        const int xo0 = ((ks * 4 + fa.hi * 2) ^ fa.fl) << 4, xo1 = ((ks * 4 + fa.hi * 2 + 1) ^ fa.fl) << 4;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) af[i] = *reinterpret_cast<const v4i*>(pa + i * 32 * BK + xo);
-#pragma unroll
-            for (int j = 0; j < 4; ++j) bf[j] = *reinterpret_cast<const v4i*>(pb + j * 32 * BK + xo);
-        } else {
-            const int xo0 = ((ks * 4 + hi * 2) ^ fl) << 4, xo1 = ((ks * 4 + hi * 2 + 1) ^ fl) << 4;
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                v4i lo = *reinterpret_cast<const v4i*>(pa + i * 32 * BK + xo0);
-                v4i up = *reinterpret_cast<const v4i*>(pa + i * 32 * BK + xo1);
-                af[i] = __builtin_shufflevector(lo, up, 0, 1, 2, 3, 4, 5, 6, 7);
-            }
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                v4i lo = *reinterpret_cast<const v4i*>(pb + j * 32 * BK + xo0);
-                v4i up = *reinterpret_cast<const v4i*>(pb + j * 32 * BK + xo1);
-                bf[j] = __builtin_shufflevector(lo, up, 0, 1, 2, 3, 4, 5, 6, 7);
-            }
+        for (int i = 0; i < 4; ++i) {
+            v4i lo = *reinterpret_cast<const v4i*>(pa + i * 32 * BK + xo0);
+            v4i up = *reinterpret_cast<const v4i*>(pa + i * 32 * BK + xo1);
+            af[i] = __builtin_shufflevector(lo, up, 0, 1, 2, 3, 4, 5, 6, 7);
         }
-    };
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            v4i lo = *reinterpret_cast<const v4i*>(pb + j * 32 * BK + xo0);
+            v4i up = *reinterpret_cast<const v4i*>(pb + j * 32 * BK + xo1);
+            bf[j] = __builtin_shufflevector(lo, up, 0, 1, 2, 3, 4, 5, 6, 7);
+        }
+    }
+}
 
-    // acc[j][i]: 32x32 block with rows = n (W rows, MFMA "A" operand) and columns = m (X rows, "B"
-    // operand), so that a lane ends up owning one output row m and runs of 4 consecutive n.
-    acc_t acc[4][4];
+// one fragment of the next slice's step 0: g = 0..3 -> A block g, g = 4..7 -> B block g-4 (INT8: one
+// ds_read_b128; FP8: two)
+template <bool FP8>
+__device__ __forceinline__ void load_one_frag(const FragAddr& fa, int stage, int g, typename Frag<FP8>::type (&af)[4],
+                                              typename Frag<FP8>::type (&bf)[4]) {
+    using namespace t256;
+    const uint8_t* pr = (g < 4 ? fa.a_rd : fa.b_rd) + stage * STAGE + (g & 3) * 32 * BK;
+    if constexpr (!FP8) {
+        const int xo = (fa.hi ^ fa.fl) << 4;
+        (g < 4 ? af[g & 3] : bf[g & 3]) = *reinterpret_cast<const v4i*>(pr + xo);
+    } else {
+        const int xo0 = ((fa.hi * 2) ^ fa.fl) << 4, xo1 = ((fa.hi * 2 + 1) ^ fa.fl) << 4;
+        v4i lo = *reinterpret_cast<const v4i*>(pr + xo0);
+        v4i up = *reinterpret_cast<const v4i*>(pr + xo1);
+        (g < 4 ? af[g & 3] : bf[g & 3]) = __builtin_shufflevector(lo, up, 0, 1, 2, 3, 4, 5, 6, 7);
+    }
+}
+
+template <bool FP8>
+__device__ __forceinline__ void mfma_one(typename AccT<FP8>::type (&acc)[4][4], int g, const typename Frag<FP8>::type (&af)[4],
+                                         const typename Frag<FP8>::type (&bf)[4]) {
+    const int j = g >> 2, i = g & 3;
+    if constexpr (!FP8)
+        acc[j][i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[j], af[i], acc[j][i], 0, 0, 0);
+    else
+        acc[j][i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bf[j], af[i], acc[j][i], 0, 0, 0, 0, 0, 0);
+}
+
+// acc[j][i]: 32x32 block with rows = n (W rows, MFMA "A" operand) and columns = m (X rows, "B"
+// operand), so that a lane ends up owning one output row m and runs of 4 consecutive n.
+template <bool FP8>
+__device__ __forceinline__ void mfma_step(typename AccT<FP8>::type (&acc)[4][4], const typename Frag<FP8>::type (&af)[4],
+                                          const typename Frag<FP8>::type (&bf)[4]) {
 #pragma unroll
     for (int j = 0; j < 4; ++j)
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) acc[j][i][v] = 0;
-
-    auto mfma_step = [&](const frag_t (&af)[4], const frag_t (&bf)[4]) {
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                if constexpr (!FP8)
-                    acc[j][i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[j], af[i], acc[j][i], 0, 0, 0);
-                else
-                    acc[j][i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bf[j], af[i], acc[j][i], 0, 0, 0, 0, 0, 0);
-            }
-    };
-
-    const int KT = p.k / BK;
-    frag_t fa0[4], fb0[4], fa1[4], fb1[4];
-
-    // One K slice.  ISSUE: start the loads of slice kt+2 into the buffer slice kt leaves;
-    // NEXT: prefetch the first fragments of slice kt+1.  Both are compile-time so that the body is a
-    // single basic block the scheduler can interleave.
-    auto slice = [&](int cur, auto ISSUE, auto NEXT) {
-        if constexpr (!FP8) {
-            load_frags(cur, 1, fa1, fb1);
-            mfma_step(fa0, fb0);
-#pragma unroll
-            for (int g = 0; g < 8; ++g) {
-                __builtin_amdgcn_sched_group_barrier(DAXQ_SG_DS_RD, 1, 0);
-                __builtin_amdgcn_sched_group_barrier(DAXQ_SG_MFMA, 2, 0);
-            }
-            load_frags(cur, 2, fa0, fb0);
-            mfma_step(fa1, fb1);
-#pragma unroll
-            for (int g = 0; g < 8; ++g) {
-                __builtin_amdgcn_sched_group_barrier(DAXQ_SG_DS_RD, 1, 0);
-                __builtin_amdgcn_sched_group_barrier(DAXQ_SG_MFMA, 2, 0);
-            }
-            load_frags(cur, 3, fa1, fb1);
-            mfma_step(fa0, fb0);
-#pragma unroll
-            for (int g = 0; g < 8; ++g) {
-                __builtin_amdgcn_sched_group_barrier(DAXQ_SG_DS_RD, 1, 0);
-                __builtin_amdgcn_sched_group_barrier(DAXQ_SG_MFMA, 2, 0);
-            }
-        } else {
-            load_frags(cur, 1, fa1, fb1);
-            mfma_step(fa0, fb0);
-#pragma unroll
-            for (int g = 0; g < 16; ++g) {
-                __builtin_amdgcn_sched_group_barrier(DAXQ_SG_DS_RD, 1, 0);
-                __builtin_amdgcn_sched_group_barrier(DAXQ_SG_MFMA, 1, 0);
-            }
+        for (int i = 0; i < 4; ++i) {
+            if constexpr (!FP8)
+                acc[j][i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[j], af[i], acc[j][i], 0, 0, 0);
+            else
+                acc[j][i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bf[j], af[i], acc[j][i], 0, 0, 0, 0, 0, 0);
         }
-        // slice kt+1 must have landed for every wave, and every wave must be done reading slice kt
-        __syncthreads();
-        if constexpr (ISSUE.value) issue(cur);
-        if constexpr (NEXT.value) load_frags(cur ^ 1, 0, fa0, fb0);
-        mfma_step(fa1, fb1);
-        if constexpr (ISSUE.value && NEXT.value) {
-#pragma unroll
-            for (int g = 0; g < 16; ++g) {
-                __builtin_amdgcn_sched_group_barrier(DAXQ_SG_MFMA, 1, 0);
-                __builtin_amdgcn_sched_group_barrier(DAXQ_SG_VMEM_RD, 1, 0);
-                if (FP8 || g < 8) __builtin_amdgcn_sched_group_barrier(DAXQ_SG_DS_RD, 1, 0);
-            }
-        }
-    };
+}
 
-    issue(0);
-    if (KT > 1) {
-        issue(1);
-        __builtin_amdgcn_s_waitcnt(vmcnt_imm(LOADS));  // slice 0 has landed, slice 1 may be in flight
-    } else {
-        __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
-    }
-    __builtin_amdgcn_s_barrier();
-    load_frags(0, 0, fa0, fb0);
-
-    int kt = 0;
-    for (; kt + 2 < KT; ++kt) slice(kt & 1, Yes{}, Yes{});
-    if (kt + 1 < KT) {
-        slice(kt & 1, No{}, Yes{});
-        ++kt;
-    }
-    slice(kt & 1, No{}, No{});
-
-    // ---- epilogue.  In a 32x32 block a lane owns output row m = l%32 and, in registers 4q..4q+3,
-    //      the columns n = 8q + 4*(l/32) + {0..3}.  Two v_permlane32_swap per pair of q give each
-    //      lane 8 consecutive columns, stored as one 16-byte write.
+// Epilogue.  In a 32x32 block a lane owns output row m = l%32 and, in registers 4q..4q+3, the
+// columns n = 8q + 4*(l/32) + {0..3}.  Two v_permlane32_swap per pair of q give each lane 8
+// consecutive columns, stored as one 16-byte write.  The tile's scales and bias are staged in LDS.
+template <bool FP8, bool DUMP>
+__device__ __forceinline__ void tile256_epilogue(const GemmArgs& p, typename AccT<FP8>::type (&acc)[4][4], uint8_t* smem,
+                                                 int m0, int n0, int t, int wm, int wn, int l31, int hi) {
     float* s_sx = reinterpret_cast<float*>(smem);
     float* s_sw = s_sx + 256;
     float* s_bias = s_sw + 256;
@@ -287,27 +204,178 @@ __global__ __launch_bounds__(256) void gemm_tile256_kernel(const GemmArgs p) {
                 // lanes 32-63 receive the lower lanes' half of q=2qp+1 and keep their own
                 v2u s0 = __builtin_amdgcn_permlane32_swap(pk[2 * qp][0], pk[2 * qp + 1][0], false, false);
                 v2u s1 = __builtin_amdgcn_permlane32_swap(pk[2 * qp][1], pk[2 * qp + 1][1], false, false);
-                // lower lanes: (own q0 n0..3) then (upper's q0 n4..7); upper lanes: (lower's q1 n0..3) then (own q1 n4..7)
                 *reinterpret_cast<uint4*>(orow + j * 32 + 16 * qp) = make_uint4(s0.x, s1.x, s0.y, s1.y);
             }
         }
     }
 }
 
-template <bool FP8, bool DUMP>
+// DUMP: also write the raw accumulators to p.acc (tests); a separate instantiation so that the
+// production kernel carries none of that code.
+// EXP:  timing experiments with wrong results by construction: 1 = no HBM loads in the steady
+//       state, 2 = loads only (no LDS reads, no MFMA).
+template <bool FP8, bool DUMP, int EXP = 0>
+__global__ __launch_bounds__(256) void gemm_tile256_kernel(const GemmArgs p) {
+    using namespace t256;
+    typedef typename AccT<FP8>::type acc_t;
+    typedef typename Frag<FP8>::type frag_t;
+
+    extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    int tm, tn;
+    tile_of_block<8>(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn);
+    int m0 = tm * BM, n0 = tn * BN;
+    m0 = m0 + BM <= p.m ? m0 : p.m - BM;
+    n0 = n0 + BN <= p.n ? n0 : p.n - BN;
+
+    // ---- HBM side: load instruction j of a thread covers tile row j*32 + t/8 and LDS chunk slot t%8,
+    //      i.e. global chunk (t%8) ^ f(row).  Global address = uniform row-block base (SGPR pair) +
+    //      per-lane 32-bit offset (one VGPR per operand, advanced by 128 per slice).
+    const int r8 = t >> 3, slot = t & 7;
+    const uint32_t chunk = (uint32_t)((slot ^ swz(r8)) << 4);
+    uint32_t voff_a = (uint32_t)r8 * (uint32_t)p.lda + chunk;
+    uint32_t voff_b = (uint32_t)r8 * (uint32_t)p.ldb + chunk;
+    const uint8_t* abase = p.a + (int64_t)m0 * p.lda;
+    const uint8_t* bbase = p.b + (int64_t)n0 * p.ldb;
+    const int64_t a_step = 32 * p.lda, b_step = 32 * p.ldb;
+
+    // ---- LDS side
+    FragAddr fa;
+    const int l31 = lane & 31, hi = lane >> 5;
+    fa.hi = hi;
+    fa.fl = swz(l31);
+    fa.a_rd = smem + (wm * 128 + l31) * BK;
+    fa.b_rd = smem + A_BYTES + (wn * 128 + l31) * BK;
+
+    acc_t acc[4][4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[j][i][v] = 0;
+
+    const int KT = p.k / BK;
+    frag_t fa0[4] = {}, fb0[4] = {}, fa1[4] = {}, fb1[4] = {};
+
+    // MFMA steps 0 .. n-2 of a slice, each overlapped with the fragment reads of the next step
+    auto steps_but_last = [&](int cur) {
+        if constexpr (EXP == 2) return;
+        if constexpr (!FP8) {
+            load_frags<FP8>(fa, cur, 1, fa1, fb1);
+            mfma_step<FP8>(acc, fa0, fb0);
+#pragma unroll
+            for (int g = 0; g < 8; ++g) {
+                __builtin_amdgcn_sched_group_barrier(DAXQ_SG_DS_RD, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(DAXQ_SG_MFMA, 2, 0);
+            }
+            load_frags<FP8>(fa, cur, 2, fa0, fb0);
+            mfma_step<FP8>(acc, fa1, fb1);
+#pragma unroll
+            for (int g = 0; g < 8; ++g) {
+                __builtin_amdgcn_sched_group_barrier(DAXQ_SG_DS_RD, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(DAXQ_SG_MFMA, 2, 0);
+            }
+            load_frags<FP8>(fa, cur, 3, fa1, fb1);
+            mfma_step<FP8>(acc, fa0, fb0);
+#pragma unroll
+            for (int g = 0; g < 8; ++g) {
+                __builtin_amdgcn_sched_group_barrier(DAXQ_SG_DS_RD, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(DAXQ_SG_MFMA, 2, 0);
+            }
+        } else {
+            load_frags<FP8>(fa, cur, 1, fa1, fb1);
+            mfma_step<FP8>(acc, fa0, fb0);
+#pragma unroll
+            for (int g = 0; g < 16; ++g) {
+                __builtin_amdgcn_sched_group_barrier(DAXQ_SG_DS_RD, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(DAXQ_SG_MFMA, 1, 0);
+            }
+        }
+    };
+    auto next_frags = [&](int nxt) {
+        if constexpr (EXP != 2) load_frags<FP8>(fa, nxt, 0, fa0, fb0);
+    };
+
+    {
+        // LDS address of a DMA load is wave-uniform (M0): 64 lanes x 16 B land in a row.
+        const uint32_t lds0 = (uint32_t)(uintptr_t)(DAXQ_LDS uint8_t*)smem;
+        const uint32_t wave_lds = lds0 + (uint32_t)__builtin_amdgcn_readfirstlane(wave * 1024);
+        auto issue_one = [&](int stage, int g) {  // g = 0..7: A rows g*32.., g = 8..15: B rows (g-8)*32..
+            if constexpr (EXP == 1) return;
+            if (g < 8)
+                __builtin_amdgcn_global_load_lds((const DAXQ_GLOBAL void*)(abase + g * a_step + voff_a),
+                                                 (DAXQ_LDS void*)(uintptr_t)(wave_lds + stage * STAGE + g * 4096), 16, 0, 0);
+            else
+                __builtin_amdgcn_global_load_lds((const DAXQ_GLOBAL void*)(bbase + (g - 8) * b_step + voff_b),
+                                                 (DAXQ_LDS void*)(uintptr_t)(wave_lds + stage * STAGE + A_BYTES + (g - 8) * 4096), 16, 0, 0);
+        };
+        auto advance = [&]() {
+            voff_a += BK;
+            voff_b += BK;
+        };
+        auto issue = [&](int stage) {
+#pragma unroll
+            for (int g = 0; g < 16; ++g) issue_one(stage, g);
+            advance();
+        };
+        // One K slice.  ISSUE: start the loads of slice kt+2 into the buffer slice kt leaves; NEXT:
+        // prefetch the first fragments of slice kt+1.  Compile-time, so the body is one basic block.
+        // The last MFMA step is cut into 16 scheduling regions of one MFMA, one DMA load and (for the
+        // first 8) one fragment read each: issued as a burst, the loads back up the address unit and
+        // block the in-order instruction stream, MFMAs included, behind them.
+        auto slice = [&](int cur, auto ISSUE, auto NEXT) {
+            steps_but_last(cur);
+            // slice kt+1 has landed for every wave, and every wave is done reading slice kt
+            __builtin_amdgcn_s_waitcnt(vmcnt_imm(0) & lgkmcnt0_mask());
+            __builtin_amdgcn_s_barrier();
+#pragma unroll
+            for (int g = 0; g < 16; ++g) {
+                if constexpr (ISSUE.value) issue_one(cur, g);
+                if constexpr (NEXT.value && EXP != 2)
+                    if (g < 8) load_one_frag<FP8>(fa, cur ^ 1, g, fa0, fb0);
+                if constexpr (EXP != 2) mfma_one<FP8>(acc, g, fa1, fb1);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            if constexpr (ISSUE.value) advance();
+        };
+        issue(0);
+        if (KT > 1) {
+            issue(1);
+            __builtin_amdgcn_s_waitcnt(vmcnt_imm(LOADS));  // slice 0 has landed, slice 1 may be in flight
+        } else {
+            __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+        }
+        __builtin_amdgcn_s_barrier();
+        next_frags(0);
+        int kt = 0;
+        for (; kt + 2 < KT; ++kt) slice(kt & 1, Yes{}, Yes{});
+        if (kt + 1 < KT) {
+            slice(kt & 1, No{}, Yes{});
+            ++kt;
+        }
+        slice(kt & 1, No{}, No{});
+    }
+
+    __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+    tile256_epilogue<FP8, DUMP>(p, acc, smem, m0, n0, t, wm, wn, l31, hi);
+}
+
+template <bool FP8, bool DUMP, int EXP = 0>
 static int launch_tile256_impl(const GemmArgs& a, hipStream_t st) {
     using namespace t256;
-    constexpr int smem = 2 * STAGE;
-    auto kern = gemm_tile256_kernel<FP8, DUMP>;
+    auto kern = gemm_tile256_kernel<FP8, DUMP, EXP>;
     static bool attr_done = false;
     if (!attr_done) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, smem);
-        if (e != hipSuccess) return fail(DAXQ_ERR_LAUNCH, "hipFuncSetAttribute(%d bytes LDS): %s", smem, hipGetErrorString(e));
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, SMEM);
+        if (e != hipSuccess) return fail(DAXQ_ERR_LAUNCH, "hipFuncSetAttribute(%d bytes LDS): %s", SMEM, hipGetErrorString(e));
         attr_done = true;
     }
     const int64_t nt = (int64_t)a.tiles_m * a.tiles_n;
     if (nt > 0x7fffffff) return fail(DAXQ_ERR_ARG, "gemm: too many tiles");
-    hipLaunchKernelGGL(kern, dim3((unsigned)nt), dim3(T), smem, st, a);
+    hipLaunchKernelGGL(kern, dim3((unsigned)nt), dim3(T), SMEM, st, a);
     return check_launch("gemm_tile256");
 }
 
@@ -318,6 +386,15 @@ int launch_tile256(const GemmArgs& a0, hipStream_t st) {
     a.tiles_m = (a.m + BM - 1) / BM;
     a.tiles_n = (a.n + BN - 1) / BN;
     return a.acc ? launch_tile256_impl<FP8, true>(a, st) : launch_tile256_impl<FP8, false>(a, st);
+}
+
+// timing experiments (INT8 only): exp 1 = no HBM loads in the steady state, 2 = loads only
+int launch_tile256_experiment(const GemmArgs& a0, int exp, hipStream_t st) {
+    using namespace t256;
+    GemmArgs a = a0;
+    a.tiles_m = (a.m + BM - 1) / BM;
+    a.tiles_n = (a.n + BN - 1) / BN;
+    return exp == 1 ? launch_tile256_impl<false, false, 1>(a, st) : launch_tile256_impl<false, false, 2>(a, st);
 }
 
 // the kernel applies: both dimensions hold a whole tile and the 32-bit row offsets cannot overflow

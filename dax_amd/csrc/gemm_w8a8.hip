@@ -212,6 +212,7 @@ static int g_variant = 0;
 template <bool FP8>
 int launch_tile256(const GemmArgs& a, hipStream_t st);
 bool tile256_applies(const GemmArgs& a);
+int launch_tile256_experiment(const GemmArgs& a, int exp, hipStream_t st);
 
 template <bool FP8, int BM, int BN, int BK, int WM, int WN, bool DIRECT>
 static int launch_cfg(const GemmArgs& a0, hipStream_t st) {
@@ -271,6 +272,8 @@ static int launch_gemm(const void* xq, int64_t ld_xq, const float* sx, const voi
         case 6:
             if (!tile256_applies(a)) return fail(DAXQ_ERR_ARG, "linear: the 256x256 kernel needs m, n >= 256");
             return launch_tile256<FP8>(a, st);
+        case 101:
+        case 102: return launch_tile256_experiment(a, g_variant - 100, st);
         default: return fail(DAXQ_ERR_ARG, "linear: unknown gemm variant %d", g_variant);
     }
 }
@@ -280,7 +283,8 @@ static int launch_gemm(const void* xq, int64_t ld_xq, const float* sx, const voi
 extern "C" {
 
 int daxq_set_gemm_variant(int variant) {
-    if (variant != 0 && variant != 2 && variant != 5 && variant != 6) return daxq::fail(DAXQ_ERR_ARG, "unknown gemm variant %d", variant);
+    if (variant != 0 && variant != 2 && variant != 5 && variant != 6 && variant != 101 && variant != 102)
+        return daxq::fail(DAXQ_ERR_ARG, "unknown gemm variant %d", variant);
     daxq::g_variant = variant;
     return DAXQ_OK;
 }

@@ -1,0 +1,262 @@
+"""CPU-only checks: the C-ABI library loads and exports what include/daxq.h declares, and the host
+side of the DAX module-swap API (qscheme, qconfig resolution, swap rules, constructor validation,
+state layout, fake kernels) behaves like the reference describes.  No GPU compute is called."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+from torch import nn
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "daxq.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(daxq_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    from dax_amd import _capi
+
+    lib = ctypes.CDLL(_capi.LIB_PATH)
+    declared = _declared_symbols()
+    assert len(declared) >= 12
+    for name in declared:
+        assert hasattr(lib, name), f"{name} declared in include/daxq.h but not exported"
+    assert set(declared) == set(_capi.SIGNATURES), "binding table and header disagree"
+    assert _capi.lib().daxq_abi_version() == 1
+    assert "undefined symbol" not in _capi.last_error()
+
+
+def test_no_cpu_kernels_and_clear_errors():
+    import dax_amd.ops as ops
+
+    x = torch.zeros(4, 128, dtype=torch.bfloat16)
+    for fn in (ops.act_quant_i8, ops.act_quant_e4m3, ops.row_minmax):
+        with pytest.raises(NotImplementedError):
+            fn(x)
+    with pytest.raises(NotImplementedError):
+        ops.linear_i8(torch.zeros(4, 128, dtype=torch.int8), torch.ones(4), torch.zeros(8, 128, dtype=torch.int8),
+                      torch.ones(8), None)
+
+
+def test_fake_kernels_give_shapes_for_tracing():
+    import dax_amd.ops as ops  # noqa: F401
+
+    x = torch.empty(10, 200, dtype=torch.bfloat16, device="meta")
+    q, s = torch.ops.daxq.act_quant_i8(x)
+    assert q.shape == (10, 256) and q.dtype == torch.int8 and s.shape == (10,) and s.dtype == torch.float32
+    q8, _ = torch.ops.daxq.act_quant_e4m3(x)
+    assert q8.dtype == torch.uint8
+    w = torch.empty(24, 256, dtype=torch.int8, device="meta")
+    out = torch.ops.daxq.linear_i8(q, s, w, torch.empty(24, device="meta"), None)
+    assert out.shape == (10, 24) and out.dtype == torch.bfloat16
+    out, acc = torch.ops.daxq.linear_i8_acc(q, s, w, torch.empty(24, device="meta"), None)
+    assert acc.dtype == torch.int32 and acc.shape == (10, 24)
+    qw = torch.ops.daxq.quantize_rows_i8(x, torch.empty(10, device="meta"), True)
+    assert qw.shape == (10, 256)
+
+
+def test_get_block_size_and_reduction_params():
+    from dax_amd.quant.nn.dynamic.functional import _get_reduction_params
+    from dax_amd.quant.qscheme import (get_block_size, per_channel_symmetric, per_tensor_symmetric,
+                                       per_token_symmetric)
+
+    assert per_token_symmetric == "dax.quant.per_token_symmetric"
+    assert get_block_size((2, 3, 8), per_token_symmetric) == (1, 1, 8)
+    assert get_block_size((2, 3, 8), per_tensor_symmetric) == (2, 3, 8)
+    assert get_block_size((4, 8), per_channel_symmetric) == (4, 1)
+    with pytest.raises(ValueError):
+        get_block_size((4, 8), "nope")
+    # the worked example of the reference docstring (dynamic/functional.py:20-27)
+    assert _get_reduction_params((3, 3, 2, 10), (3, 3, 10, 10)) == ([3, 3, 5, 2, 10], [0, 1, 3, 4])
+    assert _get_reduction_params((1, 8), (5, 8)) == ([5, 8], [1])
+    with pytest.raises(AssertionError):
+        _get_reduction_params((3,), (10,))
+
+
+class Inner(nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.fc = nn.Linear(8, 8)
+        self.act = nn.ReLU()
+
+
+class Outer(nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.embed = Inner()
+        self.block = Inner()
+        self.proj_out = nn.Linear(8, 4)
+
+
+class Sub(nn.Linear):
+    pass
+
+
+class FakeQ(nn.Module):
+    """Stands in for the quantised module so the swap machinery can be exercised without a GPU."""
+    made = []
+
+    def __init__(self, src):
+        super().__init__()
+        self.src_shape = tuple(src.weight.shape)
+
+    @classmethod
+    def from_float(cls, mod, reserve_float_weight=False):
+        FakeQ.made.append(mod)
+        return cls(mod)
+
+
+def _cfg():
+    from dax_amd.quant.quantization.qconfig import get_dynamic_int8_per_token_act_per_channel_weight_qconfig
+
+    return get_dynamic_int8_per_token_act_per_channel_weight_qconfig()
+
+
+def test_qconfig_resolution_prefix_type_attr_and_inheritance():
+    from dax_amd.quant.quantization.quantize import propagate_qconfig_
+
+    m = Outer()
+    cfg, other = _cfg(), _cfg()
+    m.block.act.qconfig = other          # an existing attribute wins
+    propagate_qconfig_(m, {"": cfg, "embed": None})
+    assert m.qconfig is cfg and m.block.qconfig is cfg and m.block.fc.qconfig is cfg
+    assert m.embed.qconfig is None and m.embed.fc.qconfig is None      # the subtree inherits None
+    assert m.block.act.qconfig is other
+    m2 = Outer()
+    propagate_qconfig_(m2, {nn.Linear: cfg})                           # keyed by type
+    assert m2.qconfig is None and m2.block.fc.qconfig is cfg and m2.proj_out.qconfig is cfg
+    m3 = Outer()
+    propagate_qconfig_(m3, {"": cfg, "block.fc": None})                # dotted child name
+    assert m3.block.fc.qconfig is None and m3.embed.fc.qconfig is cfg
+    with pytest.raises(AssertionError):
+        propagate_qconfig_(Outer(), {"": object()})
+
+
+def test_swap_rules_exact_type_none_subtree_hooks_and_cleanup():
+    from dax_amd.quant.quantization import quantize_dynamic
+
+    FakeQ.made.clear()
+    m = Outer()
+    m.block.sub = Sub(8, 8)              # a subclass of nn.Linear is not swapped
+    seen = []
+    m.block.fc.register_forward_pre_hook(lambda mod, inp: seen.append("pre"))
+    m.block.fc.register_forward_hook(lambda mod, inp, out: seen.append("post"))
+    out = quantize_dynamic(m, {"": _cfg(), "embed": None, "proj_out": None}, mapping={nn.Linear: FakeQ})
+    assert out is m                                                    # in place by default
+    assert isinstance(m.block.fc, FakeQ) and m.block.fc.src_shape == (8, 8)
+    assert type(m.embed.fc) is nn.Linear and type(m.proj_out) is nn.Linear and type(m.block.sub) is Sub
+    assert len(FakeQ.made) == 1
+    assert len(m.block.fc._forward_pre_hooks) == 1 and len(m.block.fc._forward_hooks) == 1
+    assert not any(hasattr(mod, "qconfig") for mod in m.modules())     # remove_qconfig=True
+    m2 = Outer()
+    q2 = quantize_dynamic(m2, {"": _cfg()}, mapping={nn.Linear: FakeQ}, inplace=False, remove_qconfig=False)
+    assert q2 is not m2 and type(m2.block.fc) is nn.Linear and isinstance(q2.block.fc, FakeQ)
+    assert hasattr(q2.block, "qconfig")
+
+
+def test_default_mapping_and_static_entry_points():
+    from dax_amd.quant.nn.dynamic import Linear
+    from dax_amd.quant.quantization import convert, prepare
+    from dax_amd.quant.quantization.quantization_mappings import get_default_dynamic_quant_module_mappings
+
+    assert get_default_dynamic_quant_module_mappings() == {nn.Linear: Linear}
+    with pytest.raises(NotImplementedError):
+        prepare(Outer())
+    with pytest.raises(NotImplementedError):
+        convert(Outer())
+
+
+def test_linear_constructor_validation_and_state_layout():
+    from dax_amd.quant.nn.dynamic import Linear
+    from dax_amd.quant.qscheme import per_channel_symmetric as ch, per_tensor_symmetric as te, per_token_symmetric as tok
+
+    lin = Linear(256, 128, True, None, torch.int8, torch.int8, torch.bfloat16, ch, tok)
+    sd = lin.state_dict()
+    assert set(sd) == {"qweight", "weight_scale", "bias"}
+    assert sd["qweight"].shape == (128, 256) and sd["qweight"].dtype == torch.int8
+    assert sd["weight_scale"].shape == (1, 128) and sd["weight_scale"].dtype == torch.float32
+    assert sd["bias"].dtype == torch.bfloat16 and lin.compute_dtype == "INT8"
+    assert "in_features=256, out_features=128" in lin.extra_repr() and lin._FLOAT_MODULE is nn.Linear
+    f8 = Linear(64, 32, False, None, torch.float8_e4m3fn, torch.float8_e4m3fn, torch.bfloat16, ch, tok)
+    assert f8.compute_dtype == "FP8" and f8.bias is None and f8.qweight.dtype == torch.float8_e4m3fn
+    assert "bias=False" in f8.extra_repr()
+    with pytest.raises(ValueError):      # mixed int8 / fp8
+        Linear(8, 8, True, None, torch.int8, torch.float8_e4m3fn, torch.bfloat16, ch, tok)
+    with pytest.raises(ValueError):      # fp8 with a qscheme pair the reference rejects
+        Linear(8, 8, True, None, torch.float8_e4m3fn, torch.float8_e4m3fn, torch.bfloat16, ch, te)
+    with pytest.raises(ValueError):
+        Linear(8, 8, True, None, torch.float32, torch.float32, torch.bfloat16, ch, tok)
+    with pytest.raises(NotImplementedError):   # valid in the reference, not built here
+        Linear(8, 8, True, None, torch.int8, torch.int8, torch.bfloat16, te, te)
+    with pytest.raises(NotImplementedError):
+        Linear(8, 8, True, None, torch.float8_e4m3fn, torch.float8_e5m2, torch.bfloat16, ch, tok)
+    # dequantised weight property is plain tensor algebra on the stored state
+    with torch.no_grad():
+        lin.qweight.copy_(torch.randint(-127, 128, (128, 256), dtype=torch.int8))
+        lin.weight_scale.copy_(torch.rand(1, 128) * 0.01)
+    w = lin.weight
+    assert w.shape == (128, 256) and w.dtype == torch.bfloat16
+    assert torch.equal(w, lin.qweight.bfloat16() * lin.weight_scale.T.bfloat16())
+
+
+def test_from_float_asserts_and_loud_failure_without_gpu():
+    from dax_amd.quant.nn.dynamic import Linear
+
+    with pytest.raises(AssertionError):
+        Linear.from_float(Sub(8, 8))
+    with pytest.raises(AssertionError):
+        Linear.from_float(nn.Linear(8, 8))             # no qconfig
+    lin = nn.Linear(8, 8).bfloat16()
+    lin.qconfig = _cfg()
+    if not torch.cuda.is_available():
+        with pytest.raises(RuntimeError, match="no ROCm device"):
+            Linear.from_float(lin)
+    from dax_amd.quant.quantization.observer import DynamicObserverPlaceholder
+
+    with pytest.raises(ValueError, match="Input must be quantized"):
+        Linear.get_qlinear(nn.Linear(8, 8), None, _cfg().weight(), False)
+    ph = DynamicObserverPlaceholder(dtype=torch.int8, qscheme="dax.quant.per_token_symmetric", is_dynamic=True)
+    assert ph.quant_max == 127 and ph.forward(torch.zeros(1)) is None and float(ph.eps) == 2.0 ** -23
+
+
+def test_qconfig_factories_defaults():
+    from dax_amd.quant.qscheme import per_channel_symmetric, per_token_symmetric
+    from dax_amd.quant.quantization.qconfig import (get_dynamic_fp8_per_token_act_per_channel_weight_qconfig as f8,
+                                                    get_dynamic_int8_per_token_act_per_channel_weight_qconfig as i8)
+
+    c = i8()
+    a, w = c.activation(), c.weight()
+    assert a.dtype == torch.int8 and a.qscheme == per_token_symmetric and a.is_dynamic
+    assert w.dtype == torch.int8 and w.qscheme == per_channel_symmetric and w.quant_max == 127
+    c8 = f8()
+    assert c8.activation().dtype == torch.float8_e5m2         # the reference's default
+    assert c8.weight().dtype == torch.float8_e4m3fn and c8.weight().quant_max == 448.0
+    assert f8(activation_dtype=torch.float8_e4m3fn).activation().dtype == torch.float8_e4m3fn
+    assert w.calculate_qparams() is None                       # nothing observed yet
+
+
+def test_optimize_pipe_switches():
+    from dax_amd.adapters.wan import optimize_pipe
+
+    class Pipe:
+        transformer = nn.Sequential()
+
+    with pytest.raises(NotImplementedError):
+        optimize_pipe(Pipe(), sequence_parallel=True)
+    with pytest.raises(ValueError):
+        optimize_pipe(Pipe(), int8_linear=True, fp8_linear=True)
+    p = Pipe()
+    assert optimize_pipe(p) is p
+
+
+def test_bench_refuses_more_than_one_gpu():
+    import subprocess
+    import sys
+
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
+    assert r.returncode != 0 and "one GPU" in (r.stderr + r.stdout)
