@@ -21,6 +21,10 @@ if ROOT not in sys.path:
 M_TOKENS = 75600
 SHAPES = [("qkv", 5120, 15360), ("out", 5120, 5120), ("ffn_up", 5120, 13824), ("ffn_down", 13824, 5120)]
 PEAK_TOPS = {"int8": 5000.0, "fp8": 5000.0}  # MI355X dense 8-bit MFMA peak
+# Bytes that left L2 towards the fabric per GEMM launch (average of the four shapes), from the rocprofv3
+# FETCH_SIZE / WRITE_SIZE passes over this same command, scaled by the 1 GiB copy in the same run
+# (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0): (9342534 + 1456787) KiB.  Includes Infinity Cache hits.
+GEMM_TRAFFIC_BYTES = {"int8": (9342534 + 1456787) * 1024, "fp8": None}
 
 
 def cpu_baseline(dtype: str, rows: int):
@@ -48,6 +52,22 @@ def cpu_baseline(dtype: str, rows: int):
                       f"os.cpu_count()={os.cpu_count()}"}
 
 
+def mfma_sustained(dtype: str):
+    """Runs the register-only MFMA microbenchmark (dax_amd/lib/mfma_rate) as a child process: the MFMA
+    rate this board sustains under its power limit for constant / uniform-random / workload-like operands."""
+    import subprocess
+
+    exe = os.path.join(ROOT, "dax_amd", "lib", "mfma_rate")
+    if not os.path.exists(exe):
+        return None
+    r = subprocess.run([exe], capture_output=True, text=True, timeout=120)
+    if r.returncode != 0:
+        return {"error": r.stderr.strip()[-200:]}
+    want = "int8" if dtype == "int8" else "fp8_e4m3fn"
+    rows = [json.loads(line) for line in r.stdout.splitlines() if line.startswith("{")]
+    return {row["data"]: row["sustained_tops"] for row in rows if row["dtype"] == want}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -56,8 +76,9 @@ def main():
     ap.add_argument("--dtype", choices=["int8", "fp8"], default="int8")
     ap.add_argument("--variant", type=int, default=0)
     ap.add_argument("--m", type=int, default=M_TOKENS)
-    ap.add_argument("--cpu-rows", type=int, default=4096)
+    ap.add_argument("--cpu-rows", type=int, default=0, help="tokens in the CPU-baseline sample (0 = pick for 10-30 s)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-mfma-ceiling", action="store_true")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also run one plain 1 GiB device copy (reference point for HBM traffic counters)")
     args = ap.parse_args()
@@ -165,14 +186,23 @@ def main():
                    "gemm_variant": args.variant},
         "pct_of_mfma_peak": round(100.0 * value / peak, 2),
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": peak, "unit": "TFLOP/s",
-                     "frac": round(achieved / peak, 4), "traffic": None,
-                     "kernel": "gemm_w8a8_kernel (all four shapes; 8-bit ops counted as 2*M*N*K)",
+                     "frac": round(achieved / peak, 4), "traffic": GEMM_TRAFFIC_BYTES[args.dtype] if m == M_TOKENS else None,
+                     "kernel": "gemm_tile256_kernel, average launch over the four shapes; 8-bit ops counted as 2*M*N*K",
                      "gemm_ms_per_step": round(gemm_ms_sum, 4), "quant_ms_per_step": round(quant_ms_sum, 4)},
         "per_linear": per_layer,
         "device": {"arch": info["arch"], "cu_count": info["cu_count"], "max_clock_mhz": info["clock_khz"] / 1000.0},
     }
+    if not args.no_mfma_ceiling:
+        sus = mfma_sustained(args.dtype)
+        if sus and "workload" in sus:
+            res["mfma_sustained"] = {
+                "unit": "TOPS", **sus,
+                "note": "register-only MFMA loop, no memory traffic: the rate the board holds under its power limit "
+                        "depends on operand bit activity; 'workload' uses this benchmark's value distribution",
+                "gemm_frac_of_workload_ceiling": round(achieved / sus["workload"], 4)}
     if not args.no_cpu_baseline:
-        res["cpu_baseline"] = cpu_baseline(args.dtype, args.cpu_rows)
+        rows = args.cpu_rows or (49152 if not fp8 else 24576)
+        res["cpu_baseline"] = cpu_baseline(args.dtype, min(rows, m))
     print(json.dumps(res), flush=True)
 
 

@@ -14,6 +14,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 LIB = os.path.join(LIBDIR, "libdaxq.so")
+MFMA_RATE = os.path.join(LIBDIR, "mfma_rate")
 SOURCES = ["capi.hip", "quant_rows.hip", "gemm_w8a8.hip", "gemm_tile256.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
@@ -48,6 +49,13 @@ def build(verbose: bool = False) -> str:
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError(f"link failed:\n{r.stderr}")
+    # stand-alone microbenchmark behind bench.py's sustained-MFMA-rate figure
+    cmd = [HIPCC, *FLAGS, os.path.join(CSRC, "microbench", "mfma_rate.hip"), "-o", MFMA_RATE]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"hipcc failed on mfma_rate.hip:\n{r.stderr}")
     return LIB
 
 

@@ -1,0 +1,161 @@
+// Sustained MFMA issue rate of the device with no memory traffic at all, as a function of the operand
+// data.  The 8-bit MFMA datasheet peak (256 CUs x 4 SIMDs x 2048 op/clk x 2.4 GHz = 5.03 P-op/s) assumes
+// the boost clock; under the board power limit the clock the chip sustains depends on how many bits
+// toggle in the multiplier array, so the attainable ceiling for a GEMM is set by its operand statistics.
+// This program measures that ceiling: every wavefront loops over register-resident operands only.
+//
+//   mfma_rate            prints one JSON line per (dtype, data) case
+//
+// data: "constant" (all bytes 0x01), "uniform" (independent uniform random bytes), "workload"
+// (what the W8A8 linear feeds the MFMA at the benchmark's value distribution: int8 activations
+// round(N(0, 2.1)) against weights round(N(0, 32)); e4m3 activations N(0, 7.5) against weights N(0, 112)).
+#include <hip/hip_runtime.h>
+#include <math.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdlib.h>
+
+#include <random>
+#include <vector>
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+#define CHECK(x)                                                               \
+    do {                                                                       \
+        hipError_t e = (x);                                                    \
+        if (e != hipSuccess) {                                                 \
+            fprintf(stderr, "%s: %s\n", #x, hipGetErrorString(e));             \
+            return 1;                                                          \
+        }                                                                      \
+    } while (0)
+
+// a, b: 8 operand sets per lane (256 lanes per block share the pattern across blocks)
+template <bool FP8>
+__global__ __launch_bounds__(256) void spin(const int* __restrict__ a_src, const int* __restrict__ b_src, int iters, int* out) {
+    constexpr int W = FP8 ? 8 : 4;
+    int a[8][W], b[8][W];
+    for (int s = 0; s < 8; ++s)
+        for (int w = 0; w < W; ++w) {
+            a[s][w] = a_src[(s * W + w) * 256 + threadIdx.x];
+            b[s][w] = b_src[(s * W + w) * 256 + threadIdx.x];
+        }
+    if constexpr (!FP8) {
+        v16i c[8];
+        for (int s = 0; s < 8; ++s)
+            for (int v = 0; v < 16; ++v) c[s][v] = 0;
+        for (int it = 0; it < iters; ++it) {
+#pragma unroll
+            for (int s = 0; s < 8; ++s) {
+                v4i av = {a[s][0], a[s][1], a[s][2], a[s][3]};
+                const int t = (s + it) & 7;
+                v4i bv = {b[t][0], b[t][1], b[t][2], b[t][3]};
+                c[s] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av, bv, c[s], 0, 0, 0);
+            }
+        }
+        int r = 0;
+        for (int s = 0; s < 8; ++s) r += c[s][0];
+        out[blockIdx.x * 256 + threadIdx.x] = r;
+    } else {
+        v16f c[8];
+        for (int s = 0; s < 8; ++s)
+            for (int v = 0; v < 16; ++v) c[s][v] = 0;
+        for (int it = 0; it < iters; ++it) {
+#pragma unroll
+            for (int s = 0; s < 8; ++s) {
+                v8i av = {a[s][0], a[s][1], a[s][2], a[s][3], a[s][4], a[s][5], a[s][6], a[s][7]};
+                const int t = (s + it) & 7;
+                v8i bv = {b[t][0], b[t][1], b[t][2], b[t][3], b[t][4], b[t][5], b[t][6], b[t][7]};
+                c[s] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, bv, c[s], 0, 0, 0, 0, 0, 0);
+            }
+        }
+        float r = 0;
+        for (int s = 0; s < 8; ++s) r += c[s][0];
+        out[blockIdx.x * 256 + threadIdx.x] = (int)r;
+    }
+}
+
+static uint8_t to_e4m3(float v) {  // nearest e4m3fn by search over the 254 finite codes (host, tiny inputs)
+    float best = 1e30f;
+    uint8_t code = 0;
+    for (int b = 0; b < 256; ++b) {
+        const int e = (b >> 3) & 15, m = b & 7;
+        if (e == 15 && m == 7) continue;
+        float mag = e == 0 ? ldexpf((float)m, -9) : ldexpf((float)(8 + m), e - 10);
+        float val = (b & 0x80) ? -mag : mag;
+        float d = fabsf(val - v);
+        if (d < best) {
+            best = d;
+            code = (uint8_t)b;
+        }
+    }
+    return code;
+}
+
+int main() {
+    hipDeviceProp_t prop;
+    CHECK(hipGetDeviceProperties(&prop, 0));
+    const int blocks = 2 * prop.multiProcessorCount;  // two workgroups of 4 waves per CU: 2 waves per SIMD
+    int *da, *db, *dout;
+    const size_t words = 8 * 8 * 256;
+    CHECK(hipMalloc(&da, words * 4));
+    CHECK(hipMalloc(&db, words * 4));
+    CHECK(hipMalloc(&dout, (size_t)blocks * 256 * 4));
+    hipEvent_t e0, e1;
+    CHECK(hipEventCreate(&e0));
+    CHECK(hipEventCreate(&e1));
+    std::mt19937 rng(1234);
+    std::normal_distribution<float> nrm(0.0f, 1.0f);
+    const char* data_names[3] = {"constant", "uniform", "workload"};
+    for (int fp8 = 0; fp8 < 2; ++fp8) {
+        for (int data = 0; data < 3; ++data) {
+            std::vector<uint8_t> ha(words * 4), hb(words * 4);
+            for (size_t i = 0; i < ha.size(); ++i) {
+                if (data == 0) {
+                    ha[i] = hb[i] = fp8 ? 0x38 : 0x01;  // e4m3 1.0 / int8 1
+                } else if (data == 1) {
+                    ha[i] = (uint8_t)rng();
+                    hb[i] = (uint8_t)rng();
+                    if (fp8) {
+                        if ((ha[i] & 0x7f) == 0x7f) ha[i] &= 0xfe;
+                        if ((hb[i] & 0x7f) == 0x7f) hb[i] &= 0xfe;
+                    }
+                } else if (!fp8) {
+                    float x = nrm(rng) * 2.1f, w = nrm(rng) * 32.0f;
+                    ha[i] = (uint8_t)(int8_t)lrintf(fminf(fmaxf(x, -127.f), 127.f));
+                    hb[i] = (uint8_t)(int8_t)lrintf(fminf(fmaxf(w, -127.f), 127.f));
+                } else {
+                    ha[i] = to_e4m3(fminf(fmaxf(nrm(rng) * 7.5f, -448.f), 448.f));
+                    hb[i] = to_e4m3(fminf(fmaxf(nrm(rng) * 112.0f, -448.f), 448.f));
+                }
+            }
+            CHECK(hipMemcpy(da, ha.data(), ha.size(), hipMemcpyHostToDevice));
+            CHECK(hipMemcpy(db, hb.data(), hb.size(), hipMemcpyHostToDevice));
+            const int iters = fp8 ? 100000 : 200000;  // ~50-100 ms per launch
+            const double ops_per_mfma = fp8 ? 2.0 * 32 * 32 * 64 : 2.0 * 32 * 32 * 32;
+            double best = 0, last = 0;
+            for (int rep = 0; rep < 3; ++rep) {
+                CHECK(hipEventRecord(e0));
+                if (fp8)
+                    hipLaunchKernelGGL(spin<true>, dim3(blocks), dim3(256), 0, 0, da, db, iters, dout);
+                else
+                    hipLaunchKernelGGL(spin<false>, dim3(blocks), dim3(256), 0, 0, da, db, iters, dout);
+                CHECK(hipEventRecord(e1));
+                CHECK(hipEventSynchronize(e1));
+                float ms;
+                CHECK(hipEventElapsedTime(&ms, e0, e1));
+                last = (double)blocks * 4 * iters * 8 * ops_per_mfma / ms / 1e9;
+                if (last > best) best = last;
+            }
+            // the last repetition is the one at thermal / power steady state
+            printf("{\"dtype\": \"%s\", \"data\": \"%s\", \"sustained_tops\": %.1f, \"best_tops\": %.1f, "
+                   "\"implied_clock_ghz\": %.3f, \"cus\": %d}\n",
+                   fp8 ? "fp8_e4m3fn" : "int8", data_names[data], last, best,
+                   last * 1e12 / (prop.multiProcessorCount * 4.0 * 2048.0) / 1e9, prop.multiProcessorCount);
+            fflush(stdout);
+        }
+    }
+    return 0;
+}
