@@ -26,4 +26,12 @@ __device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
     return u >> 16;
 }
 
+// two f32 -> two bf16 in one word (lo = first), round to nearest even: v_cvt_pk_bf16_f32
+typedef __bf16 daxq_bf16x2 __attribute__((ext_vector_type(2)));
+typedef float daxq_f32x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pack_bf16_rne(float lo, float hi) {
+    daxq_f32x2 v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, daxq_bf16x2));
+}
+
 }  // namespace daxq

@@ -182,21 +182,25 @@ __device__ __forceinline__ void tile256_epilogue(const GemmArgs& p, typename Acc
                 const float4 b4 = *reinterpret_cast<const float4*>(s_bias + nl);
                 const float sws[4] = {sw4.x, sw4.y, sw4.z, sw4.w};
                 const float bs[4] = {b4.x, b4.y, b4.z, b4.w};
-                uint32_t o[4];
 #pragma unroll
-                for (int r = 0; r < 4; ++r) {
+                for (int h = 0; h < 2; ++h) {  // two columns at a time: v_cvt_pk_bf16_f32 rounds a pair (RNE)
+                    const int r = 2 * h;
                     if constexpr (!FP8) {
-                        float y = (float)acc[j][i][q * 4 + r];  // v_cvt_f32_i32, round to nearest even
-                        y = y * sxv;
-                        y = y * sws[r];
-                        const uint32_t o1 = f32_to_bf16_bits(y);
-                        o[r] = f32_to_bf16_bits(bf16_bits_to_f32(o1) + bs[r]);
+                        float y0 = (float)acc[j][i][q * 4 + r];  // v_cvt_f32_i32, round to nearest even
+                        float y1 = (float)acc[j][i][q * 4 + r + 1];
+                        y0 = y0 * sxv;
+                        y1 = y1 * sxv;
+                        y0 = y0 * sws[r];
+                        y1 = y1 * sws[r + 1];
+                        const uint32_t o1 = pack_bf16_rne(y0, y1);
+                        // second rounding: the bias is added to the bf16 value
+                        pk[q][h] = pack_bf16_rne(__uint_as_float(o1 << 16) + bs[r],
+                                                 __uint_as_float(o1 & 0xffff0000u) + bs[r + 1]);
                     } else {
-                        o[r] = f32_to_bf16_bits(acc[j][i][q * 4 + r] * sxv * sws[r] + bs[r]);
+                        pk[q][h] = pack_bf16_rne(acc[j][i][q * 4 + r] * sxv * sws[r] + bs[r],
+                                                 acc[j][i][q * 4 + r + 1] * sxv * sws[r + 1] + bs[r + 1]);
                     }
                 }
-                pk[q][0] = o[0] | (o[1] << 16);
-                pk[q][1] = o[2] | (o[3] << 16);
             }
 #pragma unroll
             for (int qp = 0; qp < 2; ++qp) {

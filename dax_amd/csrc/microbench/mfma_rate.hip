@@ -46,14 +46,17 @@ __global__ __launch_bounds__(256) void spin(const int* __restrict__ a_src, const
         v16i c[8];
         for (int s = 0; s < 8; ++s)
             for (int v = 0; v < 16; ++v) c[s][v] = 0;
-        for (int it = 0; it < iters; ++it) {
+        v4i av[8], bv[8];
 #pragma unroll
-            for (int s = 0; s < 8; ++s) {
-                v4i av = {a[s][0], a[s][1], a[s][2], a[s][3]};
-                const int t = (s + it) & 7;
-                v4i bv = {b[t][0], b[t][1], b[t][2], b[t][3]};
-                c[s] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av, bv, c[s], 0, 0, 0);
-            }
+        for (int s = 0; s < 8; ++s) {
+            av[s] = v4i{a[s][0], a[s][1], a[s][2], a[s][3]};
+            bv[s] = v4i{b[s][0], b[s][1], b[s][2], b[s][3]};
+        }
+        for (int it = 0; it < iters; it += 8) {
+#pragma unroll
+            for (int u = 0; u < 8; ++u)  // static operand rotation: every accumulator sees every B set
+#pragma unroll
+                for (int s = 0; s < 8; ++s) c[s] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av[s], bv[(s + u) & 7], c[s], 0, 0, 0);
         }
         int r = 0;
         for (int s = 0; s < 8; ++s) r += c[s][0];
@@ -62,14 +65,18 @@ __global__ __launch_bounds__(256) void spin(const int* __restrict__ a_src, const
         v16f c[8];
         for (int s = 0; s < 8; ++s)
             for (int v = 0; v < 16; ++v) c[s][v] = 0;
-        for (int it = 0; it < iters; ++it) {
+        v8i av[8], bv[8];
 #pragma unroll
-            for (int s = 0; s < 8; ++s) {
-                v8i av = {a[s][0], a[s][1], a[s][2], a[s][3], a[s][4], a[s][5], a[s][6], a[s][7]};
-                const int t = (s + it) & 7;
-                v8i bv = {b[t][0], b[t][1], b[t][2], b[t][3], b[t][4], b[t][5], b[t][6], b[t][7]};
-                c[s] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, bv, c[s], 0, 0, 0, 0, 0, 0);
-            }
+        for (int s = 0; s < 8; ++s) {
+            av[s] = v8i{a[s][0], a[s][1], a[s][2], a[s][3], a[s][4], a[s][5], a[s][6], a[s][7]};
+            bv[s] = v8i{b[s][0], b[s][1], b[s][2], b[s][3], b[s][4], b[s][5], b[s][6], b[s][7]};
+        }
+        for (int it = 0; it < iters; it += 8) {
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+#pragma unroll
+                for (int s = 0; s < 8; ++s)
+                    c[s] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av[s], bv[(s + u) & 7], c[s], 0, 0, 0, 0, 0, 0);
         }
         float r = 0;
         for (int s = 0; s < 8; ++s) r += c[s][0];
