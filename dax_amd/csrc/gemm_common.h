@@ -34,6 +34,7 @@ struct GemmArgs {
     int64_t lda, ldb, ldo, ldacc;
     int m, n, k;
     int tiles_m, tiles_n;
+    int gm;  // depth (in tile rows) of the groups the tile order walks through
 };
 
 // s_waitcnt immediate that waits for vmcnt <= n only (gfx9 encoding: vmcnt in bits 3:0 and 15:14,
@@ -48,8 +49,7 @@ __device__ __forceinline__ int swz(int row) { return (row & 7) ^ ((row >> 3) & 1
 // Maps the flat workgroup id to an output tile.  Hardware deals consecutive ids round-robin
 // over the 8 XCDs; give each XCD one contiguous range of the tile sequence, and order the
 // sequence in groups of GM tile rows so a range covers a near-square patch.
-template <int GM>
-__device__ __forceinline__ void tile_of_block(int pid, int tiles_m, int tiles_n, int& tm, int& tn) {
+__device__ __forceinline__ void tile_of_block(int GM, int pid, int tiles_m, int tiles_n, int& tm, int& tn) {
     const int nt = tiles_m * tiles_n;
     const int xcd = pid & 7, q = nt >> 3, r = nt & 7;
     const int id = xcd * q + (xcd < r ? xcd : r) + (pid >> 3);

@@ -229,7 +229,7 @@ __global__ __launch_bounds__(256) void gemm_tile256_kernel(const GemmArgs p) {
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
     const int wm = wave >> 1, wn = wave & 1;
     int tm, tn;
-    tile_of_block<8>(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn);
+    tile_of_block(p.gm, blockIdx.x, p.tiles_m, p.tiles_n, tm, tn);
     int m0 = tm * BM, n0 = tn * BN;
     m0 = m0 + BM <= p.m ? m0 : p.m - BM;
     n0 = n0 + BN <= p.n ? n0 : p.n - BN;
