@@ -26,12 +26,14 @@ SIGNATURES = {
     "daxq_device_info": [_INT, C.POINTER(_INT), C.POINTER(_INT), C.POINTER(_INT), C.c_char_p, _INT],
     "daxq_act_quant_i8": [_P, _I64, _I64, _I64, _P, _I64, _P, _P],
     "daxq_act_quant_e4m3": [_P, _I64, _I64, _I64, _P, _I64, _P, _P],
+    "daxq_act_quant_e5m2": [_P, _I64, _I64, _I64, _P, _I64, _P, _P],
     "daxq_quantize_rows_i8": [_P, _I64, _I64, _I64, _P, _P, _I64, _P],
     "daxq_quantize_rows_e4m3": [_P, _I64, _I64, _I64, _P, _P, _I64, _P],
     "daxq_row_minmax": [_P, _I64, _I64, _I64, _P, _P, _P],
     "daxq_scale_from_minmax": [_P, _P, _I64, _F32, _P, _P],
     "daxq_linear_i8": [_P, _I64, _P, _P, _I64, _P, _P, _P, _I64, _P, _I64, _I64, _I64, _I64, _P],
     "daxq_linear_e4m3": [_P, _I64, _P, _P, _I64, _P, _P, _P, _I64, _P, _I64, _I64, _I64, _I64, _P],
+    "daxq_linear_e5m2_e4m3": [_P, _I64, _P, _P, _I64, _P, _P, _P, _I64, _P, _I64, _I64, _I64, _I64, _P],
     "daxq_set_gemm_variant": [_INT],
 }
 

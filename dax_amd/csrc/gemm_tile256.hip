@@ -110,19 +110,20 @@ __device__ __forceinline__ void load_one_frag(const FragAddr& fa, int stage, int
     }
 }
 
-template <bool FP8>
+template <bool FP8, bool XE5>
 __device__ __forceinline__ void mfma_one(typename AccT<FP8>::type (&acc)[4][4], int g, const typename Frag<FP8>::type (&af)[4],
                                          const typename Frag<FP8>::type (&bf)[4]) {
     const int j = g >> 2, i = g & 3;
     if constexpr (!FP8)
         acc[j][i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[j], af[i], acc[j][i], 0, 0, 0);
     else
-        acc[j][i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bf[j], af[i], acc[j][i], 0, 0, 0, 0, 0, 0);
+        acc[j][i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bf[j], af[i], acc[j][i], 0, XE5 ? 1 : 0, 0, 0, 0, 0);
 }
 
 // acc[j][i]: 32x32 block with rows = n (W rows, MFMA "A" operand) and columns = m (X rows, "B"
 // operand), so that a lane ends up owning one output row m and runs of 4 consecutive n.
-template <bool FP8>
+// XE5: the activation bytes are e5m2 instead of e4m3fn (format select of the MFMA "B" operand).
+template <bool FP8, bool XE5>
 __device__ __forceinline__ void mfma_step(typename AccT<FP8>::type (&acc)[4][4], const typename Frag<FP8>::type (&af)[4],
                                           const typename Frag<FP8>::type (&bf)[4]) {
 #pragma unroll
@@ -132,7 +133,7 @@ __device__ __forceinline__ void mfma_step(typename AccT<FP8>::type (&acc)[4][4],
             if constexpr (!FP8)
                 acc[j][i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[j], af[i], acc[j][i], 0, 0, 0);
             else
-                acc[j][i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bf[j], af[i], acc[j][i], 0, 0, 0, 0, 0, 0);
+                acc[j][i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bf[j], af[i], acc[j][i], 0, XE5 ? 1 : 0, 0, 0, 0, 0);
         }
 }
 
@@ -218,7 +219,7 @@ __device__ __forceinline__ void tile256_epilogue(const GemmArgs& p, typename Acc
 // production kernel carries none of that code.
 // EXP:  timing experiments with wrong results by construction: 1 = no HBM loads in the steady
 //       state, 2 = loads only (no LDS reads, no MFMA).
-template <bool FP8, bool DUMP, int EXP = 0>
+template <bool FP8, bool DUMP, int EXP = 0, bool XE5 = false>
 __global__ __launch_bounds__(256) void gemm_tile256_kernel(const GemmArgs p) {
     using namespace t256;
     typedef typename AccT<FP8>::type acc_t;
@@ -269,21 +270,21 @@ __global__ __launch_bounds__(256) void gemm_tile256_kernel(const GemmArgs p) {
         if constexpr (EXP == 2) return;
         if constexpr (!FP8) {
             load_frags<FP8>(fa, cur, 1, fa1, fb1);
-            mfma_step<FP8>(acc, fa0, fb0);
+            mfma_step<FP8, XE5>(acc, fa0, fb0);
 #pragma unroll
             for (int g = 0; g < 8; ++g) {
                 __builtin_amdgcn_sched_group_barrier(DAXQ_SG_DS_RD, 1, 0);
                 __builtin_amdgcn_sched_group_barrier(DAXQ_SG_MFMA, 2, 0);
             }
             load_frags<FP8>(fa, cur, 2, fa0, fb0);
-            mfma_step<FP8>(acc, fa1, fb1);
+            mfma_step<FP8, XE5>(acc, fa1, fb1);
 #pragma unroll
             for (int g = 0; g < 8; ++g) {
                 __builtin_amdgcn_sched_group_barrier(DAXQ_SG_DS_RD, 1, 0);
                 __builtin_amdgcn_sched_group_barrier(DAXQ_SG_MFMA, 2, 0);
             }
             load_frags<FP8>(fa, cur, 3, fa1, fb1);
-            mfma_step<FP8>(acc, fa0, fb0);
+            mfma_step<FP8, XE5>(acc, fa0, fb0);
 #pragma unroll
             for (int g = 0; g < 8; ++g) {
                 __builtin_amdgcn_sched_group_barrier(DAXQ_SG_DS_RD, 1, 0);
@@ -291,7 +292,7 @@ __global__ __launch_bounds__(256) void gemm_tile256_kernel(const GemmArgs p) {
             }
         } else {
             load_frags<FP8>(fa, cur, 1, fa1, fb1);
-            mfma_step<FP8>(acc, fa0, fb0);
+            mfma_step<FP8, XE5>(acc, fa0, fb0);
 #pragma unroll
             for (int g = 0; g < 16; ++g) {
                 __builtin_amdgcn_sched_group_barrier(DAXQ_SG_DS_RD, 1, 0);
@@ -340,7 +341,7 @@ __global__ __launch_bounds__(256) void gemm_tile256_kernel(const GemmArgs p) {
                 if constexpr (ISSUE.value) issue_one(cur, g);
                 if constexpr (NEXT.value && EXP != 2)
                     if (g < 8) load_one_frag<FP8>(fa, cur ^ 1, g, fa0, fb0);
-                if constexpr (EXP != 2) mfma_one<FP8>(acc, g, fa1, fb1);
+                if constexpr (EXP != 2) mfma_one<FP8, XE5>(acc, g, fa1, fb1);
                 __builtin_amdgcn_sched_barrier(0);
             }
             if constexpr (ISSUE.value) advance();
@@ -367,10 +368,10 @@ __global__ __launch_bounds__(256) void gemm_tile256_kernel(const GemmArgs p) {
     tile256_epilogue<FP8, DUMP>(p, acc, smem, m0, n0, t, wm, wn, l31, hi);
 }
 
-template <bool FP8, bool DUMP, int EXP = 0>
+template <bool FP8, bool DUMP, int EXP = 0, bool XE5 = false>
 static int launch_tile256_impl(const GemmArgs& a, hipStream_t st) {
     using namespace t256;
-    auto kern = gemm_tile256_kernel<FP8, DUMP, EXP>;
+    auto kern = gemm_tile256_kernel<FP8, DUMP, EXP, XE5>;
     static bool attr_done = false;
     if (!attr_done) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, SMEM);
@@ -384,11 +385,15 @@ static int launch_tile256_impl(const GemmArgs& a, hipStream_t st) {
 }
 
 template <bool FP8>
-int launch_tile256(const GemmArgs& a0, hipStream_t st) {
+int launch_tile256(const GemmArgs& a0, bool x_e5m2, hipStream_t st) {
     using namespace t256;
     GemmArgs a = a0;
     a.tiles_m = (a.m + BM - 1) / BM;
     a.tiles_n = (a.n + BN - 1) / BN;
+    if constexpr (FP8) {
+        if (x_e5m2)
+            return a.acc ? launch_tile256_impl<true, true, 0, true>(a, st) : launch_tile256_impl<true, false, 0, true>(a, st);
+    }
     return a.acc ? launch_tile256_impl<FP8, true>(a, st) : launch_tile256_impl<FP8, false>(a, st);
 }
 
@@ -406,7 +411,7 @@ bool tile256_applies(const GemmArgs& a) {
     return a.m >= t256::BM && a.n >= t256::BN && a.lda < (1 << 26) && a.ldb < (1 << 26);
 }
 
-template int launch_tile256<false>(const GemmArgs&, hipStream_t);
-template int launch_tile256<true>(const GemmArgs&, hipStream_t);
+template int launch_tile256<false>(const GemmArgs&, bool, hipStream_t);
+template int launch_tile256<true>(const GemmArgs&, bool, hipStream_t);
 
 }  // namespace daxq

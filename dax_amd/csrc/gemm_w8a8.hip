@@ -21,7 +21,8 @@
 
 namespace daxq {
 
-template <bool FP8, int BM, int BN, int BK, int WM, int WN, bool DIRECT>
+// XE5: the activation bytes (MFMA "A" operand here) are e5m2 instead of e4m3fn
+template <bool FP8, int BM, int BN, int BK, int WM, int WN, bool DIRECT, bool XE5 = false>
 __global__ __launch_bounds__(WM* WN * 64) void gemm_w8a8_kernel(const GemmArgs p) {
     constexpr int T = WM * WN * 64;
     constexpr int TM = BM / WM, TN = BN / WN;  // wave tile
@@ -117,7 +118,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_w8a8_kernel(const GemmArgs p
                 for (int i = 0; i < MB; ++i)
 #pragma unroll
                     for (int j = 0; j < NB; ++j)
-                        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(af[i], bf[j], acc[i][j], 0, 0, 0, 0, 0, 0);
+                        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(af[i], bf[j], acc[i][j], XE5 ? 1 : 0, 0, 0, 0, 0, 0);
             }
         }
     };
@@ -211,17 +212,17 @@ static int g_variant = 0;
 static int g_gm = 8;
 
 template <bool FP8>
-int launch_tile256(const GemmArgs& a, hipStream_t st);
+int launch_tile256(const GemmArgs& a, bool x_e5m2, hipStream_t st);
 bool tile256_applies(const GemmArgs& a);
 int launch_tile256_experiment(const GemmArgs& a, int exp, hipStream_t st);
 
-template <bool FP8, int BM, int BN, int BK, int WM, int WN, bool DIRECT>
+template <bool FP8, int BM, int BN, int BK, int WM, int WN, bool DIRECT, bool XE5 = false>
 static int launch_cfg(const GemmArgs& a0, hipStream_t st) {
     GemmArgs a = a0;
     a.tiles_m = (a.m + BM - 1) / BM;
     a.tiles_n = (a.n + BN - 1) / BN;
     constexpr int smem = 2 * (BM + BN) * BK;
-    auto kern = gemm_w8a8_kernel<FP8, BM, BN, BK, WM, WN, DIRECT>;
+    auto kern = gemm_w8a8_kernel<FP8, BM, BN, BK, WM, WN, DIRECT, XE5>;
     static bool attr_done = false;  // per instantiation; benign if two threads race to set the same value
     if (!attr_done) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, smem);
@@ -237,7 +238,7 @@ static int launch_cfg(const GemmArgs& a0, hipStream_t st) {
 template <bool FP8>
 static int launch_gemm(const void* xq, int64_t ld_xq, const float* sx, const void* wq, int64_t ld_wq, const float* sw,
                        const void* bias, void* out, int64_t ld_out, void* acc, int64_t ld_acc, int64_t m, int64_t n,
-                       int64_t k, hipStream_t st) {
+                       int64_t k, hipStream_t st, bool x_e5m2 = false) {
     if (m < 0 || n < 0 || k <= 0 || ld_xq < k || ld_wq < k || ld_out < n || (acc && ld_acc < n))
         return fail(DAXQ_ERR_ARG, "linear: bad shape m=%lld n=%lld k=%lld", (long long)m, (long long)n, (long long)k);
     if (m == 0 || n == 0) return DAXQ_OK;
@@ -266,14 +267,28 @@ static int launch_gemm(const void* xq, int64_t ld_xq, const float* sx, const voi
     a.tiles_m = a.tiles_n = 0;
     a.gm = g_gm;
     switch (g_variant) {
-        case 0:  // library default: the 256x256 kernel when both dimensions hold a tile, else the generic one
-            if (tile256_applies(a)) return launch_tile256<FP8>(a, st);
+        case 0: {
+            // library default: the 256x256 kernel once its tiles fill at least half of the 256 CUs,
+            // otherwise 128x128 tiles (4x as many workgroups; measured cross-over between M = 1024
+            // and M = 2048 at N = K = 5120)
+            const int64_t tiles256 = ((m + 255) / 256) * ((n + 255) / 256);
+            if (tile256_applies(a) && tiles256 >= 128) return launch_tile256<FP8>(a, x_e5m2, st);
+            if constexpr (FP8) {
+                if (x_e5m2) return launch_cfg<true, 128, 128, 128, 2, 2, true, true>(a, st);
+            }
             return launch_cfg<FP8, 128, 128, 128, 2, 2, true>(a, st);
-        case 2: return launch_cfg<FP8, 256, 256, 128, 2, 4, true>(a, st);
-        case 5: return launch_cfg<FP8, 128, 128, 128, 2, 2, true>(a, st);
+        }
+        case 2:
+            if (x_e5m2) return fail(DAXQ_ERR_ARG, "linear: gemm variant 2 has no e5m2 form");
+            return launch_cfg<FP8, 256, 256, 128, 2, 4, true>(a, st);
+        case 5:
+            if constexpr (FP8) {
+                if (x_e5m2) return launch_cfg<true, 128, 128, 128, 2, 2, true, true>(a, st);
+            }
+            return launch_cfg<FP8, 128, 128, 128, 2, 2, true>(a, st);
         case 6:
             if (!tile256_applies(a)) return fail(DAXQ_ERR_ARG, "linear: the 256x256 kernel needs m, n >= 256");
-            return launch_tile256<FP8>(a, st);
+            return launch_tile256<FP8>(a, x_e5m2, st);
         case 101:
         case 102: return launch_tile256_experiment(a, g_variant - 100, st);
         default: return fail(DAXQ_ERR_ARG, "linear: unknown gemm variant %d", g_variant);
@@ -307,6 +322,14 @@ int daxq_linear_e4m3(const uint8_t* xq, int64_t ld_xq, const float* sx, const ui
                      int64_t m, int64_t n, int64_t k, daxq_stream_t stream) {
     return daxq::launch_gemm<true>(xq, ld_xq, sx, wq, ld_wq, sw, bias, out, ld_out, acc, ld_acc, m, n, k,
                                    (hipStream_t)stream);
+}
+
+
+int daxq_linear_e5m2_e4m3(const uint8_t* xq, int64_t ld_xq, const float* sx, const uint8_t* wq, int64_t ld_wq,
+                          const float* sw, const void* bias, void* out, int64_t ld_out, float* acc, int64_t ld_acc,
+                          int64_t m, int64_t n, int64_t k, daxq_stream_t stream) {
+    return daxq::launch_gemm<true>(xq, ld_xq, sx, wq, ld_wq, sw, bias, out, ld_out, acc, ld_acc, m, n, k,
+                                   (hipStream_t)stream, true);
 }
 
 }  // extern "C"

@@ -8,6 +8,7 @@
 // The element rule is the leaf quantiser of dax/quant/nn/quantized/functional.py:11-20:
 //   int8:  clamp(rint(f32(x) * (1.0f / s)), -128, 127)      reciprocal-multiply
 //   e4m3:  e4m3fn_rne(clamp(f32(x) / s, -448, 448))         true division
+//   e5m2:  e5m2_rne(clamp(f32(x) / s, -57344, 57344))       true division (activations only)
 //
 // HBM-bound: 2 B read + 1 B written per element.  The fast kernel gives one
 // 64-lane wavefront a whole row, keeps the row in VGPRs between the abs-max pass
@@ -49,13 +50,24 @@ __device__ __forceinline__ int q_i8(float x, float inv) {
     return (int)r;
 }
 
+// FMT: 0 = int8, 1 = OCP e4m3fn (max 448), 2 = OCP e5m2 (max 57344)
+template <int FMT>
 __device__ __forceinline__ float q_f8_pre(float x, float s) {
+    constexpr float kMax = FMT == 2 ? 57344.0f : 448.0f;
     float v = x / s;  // IEEE division per element
-    return fminf(fmaxf(v, -448.0f), 448.0f);
+    return fminf(fmaxf(v, -kMax), kMax);
+}
+
+template <int FMT>
+__device__ __forceinline__ int cvt_pk_f8(float a, float b, int old, bool hi) {
+    if constexpr (FMT == 2)
+        return hi ? __builtin_amdgcn_cvt_pk_bf8_f32(a, b, old, true) : __builtin_amdgcn_cvt_pk_bf8_f32(a, b, old, false);
+    else
+        return hi ? __builtin_amdgcn_cvt_pk_fp8_f32(a, b, old, true) : __builtin_amdgcn_cvt_pk_fp8_f32(a, b, old, false);
 }
 
 // 8 bf16 (one 16-byte chunk) -> 8 quantised bytes
-template <bool FP8>
+template <int FMT>
 __device__ __forceinline__ uint2 quant_chunk(const uint4& v, float s, float inv) {
     const uint32_t w[4] = {v.x, v.y, v.z, v.w};
     uint32_t o[2];
@@ -65,9 +77,9 @@ __device__ __forceinline__ uint2 quant_chunk(const uint4& v, float s, float inv)
         float f1 = __uint_as_float(w[2 * h] & 0xffff0000u);
         float f2 = __uint_as_float(w[2 * h + 1] << 16);
         float f3 = __uint_as_float(w[2 * h + 1] & 0xffff0000u);
-        if (FP8) {
-            int p = __builtin_amdgcn_cvt_pk_fp8_f32(q_f8_pre(f0, s), q_f8_pre(f1, s), 0, false);
-            p = __builtin_amdgcn_cvt_pk_fp8_f32(q_f8_pre(f2, s), q_f8_pre(f3, s), p, true);
+        if (FMT != 0) {
+            int p = cvt_pk_f8<FMT>(q_f8_pre<FMT>(f0, s), q_f8_pre<FMT>(f1, s), 0, false);
+            p = cvt_pk_f8<FMT>(q_f8_pre<FMT>(f2, s), q_f8_pre<FMT>(f3, s), p, true);
             o[h] = (uint32_t)p;
         } else {
             uint32_t b0 = (uint32_t)q_i8(f0, inv) & 0xffu;
@@ -84,7 +96,7 @@ __device__ __forceinline__ uint2 quant_chunk(const uint4& v, float s, float inv)
 // Requires k % 8 == 0, ld_x % 8 == 0, ld_q % 8 == 0, 16-byte aligned x, 8-byte aligned q,
 // and ld_q / 8 <= NCH * 64.
 // SCALE_IN: the per-row scale is an input (leaf quantiser) instead of being derived from the row.
-template <int NCH, bool FP8, bool ROUND_BF16, bool SCALE_IN>
+template <int NCH, int FMT, bool ROUND_BF16, bool SCALE_IN>
 __global__ __launch_bounds__(256) void quant_rows_wave(const uint16_t* __restrict__ x, int64_t m, int k,
                                                        int64_t ld_x, uint8_t* __restrict__ q, int64_t ld_q,
                                                        float* __restrict__ scale, float qmax) {
@@ -129,7 +141,7 @@ __global__ __launch_bounds__(256) void quant_rows_wave(const uint16_t* __restric
     for (int i = 0; i < NCH; ++i) {
         const int c = i * 64 + lane;
         if (c < nch) {
-            qr[c] = quant_chunk<FP8>(v[i], s, inv);
+            qr[c] = quant_chunk<FMT>(v[i], s, inv);
         } else if (c < npad) {
             qr[c] = make_uint2(0, 0);
         }
@@ -137,7 +149,7 @@ __global__ __launch_bounds__(256) void quant_rows_wave(const uint16_t* __restric
 }
 
 // General path: any k / alignment / row length; one 256-thread block per row, two passes.
-template <bool FP8, bool ROUND_BF16, bool SCALE_IN>
+template <int FMT, bool ROUND_BF16, bool SCALE_IN>
 __global__ __launch_bounds__(256) void quant_rows_block(const uint16_t* __restrict__ x, int64_t m, int64_t k,
                                                         int64_t ld_x, uint8_t* __restrict__ q, int64_t ld_q,
                                                         float* __restrict__ scale, float qmax) {
@@ -169,8 +181,8 @@ __global__ __launch_bounds__(256) void quant_rows_block(const uint16_t* __restri
         uint8_t o = 0;
         if (c < k) {
             float f = bf16_bits_to_f32(xr[c]);
-            if (FP8) {
-                o = (uint8_t)(__builtin_amdgcn_cvt_pk_fp8_f32(q_f8_pre(f, s), 0.0f, 0, false) & 0xff);
+            if (FMT != 0) {
+                o = (uint8_t)(cvt_pk_f8<FMT>(q_f8_pre<FMT>(f, s), 0.0f, 0, false) & 0xff);
             } else {
                 o = (uint8_t)(q_i8(f, inv) & 0xff);
             }
@@ -179,7 +191,7 @@ __global__ __launch_bounds__(256) void quant_rows_block(const uint16_t* __restri
     }
 }
 
-template <bool FP8, bool ROUND_BF16, bool SCALE_IN>
+template <int FMT, bool ROUND_BF16, bool SCALE_IN>
 static int launch_quant_rows(const void* x, int64_t m, int64_t k, int64_t ld_x, void* q, int64_t ld_q, float* scale,
                              float qmax, hipStream_t st) {
     if (m < 0 || k <= 0 || ld_x < k || ld_q < k) return fail(DAXQ_ERR_ARG, "quant_rows: bad shape m=%lld k=%lld ld_x=%lld ld_q=%lld",
@@ -196,7 +208,7 @@ static int launch_quant_rows(const void* x, int64_t m, int64_t k, int64_t ld_x, 
         const dim3 grid((unsigned)((m + 3) / 4)), block(256);
 #define DAXQ_Q_CASE(N)                                                                                      \
     if (nchunks <= N) {                                                                                     \
-        hipLaunchKernelGGL((quant_rows_wave<N, FP8, ROUND_BF16, SCALE_IN>), grid, block, 0, st, xp, m, (int)k, ld_x, qp, \
+        hipLaunchKernelGGL((quant_rows_wave<N, FMT, ROUND_BF16, SCALE_IN>), grid, block, 0, st, xp, m, (int)k, ld_x, qp, \
                            ld_q, scale, qmax);                                                              \
         return check_launch("quant_rows_wave");                                                             \
     }
@@ -210,7 +222,7 @@ static int launch_quant_rows(const void* x, int64_t m, int64_t k, int64_t ld_x, 
 #undef DAXQ_Q_CASE
     }
     if (m > 0x7fffffff) return fail(DAXQ_ERR_ARG, "quant_rows: too many rows for the general kernel");
-    hipLaunchKernelGGL((quant_rows_block<FP8, ROUND_BF16, SCALE_IN>), dim3((unsigned)m), dim3(256), 0, st, xp, m, k, ld_x, qp,
+    hipLaunchKernelGGL((quant_rows_block<FMT, ROUND_BF16, SCALE_IN>), dim3((unsigned)m), dim3(256), 0, st, xp, m, k, ld_x, qp,
                        ld_q, scale, qmax);
     return check_launch("quant_rows_block");
 }
@@ -260,23 +272,28 @@ extern "C" {
 
 int daxq_act_quant_i8(const void* x, int64_t m, int64_t k, int64_t ld_x, int8_t* q, int64_t ld_q, float* scale,
                       daxq_stream_t stream) {
-    return daxq::launch_quant_rows<false, true, false>(x, m, k, ld_x, q, ld_q, scale, 127.0f, (hipStream_t)stream);
+    return daxq::launch_quant_rows<0, true, false>(x, m, k, ld_x, q, ld_q, scale, 127.0f, (hipStream_t)stream);
 }
 
 int daxq_act_quant_e4m3(const void* x, int64_t m, int64_t k, int64_t ld_x, uint8_t* q, int64_t ld_q, float* scale,
                         daxq_stream_t stream) {
-    return daxq::launch_quant_rows<true, true, false>(x, m, k, ld_x, q, ld_q, scale, 448.0f, (hipStream_t)stream);
+    return daxq::launch_quant_rows<1, true, false>(x, m, k, ld_x, q, ld_q, scale, 448.0f, (hipStream_t)stream);
+}
+
+int daxq_act_quant_e5m2(const void* x, int64_t m, int64_t k, int64_t ld_x, uint8_t* q, int64_t ld_q, float* scale,
+                        daxq_stream_t stream) {
+    return daxq::launch_quant_rows<2, true, false>(x, m, k, ld_x, q, ld_q, scale, 57344.0f, (hipStream_t)stream);
 }
 
 int daxq_quantize_rows_i8(const void* x, int64_t m, int64_t k, int64_t ld_x, const float* scale, int8_t* q,
                           int64_t ld_q, daxq_stream_t stream) {
-    return daxq::launch_quant_rows<false, false, true>(x, m, k, ld_x, q, ld_q, const_cast<float*>(scale), 127.0f,
+    return daxq::launch_quant_rows<0, false, true>(x, m, k, ld_x, q, ld_q, const_cast<float*>(scale), 127.0f,
                                                        (hipStream_t)stream);
 }
 
 int daxq_quantize_rows_e4m3(const void* x, int64_t m, int64_t k, int64_t ld_x, const float* scale, uint8_t* q,
                             int64_t ld_q, daxq_stream_t stream) {
-    return daxq::launch_quant_rows<true, false, true>(x, m, k, ld_x, q, ld_q, const_cast<float*>(scale), 448.0f,
+    return daxq::launch_quant_rows<1, false, true>(x, m, k, ld_x, q, ld_q, const_cast<float*>(scale), 448.0f,
                                                       (hipStream_t)stream);
 }
 

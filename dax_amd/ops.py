@@ -40,8 +40,8 @@ def _rows_bf16(x: torch.Tensor, what: str) -> None:
 
 
 # ----------------------------------------------------------------------------- act quant
-def _act_quant(x: torch.Tensor, fp8: bool) -> Tuple[torch.Tensor, torch.Tensor]:
-    name = "act_quant_e4m3" if fp8 else "act_quant_i8"
+def _act_quant(x: torch.Tensor, fp8, e5m2: bool = False) -> Tuple[torch.Tensor, torch.Tensor]:
+    name = "act_quant_e5m2" if e5m2 else "act_quant_e4m3" if fp8 else "act_quant_i8"
     _rows_bf16(x, name)
     m, k = x.shape
     kp = pad_k(k)
@@ -49,7 +49,7 @@ def _act_quant(x: torch.Tensor, fp8: bool) -> Tuple[torch.Tensor, torch.Tensor]:
         q = torch.empty((m, kp), dtype=torch.uint8 if fp8 else torch.int8, device=x.device)
         s = torch.empty((m,), dtype=torch.float32, device=x.device)
         if m:
-            fn = _capi.lib().daxq_act_quant_e4m3 if fp8 else _capi.lib().daxq_act_quant_i8
+            fn = getattr(_capi.lib(), "daxq_" + name)
             ld_x = x.stride(0) if m > 1 else k
             _capi.check(fn(x.data_ptr(), m, k, ld_x, q.data_ptr(), kp, s.data_ptr(), _stream(x)), name)
     return q, s
@@ -67,12 +67,19 @@ def act_quant_e4m3(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
     return _act_quant(x, True)
 
 
+@torch.library.custom_op("daxq::act_quant_e5m2", mutates_args=(), device_types="cuda")
+def act_quant_e5m2(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """bf16 [M,K] -> (e5m2 bytes as uint8 [M, pad128(K)], fp32 [M] per-token scale)."""
+    return _act_quant(x, True, True)
+
+
 def _act_quant_fake(x, dtype):
     return x.new_empty((x.shape[0], pad_k(x.shape[1])), dtype=dtype), x.new_empty((x.shape[0],), dtype=torch.float32)
 
 
 act_quant_i8.register_fake(lambda x: _act_quant_fake(x, torch.int8))
 act_quant_e4m3.register_fake(lambda x: _act_quant_fake(x, torch.uint8))
+act_quant_e5m2.register_fake(lambda x: _act_quant_fake(x, torch.uint8))
 
 
 # ----------------------------------------------------------------------------- leaf quantisers
@@ -147,8 +154,8 @@ scale_from_minmax.register_fake(lambda min_val, max_val, qmax: torch.empty_like(
 
 
 # ----------------------------------------------------------------------------- GEMM + epilogue
-def _linear(xq, sx, wq, sw, bias, fp8: bool, want_acc: bool):
-    name = "linear_e4m3" if fp8 else "linear_i8"
+def _linear(xq, sx, wq, sw, bias, fp8: bool, want_acc: bool, x_e5m2: bool = False):
+    name = "linear_e5m2_e4m3" if x_e5m2 else "linear_e4m3" if fp8 else "linear_i8"
     _need_gpu(xq, name)
     qdt = torch.uint8 if fp8 else torch.int8
     if xq.dtype != qdt or wq.dtype != qdt:
@@ -169,7 +176,7 @@ def _linear(xq, sx, wq, sw, bias, fp8: bool, want_acc: bool):
         out = torch.empty((m, n), dtype=torch.bfloat16, device=xq.device)
         acc = torch.empty((m, n), dtype=torch.float32 if fp8 else torch.int32, device=xq.device) if want_acc else None
         if m and n:
-            fn = _capi.lib().daxq_linear_e4m3 if fp8 else _capi.lib().daxq_linear_i8
+            fn = getattr(_capi.lib(), "daxq_" + name)
             ld_x = xq.stride(0) if m > 1 else k
             ld_w = wq.stride(0) if n > 1 else k
             _capi.check(fn(xq.data_ptr(), ld_x, sx.data_ptr(), wq.data_ptr(), ld_w, sw.data_ptr(),
@@ -205,12 +212,28 @@ def linear_e4m3_acc(xq: torch.Tensor, sx: torch.Tensor, wq: torch.Tensor, sw: to
     return _linear(xq, sx, wq, sw, bias, True, True)
 
 
+@torch.library.custom_op("daxq::linear_e5m2_e4m3", mutates_args=(), device_types="cuda")
+def linear_e5m2_e4m3(xq: torch.Tensor, sx: torch.Tensor, wq: torch.Tensor, sw: torch.Tensor,
+                     bias: Optional[torch.Tensor]) -> torch.Tensor:
+    """e5m2 activation bytes [M,Kp] x e4m3fn weight bytes [N,Kp]^T, fp32 accumulate, fused epilogue."""
+    return _linear(xq, sx, wq, sw, bias, True, False, True)[0]
+
+
+@torch.library.custom_op("daxq::linear_e5m2_e4m3_acc", mutates_args=(), device_types="cuda")
+def linear_e5m2_e4m3_acc(xq: torch.Tensor, sx: torch.Tensor, wq: torch.Tensor, sw: torch.Tensor,
+                         bias: Optional[torch.Tensor]) -> Tuple[torch.Tensor, torch.Tensor]:
+    return _linear(xq, sx, wq, sw, bias, True, True, True)
+
+
 def _lin_fake(xq, sx, wq, sw, bias):
     return xq.new_empty((xq.shape[0], wq.shape[0]), dtype=torch.bfloat16)
 
 
 linear_i8.register_fake(_lin_fake)
 linear_e4m3.register_fake(_lin_fake)
+linear_e5m2_e4m3.register_fake(_lin_fake)
+linear_e5m2_e4m3_acc.register_fake(lambda xq, sx, wq, sw, bias: (
+    _lin_fake(xq, sx, wq, sw, bias), xq.new_empty((xq.shape[0], wq.shape[0]), dtype=torch.float32)))
 linear_i8_acc.register_fake(lambda xq, sx, wq, sw, bias: (
     _lin_fake(xq, sx, wq, sw, bias), xq.new_empty((xq.shape[0], wq.shape[0]), dtype=torch.int32)))
 linear_e4m3_acc.register_fake(lambda xq, sx, wq, sw, bias: (

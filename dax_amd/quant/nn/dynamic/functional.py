@@ -55,8 +55,6 @@ def _dynamic_quantize_func(
     assert len(block_size) == input.dim(), f"Got input dim:{input.dim()}, block_size: {block_size}"
     if target_dtype not in FP8_ALLOWED_DTYPES and target_dtype != torch.int8:
         raise NotImplementedError(f"Unsupported dtype {target_dtype}")
-    if target_dtype == torch.float8_e5m2:
-        raise NotImplementedError("daxq implements float8_e4m3fn and int8 activations; float8_e5m2 is not built")
     if not _is_per_token(block_size, input.shape):
         raise NotImplementedError("daxq implements the per-token dynamic scheme; per-tensor / grouped blocks are not built")
     if scale_dtype not in (None, torch.float32) or (eps is not None and eps != torch.finfo(torch.float32).eps):
@@ -65,6 +63,9 @@ def _dynamic_quantize_func(
     x2 = input.reshape(-1, k)
     if target_dtype == torch.int8:
         q, s = ops.act_quant_i8(x2)
+    elif target_dtype == torch.float8_e5m2:
+        q, s = ops.act_quant_e5m2(x2)
+        q = q.view(torch.float8_e5m2)
     else:
         q, s = ops.act_quant_e4m3(x2)
         q = q.view(torch.float8_e4m3fn)

@@ -61,10 +61,9 @@ class Linear(nn.Module):
             raise NotImplementedError(
                 "daxq implements per-token activations with per-channel weights; "
                 f"got input_qscheme={input_qscheme}, weight_qscheme={weight_qscheme}")
-        if compute_dtype == "FP8" and not (weight_dtype == input_dtype == torch.float8_e4m3fn):
+        if compute_dtype == "FP8" and weight_dtype != torch.float8_e4m3fn:
             raise NotImplementedError(
-                f"daxq implements float8_e4m3fn x float8_e4m3fn; got weight {weight_dtype}, input {input_dtype} "
-                "(pass activation_dtype=torch.float8_e4m3fn to the fp8 qconfig factory)")
+                f"daxq implements float8_e4m3fn weights (with e4m3fn or e5m2 activations); got weight {weight_dtype}")
         if out_dtype not in (None, torch.bfloat16):
             raise NotImplementedError(f"daxq kernels produce bfloat16 outputs, got out_dtype={out_dtype}")
 
@@ -120,7 +119,10 @@ class Linear(nn.Module):
         flat = input.view(-1, self.in_features)
         wq = self._gemm_weight()
         sw = self.weight_scale.view(-1)
-        if self.compute_dtype == "FP8":
+        if self.compute_dtype == "FP8" and self.input_dtype == torch.float8_e5m2:
+            xq, sx = ops.act_quant_e5m2(flat)
+            out = ops.linear_e5m2_e4m3(xq, sx, wq, sw, self.bias)
+        elif self.compute_dtype == "FP8":
             xq, sx = ops.act_quant_e4m3(flat)
             out = ops.linear_e4m3(xq, sx, wq, sw, self.bias)
         else:

@@ -69,6 +69,13 @@ int daxq_act_quant_e4m3(const void* x, int64_t m, int64_t k, int64_t ld_x,
                         uint8_t* q, int64_t ld_q, float* scale, daxq_stream_t stream);
 
 /*
+ * The same for OCP e5m2 activations, the default activation dtype of the reference's FP8 qconfig
+ *   dax/quant/quantization/qconfig.py:85-87;  scale with 57344, q = e5m2_rne( clamp( f32(x) / scale, -57344, 57344 ) ).
+ */
+int daxq_act_quant_e5m2(const void* x, int64_t m, int64_t k, int64_t ld_x,
+                        uint8_t* q, int64_t ld_q, float* scale, daxq_stream_t stream);
+
+/*
  * Leaf quantisers with a caller-supplied per-row scale (used once per weight at conversion).
  * Replace quantize_to_int8 / quantize_to_fp8 with a [rows,1] scale
  *   dax/quant/nn/quantized/functional.py:11-20, called from dax/quant/nn/dynamic/linear.py:292-296
@@ -122,6 +129,13 @@ int daxq_linear_e4m3(const uint8_t* xq, int64_t ld_xq, const float* sx,
                      const void* bias, void* out, int64_t ld_out,
                      float* acc, int64_t ld_acc,
                      int64_t m, int64_t n, int64_t k, daxq_stream_t stream);
+
+/* As daxq_linear_e4m3 with e5m2 activation bytes against e4m3fn weight bytes (mixed-format MFMA). */
+int daxq_linear_e5m2_e4m3(const uint8_t* xq, int64_t ld_xq, const float* sx,
+                          const uint8_t* wq, int64_t ld_wq, const float* sw,
+                          const void* bias, void* out, int64_t ld_out,
+                          float* acc, int64_t ld_acc,
+                          int64_t m, int64_t n, int64_t k, daxq_stream_t stream);
 
 /* Selects a GEMM kernel variant for tuning and tests (0 = library default).
  * Process-wide; not part of the reference interface. */

@@ -37,11 +37,16 @@ def lib():
         L.daxo_f32_to_e4m3fn.argtypes = [f32]
         L.daxo_e4m3fn_to_f32.restype = f32
         L.daxo_e4m3fn_to_f32.argtypes = [C.c_uint8]
+        L.daxo_e5m2_to_f32.restype = f32
+        L.daxo_e5m2_to_f32.argtypes = [C.c_uint8]
         L.daxo_f32_to_bf16.restype = C.c_uint16
         L.daxo_f32_to_bf16.argtypes = [f32]
         for name, args in {
             "daxo_act_quant_i8": [p, i64, i64, p, p],
             "daxo_act_quant_e4m3": [p, i64, i64, p, p],
+            "daxo_act_quant_e5m2": [p, i64, i64, p, p],
+            "daxo_f32_to_e5m2_vec": [p, i64, p],
+            "daxo_quant_e5m2_vec": [p, i64, f32, p],
             "daxo_weight_scale": [p, i64, i64, f32, p],
             "daxo_gemm_i8": [p, p, i64, i64, i64, p],
             "daxo_epilogue_i8": [p, p, p, p, i64, i64, p],
@@ -78,6 +83,33 @@ def f32_to_e4m3fn(v: np.ndarray) -> np.ndarray:
 
 def e4m3fn_table() -> np.ndarray:
     return np.array([lib().daxo_e4m3fn_to_f32(b) for b in range(256)], np.float32)
+
+
+def f32_to_e5m2(v: np.ndarray) -> np.ndarray:
+    v = np.ascontiguousarray(v, dtype=np.float32)
+    out = np.empty(v.shape, np.uint8)
+    lib().daxo_f32_to_e5m2_vec(_ptr(v), v.size, _ptr(out))
+    return out
+
+
+def e5m2_table() -> np.ndarray:
+    return np.array([lib().daxo_e5m2_to_f32(b) for b in range(256)], np.float32)
+
+
+def quant_e5m2_vec(x_bits: np.ndarray, s: float) -> np.ndarray:
+    x_bits = np.ascontiguousarray(x_bits, dtype=np.uint16)
+    out = np.empty(x_bits.shape, np.uint8)
+    lib().daxo_quant_e5m2_vec(_ptr(x_bits), x_bits.size, s, _ptr(out))
+    return out
+
+
+def act_quant_e5m2(x_bits: np.ndarray):
+    x_bits = np.ascontiguousarray(x_bits, dtype=np.uint16)
+    m, k = x_bits.shape
+    q = np.empty((m, k), np.uint8)
+    s = np.empty((m,), np.float32)
+    lib().daxo_act_quant_e5m2(_ptr(x_bits), m, k, _ptr(q), _ptr(s))
+    return q, s
 
 
 def quant_i8_vec(x_bits: np.ndarray, s: float) -> np.ndarray:

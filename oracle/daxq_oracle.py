@@ -38,6 +38,7 @@ import torch
 
 INT8_QMAX = 127  # torch.iinfo(torch.int8).max      dynamic/functional.py:199
 E4M3_QMAX = 448.0  # torch.finfo(torch.float8_e4m3fn).max   dynamic/functional.py:170
+E5M2_QMAX = 57344.0  # torch.finfo(torch.float8_e5m2).max (the FP8 qconfig's default activation dtype)
 EPS = torch.finfo(torch.float32).eps  # 2**-23     dynamic/functional.py:171,200
 
 
@@ -79,9 +80,10 @@ def quantize_to_int8(x: torch.Tensor, scale: torch.Tensor) -> torch.Tensor:
     return torch.clamp(torch.round(x * (1.0 / scale)), -128, 127).to(torch.int8)
 
 
-def quantize_to_fp8(x: torch.Tensor, scale: torch.Tensor) -> torch.Tensor:
-    """dax/quant/nn/quantized/functional.py:11-13 (true division, clamp, RNE cast)."""
-    return (x / scale).clamp(-E4M3_QMAX, E4M3_QMAX).to(torch.float8_e4m3fn)
+def quantize_to_fp8(x: torch.Tensor, scale: torch.Tensor, dtype: torch.dtype = torch.float8_e4m3fn) -> torch.Tensor:
+    """dax/quant/nn/quantized/functional.py:11-13 (true division, clamp to the dtype's max, RNE cast)."""
+    qmax = torch.finfo(dtype).max
+    return (x / scale).clamp(-qmax, qmax).to(dtype)
 
 
 def act_quant_int8(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
@@ -96,6 +98,13 @@ def act_quant_e4m3(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
     x2 = x.reshape(-1, x.shape[-1])
     s = act_scale(x2, E4M3_QMAX)
     return quantize_to_fp8(x2, s), s
+
+
+def act_quant_e5m2(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """dynamic_quantize_to_fp8, per-token, e5m2 (qconfig.py:85-87 default).  dynamic/functional.py:152-177."""
+    x2 = x.reshape(-1, x.shape[-1])
+    s = act_scale(x2, E5M2_QMAX)
+    return quantize_to_fp8(x2, s, torch.float8_e5m2), s
 
 
 # --------------------------------------------------------------------------- #
@@ -186,17 +195,20 @@ def linear_int8(x: torch.Tensor, qweight: torch.Tensor, wscale: torch.Tensor,
 
 
 def linear_e4m3(x: torch.Tensor, qweight: torch.Tensor, wscale: torch.Tensor,
-                bias: Optional[torch.Tensor], row_chunk: int = 8192) -> Dict[str, torch.Tensor]:
+                bias: Optional[torch.Tensor], row_chunk: int = 8192,
+                act_dtype: torch.dtype = torch.float8_e4m3fn) -> Dict[str, torch.Tensor]:
     """Whole FP8 forward.  dax/quant/nn/dynamic/linear.py:145-178.
 
     torch._scaled_mm with row-wise scales is CUDA-only, so the matmul is
     emulated in fp32: bf16( (Xq . Wq^T in fp32) * sx * sw + bias ), one rounding.
     The summation order of the reference (cuBLASLt, use_fast_accum=True) is not
-    specified; comparisons against this function use a tolerance.
+    specified; comparisons against this function use a tolerance.  ``act_dtype``
+    float8_e5m2 gives the reference's default FP8 pairing (e5m2 activations against
+    e4m3fn weights).
     """
     prev = x.shape[:-1]
     x2 = x.reshape(-1, x.shape[-1])
-    xq, sx = act_quant_e4m3(x2)
+    xq, sx = act_quant_e4m3(x2) if act_dtype == torch.float8_e4m3fn else act_quant_e5m2(x2)
     wf = qweight.to(torch.float32)
     outs = []
     for r0 in range(0, x2.shape[0], row_chunk):

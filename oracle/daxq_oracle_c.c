@@ -130,6 +130,54 @@ float daxo_e4m3fn_to_f32(uint8_t b) {
     return u2f(f2u(mag) | sign);
 }
 
+/* f32 -> OCP e5m2 byte, round to nearest even; e5m2 is IEEE-like (5 exponent bits, bias 15, 2 mantissa
+ * bits, infinities and NaNs): values at or above 61440 (the midpoint between 57344 and 65536) round to
+ * infinity. */
+uint8_t daxo_f32_to_e5m2(float v) {
+    uint32_t u = f2u(v);
+    uint8_t sign = (uint8_t)((u >> 24) & 0x80u);
+    uint32_t au = u & 0x7fffffffu;
+    if (au > 0x7f800000u) return (uint8_t)(sign | 0x7fu);            /* NaN */
+    if (au >= 0x47700000u) return (uint8_t)(sign | 0x7cu);           /* >= 61440 -> inf (tie goes to even = 65536 = inf) */
+    int32_t e = (int32_t)(au >> 23) - 127;
+    uint32_t man = (au & 0x7fffffu) | (au >= 0x00800000u ? 0x800000u : 0u);
+    if (au < 0x00800000u) e = -126;
+    int32_t qexp = (e >= -14) ? e - 2 : -16;                         /* quantum: 2 fraction bits, subnormal 2^-16 */
+    int32_t shift = qexp - (e - 23);
+    uint32_t q;
+    if (shift > 25) q = 0;
+    else {
+        uint32_t keep = man >> shift, rem = man & ((1u << shift) - 1u), half = 1u << (shift - 1);
+        if (rem > half || (rem == half && (keep & 1u))) keep++;
+        q = keep;
+    }
+    if (q == 0) return sign;
+    uint8_t out;
+    if (e >= -14) {
+        int32_t be = e + 15;
+        if (q == 8) { q = 4; be += 1; }
+        out = (uint8_t)((be << 2) | (q & 3u));
+    } else {
+        out = (uint8_t)q;                                            /* q == 4 is the min normal */
+    }
+    return (uint8_t)(sign | out);
+}
+
+float daxo_e5m2_to_f32(uint8_t b) {
+    uint32_t sign = (uint32_t)(b & 0x80u) << 24;
+    uint32_t be = (b >> 2) & 0x1fu, m = b & 3u;
+    if (be == 0x1f) return u2f(sign | (m ? 0x7fc00000u : 0x7f800000u));
+    float mag = be == 0 ? ldexpf((float)m, -16) : ldexpf((float)(4 + m), (int)be - 15 - 2);
+    return u2f(f2u(mag) | sign);
+}
+
+uint8_t daxo_quant_e5m2(uint16_t x_bits, float s) {
+    float v = daxo_bf16_to_f32(x_bits) / s;
+    if (v < -57344.0f) v = -57344.0f;
+    if (v > 57344.0f) v = 57344.0f;
+    return daxo_f32_to_e5m2(v);
+}
+
 /* fp8 leaf quantiser: e4m3fn_rne(clamp(f32(x) / s, -448, 448)) */
 uint8_t daxo_quant_e4m3(uint16_t x_bits, float s) {
     float v = daxo_bf16_to_f32(x_bits) / s;
@@ -161,6 +209,14 @@ void daxo_act_quant_e4m3(const uint16_t* x, int64_t m, int64_t k, uint8_t* q, fl
         float s = daxo_act_scale(row_amax_bits(x + r * k, k), 448.0f);
         scale[r] = s;
         for (int64_t i = 0; i < k; ++i) q[r * k + i] = daxo_quant_e4m3(x[r * k + i], s);
+    }
+}
+
+void daxo_act_quant_e5m2(const uint16_t* x, int64_t m, int64_t k, uint8_t* q, float* scale) {
+    for (int64_t r = 0; r < m; ++r) {
+        float s = daxo_act_scale(row_amax_bits(x + r * k, k), 57344.0f);
+        scale[r] = s;
+        for (int64_t i = 0; i < k; ++i) q[r * k + i] = daxo_quant_e5m2(x[r * k + i], s);
     }
 }
 
@@ -207,6 +263,12 @@ void daxo_epilogue_i8(const int32_t* acc, const float* sx, const float* sw, cons
 /* vector helpers used by the exhaustive tests */
 void daxo_f32_to_e4m3fn_vec(const float* v, int64_t n, uint8_t* out) {
     for (int64_t i = 0; i < n; ++i) out[i] = daxo_f32_to_e4m3fn(v[i]);
+}
+void daxo_f32_to_e5m2_vec(const float* v, int64_t n, uint8_t* out) {
+    for (int64_t i = 0; i < n; ++i) out[i] = daxo_f32_to_e5m2(v[i]);
+}
+void daxo_quant_e5m2_vec(const uint16_t* x_bits, int64_t n, float s, uint8_t* out) {
+    for (int64_t i = 0; i < n; ++i) out[i] = daxo_quant_e5m2(x_bits[i], s);
 }
 void daxo_act_scale_vec(const uint16_t* amax_bits, int64_t n, float qmax, float* out) {
     for (int64_t i = 0; i < n; ++i) out[i] = daxo_act_scale(amax_bits[i], qmax);

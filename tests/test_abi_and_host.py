@@ -193,8 +193,10 @@ def test_linear_constructor_validation_and_state_layout():
         Linear(8, 8, True, None, torch.float32, torch.float32, torch.bfloat16, ch, tok)
     with pytest.raises(NotImplementedError):   # valid in the reference, not built here
         Linear(8, 8, True, None, torch.int8, torch.int8, torch.bfloat16, te, te)
-    with pytest.raises(NotImplementedError):
-        Linear(8, 8, True, None, torch.float8_e4m3fn, torch.float8_e5m2, torch.bfloat16, ch, tok)
+    mixed = Linear(8, 8, True, None, torch.float8_e4m3fn, torch.float8_e5m2, torch.bfloat16, ch, tok)
+    assert mixed.compute_dtype == "FP8" and mixed.input_dtype == torch.float8_e5m2   # the reference's FP8 default
+    with pytest.raises(NotImplementedError):   # e5m2 weights: valid in the reference, not built here
+        Linear(8, 8, True, None, torch.float8_e5m2, torch.float8_e5m2, torch.bfloat16, ch, tok)
     # dequantised weight property is plain tensor algebra on the stored state
     with torch.no_grad():
         lin.qweight.copy_(torch.randint(-127, 128, (128, 256), dtype=torch.int8))

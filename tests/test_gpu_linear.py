@@ -14,7 +14,12 @@ from tests.util import bf16_bits, rel_l2
 
 pytestmark = pytest.mark.gpu
 
-VARIANTS = [0, 2, 5]  # 0 = library default (256x256 kernel when m, n >= 256), 2 / 5 = generic kernels
+VARIANTS = [0, 2, 5, 6]  # 0 = library default, 2 / 5 = generic kernels, 6 = the 256x256 kernel (m, n >= 256)
+
+
+def _skip_if_too_small(variant, m, n):
+    if variant == 6 and (m < 256 or n < 256):
+        pytest.skip("the 256x256 kernel needs m, n >= 256")
 FP8_TOL = 2e-2
 
 
@@ -47,6 +52,7 @@ GEMM_SHAPES = [(256, 256, 128), (300, 520, 256), (1, 8, 128), (17, 24, 384), (51
 def test_linear_i8_bit_exact(ops, variant, m, n, k):
     from dax_amd import _capi
 
+    _skip_if_too_small(variant, m, n)
     _capi.set_gemm_variant(variant)
     x, w, b = O.make_inputs(m, k, n, seed=m + n + k)
     qw, sw = O.weight_quant_int8(w)
@@ -67,7 +73,7 @@ def test_linear_i8_adversarial_extremes(ops, variant):
     from dax_amd import _capi
 
     _capi.set_gemm_variant(variant)
-    m, n, k = 130, 264, 13824
+    m, n, k = 300, 264, 13824
     xq = torch.full((m, k), -128, dtype=torch.int8)
     xq[1::2] = 127
     wq = torch.full((n, k), -128, dtype=torch.int8)
@@ -103,6 +109,7 @@ def test_linear_i8_one_hot_layout(ops):
 def test_linear_e4m3_within_tolerance(ops, variant, m, n, k):
     from dax_amd import _capi
 
+    _skip_if_too_small(variant, m, n)
     _capi.set_gemm_variant(variant)
     x, w, b = O.make_inputs(m, k, n, seed=m + n + k + 1)
     qw, sw = O.weight_quant_e4m3(w)
@@ -117,6 +124,24 @@ def test_linear_e4m3_within_tolerance(ops, variant, m, n, k):
     r = rel_l2(out, ref["out"])
     assert r < FP8_TOL, r
     assert r < 3e-3, r                          # what fp32 accumulation actually delivers
+
+
+@pytest.mark.parametrize("variant", [0, 5, 6])
+@pytest.mark.parametrize("m,n,k", [(300, 520, 256), (17, 24, 384), (512, 1536, 1536), (4096, 1536, 1536)])
+def test_linear_e5m2_activations_within_tolerance(ops, variant, m, n, k):
+    from dax_amd import _capi
+
+    _skip_if_too_small(variant, m, n)
+    _capi.set_gemm_variant(variant)
+    x, w, b = O.make_inputs(m, k, n, seed=m + n + k + 2)
+    qw, sw = O.weight_quant_e4m3(w)
+    ref = O.linear_e4m3(x, qw, sw, b, act_dtype=torch.float8_e5m2)
+    xq, sx = ops.act_quant_e5m2(dev(x))
+    assert torch.equal(xq[:, :k].cpu(), ref["xq"].view(torch.uint8))
+    out, acc = ops.linear_e5m2_e4m3_acc(xq, sx, dev(qw.view(torch.uint8)), dev(sw.view(-1)), dev(b))
+    acc_ref = ref["xq"].float() @ qw.float().t()
+    assert rel_l2(acc, acc_ref) < 2e-4          # a wrong operand format would be off by orders of magnitude
+    assert rel_l2(out, ref["out"]) < 3e-3
 
 
 def test_linear_rejects_unaligned_k(ops):
@@ -207,13 +232,26 @@ def test_quantize_dynamic_fp8_module_matches_oracle():
     assert rel_l2(y, ref) < FP8_TOL
 
 
-def test_fp8_default_e5m2_activation_keeps_float_module():
+def test_fp8_default_qconfig_e5m2_activations_e4m3_weights():
+    from dax_amd.quant.nn.dynamic import Linear as QLinear
     from dax_amd.quant.quantization import quantize_dynamic
     from dax_amd.quant.quantization.qconfig import get_dynamic_fp8_per_token_act_per_channel_weight_qconfig as cfg
 
     model = _toy(2).to("cuda")
-    quantize_dynamic(model, {"": cfg()})       # reference default: e5m2 activations, not built
-    assert type(model.to_q) is nn.Linear
+    w = model.to_q.weight.detach().cpu().clone()
+    b = model.to_q.bias.detach().cpu().clone()
+    quantize_dynamic(model, {"": cfg(), "proj_out": None})       # the reference's default FP8 pairing
+    assert isinstance(model.to_q, QLinear) and model.to_q.input_dtype == torch.float8_e5m2
+    assert model.to_q.qweight.dtype == torch.float8_e4m3fn
+    qw, sw = O.weight_quant_e4m3(w)
+    x, _, _ = O.make_inputs(150, 256, 8, seed=5)
+    y = model.to_q(x.to("cuda"))
+    ref = O.linear_e4m3(x, qw, sw, b, act_dtype=torch.float8_e5m2)["out"]
+    assert rel_l2(y, ref) < FP8_TOL
+    # e5m2 weights are not built: the layer stays a float module, as the reference does on NotImplementedError
+    model2 = _toy(3).to("cuda")
+    quantize_dynamic(model2, {"": cfg(weight_dtype=torch.float8_e5m2)})
+    assert type(model2.to_q) is nn.Linear
 
 
 def test_state_dict_round_trip_and_hooks():

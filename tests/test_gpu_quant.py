@@ -66,6 +66,35 @@ def test_act_quant_e4m3_matches_oracle(ops, m, k):
     assert not q[:, k:].any()
 
 
+@pytest.mark.parametrize("m,k", SHAPES)
+def test_act_quant_e5m2_matches_oracle(ops, m, k):
+    x, _, _ = O.make_inputs(m, k, 8, seed=m * 13 + k)
+    if m > 2:
+        x[1] = 0
+    q, s = ops.act_quant_e5m2(dev(x))
+    torch.cuda.synchronize()
+    qo, so = O.act_quant_e5m2(x)
+    np.testing.assert_array_equal(s.cpu().numpy().view(np.uint32), so.view(-1).numpy().view(np.uint32))
+    np.testing.assert_array_equal(q[:, :k].cpu().numpy(), qo.view(torch.uint8).numpy())
+    assert not q[:, k:].any()
+
+
+def test_act_quant_e5m2_every_bf16_amax_and_value(ops):
+    # rows: every finite bf16 value once as the row abs-max (alternating sign), and a second block
+    # where every finite bf16 value appears under a large fixed abs-max
+    n = ALL_POS_FINITE.size
+    x = torch.zeros(n, 64, dtype=torch.bfloat16)
+    vals = from_bits(ALL_POS_FINITE)
+    sign = torch.where(torch.arange(n) % 2 == 1, -1.0, 1.0).bfloat16()
+    x[torch.arange(n), torch.arange(n) % 64] = vals * sign
+    allv = from_bits(FINITE_BF16).view(-1, 64)            # 1020 rows of 64 distinct values
+    xs = torch.cat([x, allv])
+    q, s = ops.act_quant_e5m2(dev(xs))
+    qo, so = O.act_quant_e5m2(xs)
+    np.testing.assert_array_equal(s.cpu().numpy().view(np.uint32), so.view(-1).numpy().view(np.uint32))
+    np.testing.assert_array_equal(q[:, :64].cpu().numpy(), qo.view(torch.uint8).numpy())
+
+
 def test_act_quant_strided_rows(ops):
     x, _, _ = O.make_inputs(40, 512, 8, seed=5)
     big = torch.zeros(40, 640, dtype=torch.bfloat16)

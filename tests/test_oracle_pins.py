@@ -167,6 +167,59 @@ def test_quant_fp8_clamp_is_live_and_saturates_to_448():
     assert O.quantize_to_fp8(xs, sc).float().item() == 1.0
 
 
+# ------------------------------------------------------------------ e5m2 (the FP8 qconfig's default activation dtype)
+def test_e5m2_cast_torch_vs_closed_form(closed_form):
+    table = closed_form.e5m2_table()
+    tt = torch.arange(256, dtype=torch.uint8).view(torch.float8_e5m2).float().numpy()
+    ok = ~np.isnan(table)
+    np.testing.assert_array_equal(table[ok].view(np.uint32), tt[ok].view(np.uint32))
+    assert table[0x7B] == 57344.0 and table[0x01] == 2.0 ** -16 and np.isinf(table[0x7C])
+    v = np.array([57344, 61439.9, 61440, 3.0, 3.5, 4.5, 2.0 ** -17, 1.5 * 2.0 ** -17, 2.0 ** -16, -57344, 1.125, 1.375],
+                 np.float32)
+    want = np.array([57344, 57344, np.inf, 3.0, 3.5, 4.0, 0.0, 2.0 ** -16, 2.0 ** -16, -57344, 1.0, 1.5], np.float32)
+    np.testing.assert_array_equal(table[closed_form.f32_to_e5m2(v)], want)
+    np.testing.assert_array_equal(torch.from_numpy(v).to(torch.float8_e5m2).float().numpy(), want)
+    hi = np.float32(61440.0).view(np.uint32)
+    pats = np.arange(0, int(hi) + 2048, 53, dtype=np.uint32)
+    vals = np.unique(np.abs(table[np.isfinite(table)]))
+    mids = ((vals[:-1].astype(np.float64) + vals[1:].astype(np.float64)) / 2).astype(np.float32)
+    near = (np.concatenate([vals, mids]).view(np.uint32)[:, None].astype(np.int64) + np.arange(-64, 65)[None, :]).reshape(-1)
+    near = near[(near >= 0) & (near <= int(hi) + 2048)].astype(np.uint32)
+    pats = np.unique(np.concatenate([pats, near]))
+    for sign in (0, 0x80000000):
+        f = (pats | np.uint32(sign)).view(np.float32)
+        got_t = torch.from_numpy(f.copy()).to(torch.float8_e5m2).view(torch.uint8).numpy()
+        np.testing.assert_array_equal(got_t, closed_form.f32_to_e5m2(f))
+
+
+def test_quant_e5m2_closed_form_all_bf16_x_sampled_scales(closed_form):
+    scales = reachable_scales(57344.0)
+    rng = np.random.default_rng(2)
+    pick = np.concatenate([scales[:4], scales[-4:], rng.choice(scales, 100, replace=False)])
+    finite = np.concatenate([np.arange(0, 0x7F80), np.arange(0x8000, 0xFF80)]).astype(np.uint16)
+    xt = from_bits(finite)
+    for s in pick:
+        got = O.quantize_to_fp8(xt, torch.tensor([float(s)], dtype=torch.float32), torch.float8_e5m2)
+        np.testing.assert_array_equal(got.view(torch.uint8).numpy(), closed_form.quant_e5m2_vec(finite, float(s)))
+    # +-amax lands on +-57344 (never inf): the clamp is what keeps it finite
+    amax = ALL_POS_FINITE[ALL_POS_FINITE > 0]
+    x = from_bits(amax).view(-1, 1)
+    s = O.act_scale(x, 57344.0)
+    live = (s.view(-1) > 2.0 ** -23)
+    q = O.quantize_to_fp8(x, s, torch.float8_e5m2).float().view(-1)
+    assert (q[live] == 57344).all() and ((x.float() / s).view(-1)[live] > 57344).any()
+
+
+def test_act_quant_e5m2_rows_vs_closed_form(closed_form):
+    x, _, _ = O.make_inputs(48, 320, 8, seed=13)
+    x[3] = 0
+    q, s = O.act_quant_e5m2(x)
+    qc, sc = closed_form.act_quant_e5m2(bf16_bits(x))
+    np.testing.assert_array_equal(q.view(torch.uint8).numpy(), qc)
+    np.testing.assert_array_equal(s.view(-1).numpy(), sc)
+    assert q.dtype == torch.float8_e5m2
+
+
 # ------------------------------------------------------------------ whole rows
 def test_act_quant_rows_vs_closed_form(closed_form):
     x, _, _ = O.make_inputs(64, 384, 8, seed=3)
