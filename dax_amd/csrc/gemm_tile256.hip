@@ -218,7 +218,7 @@ __device__ __forceinline__ void tile256_epilogue(const GemmArgs& p, typename Acc
 // DUMP: also write the raw accumulators to p.acc (tests); a separate instantiation so that the
 // production kernel carries none of that code.
 // EXP:  timing experiments with wrong results by construction: 1 = no HBM loads in the steady
-//       state, 2 = loads only (no LDS reads, no MFMA).
+//       state, 2 = loads only (no LDS reads, no MFMA), 3 = all tiles load tile (0,0)'s panels (L2 hits).
 template <bool FP8, bool DUMP, int EXP = 0, bool XE5 = false>
 __global__ __launch_bounds__(256) void gemm_tile256_kernel(const GemmArgs p) {
     using namespace t256;
@@ -242,8 +242,9 @@ __global__ __launch_bounds__(256) void gemm_tile256_kernel(const GemmArgs p) {
     const uint32_t chunk = (uint32_t)((slot ^ swz(r8)) << 4);
     uint32_t voff_a = (uint32_t)r8 * (uint32_t)p.lda + chunk;
     uint32_t voff_b = (uint32_t)r8 * (uint32_t)p.ldb + chunk;
-    const uint8_t* abase = p.a + (int64_t)m0 * p.lda;
-    const uint8_t* bbase = p.b + (int64_t)n0 * p.ldb;
+    // EXP 3: every tile loads the panels of tile (0, 0), so that all loads hit L2
+    const uint8_t* abase = p.a + (EXP == 3 ? 0 : (int64_t)m0 * p.lda);
+    const uint8_t* bbase = p.b + (EXP == 3 ? 0 : (int64_t)n0 * p.ldb);
     const int64_t a_step = 32 * p.lda, b_step = 32 * p.ldb;
 
     // ---- LDS side
@@ -331,20 +332,68 @@ __global__ __launch_bounds__(256) void gemm_tile256_kernel(const GemmArgs p) {
         // The last MFMA step is cut into 16 scheduling regions of one MFMA, one DMA load and (for the
         // first 8) one fragment read each: issued as a burst, the loads back up the address unit and
         // block the in-order instruction stream, MFMAs included, behind them.
+        // INT8 keeps four fragment sets, one per MFMA step of a slice, and reads them two steps ahead:
+        // the HBM->LDS writes of the slice in flight share the LDS with these reads, and one step
+        // (16 MFMAs) of slack did not cover the delays that causes.  The barrier sits after step 1, when
+        // all fragments of the slice have been read; steps 2 and 3 then pull the next slice's first two
+        // fragment sets while step 2 also issues the loads of slice kt+2.
+        frag_t fa2[4] = {}, fb2[4] = {}, fa3[4] = {}, fb3[4] = {};
         auto slice = [&](int cur, auto ISSUE, auto NEXT) {
-            steps_but_last(cur);
-            // slice kt+1 has landed for every wave, and every wave is done reading slice kt
-            __builtin_amdgcn_s_waitcnt(vmcnt_imm(0) & lgkmcnt0_mask());
-            __builtin_amdgcn_s_barrier();
+            if constexpr (FP8) {
+                steps_but_last(cur);
+                // slice kt+1 has landed for every wave, and every wave is done reading slice kt
+                __builtin_amdgcn_s_waitcnt(vmcnt_imm(0) & lgkmcnt0_mask());
+                __builtin_amdgcn_s_barrier();
 #pragma unroll
-            for (int g = 0; g < 16; ++g) {
-                if constexpr (ISSUE.value) issue_one(cur, g);
-                if constexpr (NEXT.value && EXP != 2)
-                    if (g < 8) load_one_frag<FP8>(fa, cur ^ 1, g, fa0, fb0);
-                if constexpr (EXP != 2) mfma_one<FP8, XE5>(acc, g, fa1, fb1);
-                __builtin_amdgcn_sched_barrier(0);
+                for (int g = 0; g < 16; ++g) {
+                    if constexpr (ISSUE.value) issue_one(cur, g);
+                    if constexpr (NEXT.value && EXP != 2)
+                        if (g < 8) load_one_frag<FP8>(fa, cur ^ 1, g, fa0, fb0);
+                    if constexpr (EXP != 2) mfma_one<FP8, XE5>(acc, g, fa1, fb1);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                if constexpr (ISSUE.value) advance();
+            } else {
+                if constexpr (EXP != 2) {
+                    load_frags<FP8>(fa, cur, 2, fa2, fb2);
+                    mfma_step<FP8, XE5>(acc, fa0, fb0);
+#pragma unroll
+                    for (int g = 0; g < 8; ++g) {
+                        __builtin_amdgcn_sched_group_barrier(DAXQ_SG_DS_RD, 1, 0);
+                        __builtin_amdgcn_sched_group_barrier(DAXQ_SG_MFMA, 2, 0);
+                    }
+                    load_frags<FP8>(fa, cur, 3, fa3, fb3);
+                    mfma_step<FP8, XE5>(acc, fa1, fb1);
+#pragma unroll
+                    for (int g = 0; g < 8; ++g) {  // reads first, so that they are over when the barrier comes
+                        __builtin_amdgcn_sched_group_barrier(DAXQ_SG_DS_RD, 1, 0);
+                        __builtin_amdgcn_sched_group_barrier(DAXQ_SG_MFMA, 1, 0);
+                    }
+                }
+                // slice kt+1 has landed for every wave, and every wave has read all of slice kt
+                __builtin_amdgcn_s_waitcnt(vmcnt_imm(0) & lgkmcnt0_mask());
+                __builtin_amdgcn_s_barrier();
+#pragma unroll
+                for (int g = 0; g < 16; ++g) {
+                    if constexpr (ISSUE.value) issue_one(cur, g);
+                    if constexpr (NEXT.value && EXP != 2)
+                        if (g < 8) load_one_frag<FP8>(fa, cur ^ 1, g, fa0, fb0);
+                    if constexpr (EXP != 2) mfma_one<FP8, XE5>(acc, g, fa2, fb2);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                if constexpr (ISSUE.value) advance();
+                if constexpr (EXP != 2) {
+                    if constexpr (NEXT.value) load_frags<FP8>(fa, cur ^ 1, 1, fa1, fb1);
+                    mfma_step<FP8, XE5>(acc, fa3, fb3);
+                    if constexpr (NEXT.value) {
+#pragma unroll
+                        for (int g = 0; g < 8; ++g) {
+                            __builtin_amdgcn_sched_group_barrier(DAXQ_SG_DS_RD, 1, 0);
+                            __builtin_amdgcn_sched_group_barrier(DAXQ_SG_MFMA, 2, 0);
+                        }
+                    }
+                }
             }
-            if constexpr (ISSUE.value) advance();
         };
         issue(0);
         if (KT > 1) {
@@ -355,6 +404,7 @@ __global__ __launch_bounds__(256) void gemm_tile256_kernel(const GemmArgs p) {
         }
         __builtin_amdgcn_s_barrier();
         next_frags(0);
+        if constexpr (!FP8 && EXP != 2) load_frags<FP8>(fa, 0, 1, fa1, fb1);
         int kt = 0;
         for (; kt + 2 < KT; ++kt) slice(kt & 1, Yes{}, Yes{});
         if (kt + 1 < KT) {
@@ -403,6 +453,7 @@ int launch_tile256_experiment(const GemmArgs& a0, int exp, hipStream_t st) {
     GemmArgs a = a0;
     a.tiles_m = (a.m + BM - 1) / BM;
     a.tiles_n = (a.n + BN - 1) / BN;
+    if (exp == 3) return launch_tile256_impl<false, false, 3>(a, st);
     return exp == 1 ? launch_tile256_impl<false, false, 1>(a, st) : launch_tile256_impl<false, false, 2>(a, st);
 }
 

@@ -290,7 +290,8 @@ static int launch_gemm(const void* xq, int64_t ld_xq, const float* sx, const voi
             if (!tile256_applies(a)) return fail(DAXQ_ERR_ARG, "linear: the 256x256 kernel needs m, n >= 256");
             return launch_tile256<FP8>(a, x_e5m2, st);
         case 101:
-        case 102: return launch_tile256_experiment(a, g_variant - 100, st);
+        case 102:
+        case 103: return launch_tile256_experiment(a, g_variant - 100, st);
         default: return fail(DAXQ_ERR_ARG, "linear: unknown gemm variant %d", g_variant);
     }
 }
@@ -304,7 +305,7 @@ int daxq_set_gemm_variant(int variant) {
         daxq::g_gm = variant - 1000 > 0 ? variant - 1000 : 8;
         return DAXQ_OK;
     }
-    if (variant != 0 && variant != 2 && variant != 5 && variant != 6 && variant != 101 && variant != 102)
+    if (variant != 0 && variant != 2 && variant != 5 && variant != 6 && variant != 101 && variant != 102 && variant != 103)
         return daxq::fail(DAXQ_ERR_ARG, "unknown gemm variant %d", variant);
     daxq::g_variant = variant;
     return DAXQ_OK;
