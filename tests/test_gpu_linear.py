@@ -44,7 +44,7 @@ def dev(t):
 
 
 GEMM_SHAPES = [(256, 256, 128), (300, 520, 256), (1, 8, 128), (17, 24, 384), (512, 1536, 1536), (1000, 72, 640),
-               (257, 257, 128), (4096, 1536, 1536)]
+               (257, 257, 128), (4096, 1536, 1536), (200, 392, 384)]
 
 
 @pytest.mark.parametrize("variant", VARIANTS)
