@@ -75,6 +75,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--dtype", choices=["int8", "fp8"], default="int8")
     ap.add_argument("--variant", type=int, default=0)
+    ap.add_argument("--tile-group", type=int, default=0, help="tile-order group depth (0 = library default)")
     ap.add_argument("--m", type=int, default=M_TOKENS)
     ap.add_argument("--cpu-rows", type=int, default=0, help="tokens in the CPU-baseline sample (0 = pick for 10-30 s)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -94,6 +95,8 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs an MI355X"
     _capi.require_gfx950(0)
     _capi.set_gemm_variant(args.variant)
+    if args.tile_group:
+        _capi.set_gemm_variant(1000 + args.tile_group)
     dev = torch.device("cuda:0")
     fp8 = args.dtype == "fp8"
     m = args.m
@@ -187,7 +190,7 @@ def main():
         "pct_of_mfma_peak": round(100.0 * value / peak, 2),
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": peak, "unit": "TFLOP/s",
                      "frac": round(achieved / peak, 4), "traffic": GEMM_TRAFFIC_BYTES[args.dtype] if m == M_TOKENS else None,
-                     "kernel": "gemm_tile256_kernel, average launch over the four shapes; 8-bit ops counted as 2*M*N*K",
+                     "kernel": "gemm_tile256s5_kernel, average launch over the four shapes; 8-bit ops counted as 2*M*N*K",
                      "gemm_ms_per_step": round(gemm_ms_sum, 4), "quant_ms_per_step": round(quant_ms_sum, 4)},
         "per_linear": per_layer,
         "device": {"arch": info["arch"], "cu_count": info["cu_count"], "max_clock_mhz": info["clock_khz"] / 1000.0},

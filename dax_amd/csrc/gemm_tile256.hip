@@ -447,6 +447,220 @@ int launch_tile256(const GemmArgs& a0, bool x_e5m2, hipStream_t st) {
     return a.acc ? launch_tile256_impl<FP8, true>(a, st) : launch_tile256_impl<FP8, false>(a, st);
 }
 
+// ---------------------------------------------------------------------------------------------
+// Five-stage form of the same tile: K in 64-byte slices, five 32 KB LDS stages (all 160 KB).
+//
+// The two-stage kernel above issues the 16 loads of a 128-byte slice in a burst (one per MFMA of one
+// step) and gives them between one and two MFMA steps less than a slice time to land.  Here a stage is
+// half as deep, so the same LDS holds the slice being read plus four more, and the load stream is
+// even: 8 loads per 64-byte slice, one every fourth (INT8) or second (FP8) MFMA.
+//   * loads are issued in pairs of slices (2q, 2q+1) so that the two 64-byte halves of a 128-byte
+//     line are requested by adjacent instructions (the second hits L1: measured at the full-line
+//     rate, whereas half lines requested a slice apart run at half of it);
+//   * the A loads of pair q+2 go out during slice 2q, its B loads during slice 2q+1; the pair has to
+//     have landed at the barrier of slice 2q+3;
+//   * fragments of slice s+1 are read during slice s into the other of two register sets.
+// LDS layout of an operand part: [256 rows][64 B], 16-byte chunk c of row r stored at chunk
+// c ^ ((r >> 2) & 3): 16 consecutive lanes (rows) of a ds_read_b128 then cover all 64 banks once.
+namespace t5 {
+constexpr int BKS = 64, NST = 5, T = 256;
+constexpr int A_BYTES = 256 * BKS, STAGE = 2 * A_BYTES;  // 16 KB, 32 KB
+constexpr int SMEM = NST * STAGE;                        // 163840
+constexpr int PAIR_LOADS = 16;                           // per thread and pair of slices
+}  // namespace t5
+
+template <bool FP8, bool DUMP, bool XE5>
+__global__ __launch_bounds__(256) void gemm_tile256s5_kernel(const GemmArgs p) {
+    using namespace t5;
+    typedef typename AccT<FP8>::type acc_t;
+    typedef typename Frag<FP8>::type frag_t;
+    constexpr int STEPS = FP8 ? 1 : 2;               // MFMA steps per 64-byte slice
+    constexpr int NREG = 16 * STEPS;                 // MFMAs = scheduling regions per slice
+    constexpr int DMA_EVERY = NREG / (PAIR_LOADS / 2);  // regions per DMA load
+
+    extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    int tm, tn;
+    tile_of_block(p.gm, blockIdx.x, p.tiles_m, p.tiles_n, tm, tn);
+    int m0 = tm * 256, n0 = tn * 256;
+    m0 = m0 + 256 <= p.m ? m0 : p.m - 256;
+    n0 = n0 + 256 <= p.n ? n0 : p.n - 256;
+
+    // ---- HBM side.  One wave instruction fills 1 KB of LDS = 16 rows x 64 B: lane l -> row l/4,
+    //      stored chunk l%4, i.e. global chunk (l%4) ^ ((row>>2)&3).  Instruction j of a thread
+    //      covers tile rows j*64 + t/4.
+    const uint32_t gsw = (uint32_t)(((t & 3) ^ ((t >> 4) & 3)) << 4);
+    uint32_t voff_a = (uint32_t)(t >> 2) * (uint32_t)p.lda + gsw;
+    uint32_t voff_b = (uint32_t)(t >> 2) * (uint32_t)p.ldb + gsw;
+    const uint8_t* abase = p.a + (int64_t)m0 * p.lda;
+    const uint8_t* bbase = p.b + (int64_t)n0 * p.ldb;
+    const int64_t a_step = 64 * p.lda, b_step = 64 * p.ldb;
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(DAXQ_LDS uint8_t*)smem;
+    const uint32_t wave_lds = lds0 + (uint32_t)__builtin_amdgcn_readfirstlane(wave * 1024);
+    // load g = 0..15 of a pair: operand g/8 (0 = A), row block (g/2)%4, half g%2 -> stage o0 / o1
+    auto issue_one = [&](uint32_t o0, uint32_t o1, int g) {
+        const int opnd = g >> 3, j = (g >> 1) & 3, half = g & 1;
+        const uint8_t* src = (opnd ? bbase + j * b_step : abase + j * a_step) + half * BKS;
+        const uint32_t dst = wave_lds + (half ? o1 : o0) + opnd * A_BYTES + j * 4096;
+        __builtin_amdgcn_global_load_lds((const DAXQ_GLOBAL void*)(src + (opnd ? voff_b : voff_a)), (DAXQ_LDS void*)(uintptr_t)dst, 16, 0, 0);
+    };
+    auto advance = [&]() {
+        voff_a += 2 * BKS;
+        voff_b += 2 * BKS;
+    };
+
+    // ---- LDS side: row (w*128 + i*32 + l%32), chunk c of the slice at (c ^ g) * 16, g = (l%32 >> 2) & 3
+    const int l31 = lane & 31, hi = lane >> 5;
+    const int gq = (l31 >> 2) & 3;
+    const uint8_t* a_rd = smem + (wm * 128 + l31) * BKS;
+    const uint8_t* b_rd = smem + A_BYTES + (wn * 128 + l31) * BKS;
+    // one fragment: f = 0..3 A block f, 4..7 B block f-4; step ks of the slice in the stage at offset o
+    auto read_frag = [&](uint32_t o, int ks, int f, frag_t (&af)[4], frag_t (&bf)[4]) {
+        const uint8_t* pr = (f < 4 ? a_rd : b_rd) + o + (f & 3) * 32 * BKS;
+        if constexpr (!FP8) {
+            const int xo = ((ks * 2 + hi) ^ gq) << 4;
+            (f < 4 ? af[f & 3] : bf[f & 3]) = *reinterpret_cast<const v4i*>(pr + xo);
+        } else {
+            const int xo0 = ((hi * 2) ^ gq) << 4, xo1 = ((hi * 2 + 1) ^ gq) << 4;
+            v4i lo = *reinterpret_cast<const v4i*>(pr + xo0);
+            v4i up = *reinterpret_cast<const v4i*>(pr + xo1);
+            (f < 4 ? af[f & 3] : bf[f & 3]) = __builtin_shufflevector(lo, up, 0, 1, 2, 3, 4, 5, 6, 7);
+        }
+    };
+
+    acc_t acc[4][4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[j][i][v] = 0;
+
+    // fragment sets: [slice parity][MFMA step]
+    frag_t fa00[4] = {}, fb00[4] = {}, fa01[4] = {}, fb01[4] = {}, fa10[4] = {}, fb10[4] = {}, fa11[4] = {}, fb11[4] = {};
+
+    const int S = p.k / BKS;  // slices; even because K is a multiple of 128
+    // stage offsets of slices s .. s+4 (s = the even slice of the current pair)
+    uint32_t st0 = 0, st1 = STAGE, st2 = 2 * STAGE, st3 = 3 * STAGE, st4 = 4 * STAGE;
+
+    // One slice.  ODD: slice parity (which register set is consumed).  At its barrier slice s+1 has
+    // landed for every wave and every wave has the fragments of slice s in registers.
+    //   ISSUE  start half of pair (s+4, s+5) (s even: the A loads; s odd: the B loads of the same
+    //          pair) into the stages o_ld0 / o_ld1 that slices s-1 and s have left
+    //   NEXT   slice s+1 exists: read its fragments into the other set
+    //   YOUNG  loads issued after those of slice s+1 exist and may stay in flight: a whole pair at
+    //          an even slice, the A half of the newest pair at an odd one (vmcnt retires in order)
+    auto slice = [&](auto ODD, auto ISSUE, auto NEXT, auto YOUNG, uint32_t o_next, uint32_t o_ld0, uint32_t o_ld1) {
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm(YOUNG.value ? (ODD.value ? PAIR_LOADS / 2 : PAIR_LOADS) : 0) & lgkmcnt0_mask());
+        __builtin_amdgcn_s_barrier();
+#pragma unroll
+        for (int g = 0; g < NREG; ++g) {
+            if constexpr (ISSUE.value) {
+                if (g % DMA_EVERY == 0) issue_one(o_ld0, o_ld1, g / DMA_EVERY + (ODD.value ? PAIR_LOADS / 2 : 0));
+            }
+            if constexpr (NEXT.value) {
+                if constexpr (!FP8) {  // 16 reads: step 0 set in regions 0..7, step 1 set in regions 8..15
+                    if (g < 8) {
+                        if constexpr (ODD.value) read_frag(o_next, 0, g, fa00, fb00);
+                        else read_frag(o_next, 0, g, fa10, fb10);
+                    } else if (g < 16) {
+                        if constexpr (ODD.value) read_frag(o_next, 1, g - 8, fa01, fb01);
+                        else read_frag(o_next, 1, g - 8, fa11, fb11);
+                    }
+                } else {
+                    if (g < 8) {
+                        if constexpr (ODD.value) read_frag(o_next, 0, g, fa00, fb00);
+                        else read_frag(o_next, 0, g, fa10, fb10);
+                    }
+                }
+            }
+            if constexpr (!FP8) {
+                if constexpr (ODD.value) {
+                    if (g < 16) mfma_one<FP8, XE5>(acc, g, fa10, fb10);
+                    else mfma_one<FP8, XE5>(acc, g - 16, fa11, fb11);
+                } else {
+                    if (g < 16) mfma_one<FP8, XE5>(acc, g, fa00, fb00);
+                    else mfma_one<FP8, XE5>(acc, g - 16, fa01, fb01);
+                }
+            } else {
+                if constexpr (ODD.value) mfma_one<FP8, XE5>(acc, g, fa10, fb10);
+                else mfma_one<FP8, XE5>(acc, g, fa00, fb00);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        if constexpr (ISSUE.value && ODD.value) advance();
+    };
+    // a pair of slices (s, s+1), s even; YOUNG of the odd slice equals ISSUE (the pair this one started)
+    auto pair = [&](auto ISSUE, auto YOUNG_E, auto NEXT_O) {
+        slice(No{}, ISSUE, Yes{}, YOUNG_E, st1, st4, st0);
+        slice(Yes{}, ISSUE, NEXT_O, ISSUE, st2, st4, st0);
+        const uint32_t r0 = st0, r1 = st1;
+        st0 = st2;
+        st1 = st3;
+        st2 = st4;
+        st3 = r0;
+        st4 = r1;
+    };
+
+    // ---- prologue: pairs 0 and 1 in flight, pair 0 landed, fragments of slice 0 in set 0
+#pragma unroll
+    for (int g = 0; g < PAIR_LOADS; ++g) issue_one(0, STAGE, g);
+    advance();
+    if (S >= 4) {
+#pragma unroll
+        for (int g = 0; g < PAIR_LOADS; ++g) issue_one(2 * STAGE, 3 * STAGE, g);
+        advance();
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm(PAIR_LOADS));
+    } else {
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+    }
+    __builtin_amdgcn_s_barrier();
+#pragma unroll
+    for (int f = 0; f < 8; ++f) {
+        read_frag(0, 0, f, fa00, fb00);
+        if constexpr (!FP8) read_frag(0, 1, f, fa01, fb01);
+    }
+
+    const int Q = S >> 1;  // pairs
+    for (int q = 0; q + 2 < Q; ++q) pair(Yes{}, Yes{}, Yes{});
+    if (Q >= 2) pair(No{}, Yes{}, Yes{});
+    pair(No{}, No{}, No{});
+
+    tile256_epilogue<FP8, DUMP>(p, acc, smem, m0, n0, t, wm, wn, l31, hi);
+}
+
+template <bool FP8, bool DUMP, bool XE5>
+static int launch_tile256s5_impl(const GemmArgs& a, hipStream_t st) {
+    using namespace t5;
+    auto kern = gemm_tile256s5_kernel<FP8, DUMP, XE5>;
+    static bool attr_done = false;
+    if (!attr_done) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, SMEM);
+        if (e != hipSuccess) return fail(DAXQ_ERR_LAUNCH, "hipFuncSetAttribute(%d bytes LDS): %s", SMEM, hipGetErrorString(e));
+        attr_done = true;
+    }
+    const int64_t nt = (int64_t)a.tiles_m * a.tiles_n;
+    if (nt > 0x7fffffff) return fail(DAXQ_ERR_ARG, "gemm: too many tiles");
+    hipLaunchKernelGGL(kern, dim3((unsigned)nt), dim3(T), SMEM, st, a);
+    return check_launch("gemm_tile256s5");
+}
+
+template <bool FP8>
+int launch_tile256s5(const GemmArgs& a0, bool x_e5m2, hipStream_t st) {
+    GemmArgs a = a0;
+    a.tiles_m = (a.m + 255) / 256;
+    a.tiles_n = (a.n + 255) / 256;
+    if constexpr (FP8) {
+        if (x_e5m2) return a.acc ? launch_tile256s5_impl<true, true, true>(a, st) : launch_tile256s5_impl<true, false, true>(a, st);
+    }
+    return a.acc ? launch_tile256s5_impl<FP8, true, false>(a, st) : launch_tile256s5_impl<FP8, false, false>(a, st);
+}
+
+template int launch_tile256s5<false>(const GemmArgs&, bool, hipStream_t);
+template int launch_tile256s5<true>(const GemmArgs&, bool, hipStream_t);
+
 // timing experiments (INT8 only): exp 1 = no HBM loads in the steady state, 2 = loads only
 int launch_tile256_experiment(const GemmArgs& a0, int exp, hipStream_t st) {
     using namespace t256;

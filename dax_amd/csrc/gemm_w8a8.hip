@@ -209,12 +209,14 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_w8a8_kernel(const GemmArgs p
 }
 
 static int g_variant = 0;
-static int g_gm = 8;
+static int g_gm = 4;
 
 template <bool FP8>
 int launch_tile256(const GemmArgs& a, bool x_e5m2, hipStream_t st);
 bool tile256_applies(const GemmArgs& a);
 int launch_tile256_experiment(const GemmArgs& a, int exp, hipStream_t st);
+template <bool FP8>
+int launch_tile256s5(const GemmArgs& a, bool x_e5m2, hipStream_t st);
 
 template <bool FP8, int BM, int BN, int BK, int WM, int WN, bool DIRECT, bool XE5 = false>
 static int launch_cfg(const GemmArgs& a0, hipStream_t st) {
@@ -268,11 +270,11 @@ static int launch_gemm(const void* xq, int64_t ld_xq, const float* sx, const voi
     a.gm = g_gm;
     switch (g_variant) {
         case 0: {
-            // library default: the 256x256 kernel once its tiles fill at least half of the 256 CUs,
-            // otherwise 128x128 tiles (4x as many workgroups; measured cross-over between M = 1024
-            // and M = 2048 at N = K = 5120)
+            // library default: the five-stage 256x256 kernel once its tiles fill at least half of the
+            // 256 CUs, otherwise 128x128 tiles (4x as many workgroups; measured cross-over between
+            // M = 1024 and M = 2048 at N = K = 5120)
             const int64_t tiles256 = ((m + 255) / 256) * ((n + 255) / 256);
-            if (tile256_applies(a) && tiles256 >= 128) return launch_tile256<FP8>(a, x_e5m2, st);
+            if (tile256_applies(a) && tiles256 >= 128) return launch_tile256s5<FP8>(a, x_e5m2, st);
             if constexpr (FP8) {
                 if (x_e5m2) return launch_cfg<true, 128, 128, 128, 2, 2, true, true>(a, st);
             }
@@ -289,6 +291,9 @@ static int launch_gemm(const void* xq, int64_t ld_xq, const float* sx, const voi
         case 6:
             if (!tile256_applies(a)) return fail(DAXQ_ERR_ARG, "linear: the 256x256 kernel needs m, n >= 256");
             return launch_tile256<FP8>(a, x_e5m2, st);
+        case 8:
+            if (!tile256_applies(a)) return fail(DAXQ_ERR_ARG, "linear: the 256x256 kernel needs m, n >= 256");
+            return launch_tile256s5<FP8>(a, x_e5m2, st);
         case 101:
         case 102:
         case 103: return launch_tile256_experiment(a, g_variant - 100, st);
@@ -302,10 +307,10 @@ extern "C" {
 
 int daxq_set_gemm_variant(int variant) {
     if (variant >= 1000 && variant < 1064) {  // tuning hook: 1000 + depth of the tile-order groups
-        daxq::g_gm = variant - 1000 > 0 ? variant - 1000 : 8;
+        daxq::g_gm = variant - 1000 > 0 ? variant - 1000 : 4;
         return DAXQ_OK;
     }
-    if (variant != 0 && variant != 2 && variant != 5 && variant != 6 && variant != 101 && variant != 102 && variant != 103)
+    if (variant != 0 && variant != 2 && variant != 5 && variant != 6 && variant != 8 && variant != 101 && variant != 102 && variant != 103)
         return daxq::fail(DAXQ_ERR_ARG, "unknown gemm variant %d", variant);
     daxq::g_variant = variant;
     return DAXQ_OK;
