@@ -51,6 +51,10 @@ struct Yes {
 struct No {
     static constexpr bool value = false;
 };
+template <int N>
+struct Int {
+    static constexpr int value = N;
+};
 
 // sched_group_barrier masks
 #define DAXQ_SG_MFMA 0x008
@@ -140,15 +144,17 @@ __device__ __forceinline__ void mfma_step(typename AccT<FP8>::type (&acc)[4][4],
 // Epilogue.  In a 32x32 block a lane owns output row m = l%32 and, in registers 4q..4q+3, the
 // columns n = 8q + 4*(l/32) + {0..3}.  Two v_permlane32_swap per pair of q give each lane 8
 // consecutive columns, stored as one 16-byte write.  The tile's scales and bias are staged in LDS.
+// pre_*: this thread's element (index t) of the tile's sx / sw / bias, already loaded by the caller.
 template <bool FP8, bool DUMP>
 __device__ __forceinline__ void tile256_epilogue(const GemmArgs& p, typename AccT<FP8>::type (&acc)[4][4], uint8_t* smem,
-                                                 int m0, int n0, int t, int wm, int wn, int l31, int hi) {
+                                                 int m0, int n0, int t, int wm, int wn, int l31, int hi, float pre_sx,
+                                                 float pre_sw, float pre_bias) {
     float* s_sx = reinterpret_cast<float*>(smem);
     float* s_sw = s_sx + 256;
     float* s_bias = s_sw + 256;
-    s_sx[t] = p.sx[m0 + t];
-    s_sw[t] = p.sw[n0 + t];
-    s_bias[t] = p.bias ? bf16_bits_to_f32(p.bias[n0 + t]) : -0.0f;  // x + (-0.0) == x bit for bit
+    s_sx[t] = pre_sx;
+    s_sw[t] = pre_sw;
+    s_bias[t] = pre_bias;
     __syncthreads();
 
     if constexpr (DUMP) {
@@ -415,7 +421,9 @@ __global__ __launch_bounds__(256) void gemm_tile256_kernel(const GemmArgs p) {
     }
 
     __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
-    tile256_epilogue<FP8, DUMP>(p, acc, smem, m0, n0, t, wm, wn, l31, hi);
+    // a missing bias is + (-0.0): x + (-0.0) == x bit for bit
+    tile256_epilogue<FP8, DUMP>(p, acc, smem, m0, n0, t, wm, wn, l31, hi, p.sx[m0 + t], p.sw[n0 + t],
+                                p.bias ? bf16_bits_to_f32(p.bias[n0 + t]) : -0.0f);
 }
 
 template <bool FP8, bool DUMP, int EXP = 0, bool XE5 = false>
@@ -552,8 +560,9 @@ __global__ __launch_bounds__(256) void gemm_tile256s5_kernel(const GemmArgs p) {
     //   NEXT   slice s+1 exists: read its fragments into the other set
     //   YOUNG  loads issued after those of slice s+1 exist and may stay in flight: a whole pair at
     //          an even slice, the A half of the newest pair at an odd one (vmcnt retires in order)
-    auto slice = [&](auto ODD, auto ISSUE, auto NEXT, auto YOUNG, uint32_t o_next, uint32_t o_ld0, uint32_t o_ld1) {
-        __builtin_amdgcn_s_waitcnt(vmcnt_imm(YOUNG.value ? (ODD.value ? PAIR_LOADS / 2 : PAIR_LOADS) : 0) & lgkmcnt0_mask());
+    //   EXTRA  younger loads that are not tile loads (the epilogue's scales) and may stay in flight
+    auto slice = [&](auto ODD, auto ISSUE, auto NEXT, auto YOUNG, auto EXTRA, uint32_t o_next, uint32_t o_ld0, uint32_t o_ld1) {
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm((YOUNG.value ? (ODD.value ? PAIR_LOADS / 2 : PAIR_LOADS) : 0) + EXTRA.value) & lgkmcnt0_mask());
         __builtin_amdgcn_s_barrier();
 #pragma unroll
         for (int g = 0; g < NREG; ++g) {
@@ -593,9 +602,9 @@ __global__ __launch_bounds__(256) void gemm_tile256s5_kernel(const GemmArgs p) {
         if constexpr (ISSUE.value && ODD.value) advance();
     };
     // a pair of slices (s, s+1), s even; YOUNG of the odd slice equals ISSUE (the pair this one started)
-    auto pair = [&](auto ISSUE, auto YOUNG_E, auto NEXT_O) {
-        slice(No{}, ISSUE, Yes{}, YOUNG_E, st1, st4, st0);
-        slice(Yes{}, ISSUE, NEXT_O, ISSUE, st2, st4, st0);
+    auto pair = [&](auto ISSUE, auto YOUNG_E, auto NEXT_O, auto EXTRA) {
+        slice(No{}, ISSUE, Yes{}, YOUNG_E, EXTRA, st1, st4, st0);
+        slice(Yes{}, ISSUE, NEXT_O, ISSUE, EXTRA, st2, st4, st0);
         const uint32_t r0 = st0, r1 = st1;
         st0 = st2;
         st1 = st3;
@@ -624,11 +633,20 @@ __global__ __launch_bounds__(256) void gemm_tile256s5_kernel(const GemmArgs p) {
     }
 
     const int Q = S >> 1;  // pairs
-    for (int q = 0; q + 2 < Q; ++q) pair(Yes{}, Yes{}, Yes{});
-    if (Q >= 2) pair(No{}, Yes{}, Yes{});
-    pair(No{}, No{}, No{});
+    for (int q = 0; q + 2 < Q; ++q) pair(Yes{}, Yes{}, Yes{}, Int<0>{});
 
-    tile256_epilogue<FP8, DUMP>(p, acc, smem, m0, n0, t, wm, wn, l31, hi);
+    // The epilogue's scales and bias are requested here, behind the last tile loads, so that their
+    // latency is covered by the remaining two pairs of slices.  Always three loads (a missing bias
+    // reads a scale instead and is replaced by -0.0: x + (-0.0) == x bit for bit).
+    const float pre_sx = p.sx[m0 + t], pre_sw = p.sw[n0 + t];
+    const uint16_t pre_b = (p.bias ? p.bias : reinterpret_cast<const uint16_t*>(p.sw))[n0 + t];
+    __builtin_amdgcn_sched_barrier(0);
+
+    if (Q >= 2) pair(No{}, Yes{}, Yes{}, Int<3>{});
+    pair(No{}, No{}, No{}, Int<3>{});
+
+    tile256_epilogue<FP8, DUMP>(p, acc, smem, m0, n0, t, wm, wn, l31, hi, pre_sx, pre_sw,
+                                p.bias ? bf16_bits_to_f32(pre_b) : -0.0f);
 }
 
 template <bool FP8, bool DUMP, bool XE5>
