@@ -174,21 +174,34 @@ __device__ __forceinline__ void tile256_epilogue(const GemmArgs& p, typename Acc
             }
     }
 
+    // every scale and bias value this lane needs goes into registers in one burst of LDS reads
+    // (the fragment registers of the main loop are free now): 4 x sx, 16 x 4 sw, 16 x 4 bias
+    float sxr[4];
+    float4 swr[4][4], br[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) sxr[i] = s_sx[wm * 128 + i * 32 + l31];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const int nl = wn * 128 + j * 32 + 8 * q + 4 * hi;
+            swr[j][q] = *reinterpret_cast<const float4*>(s_sw + nl);
+            br[j][q] = *reinterpret_cast<const float4*>(s_bias + nl);
+        }
+    __builtin_amdgcn_sched_barrier(0);
+
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const int ml = wm * 128 + i * 32 + l31;
-        const float sxv = s_sx[ml];
+        const float sxv = sxr[i];
         uint16_t* orow = p.out + (int64_t)(m0 + ml) * p.ldo + n0 + wn * 128 + 8 * hi;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             uint32_t pk[4][2];
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
-                const int nl = wn * 128 + j * 32 + 8 * q + 4 * hi;
-                const float4 sw4 = *reinterpret_cast<const float4*>(s_sw + nl);
-                const float4 b4 = *reinterpret_cast<const float4*>(s_bias + nl);
-                const float sws[4] = {sw4.x, sw4.y, sw4.z, sw4.w};
-                const float bs[4] = {b4.x, b4.y, b4.z, b4.w};
+                const float sws[4] = {swr[j][q].x, swr[j][q].y, swr[j][q].z, swr[j][q].w};
+                const float bs[4] = {br[j][q].x, br[j][q].y, br[j][q].z, br[j][q].w};
 #pragma unroll
                 for (int h = 0; h < 2; ++h) {  // two columns at a time: v_cvt_pk_bf16_f32 rounds a pair (RNE)
                     const int r = 2 * h;
