@@ -1,26 +1,25 @@
-// 256x256-tile W8A8 GEMM for gfx950: the kernel the large DiT shapes run on.
+// 256x256-tile W8A8 GEMMs for gfx950: the kernels the large DiT shapes run on.
+//
+// Two forms of the same tile live here.  gemm_tile256s5_kernel (second half of the file, K in
+// 64-byte slices through five 32 KB LDS stages) is the one the library launches;
+// gemm_tile256_kernel (K in 128-byte slices, two 64 KB stages) came first and stays as a second
+// implementation for the tests and for timing experiments.  They share everything but the main loop.
 //
 // Work decomposition
 //   workgroup  256 x 256 outputs, 4 wavefronts (one per SIMD) in a 2 x 2 grid
 //   wavefront  128 x 128 outputs = 4 x 4 MFMA 32x32 blocks, 256 accumulator registers (AGPRs)
-//   K          128-byte slices; two 64 KB LDS buffers (A 32 KB + B 32 KB each)
-// A 2 x 2 wave grid is what minimises LDS reads per MFMA for a square tile: each K slice is
+// A 2 x 2 wave grid is what minimises LDS reads per MFMA for a square tile: 128 bytes of K are
 // read (2 + 2) * 256 * 128 B = 128 KB per workgroup against 128 MFMAs of 32 cycles per wave.
-// Rows are kept as whole 128-byte lines because L2 serves a 64-byte half line at the price of
-// a full one (measured: 17 TB/s against 33 TB/s device-wide).
 //
-// Data movement
+// Data movement of the two-stage form
 //   HBM/L2 -> LDS   global_load_lds_dwordx4 (no VGPR staging): 16 per thread and slice.  The 16-byte
 //                   chunk c of tile row r lands in LDS at chunk slot c ^ f(r); the swizzle is applied
 //                   to the global address because the LDS side of a DMA load is fixed (64 lanes in a row)
-//   LDS -> VGPR     ds_read_b128, bank-conflict free thanks to the swizzle, read one MFMA step
-//                   ahead into a second fragment register set
-//   one s_barrier per K slice, placed before the last MFMA step of the slice; that step is cut into
-//   16 scheduling regions of one MFMA + one DMA load + one fragment read so that the loads of slice
-//   kt+2 and the first fragments of slice kt+1 are spread over its MFMAs.
-// One slice is in flight while one is computed on.  A variant that staged two slices through 128
-// VGPRs to keep two slices in flight moved data faster but could not be register-allocated by the
-// compiler without spilling, and was dropped.
+//   LDS -> VGPR     ds_read_b128, bank-conflict free thanks to the swizzle, read one (FP8) or two
+//                   (INT8) MFMA steps ahead into further fragment register sets
+//   one s_barrier per K slice; the MFMA step after it is cut into 16 scheduling regions of one
+//   MFMA + one DMA load + one fragment read so that the loads of slice kt+2 and the first
+//   fragments of slice kt+1 are spread over its MFMAs.
 //
 // Tiles at the M / N edge are shifted inwards (origin min(tile*256, dim-256)) instead of being
 // predicated: the overlap rows are computed twice with identical results.  Shapes with
