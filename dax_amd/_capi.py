@@ -27,6 +27,12 @@ SIGNATURES = {
     "daxq_act_quant_i8": [_P, _I64, _I64, _I64, _P, _I64, _P, _P],
     "daxq_act_quant_e4m3": [_P, _I64, _I64, _I64, _P, _I64, _P, _P],
     "daxq_act_quant_e5m2": [_P, _I64, _I64, _I64, _P, _I64, _P, _P],
+    "daxq_layernorm_act_quant_i8": [_P, _I64, _I64, _I64, _P, _P, _I64, _F32, _P, _I64, _P, _I64, _P, _P],
+    "daxq_layernorm_act_quant_e4m3": [_P, _I64, _I64, _I64, _P, _P, _I64, _F32, _P, _I64, _P, _I64, _P, _P],
+    "daxq_layernorm_act_quant_e5m2": [_P, _I64, _I64, _I64, _P, _P, _I64, _F32, _P, _I64, _P, _I64, _P, _P],
+    "daxq_gelu_tanh_act_quant_i8": [_P, _I64, _I64, _I64, _P, _I64, _P, _I64, _P, _P],
+    "daxq_gelu_tanh_act_quant_e4m3": [_P, _I64, _I64, _I64, _P, _I64, _P, _I64, _P, _P],
+    "daxq_gelu_tanh_act_quant_e5m2": [_P, _I64, _I64, _I64, _P, _I64, _P, _I64, _P, _P],
     "daxq_quantize_rows_i8": [_P, _I64, _I64, _I64, _P, _P, _I64, _P],
     "daxq_quantize_rows_e4m3": [_P, _I64, _I64, _I64, _P, _P, _I64, _P],
     "daxq_row_minmax": [_P, _I64, _I64, _I64, _P, _P, _P],

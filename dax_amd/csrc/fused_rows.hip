@@ -1,0 +1,273 @@
+// Producer + per-token quantiser in one pass over the activation.
+//
+// Inside the DiT block the input of a quantised linear is produced by a row-local operation:
+//   * LayerNorm (fp32 statistics) followed by a per-column multiply-add -- the adaLN modulation
+//     norm(x) * (1 + scale) + shift in front of the self-attention and FFN projections, or the
+//     LayerNorm's own weight / bias in front of the cross-attention projections;
+//   * GELU (tanh form) between the two FFN linears.
+// Run eagerly, the producer writes a bf16 [M, K] tensor that the quantiser reads back; under the
+// reference's torch.compile (dax/adapters/wan/functional.py:33-36) Inductor fuses the quantiser's
+// row reduction (dax/quant/nn/dynamic/functional.py:124-129) into the producing kernel.  These
+// kernels are that fusion written out: one wavefront owns a row, keeps it in VGPRs, applies the
+// producer in fp32, rounds to bf16 exactly where the unfused graph would (the value the reference
+// quantises is the bf16 tensor), and then runs the same abs-max / scale / leaf-quantiser code as
+// quant_rows.hip.  The bf16 tensor itself is only written when the caller asks for it.
+//
+// HBM traffic: 2 B read + 1 B written per element (+ 2 B when the bf16 result is wanted), against
+// 2 + 2 + 2 + 1 for producer and quantiser run separately.  The GELU form is VALU-bound on gfx950
+// (one v_exp_f32 and one v_rcp_f32 per element), not HBM-bound.
+#include "quant_rows.h"
+
+namespace daxq {
+
+enum { PRE_LN = 1, PRE_GELU = 2 };
+
+__device__ __forceinline__ float wave_sum_f32(float v) {
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+
+__device__ __forceinline__ void unpack8(const uint4& v, float (&f)[8]) {
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int h = 0; h < 4; ++h) {
+        f[2 * h] = __uint_as_float(w[h] << 16);
+        f[2 * h + 1] = __uint_as_float(w[h] & 0xffff0000u);
+    }
+}
+
+__device__ __forceinline__ uint4 pack8(const float (&f)[8]) {
+    return make_uint4(pack_bf16_rne(f[0], f[1]), pack_bf16_rne(f[2], f[3]), pack_bf16_rne(f[4], f[5]),
+                      pack_bf16_rne(f[6], f[7]));
+}
+
+// gelu(x, approximate="tanh") = 0.5 x (1 + tanh(u)), u = sqrt(2/pi) (x + 0.044715 x^3), evaluated as
+// x / (1 + exp(-2u)): the same function without the cancellation in 1 + tanh(u) for negative x.
+__device__ __forceinline__ float gelu_tanh_f32(float x) {
+    constexpr float kBeta = 0.7978845608028654f, kKappa = 0.044715f, kLog2e = 1.4426950408889634f;
+    const float x2 = x * x;
+    const float u = kBeta * (x + kKappa * x2 * x);
+    const float e = __builtin_amdgcn_exp2f(-2.0f * kLog2e * u);  // exp(-2u); +inf for very negative x
+    return x * __builtin_amdgcn_rcpf(1.0f + e);                  // x * 0 = -0 there, as the limit
+}
+
+// One wavefront per row, 4 rows per workgroup pass, grid-stride over row quads.
+// PRE_LN: y = bf16( ((x - mean) * rstd) * mul[g][c] + add[g][c] ), g = row / rows_per_group; the two
+//         vectors of the workgroup's current group are staged in LDS (mul / add may be null: 1 / 0).
+// PRE_GELU: y = bf16( gelu_tanh(x) ).
+// Requires k % 8 == 0, 16-byte aligned rows of x (and y), 8-byte aligned rows of q, ld_q/8 <= NCH*64.
+template <int NCH, int FMT, int PRE, bool WRITE_Y>
+__global__ __launch_bounds__(256) void fused_rows_wave(const uint16_t* __restrict__ x, int64_t m, int k, int64_t ld_x,
+                                                       const float* __restrict__ mul, const float* __restrict__ add,
+                                                       int64_t rows_per_group, float eps, uint16_t* __restrict__ y,
+                                                       int64_t ld_y, uint8_t* __restrict__ q, int64_t ld_q,
+                                                       float* __restrict__ scale, float qmax) {
+    extern __shared__ __attribute__((aligned(16))) float s_vec[];  // PRE_LN: mul[k] then add[k]
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int nch = k >> 3;
+    const int npad = (int)(ld_q >> 3);
+    int64_t staged = -1;
+
+    for (int64_t row0 = (int64_t)blockIdx.x * 4; row0 < m; row0 += (int64_t)gridDim.x * 4) {
+        const int64_t row = row0 + wave;
+        if constexpr (PRE == PRE_LN) {
+            // the group of the quad's first row is staged; a wave whose row lies in another group
+            // (a quad that straddles a boundary) reads the vectors from memory instead
+            const int64_t g0 = row0 / rows_per_group;
+            if (g0 != staged) {
+                __syncthreads();  // everyone is done with the previous group's vectors
+                for (int c = threadIdx.x; c < k; c += 256) {
+                    s_vec[c] = mul ? mul[g0 * k + c] : 1.0f;
+                    s_vec[k + c] = add ? add[g0 * k + c] : 0.0f;
+                }
+                staged = g0;
+                __syncthreads();
+            }
+        }
+        if (row >= m) continue;
+
+        const uint4* xr = reinterpret_cast<const uint4*>(x + row * ld_x);
+        uint4 v[NCH];
+#pragma unroll
+        for (int i = 0; i < NCH; ++i) {
+            const int c = i * 64 + lane;
+            v[i] = c < nch ? xr[c] : make_uint4(0, 0, 0, 0);
+        }
+
+        if constexpr (PRE == PRE_LN) {
+            // mean and biased variance in fp32, two passes over the registers
+            float sum = 0.0f;
+#pragma unroll
+            for (int i = 0; i < NCH; ++i) {
+                float f[8];
+                unpack8(v[i], f);  // padding chunks are zero and add nothing
+                sum += ((f[0] + f[1]) + (f[2] + f[3])) + ((f[4] + f[5]) + (f[6] + f[7]));
+            }
+            const float mean = wave_sum_f32(sum) / (float)k;
+            float ssq = 0.0f;
+#pragma unroll
+            for (int i = 0; i < NCH; ++i) {
+                if (i * 64 + lane < nch) {
+                    float f[8];
+                    unpack8(v[i], f);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        const float d = f[e] - mean;
+                        ssq += d * d;
+                    }
+                }
+            }
+            const float var = wave_sum_f32(ssq) / (float)k;
+            const float rstd = 1.0f / sqrtf(var + eps);  // IEEE sqrt and division
+            const int64_t g = row / rows_per_group;
+            const bool in_lds = g == staged;
+#pragma unroll
+            for (int i = 0; i < NCH; ++i) {
+                const int c = i * 64 + lane;
+                if (c < nch) {
+                    float f[8], a[8], b[8];
+                    unpack8(v[i], f);
+                    if (in_lds) {
+                        const float4 a0 = *reinterpret_cast<const float4*>(s_vec + c * 8);
+                        const float4 a1 = *reinterpret_cast<const float4*>(s_vec + c * 8 + 4);
+                        const float4 b0 = *reinterpret_cast<const float4*>(s_vec + k + c * 8);
+                        const float4 b1 = *reinterpret_cast<const float4*>(s_vec + k + c * 8 + 4);
+                        a[0] = a0.x, a[1] = a0.y, a[2] = a0.z, a[3] = a0.w, a[4] = a1.x, a[5] = a1.y, a[6] = a1.z, a[7] = a1.w;
+                        b[0] = b0.x, b[1] = b0.y, b[2] = b0.z, b[3] = b0.w, b[4] = b1.x, b[5] = b1.y, b[6] = b1.z, b[7] = b1.w;
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) {
+                            a[e] = mul ? mul[g * k + c * 8 + e] : 1.0f;
+                            b[e] = add ? add[g * k + c * 8 + e] : 0.0f;
+                        }
+                    }
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        // three separately rounded fp32 operations, like the unfused graph
+                        const float xh = __fmul_rn(f[e] - mean, rstd);
+                        f[e] = __fadd_rn(__fmul_rn(xh, a[e]), b[e]);
+                    }
+                    v[i] = pack8(f);
+                }
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < NCH; ++i) {
+                if (i * 64 + lane < nch) {
+                    float f[8];
+                    unpack8(v[i], f);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) f[e] = gelu_tanh_f32(f[e]);
+                    v[i] = pack8(f);
+                }
+            }
+        }
+
+        if constexpr (WRITE_Y) {
+            uint4* yr = reinterpret_cast<uint4*>(y + row * ld_y);
+#pragma unroll
+            for (int i = 0; i < NCH; ++i) {
+                const int c = i * 64 + lane;
+                if (c < nch) yr[c] = v[i];
+            }
+        }
+
+        // ---- from here on: the per-token quantiser of quant_rows.hip on the bf16 values
+        uint32_t mx = 0;
+#pragma unroll
+        for (int i = 0; i < NCH; ++i) mx = chunk_absmax(mx, v[i]);
+        uint32_t amax = (mx & 0xffffu) > (mx >> 16) ? (mx & 0xffffu) : (mx >> 16);
+        amax = wave_max_u32(amax);
+        const float s = scale_from_amax_bits<true>(amax, qmax);
+        if (lane == 0) scale[row] = s;
+        const float inv = 1.0f / s;
+        uint2* qr = reinterpret_cast<uint2*>(q + row * ld_q);
+#pragma unroll
+        for (int i = 0; i < NCH; ++i) {
+            const int c = i * 64 + lane;
+            if (c < nch) {
+                qr[c] = quant_chunk<FMT>(v[i], s, inv);
+            } else if (c < npad) {
+                qr[c] = make_uint2(0, 0);
+            }
+        }
+    }
+}
+
+template <int FMT, int PRE>
+static int launch_fused_rows(const char* what, const void* x, int64_t m, int64_t k, int64_t ld_x, const float* mul,
+                             const float* add, int64_t rows_per_group, float eps, void* y, int64_t ld_y, void* q,
+                             int64_t ld_q, float* scale, float qmax, hipStream_t st) {
+    if (m < 0 || k <= 0 || ld_x < k || ld_q < k || (y && ld_y < k))
+        return fail(DAXQ_ERR_ARG, "%s: bad shape m=%lld k=%lld ld_x=%lld ld_q=%lld", what, (long long)m, (long long)k,
+                    (long long)ld_x, (long long)ld_q);
+    if (PRE == PRE_LN && (rows_per_group <= 0 || !(eps >= 0.0f))) return fail(DAXQ_ERR_ARG, "%s: rows_per_group and eps must be positive", what);
+    if (m == 0) return DAXQ_OK;
+    if (!x || !q || !scale) return fail(DAXQ_ERR_ARG, "%s: null pointer", what);
+    // the row has to fit the registers of one wavefront and move in 16-byte pieces
+    const bool ok = (k % 8 == 0) && (ld_x % 8 == 0) && (ld_q % 8 == 0) && (!y || ld_y % 8 == 0) && (((uintptr_t)x & 15) == 0) &&
+                    (((uintptr_t)y & 15) == 0) && (((uintptr_t)q & 7) == 0) && (((uintptr_t)scale & 3) == 0) &&
+                    (((uintptr_t)mul & 3) == 0) && (((uintptr_t)add & 3) == 0) && (ld_q / 8 <= 28 * 64) &&
+                    (PRE != PRE_LN || k <= 8192);
+    if (!ok)
+        return fail(DAXQ_ERR_ALIGN, "%s: needs k %% 8 == 0, k <= 14336 (8192 with LayerNorm), 16-byte aligned rows of x / y and 8-byte aligned rows of q", what);
+    const uint16_t* xp = static_cast<const uint16_t*>(x);
+    uint16_t* yp = static_cast<uint16_t*>(y);
+    uint8_t* qp = static_cast<uint8_t*>(q);
+    const int nchunks = (int)((ld_q / 8 + 63) / 64);
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+        return fail(DAXQ_ERR_LAUNCH, "%s: cannot read the CU count", what);
+    // PRE_LN keeps its workgroups resident (as many as their LDS allows, at most 8 per CU) so that the staged vectors are reused over many
+    // rows; the GELU form has nothing to reuse and takes one quad of rows per workgroup
+    const int64_t quads = (m + 3) / 4;
+    const size_t lds = PRE == PRE_LN ? (size_t)k * 8 : 0;
+    const int64_t resident = lds ? (int64_t)(163840 / lds < 8 ? 163840 / lds : 8) : 8;
+    const int64_t want = PRE == PRE_LN ? (int64_t)cus * resident : quads;
+    const dim3 grid((unsigned)(quads < want ? quads : want)), block(256);
+#define DAXQ_F_CASE(N)                                                                                                   \
+    if (nchunks <= N) {                                                                                                  \
+        if (yp)                                                                                                          \
+            hipLaunchKernelGGL((fused_rows_wave<N, FMT, PRE, true>), grid, block, lds, st, xp, m, (int)k, ld_x, mul, add, \
+                               rows_per_group, eps, yp, ld_y, qp, ld_q, scale, qmax);                                    \
+        else                                                                                                             \
+            hipLaunchKernelGGL((fused_rows_wave<N, FMT, PRE, false>), grid, block, lds, st, xp, m, (int)k, ld_x, mul, add, \
+                               rows_per_group, eps, yp, ld_y, qp, ld_q, scale, qmax);                                    \
+        return check_launch(what);                                                                                       \
+    }
+    DAXQ_F_CASE(4)
+    DAXQ_F_CASE(12)
+    DAXQ_F_CASE(20)
+    DAXQ_F_CASE(28)
+#undef DAXQ_F_CASE
+    return fail(DAXQ_ERR_ARG, "%s: row too long", what);
+}
+
+}  // namespace daxq
+
+extern "C" {
+
+#define DAXQ_LN_ENTRY(NAME, FMT, QT, QMAX)                                                                                \
+    int NAME(const void* x, int64_t m, int64_t k, int64_t ld_x, const float* mul, const float* add, int64_t rows_per_group, \
+             float eps, void* y, int64_t ld_y, QT* q, int64_t ld_q, float* scale, daxq_stream_t stream) {                  \
+        return daxq::launch_fused_rows<FMT, daxq::PRE_LN>(#NAME, x, m, k, ld_x, mul, add, rows_per_group, eps, y, ld_y, q,  \
+                                                          ld_q, scale, QMAX, (hipStream_t)stream);                         \
+    }
+DAXQ_LN_ENTRY(daxq_layernorm_act_quant_i8, 0, int8_t, 127.0f)
+DAXQ_LN_ENTRY(daxq_layernorm_act_quant_e4m3, 1, uint8_t, 448.0f)
+DAXQ_LN_ENTRY(daxq_layernorm_act_quant_e5m2, 2, uint8_t, 57344.0f)
+#undef DAXQ_LN_ENTRY
+
+#define DAXQ_GELU_ENTRY(NAME, FMT, QT, QMAX)                                                                           \
+    int NAME(const void* x, int64_t m, int64_t k, int64_t ld_x, void* y, int64_t ld_y, QT* q, int64_t ld_q, float* scale, \
+             daxq_stream_t stream) {                                                                                   \
+        return daxq::launch_fused_rows<FMT, daxq::PRE_GELU>(#NAME, x, m, k, ld_x, nullptr, nullptr, 1, 0.0f, y, ld_y, q,  \
+                                                            ld_q, scale, QMAX, (hipStream_t)stream);                    \
+    }
+DAXQ_GELU_ENTRY(daxq_gelu_tanh_act_quant_i8, 0, int8_t, 127.0f)
+DAXQ_GELU_ENTRY(daxq_gelu_tanh_act_quant_e4m3, 1, uint8_t, 448.0f)
+DAXQ_GELU_ENTRY(daxq_gelu_tanh_act_quant_e5m2, 2, uint8_t, 57344.0f)
+#undef DAXQ_GELU_ENTRY
+
+}  // extern "C"

@@ -82,6 +82,111 @@ act_quant_e4m3.register_fake(lambda x: _act_quant_fake(x, torch.uint8))
 act_quant_e5m2.register_fake(lambda x: _act_quant_fake(x, torch.uint8))
 
 
+# ----------------------------------------------------------------------------- producer + act quant
+_FMT_NAMES = ("i8", "e4m3", "e5m2")
+
+
+def _fused_out(x: torch.Tensor, fmt: str, want_y: bool):
+    m, k = x.shape
+    q = torch.empty((m, pad_k(k)), dtype=torch.int8 if fmt == "i8" else torch.uint8, device=x.device)
+    s = torch.empty((m,), dtype=torch.float32, device=x.device)
+    y = torch.empty((m, k) if want_y else (0, k), dtype=torch.bfloat16, device=x.device)
+    return q, s, y
+
+
+def _vec_arg(v: Optional[torch.Tensor], x: torch.Tensor, groups: int, what: str) -> int:
+    if v is None:
+        return 0
+    if v.dtype != torch.float32 or v.device != x.device or not v.is_contiguous() or v.numel() != groups * x.shape[1]:
+        raise ValueError(f"daxq::{what}: mul / add must be contiguous fp32 [{groups}, {x.shape[1]}] on {x.device}")
+    return v.data_ptr()
+
+
+def _layernorm_act_quant(fmt: str, x, mul, add, rows_per_group: int, eps: float, want_y: bool):
+    name = "layernorm_act_quant_" + fmt
+    _rows_bf16(x, name)
+    m, k = x.shape
+    if rows_per_group <= 0:
+        raise ValueError(f"daxq::{name}: rows_per_group must be positive")
+    groups = max(1, -(-m // rows_per_group))
+    with torch.cuda.device(x.device):
+        q, s, y = _fused_out(x, fmt, want_y)
+        if m:
+            fn = getattr(_capi.lib(), "daxq_" + name)
+            ld_x = x.stride(0) if m > 1 else k
+            _capi.check(fn(x.data_ptr(), m, k, ld_x, _vec_arg(mul, x, groups, name), _vec_arg(add, x, groups, name),
+                           rows_per_group, eps, y.data_ptr() if want_y else 0, k, q.data_ptr(), q.shape[1],
+                           s.data_ptr(), _stream(x)), name)
+    return q, s, y
+
+
+def _gelu_tanh_act_quant(fmt: str, x, want_y: bool):
+    name = "gelu_tanh_act_quant_" + fmt
+    _rows_bf16(x, name)
+    m, k = x.shape
+    with torch.cuda.device(x.device):
+        q, s, y = _fused_out(x, fmt, want_y)
+        if m:
+            fn = getattr(_capi.lib(), "daxq_" + name)
+            ld_x = x.stride(0) if m > 1 else k
+            _capi.check(fn(x.data_ptr(), m, k, ld_x, y.data_ptr() if want_y else 0, k, q.data_ptr(), q.shape[1],
+                           s.data_ptr(), _stream(x)), name)
+    return q, s, y
+
+
+def _fused_fake(x, fmt, want_y):
+    return (x.new_empty((x.shape[0], pad_k(x.shape[1])), dtype=torch.int8 if fmt == "i8" else torch.uint8),
+            x.new_empty((x.shape[0],), dtype=torch.float32),
+            x.new_empty((x.shape[0] if want_y else 0, x.shape[1]), dtype=torch.bfloat16))
+
+
+@torch.library.custom_op("daxq::layernorm_act_quant_i8", mutates_args=(), device_types="cuda")
+def layernorm_act_quant_i8(x: torch.Tensor, mul: Optional[torch.Tensor], add: Optional[torch.Tensor],
+                           rows_per_group: int, eps: float,
+                           want_y: bool = False) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """y = bf16(layer_norm_f32(x, eps) * mul[row // rows_per_group] + add[...]) and its per-token int8
+    quantisation in one pass: (q [M, pad128(K)], scale [M], y [M, K] or an empty [0, K])."""
+    return _layernorm_act_quant("i8", x, mul, add, rows_per_group, eps, want_y)
+
+
+@torch.library.custom_op("daxq::layernorm_act_quant_e4m3", mutates_args=(), device_types="cuda")
+def layernorm_act_quant_e4m3(x: torch.Tensor, mul: Optional[torch.Tensor], add: Optional[torch.Tensor],
+                             rows_per_group: int, eps: float,
+                             want_y: bool = False) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    return _layernorm_act_quant("e4m3", x, mul, add, rows_per_group, eps, want_y)
+
+
+@torch.library.custom_op("daxq::layernorm_act_quant_e5m2", mutates_args=(), device_types="cuda")
+def layernorm_act_quant_e5m2(x: torch.Tensor, mul: Optional[torch.Tensor], add: Optional[torch.Tensor],
+                             rows_per_group: int, eps: float,
+                             want_y: bool = False) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    return _layernorm_act_quant("e5m2", x, mul, add, rows_per_group, eps, want_y)
+
+
+@torch.library.custom_op("daxq::gelu_tanh_act_quant_i8", mutates_args=(), device_types="cuda")
+def gelu_tanh_act_quant_i8(x: torch.Tensor, want_y: bool = False) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """y = bf16(gelu(x, approximate="tanh")) and its per-token int8 quantisation in one pass."""
+    return _gelu_tanh_act_quant("i8", x, want_y)
+
+
+@torch.library.custom_op("daxq::gelu_tanh_act_quant_e4m3", mutates_args=(), device_types="cuda")
+def gelu_tanh_act_quant_e4m3(x: torch.Tensor, want_y: bool = False) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    return _gelu_tanh_act_quant("e4m3", x, want_y)
+
+
+@torch.library.custom_op("daxq::gelu_tanh_act_quant_e5m2", mutates_args=(), device_types="cuda")
+def gelu_tanh_act_quant_e5m2(x: torch.Tensor, want_y: bool = False) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    return _gelu_tanh_act_quant("e5m2", x, want_y)
+
+
+layernorm_act_quant_i8.register_fake(lambda x, mul, add, rows_per_group, eps, want_y=False: _fused_fake(x, "i8", want_y))
+layernorm_act_quant_e4m3.register_fake(lambda x, mul, add, rows_per_group, eps, want_y=False: _fused_fake(x, "e4m3", want_y))
+layernorm_act_quant_e5m2.register_fake(lambda x, mul, add, rows_per_group, eps, want_y=False: _fused_fake(x, "e5m2", want_y))
+gelu_tanh_act_quant_i8.register_fake(lambda x, want_y=False: _fused_fake(x, "i8", want_y))
+gelu_tanh_act_quant_e4m3.register_fake(lambda x, want_y=False: _fused_fake(x, "e4m3", want_y))
+gelu_tanh_act_quant_e5m2.register_fake(lambda x, want_y=False: _fused_fake(x, "e5m2", want_y))
+
+
 # ----------------------------------------------------------------------------- leaf quantisers
 def _quantize_rows(x: torch.Tensor, scale: torch.Tensor, fp8: bool, padded: bool) -> torch.Tensor:
     name = "quantize_rows_e4m3" if fp8 else "quantize_rows_i8"

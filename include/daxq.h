@@ -76,6 +76,47 @@ int daxq_act_quant_e5m2(const void* x, int64_t m, int64_t k, int64_t ld_x,
                         uint8_t* q, int64_t ld_q, float* scale, daxq_stream_t stream);
 
 /*
+ * Producer fused with the per-token quantiser: LayerNorm + per-column multiply-add.
+ *   y = bf16( layer_norm_f32(x, eps) * mul[g] + add[g] ),  g = row / rows_per_group,  then y is quantised as above.
+ * This is the adaLN pattern of the DiT, whose operation order the reference spells out at
+ *   dax/adapters/wan/transformer_adapter.py:151-153   (norm(x.float()) * (1 + scale) + shift).type_as(x)
+ * (mul = 1 + scale, add = shift, one group per batch element), and a LayerNorm with its own weight and
+ * bias (mul = weight, add = bias, one group).  Under the reference's torch.compile
+ *   dax/adapters/wan/functional.py:33-36
+ * Inductor fuses the quantiser's row reduction (dax/quant/nn/dynamic/functional.py:124-129) into this
+ * producer; eagerly the bf16 tensor y makes a round trip through memory.
+ * x bf16 [m, k]; mul, add fp32 [groups, k] or NULL (1 / 0); y bf16 [m, ld_y] or NULL when only the
+ * quantised form is wanted; q, scale as for daxq_act_quant_*.  k % 8 == 0, k <= 8192, 16-byte aligned rows.
+ * Statistics in fp32 (mean, biased variance, 1/sqrt(var + eps)); floating point: results match an fp32
+ * LayerNorm to its rounding, not bit for bit.
+ */
+int daxq_layernorm_act_quant_i8(const void* x, int64_t m, int64_t k, int64_t ld_x, const float* mul, const float* add,
+                                int64_t rows_per_group, float eps, void* y, int64_t ld_y,
+                                int8_t* q, int64_t ld_q, float* scale, daxq_stream_t stream);
+int daxq_layernorm_act_quant_e4m3(const void* x, int64_t m, int64_t k, int64_t ld_x, const float* mul, const float* add,
+                                  int64_t rows_per_group, float eps, void* y, int64_t ld_y,
+                                  uint8_t* q, int64_t ld_q, float* scale, daxq_stream_t stream);
+int daxq_layernorm_act_quant_e5m2(const void* x, int64_t m, int64_t k, int64_t ld_x, const float* mul, const float* add,
+                                  int64_t rows_per_group, float eps, void* y, int64_t ld_y,
+                                  uint8_t* q, int64_t ld_q, float* scale, daxq_stream_t stream);
+
+/*
+ * Producer fused with the per-token quantiser: GELU in its tanh form, the activation between the two
+ * FFN linears of the DiT (the second one, 13824 -> 5120, is where the unfused quantiser reads 3.1 GB).
+ *   y = bf16( gelu(f32(x), approximate="tanh") ), then y is quantised as above.
+ * Same fusion as above (dax/adapters/wan/functional.py:33-36 over dax/quant/nn/dynamic/functional.py:124-129).
+ * x bf16 [m, k], k % 8 == 0, k <= 14336; y bf16 [m, ld_y] or NULL; q, scale as for daxq_act_quant_*.
+ * Floating point: exp and reciprocal are the hardware approximations (1 ulp), results match torch's
+ * gelu to bf16 rounding, not bit for bit.
+ */
+int daxq_gelu_tanh_act_quant_i8(const void* x, int64_t m, int64_t k, int64_t ld_x, void* y, int64_t ld_y,
+                                int8_t* q, int64_t ld_q, float* scale, daxq_stream_t stream);
+int daxq_gelu_tanh_act_quant_e4m3(const void* x, int64_t m, int64_t k, int64_t ld_x, void* y, int64_t ld_y,
+                                  uint8_t* q, int64_t ld_q, float* scale, daxq_stream_t stream);
+int daxq_gelu_tanh_act_quant_e5m2(const void* x, int64_t m, int64_t k, int64_t ld_x, void* y, int64_t ld_y,
+                                  uint8_t* q, int64_t ld_q, float* scale, daxq_stream_t stream);
+
+/*
  * Leaf quantisers with a caller-supplied per-row scale (used once per weight at conversion).
  * Replace quantize_to_int8 / quantize_to_fp8 with a [rows,1] scale
  *   dax/quant/nn/quantized/functional.py:11-20, called from dax/quant/nn/dynamic/linear.py:292-296

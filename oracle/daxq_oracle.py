@@ -24,6 +24,10 @@ How each function is pinned (see tests/test_oracle_*.py):
 * weight_scale / quant     C closed form, brute force on small matrices
 * int_mm                   numpy int64 brute force, adversarial +-127 / -128
 * linear_int8 epilogue     C closed form bf16(bf16(f32(acc)*sx*sw)+bias)
+* layernorm_affine_bf16    float64 statistics on random and constant rows; the bf16
+  gelu_tanh_bf16           result may differ from an exact evaluation by one ulp
+                           at rounding boundaries (floating point: tolerance
+                           stated in the tests); gelu checked on every bf16 input
 * linear_fp8               accumulation order is not fixed by the reference
                            (cuBLASLt fast-accum): "parity unpinned" at bit
                            level, tolerance 2e-2 relative L2; the per-tensor
@@ -234,3 +238,31 @@ def make_inputs(m: int, k: int, n: int, seed: int = 0):
     w = (torch.randn(n, k, generator=g) * 0.02).bfloat16()
     b = (torch.randn(n, generator=g) * 0.01).bfloat16()
     return x, w, b
+
+
+# --------------------------------------------------------------------------- #
+# producers in front of a quantised linear (what the fused kernels restate)
+# --------------------------------------------------------------------------- #
+def layernorm_affine_bf16(x: torch.Tensor, mul: Optional[torch.Tensor], add: Optional[torch.Tensor],
+                          rows_per_group: int, eps: float) -> torch.Tensor:
+    """``(norm(x.float()) * mul + add).type_as(x)`` with an fp32 LayerNorm without affine parameters and
+    one (mul, add) pair of fp32 [K] vectors per group of ``rows_per_group`` consecutive rows.
+
+    Operation order of dax/adapters/wan/transformer_adapter.py:151-153 (mul = 1 + scale, add = shift);
+    with mul = weight, add = bias and one group it is an affine fp32 LayerNorm cast back to bf16.
+    """
+    m, k = x.shape
+    y = torch.nn.functional.layer_norm(x.float(), (k,), None, None, eps)
+    g = torch.arange(m) // rows_per_group
+    if mul is not None:
+        y = y * mul.float().reshape(-1, k)[g]
+    if add is not None:
+        y = y + add.float().reshape(-1, k)[g]
+    return y.to(x.dtype)
+
+
+def gelu_tanh_bf16(x: torch.Tensor) -> torch.Tensor:
+    """``gelu(x, approximate="tanh")`` of a bf16 tensor: evaluated in fp32, rounded once to bf16
+    (the activation between the two FFN linears of the DiT)."""
+    return torch.nn.functional.gelu(x.float(), approximate="tanh").to(x.dtype)
+

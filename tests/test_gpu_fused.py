@@ -1,0 +1,122 @@
+"""GPU tests of the fused producer + quantiser kernels, through torch.ops.daxq -> C ABI.
+
+Two-part check.  The producer (LayerNorm multiply-add, GELU-tanh) is floating point: its bf16 result y
+must agree with the oracle to one bf16 step, and only at rounding boundaries (stated fractions below).
+The quantiser behind it is integer work: the scales and quantised bytes the kernel returns must equal,
+bit for bit, the oracle's quantiser applied to the kernel's own y.
+"""
+import pytest
+import torch
+
+from oracle import daxq_oracle as O
+from tests.util import FINITE_BF16, bf16_ulps, from_bits, rel_l2
+
+pytestmark = pytest.mark.gpu
+
+QUANT = {"i8": O.act_quant_int8, "e4m3": O.act_quant_e4m3, "e5m2": O.act_quant_e5m2}
+
+
+@pytest.fixture(scope="module")
+def ops():
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    import dax_amd.ops as ops
+
+    return ops
+
+
+def dev(t):
+    return None if t is None else t.to("cuda")
+
+
+def _check_quant_of_own_y(fmt, y_gpu, q_gpu, s_gpu, k):
+    q_ref, s_ref = QUANT[fmt](y_gpu.cpu())
+    assert torch.equal(s_gpu.cpu(), s_ref.view(-1))
+    q_ref = q_ref if fmt == "i8" else q_ref.view(torch.uint8)
+    assert torch.equal(q_gpu[:, :k].cpu(), q_ref)
+    assert int(q_gpu[:, k:].cpu().to(torch.int32).abs().sum()) == 0       # K padding is zero
+
+
+def _check_y(y_gpu, y_ref, max_frac):
+    ulps = bf16_ulps(y_gpu, y_ref)
+    tiny = (y_gpu.cpu().double() - y_ref.double()).abs() < 1e-6
+    assert bool(((ulps <= 1) | tiny).all()), int(ulps.max())
+    frac = float(((ulps > 0) & ~tiny).float().mean())
+    assert frac < max_frac, frac
+
+
+@pytest.mark.parametrize("fmt", ["i8", "e4m3", "e5m2"])
+def test_gelu_tanh_every_bf16_input(ops, fmt):
+    x = from_bits(FINITE_BF16)
+    pad = (-x.numel()) % 1024
+    x = torch.cat([x, x[:pad]]).reshape(-1, 1024)
+    q, s, y = getattr(ops, "gelu_tanh_act_quant_" + fmt)(dev(x), True)
+    _check_y(y, O.gelu_tanh_bf16(x), 1e-2)
+    _check_quant_of_own_y(fmt, y, q, s, 1024)
+
+
+@pytest.mark.parametrize("m,k", [(130, 13824), (257, 8960), (33, 1536), (1, 8), (5, 200)])
+def test_gelu_tanh_shapes_and_quant_only_form(ops, m, k):
+    g = torch.Generator().manual_seed(m + k)
+    x = (torch.randn(m, k, generator=g) * 1.5).bfloat16()
+    q, s, y = ops.gelu_tanh_act_quant_i8(dev(x), True)
+    _check_y(y, O.gelu_tanh_bf16(x), 1e-2)
+    _check_quant_of_own_y("i8", y, q, s, k)
+    q2, s2, y2 = ops.gelu_tanh_act_quant_i8(dev(x), False)                # without writing y
+    assert y2.shape[0] == 0 and torch.equal(q2, q) and torch.equal(s2, s)
+
+
+@pytest.mark.parametrize("fmt", ["i8", "e4m3", "e5m2"])
+@pytest.mark.parametrize("m,k,rpg,vecs", [(300, 1536, 300, "both"), (1001, 5120, 333, "both"), (64, 5120, 64, "none"),
+                                          (9, 256, 2, "mul"), (1, 8, 1, "add"), (70, 8192, 35, "both")])
+def test_layernorm_multiply_add(ops, fmt, m, k, rpg, vecs):
+    g = torch.Generator().manual_seed(m * 7 + k)
+    x = (torch.randn(m, k, generator=g) * 2 + 0.3).bfloat16()
+    x[:, :: max(1, k // 7)] *= 12                                         # outlier channels, as in the DiT
+    groups = -(-m // rpg)
+    mul = (1 + 0.2 * torch.randn(groups, k, generator=g)) if vecs in ("both", "mul") else None
+    add = (0.1 * torch.randn(groups, k, generator=g)) if vecs in ("both", "add") else None
+    fn = getattr(ops, "layernorm_act_quant_" + fmt)
+    q, s, y = fn(dev(x), dev(mul), dev(add), rpg, 1e-6, True)
+    _check_y(y, O.layernorm_affine_bf16(x, mul, add, rpg, 1e-6), 5e-3)
+    _check_quant_of_own_y(fmt, y, q, s, k)
+    q2, s2, _ = fn(dev(x), dev(mul), dev(add), rpg, 1e-6, False)
+    assert torch.equal(q2, q) and torch.equal(s2, s)
+
+
+def test_layernorm_constant_rows_and_strided_input(ops):
+    x = torch.full((8, 512), -3.0).bfloat16()
+    add = torch.linspace(-2, 2, 512).reshape(1, 512)
+    q, s, y = ops.layernorm_act_quant_i8(dev(x), None, dev(add), 8, 1e-6, True)
+    assert torch.equal(y.cpu(), add.bfloat16().expand(8, 512))
+    big = torch.randn(16, 1024).bfloat16()
+    xs = dev(big)[:, :512]                                                # row stride 1024
+    q, s, y = ops.layernorm_act_quant_i8(xs, None, None, 16, 1e-6, True)
+    _check_y(y, O.layernorm_affine_bf16(big[:, :512].contiguous(), None, None, 16, 1e-6), 5e-3)
+
+
+def test_fused_inputs_of_a_linear_end_to_end(ops):
+    """norm -> modulate -> quantised linear and gelu -> quantised linear against the unfused oracle chain."""
+    m, k, n = 512, 1536, 1024
+    x, w, b = O.make_inputs(m, k, n, seed=11)
+    g = torch.Generator().manual_seed(5)
+    mul, add = 1 + 0.1 * torch.randn(1, k, generator=g), 0.05 * torch.randn(1, k, generator=g)
+    qw, sw = O.weight_quant_int8(w)
+    for name, y_ref, call in [
+        ("layernorm", O.layernorm_affine_bf16(x, mul, add, m, 1e-6),
+         lambda: ops.layernorm_act_quant_i8(dev(x), dev(mul), dev(add), m, 1e-6)),
+        ("gelu", O.gelu_tanh_bf16(x), lambda: ops.gelu_tanh_act_quant_i8(dev(x))),
+    ]:
+        ref = O.linear_int8(y_ref, qw, sw, b)["out"]
+        xq, sx, _ = call()
+        out = ops.linear_i8(xq, sx, dev(qw), dev(sw.view(-1)), dev(b))
+        assert rel_l2(out, ref) < 5e-3, name      # a flipped rounding of y moves one int8 step in one row
+
+
+def test_fused_errors_are_loud(ops):
+    x = torch.randn(4, 16384).bfloat16()
+    with pytest.raises(RuntimeError):
+        ops.gelu_tanh_act_quant_i8(dev(x))        # row too long for the register-resident kernel
+    with pytest.raises(RuntimeError):
+        ops.gelu_tanh_act_quant_i8(torch.randn(4, 64).bfloat16())   # CPU tensor
+    with pytest.raises(ValueError):
+        ops.layernorm_act_quant_i8(dev(torch.randn(4, 64).bfloat16()), dev(torch.ones(3, 64)), None, 4, 1e-6)
