@@ -14,7 +14,9 @@ from ...quant.quantization.qconfig import (
 )
 
 
-def quantize_transformer(transformer, fp8: bool = False):
+def quantize_transformer(transformer, fp8: bool = False, fuse_blocks: bool = False):
+    """``fuse_blocks`` additionally applies block_fusion.fuse_transformer_blocks (one quantisation per
+    produced activation; takes the place of what the reference gets from torch.compile)."""
     if fp8:
         root = get_dynamic_fp8_per_token_act_per_channel_weight_qconfig(
             activation_dtype=torch.float8_e4m3fn, weight_dtype=torch.float8_e4m3fn)
@@ -26,3 +28,7 @@ def quantize_transformer(transformer, fp8: bool = False):
         "proj_out": None,
     }
     quantize_dynamic(transformer, qconfig_dict)
+    if fuse_blocks:
+        from .block_fusion import fuse_transformer_blocks
+
+        fuse_transformer_blocks(transformer)

@@ -1,1 +1,1 @@
-from .linear import Linear  # noqa: F401
+from .linear import Linear, QuantizedActivation  # noqa: F401

@@ -27,6 +27,30 @@ from .functional import FP8_ALLOWED_DTYPES
 logger = logging.getLogger(__name__)
 
 
+class QuantizedActivation:
+    """An activation that has already been through the per-token quantiser.
+
+    Produced by ``Linear.quantize_activation`` or by a fused producer kernel (LayerNorm multiply-add,
+    GELU-tanh) and accepted by ``Linear.forward`` in place of the bf16 tensor, so that several linears
+    reading the same activation (q / k / v) share one quantisation and a producer can hand its result
+    over without the bf16 round trip through memory.  It is not a tensor: code between the producer
+    and the linears may only pass it along.
+    """
+
+    __slots__ = ("xq", "sx", "prev_dims", "in_features", "dtype", "device")
+
+    def __init__(self, xq: Tensor, sx: Tensor, prev_dims, in_features: int, dtype: torch.dtype):
+        self.xq, self.sx, self.prev_dims, self.in_features, self.dtype = xq, sx, tuple(prev_dims), in_features, dtype
+        self.device = xq.device
+
+    @property
+    def shape(self):
+        return torch.Size(self.prev_dims + (self.in_features,))
+
+
+_ACT_QUANT = {torch.int8: "act_quant_i8", torch.float8_e4m3fn: "act_quant_e4m3", torch.float8_e5m2: "act_quant_e5m2"}
+
+
 class Linear(nn.Module):
     _FLOAT_MODULE = nn.Linear
 
@@ -114,21 +138,26 @@ class Linear(nn.Module):
         return self._packed[1]
 
     # ------------------------------------------------------------------ forward
-    def forward(self, input: Tensor) -> Tensor:
-        prev_dims = input.shape[:-1]
+    def quantize_activation(self, input: Tensor) -> QuantizedActivation:
+        """Per-token quantisation of ``input`` [..., K] in this module's activation dtype (:204-208, :146-150)."""
         flat = input.view(-1, self.in_features)
+        xq, sx = getattr(ops, _ACT_QUANT[self.input_dtype])(flat)
+        return QuantizedActivation(xq, sx, input.shape[:-1], self.in_features, self.input_dtype)
+
+    def forward(self, input) -> Tensor:
+        qa = input if isinstance(input, QuantizedActivation) else self.quantize_activation(input)
+        if qa.dtype != self.input_dtype or qa.in_features != self.in_features:
+            raise ValueError(f"quantised activation ({qa.dtype}, K={qa.in_features}) does not fit this linear "
+                             f"({self.input_dtype}, K={self.in_features})")
         wq = self._gemm_weight()
         sw = self.weight_scale.view(-1)
         if self.compute_dtype == "FP8" and self.input_dtype == torch.float8_e5m2:
-            xq, sx = ops.act_quant_e5m2(flat)
-            out = ops.linear_e5m2_e4m3(xq, sx, wq, sw, self.bias)
+            out = ops.linear_e5m2_e4m3(qa.xq, qa.sx, wq, sw, self.bias)
         elif self.compute_dtype == "FP8":
-            xq, sx = ops.act_quant_e4m3(flat)
-            out = ops.linear_e4m3(xq, sx, wq, sw, self.bias)
+            out = ops.linear_e4m3(qa.xq, qa.sx, wq, sw, self.bias)
         else:
-            xq, sx = ops.act_quant_i8(flat)
-            out = ops.linear_i8(xq, sx, wq, sw, self.bias)
-        out = out.view(*prev_dims, self.out_features)
+            out = ops.linear_i8(qa.xq, qa.sx, wq, sw, self.bias)
+        out = out.view(*qa.prev_dims, self.out_features)
         if out.dtype != self.out_dtype:
             out = out.to(self.out_dtype)
         return out

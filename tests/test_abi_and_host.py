@@ -262,3 +262,36 @@ def test_bench_refuses_more_than_one_gpu():
 
     r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
     assert r.returncode != 0 and "one GPU" in (r.stderr + r.stdout)
+
+
+def test_block_fusion_host_logic_without_gpu():
+    """fuse_linears layout, what counts as a fusable block, and that the new ops are declared."""
+    import torch
+    from dax_amd.adapters.wan import block_fusion as BF
+    from dax_amd.quant.nn.dynamic import Linear, QuantizedActivation
+    from dax_amd.quant.qscheme import per_channel_symmetric, per_token_symmetric
+    from tests.wan_replica import Transformer
+
+    def lin(n, k, seed):
+        l = Linear(k, n, True, None, torch.int8, torch.int8, torch.bfloat16, per_channel_symmetric, per_token_symmetric)
+        g = torch.Generator().manual_seed(seed)
+        l.qweight.copy_(torch.randint(-127, 128, (n, k), generator=g, dtype=torch.int8))
+        l.weight_scale.copy_(torch.rand(1, n, generator=g) + 0.1)
+        with torch.no_grad():
+            l.bias.copy_(torch.randn(n, generator=g))
+        return l
+
+    a, b = lin(8, 16, 0), lin(24, 16, 1)
+    f = BF.fuse_linears([a, b])
+    assert f.out_features == 32 and torch.equal(f.qweight[:8], a.qweight) and torch.equal(f.qweight[8:], b.qweight)
+    assert torch.equal(f.weight_scale[:, 8:], b.weight_scale) and torch.equal(f.bias[:8], a.bias)
+    assert set(f.state_dict().keys()) == {"qweight", "weight_scale", "bias"}
+    with pytest.raises(ValueError):
+        BF.fuse_linears([a, lin(8, 32, 2)])                       # different in_features
+    model = Transformer(dim=64, ffn_dim=128, heads=2, layers=1)
+    assert not BF._block_is_fusable(model.blocks[0])              # float linears: nothing to fuse
+    assert BF.fuse_transformer_blocks(model) == 0
+    qa = QuantizedActivation(torch.zeros(6, 128, dtype=torch.int8), torch.ones(6), (2, 3), 16, torch.int8)
+    assert qa.shape == (2, 3, 16)
+    with pytest.raises(ValueError):
+        lin(8, 32, 3)(qa)                                         # K mismatch is reported, not mis-computed
