@@ -76,6 +76,9 @@ def main():
     ap.add_argument("--dtype", choices=["int8", "fp8"], default="int8")
     ap.add_argument("--variant", type=int, default=0)
     ap.add_argument("--tile-group", type=int, default=0, help="tile-order group depth (0 = library default)")
+    ap.add_argument("--workload", choices=["block", "model40"], default="block",
+                    help="block: the four linears of one DiT block (the headline workload); model40: 40 layers x "
+                         "{QKV, out, cross-q, cross-k, cross-v (512 text tokens), FFN up, FFN down} with distinct weights")
     ap.add_argument("--m", type=int, default=M_TOKENS)
     ap.add_argument("--cpu-rows", type=int, default=0, help="tokens in the CPU-baseline sample (0 = pick for 10-30 s)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -105,18 +108,26 @@ def main():
     g = torch.Generator(device="cpu").manual_seed(0)
     layers = []
     xs = {}
-    for i, (name, k, n) in enumerate(SHAPES):
-        if k not in xs:
-            x = torch.randn(m, k, device=dev, dtype=torch.bfloat16)
-            idx = torch.randperm(k, generator=g)[: max(1, round(0.01 * k))].to(dev)
-            x[:, idx] *= 20
-            xs[k] = x
+    for k in (5120, 13824):
+        x = torch.randn(m, k, device=dev, dtype=torch.bfloat16)
+        idx = torch.randperm(k, generator=g)[: max(1, round(0.01 * k))].to(dev)
+        x[:, idx] *= 20
+        xs[k] = x
+    text = torch.randn(512, 5120, device=dev, dtype=torch.bfloat16)
+    if args.workload == "block":
+        plan = [(name, k, n, xs[k]) for name, k, n in SHAPES]
+    else:
+        one = [("qkv", 5120, 15360, xs[5120]), ("out", 5120, 5120, xs[5120]), ("cross_q", 5120, 5120, xs[5120]),
+               ("cross_k", 5120, 5120, text), ("cross_v", 5120, 5120, text), ("ffn_up", 5120, 13824, xs[5120]),
+               ("ffn_down", 13824, 5120, xs[13824])]
+        plan = one * 40
+    for name, k, n, x in plan:
         w = (torch.randn(n, k, device=dev) * 0.02).bfloat16()
         b = (torch.randn(n, device=dev) * 0.01).bfloat16()
         lo, hi = ops.row_minmax(w)
         sw = ops.scale_from_minmax(lo, hi, 448.0 if fp8 else 127.0)
         qw = (ops.quantize_rows_e4m3 if fp8 else ops.quantize_rows_i8)(w, sw, True)
-        layers.append((name, k, n, xs[k], qw, sw, b))
+        layers.append((name, k, n, x, qw, sw, b))
         del w
     act_quant = ops.act_quant_e4m3 if fp8 else ops.act_quant_i8
     linear = ops.linear_e4m3 if fp8 else ops.linear_i8
@@ -151,27 +162,32 @@ def main():
         torch.cuda.synchronize()
 
     ms_per_step = (t1 - t0) * 1e3 / args.steps
-    total_ops = sum(2.0 * m * n * k for _, k, n in SHAPES)
+    total_ops = sum(2.0 * x.shape[0] * n * k for _, k, n, x, *_r in layers)
     value = total_ops / (ms_per_step * 1e-3) / 1e12
 
     # ---- per-kernel durations from the events recorded on the launch stream inside the timed region
     per_layer = {}
     gemm_ms_sum, quant_ms_sum = 0.0, 0.0
-    for li, (name, k, n, *_rest) in enumerate(layers):
+    for li, (name, k, n, x, *_rest) in enumerate(layers):
         q_ms = sum(evs[s][li][0].elapsed_time(evs[s][li][1]) for s in range(args.steps)) / args.steps
         g_ms = sum(evs[s][li][1].elapsed_time(evs[s][li][2]) for s in range(args.steps)) / args.steps
-        ops_l = 2.0 * m * n * k
-        per_layer[name] = {"k": k, "n": n, "quant_ms": round(q_ms, 4), "gemm_ms": round(g_ms, 4),
-                           "gemm_tops": round(ops_l / (g_ms * 1e-3) / 1e12, 1),
-                           "quant_gbps": round((3.0 * m * k + 4.0 * m) / (q_ms * 1e-3) / 1e9, 1)}
+        e = per_layer.setdefault(name, {"k": k, "n": n, "rows": x.shape[0], "launches": 0, "quant_ms": 0.0, "gemm_ms": 0.0})
+        e["launches"] += 1
+        e["quant_ms"] += q_ms
+        e["gemm_ms"] += g_ms
         gemm_ms_sum += g_ms
         quant_ms_sum += q_ms
+    for e in per_layer.values():
+        rows, k, n, cnt = e["rows"], e["k"], e["n"], e["launches"]
+        e["gemm_tops"] = round(cnt * 2.0 * rows * n * k / (e["gemm_ms"] * 1e-3) / 1e12, 1)
+        e["quant_gbps"] = round(cnt * (3.0 * rows * k + 4.0 * rows) / (e["quant_ms"] * 1e-3) / 1e9, 1)
+        e["quant_ms"], e["gemm_ms"] = round(e["quant_ms"], 4), round(e["gemm_ms"], 4)
     achieved = total_ops / (gemm_ms_sum * 1e-3) / 1e12
     peak = PEAK_TOPS[args.dtype]
 
     info = _capi.device_info(0)
     res = {
-        "metric": f"w8a8_linear_tops_wan2.1_14b_720p_{args.dtype}",
+        "metric": f"w8a8_linear_tops_wan2.1_14b_720p_{args.dtype}" + ("" if args.workload == "block" else "_40_layers"),
         "value": round(value, 2),
         "unit": "TOPS",
         "n_gpus": 1,
@@ -183,14 +199,19 @@ def main():
         "vs_baseline": None,
         "dtype": "int8" if not fp8 else "fp8_e4m3fn",
         "data": "synthetic",
-        "config": {"workload": f"Wan2.1-14B 720p linear set, {args.dtype.upper()} W8A8, M={m} tokens: "
-                               "QKV 5120->15360, out 5120->5120, FFN 5120->13824, FFN 13824->5120; "
-                               "per linear: per-token act quant + MFMA GEMM + fused scale/bias/bf16 epilogue",
+        "config": {"workload": (f"Wan2.1-14B 720p linear set, {args.dtype.upper()} W8A8, M={m} tokens: "
+                                "QKV 5120->15360, out 5120->5120, FFN 5120->13824, FFN 13824->5120; "
+                                "per linear: per-token act quant + MFMA GEMM + fused scale/bias/bf16 epilogue")
+                   if args.workload == "block" else
+                   (f"Wan2.1-14B 720p, 40 layers x (QKV 5120->15360, out, cross-q 5120->5120 at M={m}; cross-k, cross-v "
+                    "5120->5120 at 512 text tokens; FFN 5120->13824, 13824->5120), distinct weights per layer, "
+                    f"{args.dtype.upper()} W8A8, every linear with its own per-token act quant"),
                    "gemm_variant": args.variant},
         "pct_of_mfma_peak": round(100.0 * value / peak, 2),
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": peak, "unit": "TFLOP/s",
-                     "frac": round(achieved / peak, 4), "traffic": GEMM_TRAFFIC_BYTES[args.dtype] if m == M_TOKENS else None,
-                     "kernel": "gemm_tile256s5_kernel, average launch over the four shapes; 8-bit ops counted as 2*M*N*K",
+                     "frac": round(achieved / peak, 4), "traffic": GEMM_TRAFFIC_BYTES[args.dtype] if (m == M_TOKENS and args.workload == "block") else None,
+                     "kernel": "gemm_tile256s5_kernel, average launch over the four shapes; 8-bit ops counted as 2*M*N*K"
+                     if args.workload == "block" else "all GEMM launches of the step (the 512-token ones run gemm_w8a8_kernel)",
                      "gemm_ms_per_step": round(gemm_ms_sum, 4), "quant_ms_per_step": round(quant_ms_sum, 4)},
         "per_linear": per_layer,
         "device": {"arch": info["arch"], "cu_count": info["cu_count"], "max_clock_mhz": info["clock_khz"] / 1000.0},
