@@ -15,7 +15,7 @@ CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 LIB = os.path.join(LIBDIR, "libdaxq.so")
 MFMA_RATE = os.path.join(LIBDIR, "mfma_rate")
-SOURCES = ["capi.hip", "quant_rows.hip", "fused_rows.hip", "gemm_w8a8.hip", "gemm_tile256.hip"]
+SOURCES = ["capi.hip", "quant_rows.hip", "fused_rows.hip", "per_tensor.hip", "gemm_w8a8.hip", "gemm_tile256.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-fast-math",

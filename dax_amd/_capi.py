@@ -35,6 +35,10 @@ SIGNATURES = {
     "daxq_gelu_tanh_act_quant_e5m2": [_P, _I64, _I64, _I64, _P, _I64, _P, _I64, _P, _P],
     "daxq_quantize_rows_i8": [_P, _I64, _I64, _I64, _P, _P, _I64, _P],
     "daxq_quantize_rows_e4m3": [_P, _I64, _I64, _I64, _P, _P, _I64, _P],
+    "daxq_quantize_rows_e5m2": [_P, _I64, _I64, _I64, _P, _P, _I64, _P],
+    "daxq_tensor_scale": [_P, _P, _I64, _F32, _INT, _P, _P, _I64, _P],
+    "daxq_tensor_minmax_update": [_P, _P, _I64, _P, _P, _P],
+    "daxq_broadcast_f32": [_P, _P, _I64, _P],
     "daxq_row_minmax": [_P, _I64, _I64, _I64, _P, _P, _P],
     "daxq_scale_from_minmax": [_P, _P, _I64, _F32, _P, _P],
     "daxq_linear_i8": [_P, _I64, _P, _P, _I64, _P, _P, _P, _I64, _P, _I64, _I64, _I64, _I64, _P],

@@ -223,6 +223,12 @@ int daxq_quantize_rows_e4m3(const void* x, int64_t m, int64_t k, int64_t ld_x, c
                                                       (hipStream_t)stream);
 }
 
+int daxq_quantize_rows_e5m2(const void* x, int64_t m, int64_t k, int64_t ld_x, const float* scale, uint8_t* q,
+                            int64_t ld_q, daxq_stream_t stream) {
+    return daxq::launch_quant_rows<2, false, true>(x, m, k, ld_x, q, ld_q, const_cast<float*>(scale), 57344.0f,
+                                                      (hipStream_t)stream);
+}
+
 int daxq_row_minmax(const void* x, int64_t m, int64_t k, int64_t ld_x, float* min_out, float* max_out,
                     daxq_stream_t stream) {
     using namespace daxq;

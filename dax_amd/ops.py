@@ -188,8 +188,8 @@ gelu_tanh_act_quant_e5m2.register_fake(lambda x, want_y=False: _fused_fake(x, "e
 
 
 # ----------------------------------------------------------------------------- leaf quantisers
-def _quantize_rows(x: torch.Tensor, scale: torch.Tensor, fp8: bool, padded: bool) -> torch.Tensor:
-    name = "quantize_rows_e4m3" if fp8 else "quantize_rows_i8"
+def _quantize_rows(x: torch.Tensor, scale: torch.Tensor, fmt: str, padded: bool) -> torch.Tensor:
+    name = "quantize_rows_" + fmt
     _rows_bf16(x, name)
     m, k = x.shape
     if scale.dtype != torch.float32 or scale.numel() != m or scale.device != x.device:
@@ -197,9 +197,9 @@ def _quantize_rows(x: torch.Tensor, scale: torch.Tensor, fp8: bool, padded: bool
     scale = scale.reshape(-1).contiguous()
     ld_q = pad_k(k) if padded else k
     with torch.cuda.device(x.device):
-        q = torch.empty((m, ld_q), dtype=torch.uint8 if fp8 else torch.int8, device=x.device)
+        q = torch.empty((m, ld_q), dtype=torch.int8 if fmt == "i8" else torch.uint8, device=x.device)
         if m:
-            fn = _capi.lib().daxq_quantize_rows_e4m3 if fp8 else _capi.lib().daxq_quantize_rows_i8
+            fn = getattr(_capi.lib(), "daxq_" + name)
             ld_x = x.stride(0) if m > 1 else k
             _capi.check(fn(x.data_ptr(), m, k, ld_x, scale.data_ptr(), q.data_ptr(), ld_q, _stream(x)), name)
     return q
@@ -207,14 +207,21 @@ def _quantize_rows(x: torch.Tensor, scale: torch.Tensor, fp8: bool, padded: bool
 
 @torch.library.custom_op("daxq::quantize_rows_i8", mutates_args=(), device_types="cuda")
 def quantize_rows_i8(x: torch.Tensor, scale: torch.Tensor, padded: bool = False) -> torch.Tensor:
-    return _quantize_rows(x, scale, False, padded)
+    return _quantize_rows(x, scale, "i8", padded)
 
 
 @torch.library.custom_op("daxq::quantize_rows_e4m3", mutates_args=(), device_types="cuda")
 def quantize_rows_e4m3(x: torch.Tensor, scale: torch.Tensor, padded: bool = False) -> torch.Tensor:
-    return _quantize_rows(x, scale, True, padded)
+    return _quantize_rows(x, scale, "e4m3", padded)
 
 
+@torch.library.custom_op("daxq::quantize_rows_e5m2", mutates_args=(), device_types="cuda")
+def quantize_rows_e5m2(x: torch.Tensor, scale: torch.Tensor, padded: bool = False) -> torch.Tensor:
+    return _quantize_rows(x, scale, "e5m2", padded)
+
+
+quantize_rows_e5m2.register_fake(
+    lambda x, scale, padded=False: x.new_empty((x.shape[0], pad_k(x.shape[1]) if padded else x.shape[1]), dtype=torch.uint8))
 quantize_rows_i8.register_fake(
     lambda x, scale, padded=False: x.new_empty((x.shape[0], pad_k(x.shape[1]) if padded else x.shape[1]), dtype=torch.int8))
 quantize_rows_e4m3.register_fake(
@@ -343,3 +350,60 @@ linear_i8_acc.register_fake(lambda xq, sx, wq, sw, bias: (
     _lin_fake(xq, sx, wq, sw, bias), xq.new_empty((xq.shape[0], wq.shape[0]), dtype=torch.int32)))
 linear_e4m3_acc.register_fake(lambda xq, sx, wq, sw, bias: (
     _lin_fake(xq, sx, wq, sw, bias), xq.new_empty((xq.shape[0], wq.shape[0]), dtype=torch.float32)))
+
+
+# ----------------------------------------------------------------------------- per-tensor scales
+@torch.library.custom_op("daxq::tensor_scale", mutates_args=(), device_types="cuda")
+def tensor_scale(row_min: torch.Tensor, row_max: torch.Tensor, qmax: float, round_bf16: bool,
+                 n_expand: int) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Per-tensor scale from per-row (min, max): (scale fp32 [1], the same value n_expand times)."""
+    _need_gpu(row_min, "tensor_scale")
+    if row_min.dtype != torch.float32 or row_max.dtype != torch.float32 or row_min.shape != row_max.shape or row_min.numel() == 0:
+        raise ValueError("daxq::tensor_scale: row_min / row_max must be non-empty fp32 tensors of one shape")
+    lo, hi = row_min.contiguous(), row_max.contiguous()
+    with torch.cuda.device(lo.device):
+        s1 = torch.empty((1,), dtype=torch.float32, device=lo.device)
+        ex = torch.empty((n_expand,), dtype=torch.float32, device=lo.device)
+        _capi.check(_capi.lib().daxq_tensor_scale(lo.data_ptr(), hi.data_ptr(), lo.numel(), float(qmax), int(round_bf16),
+                                                  s1.data_ptr(), ex.data_ptr() if n_expand else 0, n_expand, _stream(lo)),
+                    "tensor_scale")
+    return s1, ex
+
+
+tensor_scale.register_fake(lambda row_min, row_max, qmax, round_bf16, n_expand: (
+    row_min.new_empty((1,), dtype=torch.float32), row_min.new_empty((n_expand,), dtype=torch.float32)))
+
+
+@torch.library.custom_op("daxq::tensor_minmax_update", mutates_args=("min_inout", "max_inout"), device_types="cuda")
+def tensor_minmax_update(row_min: torch.Tensor, row_max: torch.Tensor, min_inout: torch.Tensor,
+                         max_inout: torch.Tensor) -> None:
+    """min_inout[0] = min(min_inout[0], min(row_min)); max_inout likewise (fp32, one element each)."""
+    _need_gpu(row_min, "tensor_minmax_update")
+    for t in (row_min, row_max, min_inout, max_inout):
+        if t.dtype != torch.float32 or t.device != row_min.device or not t.is_contiguous():
+            raise ValueError("daxq::tensor_minmax_update: contiguous fp32 tensors on one device expected")
+    if min_inout.numel() != 1 or max_inout.numel() != 1 or row_min.numel() == 0 or row_min.numel() != row_max.numel():
+        raise ValueError("daxq::tensor_minmax_update: bad shapes")
+    with torch.cuda.device(row_min.device):
+        _capi.check(_capi.lib().daxq_tensor_minmax_update(row_min.data_ptr(), row_max.data_ptr(), row_min.numel(),
+                                                          min_inout.data_ptr(), max_inout.data_ptr(), _stream(row_min)),
+                    "tensor_minmax_update")
+
+
+tensor_minmax_update.register_fake(lambda row_min, row_max, min_inout, max_inout: None)
+
+
+@torch.library.custom_op("daxq::broadcast_f32", mutates_args=(), device_types="cuda")
+def broadcast_f32(src: torch.Tensor, n: int) -> torch.Tensor:
+    """fp32 [n] filled with src[0] (a stored per-tensor scale as the vector the kernels take)."""
+    _need_gpu(src, "broadcast_f32")
+    if src.dtype != torch.float32 or src.numel() != 1:
+        raise ValueError("daxq::broadcast_f32: src must hold one fp32 value")
+    with torch.cuda.device(src.device):
+        dst = torch.empty((n,), dtype=torch.float32, device=src.device)
+        _capi.check(_capi.lib().daxq_broadcast_f32(src.data_ptr(), dst.data_ptr(), n, _stream(src)), "broadcast_f32")
+    return dst
+
+
+broadcast_f32.register_fake(lambda src, n: src.new_empty((n,), dtype=torch.float32))
+

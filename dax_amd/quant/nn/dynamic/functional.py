@@ -4,7 +4,9 @@ Same entry points as dax/quant/nn/dynamic/functional.py:13-206.  The per-token s
 one on the DiT hot path, is a single fused HIP kernel (row abs-max with wavefront shuffles,
 bf16-rounded scale floored at 2^-23, quantise from registers).  The scale recipe follows the
 reference's eager dtype chain for a bf16 input: the division by quant_max and the clamp
-happen in bf16, and only then is the scale widened to fp32 (:124-129).
+happen in bf16, and only then is the scale widened to fp32 (:124-129).  The per-tensor scheme
+(one block = the whole tensor) runs the row statistics kernel, a single-workgroup reduction to
+the scalar scale by the same rule, and the leaf quantiser with that scale.
 """
 from typing import List, Optional, Tuple, Union
 
@@ -55,10 +57,13 @@ def _dynamic_quantize_func(
     assert len(block_size) == input.dim(), f"Got input dim:{input.dim()}, block_size: {block_size}"
     if target_dtype not in FP8_ALLOWED_DTYPES and target_dtype != torch.int8:
         raise NotImplementedError(f"Unsupported dtype {target_dtype}")
-    if not _is_per_token(block_size, input.shape):
-        raise NotImplementedError("daxq implements the per-token dynamic scheme; per-tensor / grouped blocks are not built")
+    per_tensor = tuple(block_size) == tuple(input.shape)
+    if not (per_tensor or _is_per_token(block_size, input.shape)):
+        raise NotImplementedError("daxq implements the per-token and per-tensor dynamic schemes; grouped blocks are not built")
     if scale_dtype not in (None, torch.float32) or (eps is not None and eps != torch.finfo(torch.float32).eps):
         raise NotImplementedError("daxq kernels produce fp32 scales floored at float32 eps")
+    if per_tensor and not _is_per_token(block_size, input.shape):
+        return _per_tensor_quantize(input, target_dtype, float(quant_max))
     k = input.shape[-1]
     x2 = input.reshape(-1, k)
     if target_dtype == torch.int8:
@@ -70,6 +75,27 @@ def _dynamic_quantize_func(
         q, s = ops.act_quant_e4m3(x2)
         q = q.view(torch.float8_e4m3fn)
     return q[:, :k].view(input.shape), s.view(*input.shape[:-1], 1)
+
+
+def per_tensor_scale(x2: torch.Tensor, quant_max: float):
+    """(scale fp32 [1], the same value once per row of x2) of the whole bf16 matrix x2."""
+    lo, hi = ops.row_minmax(x2)
+    return ops.tensor_scale(lo, hi, quant_max, True, x2.shape[0])
+
+
+def _per_tensor_quantize(input, target_dtype, quant_max):
+    k = input.shape[-1]
+    x2 = input.reshape(-1, k)
+    if x2.stride(1) != 1:
+        x2 = x2.contiguous()
+    s1, rows = per_tensor_scale(x2, quant_max)
+    if target_dtype == torch.int8:
+        q = ops.quantize_rows_i8(x2, rows)
+    elif target_dtype == torch.float8_e5m2:
+        q = ops.quantize_rows_e5m2(x2, rows).view(torch.float8_e5m2)
+    else:
+        q = ops.quantize_rows_e4m3(x2, rows).view(torch.float8_e4m3fn)
+    return q.view(input.shape), s1.view((1,) * input.dim())
 
 
 def dynamic_quantize_to_fp8(

@@ -81,9 +81,10 @@ class Linear(nn.Module):
 
         # --- what the gfx950 kernels cover; anything else is reported as not implemented so
         #     that get_qlinear keeps the float module, as the reference does on NotImplementedError
-        if not (input_qscheme == per_token_symmetric and weight_qscheme == per_channel_symmetric):
+        if input_qscheme not in (per_token_symmetric, per_tensor_symmetric) or \
+                weight_qscheme not in (per_channel_symmetric, per_tensor_symmetric):
             raise NotImplementedError(
-                "daxq implements per-token activations with per-channel weights; "
+                "daxq implements per-token / per-tensor activations with per-channel / per-tensor weights; "
                 f"got input_qscheme={input_qscheme}, weight_qscheme={weight_qscheme}")
         if compute_dtype == "FP8" and weight_dtype != torch.float8_e4m3fn:
             raise NotImplementedError(
@@ -102,8 +103,12 @@ class Linear(nn.Module):
             self.bias = nn.Parameter(torch.empty(out_features, device=device, dtype=torch.bfloat16))
         else:
             self.register_parameter("bias", None)
+        # [1, N] per channel, [1] per tensor (:122-130)
         self.register_buffer(
-            "weight_scale", torch.ones((1, out_features), device=device, dtype=torch.float32), persistent=True)
+            "weight_scale",
+            torch.ones((1, out_features) if weight_qscheme == per_channel_symmetric else 1, device=device,
+                       dtype=torch.float32),
+            persistent=True)
 
         self.out_dtype = out_dtype if out_dtype is not None else torch.bfloat16
         self.weight_dtype = weight_dtype
@@ -111,8 +116,10 @@ class Linear(nn.Module):
         self.compute_dtype = compute_dtype
         self.weight_qscheme = weight_qscheme
         self.input_qscheme = input_qscheme
-        # derived, never saved: (key, K-padded byte view of qweight) for the GEMM
+        # derived, never saved: (key, K-padded byte view of qweight) for the GEMM, and the per-tensor
+        # weight scale written out once per output channel
         self._packed = None
+        self._sw_vec = None
 
     # ------------------------------------------------------------------ derived views
     @property
@@ -138,10 +145,29 @@ class Linear(nn.Module):
         return self._packed[1]
 
     # ------------------------------------------------------------------ forward
+    def _weight_scale_vector(self) -> Tensor:
+        """weight_scale as the fp32 [N] vector the GEMM reads."""
+        ws = self.weight_scale
+        if ws.numel() != 1:
+            return ws.view(-1)
+        key = (ws.data_ptr(), ws._version, str(ws.device))
+        if self._sw_vec is None or self._sw_vec[0] != key:
+            self._sw_vec = (key, ops.broadcast_f32(ws.reshape(1).contiguous(), self.out_features))
+        return self._sw_vec[1]
+
     def quantize_activation(self, input: Tensor) -> QuantizedActivation:
-        """Per-token quantisation of ``input`` [..., K] in this module's activation dtype (:204-208, :146-150)."""
+        """Dynamic quantisation of ``input`` [..., K] in this module's activation dtype and scheme
+        (:204-208, :146-150): one scale per token, or one for the whole tensor written out per token."""
         flat = input.view(-1, self.in_features)
-        xq, sx = getattr(ops, _ACT_QUANT[self.input_dtype])(flat)
+        if self.input_qscheme == per_token_symmetric:
+            xq, sx = getattr(ops, _ACT_QUANT[self.input_dtype])(flat)
+        else:
+            from .functional import per_tensor_scale
+
+            qmax = 127.0 if self.input_dtype == torch.int8 else float(torch.finfo(self.input_dtype).max)
+            _, sx = per_tensor_scale(flat, qmax)
+            xq = getattr(ops, "quantize_rows_" + {torch.int8: "i8", torch.float8_e4m3fn: "e4m3",
+                                                 torch.float8_e5m2: "e5m2"}[self.input_dtype])(flat, sx, True)
         return QuantizedActivation(xq, sx, input.shape[:-1], self.in_features, self.input_dtype)
 
     def forward(self, input) -> Tensor:
@@ -150,7 +176,7 @@ class Linear(nn.Module):
             raise ValueError(f"quantised activation ({qa.dtype}, K={qa.in_features}) does not fit this linear "
                              f"({self.input_dtype}, K={self.in_features})")
         wq = self._gemm_weight()
-        sw = self.weight_scale.view(-1)
+        sw = self._weight_scale_vector()
         if self.compute_dtype == "FP8" and self.input_dtype == torch.float8_e5m2:
             out = ops.linear_e5m2_e4m3(qa.xq, qa.sx, wq, sw, self.bias)
         elif self.compute_dtype == "FP8":
@@ -217,8 +243,12 @@ class Linear(nn.Module):
 
         weight_scale = weight_post_process.calculate_qparams()
         if weight_scale is not None:
-            assert mod.weight.shape[0] == weight_scale.numel()
-            qweight = quantize_func(w, scale=weight_scale.reshape(-1, 1), dtype=weight_post_process.dtype)
+            if weight_scale.numel() > 1:
+                assert mod.weight.shape[0] == weight_scale.numel()
+                scale_arg = weight_scale.reshape(-1, 1)
+            else:
+                scale_arg = weight_scale.reshape(1)
+            qweight = quantize_func(w, scale=scale_arg, dtype=weight_post_process.dtype)
             qlinear.qweight = qweight.to(home)
             qlinear.weight_scale.copy_(weight_scale.reshape(qlinear.weight_scale.shape))
         if qlinear.bias is not None:

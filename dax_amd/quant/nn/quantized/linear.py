@@ -1,0 +1,165 @@
+"""Static FP8 ``Linear``: calibrated per-tensor activation scale, per-tensor or per-channel weight.
+
+Drop-in for dax/quant/nn/quantized/linear.py:28-251 -- same constructor signature and state
+(``qweight`` parameter [N, K] in the fp8 weight dtype, ``weight_scale`` fp32 [1] or [1, N],
+``input_scale`` fp32 [1], ``bias``), the same ``from_float`` / ``get_qlinear`` / ``weight`` /
+``extra_repr`` surface.  ``forward`` (:91-118) is the leaf quantiser with the stored input scale
+followed by the same MFMA GEMM as the dynamic module; the scalar scales are written out as the
+per-row / per-channel vectors that kernel reads, which leaves the arithmetic per element unchanged:
+``bf16((sum_k a*b) * input_scale * weight_scale + bias)``.
+
+A pre-quantised checkpoint is loaded the way the reference does it: convert an uncalibrated model
+(observers that have seen nothing give no scales, :170-176) and ``load_state_dict`` into it.
+"""
+from __future__ import annotations
+
+import warnings
+
+import torch
+from torch import Tensor, nn
+
+from .... import ops
+from ...qscheme import per_channel_symmetric
+from .functional import FP8_ALLOWED_DTYPES, quantize_to_fp8
+
+
+class Linear(nn.Module):
+    _FLOAT_MODULE = nn.Linear
+
+    def __init__(self, in_features: int, out_features: int, bias: bool = True, device=None, weight_dtype=None,
+                 input_dtype=None, out_dtype=None, row_wise_scale=False) -> None:
+        if weight_dtype is not None and weight_dtype != torch.float8_e4m3fn:
+            raise NotImplementedError(f"daxq implements float8_e4m3fn weights, got {weight_dtype}")
+        if input_dtype is not None and input_dtype not in FP8_ALLOWED_DTYPES:
+            raise NotImplementedError(f"the static linear is an FP8 module, got input dtype {input_dtype}")
+        if out_dtype not in (None, torch.bfloat16):
+            raise NotImplementedError(f"daxq kernels produce bfloat16 outputs, got out_dtype={out_dtype}")
+        super().__init__()
+        self.in_features = in_features
+        self.out_features = out_features
+        self.qweight = nn.Parameter(
+            torch.empty((out_features, in_features), device=device, dtype=weight_dtype or torch.float8_e4m3fn),
+            requires_grad=False)
+        if bias:
+            self.bias = nn.Parameter(torch.empty(out_features, device=device, dtype=torch.bfloat16))
+        else:
+            self.register_parameter("bias", None)
+        self.register_buffer(
+            "weight_scale", torch.ones((1, out_features) if row_wise_scale else 1, device=device, dtype=torch.float32),
+            persistent=True)
+        self.register_buffer("input_scale", torch.tensor([1.0], device=device, dtype=torch.float32), persistent=True)
+        self.out_dtype = out_dtype if out_dtype is not None else torch.bfloat16
+        self.weight_dtype = weight_dtype or torch.float8_e4m3fn
+        self.input_dtype = input_dtype or torch.float8_e4m3fn
+        self.row_wise_scale = row_wise_scale
+        self._packed = None
+        self._sw_vec = None
+
+    @property
+    def weight(self):
+        """De-quantised weight in out_dtype (:87-89)."""
+        return self.qweight.to(self.out_dtype) * self.weight_scale.reshape(-1, 1).to(self.out_dtype)
+
+    def _gemm_weight(self) -> Tensor:
+        qw = self.qweight.detach().view(torch.uint8)
+        k = qw.shape[1]
+        kp = ops.pad_k(k)
+        if kp == k and qw.is_contiguous():
+            return qw
+        key = (self.qweight.data_ptr(), self.qweight._version, str(qw.device))
+        if self._packed is None or self._packed[0] != key:
+            buf = torch.zeros((qw.shape[0], kp), dtype=qw.dtype, device=qw.device)
+            buf[:, :k] = qw
+            self._packed = (key, buf)
+        return self._packed[1]
+
+    def _weight_scale_vector(self) -> Tensor:
+        ws = self.weight_scale
+        if ws.numel() != 1:
+            return ws.view(-1)
+        key = (ws.data_ptr(), ws._version, str(ws.device))
+        if self._sw_vec is None or self._sw_vec[0] != key:
+            self._sw_vec = (key, ops.broadcast_f32(ws.reshape(1).contiguous(), self.out_features))
+        return self._sw_vec[1]
+
+    def forward(self, input: Tensor) -> Tensor:
+        prev_dims = input.shape[:-1]
+        flat = input.view(-1, self.in_features)
+        sx = ops.broadcast_f32(self.input_scale.reshape(1), flat.shape[0])
+        if self.input_dtype == torch.float8_e5m2:
+            xq = ops.quantize_rows_e5m2(flat, sx, True)
+            out = ops.linear_e5m2_e4m3(xq, sx, self._gemm_weight(), self._weight_scale_vector(), self.bias)
+        else:
+            xq = ops.quantize_rows_e4m3(flat, sx, True)
+            out = ops.linear_e4m3(xq, sx, self._gemm_weight(), self._weight_scale_vector(), self.bias)
+        out = out.view(*prev_dims, self.out_features)
+        if out.dtype != self.out_dtype:
+            out = out.to(self.out_dtype)
+        return out
+
+    def extra_repr(self) -> str:
+        s = f"in_features={self.in_features}, out_features={self.out_features}"
+        if self.bias is None:
+            s += ", bias=False"
+        s += f", weight_scale={self.weight_scale}, input_scale={self.input_scale}"
+        return s
+
+    @classmethod
+    @torch.no_grad()
+    def get_qlinear(cls, mod, activation_post_process, weight_post_process, reserve_float_weight):
+        """Builds the static module from a float ``nn.Linear`` and its observers (:132-214).  With a
+        calibrated activation observer the weight is observed and quantised too; without one (nothing
+        observed) scales and quantised weight are left for a checkpoint to fill."""
+        if activation_post_process is None or activation_post_process.dtype == torch.float:
+            raise ValueError("Input must be quantized!")
+        try:
+            qlinear = cls(mod.in_features, mod.out_features, mod.bias is not None, mod.weight.device,
+                          weight_post_process.dtype, activation_post_process.dtype, mod.weight.dtype,
+                          weight_post_process.qscheme == per_channel_symmetric)
+        except NotImplementedError as e:
+            warnings.warn("Quantized linear is not supported for this combination of arguments. "
+                          f"Falling back to float module. Message: {e}")
+            return mod
+
+        input_scale = activation_post_process.calculate_qparams()
+        if input_scale is not None:
+            qlinear.input_scale.copy_(input_scale.reshape(qlinear.input_scale.shape))
+            home = mod.weight.device
+            w = mod.weight.detach()
+            if home.type != "cuda":
+                if not torch.cuda.is_available():
+                    raise RuntimeError("daxq converts weights with HIP kernels and found no ROCm device "
+                                       f"(module is on {home}); there is no CPU implementation")
+                w = w.to(torch.device("cuda", torch.cuda.current_device()))
+            weight_post_process.to(w.device)
+            weight_post_process(w)
+            weight_scale = weight_post_process.calculate_qparams()
+            if weight_scale is not None:
+                if weight_scale.numel() > 1:
+                    assert mod.weight.shape[0] == weight_scale.numel()
+                    scale_arg = weight_scale.reshape(-1, 1)
+                else:
+                    scale_arg = weight_scale.reshape(1)
+                qweight = quantize_to_fp8(w, scale=scale_arg, dtype=weight_post_process.dtype)
+                qlinear.qweight = nn.Parameter(qweight.to(home), requires_grad=False)
+                qlinear.weight_scale.copy_(weight_scale.reshape(qlinear.weight_scale.shape))
+        if qlinear.bias is not None:
+            qlinear.bias.copy_(mod.bias)
+        if not reserve_float_weight:  # release the float parameters' memory
+            del mod.weight
+            del mod.bias
+        return qlinear
+
+    @classmethod
+    def from_float(cls, mod, reserve_float_weight=False):
+        if hasattr(mod, "weight_fake_quant"):  # QAT module carrying its own observers
+            assert hasattr(mod, "activation_post_process"), "Input QAT module must have observer attached"
+            weight_post_process = mod.weight_fake_quant
+            activation_post_process = mod.activation_post_process
+        else:
+            assert type(mod) == cls._FLOAT_MODULE, (
+                f" nnq.{cls.__name__}.from_float only works for {cls._FLOAT_MODULE.__name__} but got:{type(mod)}")
+            assert hasattr(mod, "qconfig"), "Input float module must have qconfig defined."
+            activation_post_process = getattr(mod, "activation_post_process", None)
+            weight_post_process = mod.qconfig.weight()
+        return cls.get_qlinear(mod, activation_post_process, weight_post_process, reserve_float_weight)

@@ -8,8 +8,10 @@ Counterparts of dax/quant/quantization/observer.py.  Two are on the dynamic W8A8
 * ``DynamicObserverPlaceholder`` (:453-477) -- an inert carrier of dtype and qscheme for a
   dynamically quantised activation.
 
-Static calibration (``MinMaxObserver``) and the histogram profiler are not on this path and
-are not built.
+``MinMaxObserver`` (:141-226) is the per-tensor observer of the static and per-tensor variants:
+running min / max of everything shown to it, reduced on the device (``daxq_row_minmax`` +
+``daxq_tensor_minmax_update``).  The histogram profiler (``DistributionProfileObserver``, a
+calibration diagnostic that writes plots) is not built.
 """
 from __future__ import annotations
 
@@ -57,6 +59,55 @@ class UniformQuantizationObserverBase(nn.Module):
 
     def reset_min_max_vals(self):
         raise NotImplementedError("Cannot reset min/max values in the given observer.")
+
+
+class MinMaxObserver(UniformQuantizationObserverBase):
+    """Running per-tensor min / max (:141-226); ``calculate_qparams`` gives the fp32 scale [1] or None
+    while nothing has been observed."""
+
+    def __init__(self, dtype=torch.float8_e4m3fn, qscheme=per_tensor_symmetric, factory_kwargs=None,
+                 eps=torch.finfo(torch.float32).eps, is_dynamic=False, **kwargs) -> None:
+        assert qscheme == per_tensor_symmetric, "MinMaxObserver's qscheme only support per_tensor_symmetric"
+        super().__init__(dtype=dtype, qscheme=qscheme, factory_kwargs=factory_kwargs, eps=eps,
+                         is_dynamic=is_dynamic, **kwargs)
+        fk = factory_kwargs or {}
+        self.register_buffer("min_val", torch.tensor(float("inf"), **fk))
+        self.register_buffer("max_val", torch.tensor(float("-inf"), **fk))
+
+    def forward(self, x_orig):
+        if x_orig.numel() == 0:
+            return x_orig
+        x = x_orig.detach()
+        x = x.reshape(-1, x.shape[-1]) if x.dim() > 1 else x.reshape(1, -1)
+        if x.stride(1) != 1:
+            x = x.contiguous()
+        lo, hi = ops.row_minmax(x)
+        if self.min_val.device != lo.device:
+            self.min_val = self.min_val.to(lo.device)
+            self.max_val = self.max_val.to(lo.device)
+        lo1, hi1 = self.min_val.reshape(1).clone(), self.max_val.reshape(1).clone()
+        ops.tensor_minmax_update(lo, hi, lo1, hi1)
+        self.min_val.copy_(lo1.reshape(()))
+        self.max_val.copy_(hi1.reshape(()))
+        self._sync_state()
+        return x_orig
+
+    def _sync_state(self):
+        if self.sync_state and torch.distributed.is_available() and torch.distributed.is_initialized():
+            raise NotImplementedError("daxq is built for one GPU: observers with sync_state=True cannot reduce over ranks")
+
+    def calculate_qparams(self):
+        lo, hi = self.min_val.reshape(1), self.max_val.reshape(1)
+        if bool(torch.isinf(lo).any()) or bool(torch.isinf(hi).any()):
+            return None  # nothing observed yet: a pre-quantised checkpoint supplies the scales (:116-120)
+        return self._calculate_qparams(lo, hi)
+
+    def extra_repr(self):
+        return f"min_val={self.min_val}, max_val={self.max_val}"
+
+    def reset_min_max_vals(self):
+        self.min_val.fill_(float("inf"))
+        self.max_val.fill_(float("-inf"))
 
 
 class PerChannelMinMaxObserver(UniformQuantizationObserverBase):

@@ -1,7 +1,9 @@
 """Module-swap machinery: resolve a qconfig for every submodule, then replace the mapped ones.
 
 Same entry point and semantics as dax/quant/quantization/quantize.py:
-``quantize_dynamic(model, qconfig_dict, mapping, inplace, remove_qconfig)`` (:394-444).
+``quantize_dynamic(model, qconfig_dict, mapping, inplace, remove_qconfig)`` (:394-444), and for the
+static variant ``prepare`` (:250-301: attach an activation observer to every leaf module that is to be
+quantised, called from a forward pre-hook) and ``convert`` (:360-391: swap by the static mapping).
 
 qconfig resolution per module (:67-93): a key equal to the module's *type* wins over what the
 parent resolved to; a key equal to the module's dotted *name* ("" is the root) wins over that;
@@ -18,7 +20,11 @@ import copy
 from torch import nn
 from torch.nn.utils.parametrize import type_before_parametrizations
 
-from .quantization_mappings import get_default_dynamic_quant_module_mappings
+from .quantization_mappings import (
+    get_default_dynamic_quant_module_mappings,
+    get_default_qconfig_propagation_list,
+    get_default_static_quant_module_mappings,
+)
 
 _UNSET = object()
 
@@ -56,7 +62,8 @@ def swap_module(mod, mapping, reserve_float_weight=False):
     if new_mod is mod:
         return mod
     for pre_hook in mod._forward_pre_hooks.values():
-        new_mod.register_forward_pre_hook(pre_hook)
+        if pre_hook is not _observer_forward_pre_hook:  # the calibration observer goes away with the float module
+            new_mod.register_forward_pre_hook(pre_hook)
     for hook in mod._forward_hooks.values():
         new_mod.register_forward_hook(hook)
     if devices:
@@ -72,11 +79,24 @@ def _convert(module, mapping):
     return module
 
 
+def _observer_forward_pre_hook(self, input):
+    """Shows the module's input to its activation observer (:28-31)."""
+    self.activation_post_process(input[0])
+    return None
+
+
 def _remove_qconfig(module):
+    """Drops qconfig attributes, activation observers and their hooks from the tree (:304-357)."""
     for child in module.children():
         _remove_qconfig(child)
     if hasattr(module, "qconfig"):
         del module.qconfig
+    if "activation_post_process" in getattr(module, "_modules", {}):
+        del module._modules["activation_post_process"]
+    hooks = getattr(module, "_forward_pre_hooks", None)
+    if hooks:
+        for key in [k for k, fn in hooks.items() if fn is _observer_forward_pre_hook]:
+            hooks.pop(key)
 
 
 def quantize_dynamic(model, qconfig_dict=None, mapping=None, inplace=True, remove_qconfig=True):
@@ -92,11 +112,49 @@ def quantize_dynamic(model, qconfig_dict=None, mapping=None, inplace=True, remov
     return model
 
 
-def prepare(model, *args, **kwargs):
-    """Static-calibration entry point of the reference (:250-301); not part of the dynamic W8A8 path."""
-    raise NotImplementedError("static calibration (prepare/convert) is not built; use quantize_dynamic")
+def _add_observer_(module, qconfig_propagation_list, device=None):
+    """Gives every leaf module of a listed type with a qconfig an ``activation_post_process`` observer on
+    the module's device, called first among its forward pre-hooks (:123-247)."""
+    for child in module.children():
+        if isinstance(child, nn.Dropout):
+            continue
+        _add_observer_(child, qconfig_propagation_list, device)
+    is_leaf = not any(True for _ in module.children())
+    if (is_leaf and not isinstance(module, nn.Sequential) and type_before_parametrizations(module) in qconfig_propagation_list
+            and getattr(module, "qconfig", None) is not None):
+        observer = module.qconfig.activation()
+        devices = _module_devices(module)
+        assert len(devices) <= 1, f"_add_observer_ only works with cpu or single-device CUDA modules, but got devices {devices}"
+        if devices:
+            observer.to(next(iter(devices)))
+        module.add_module("activation_post_process", observer)
+        module.register_forward_pre_hook(_observer_forward_pre_hook, prepend=True)
 
 
-def convert(model, *args, **kwargs):
-    """Static-calibration entry point of the reference (:360-391); not part of the dynamic W8A8 path."""
-    raise NotImplementedError("static calibration (prepare/convert) is not built; use quantize_dynamic")
+def prepare(model, qconfig_dict=None, inplace=True, observer_non_leaf_module_list=None):
+    """Attaches qconfigs and activation observers for calibration (:250-301); run data through the model
+    afterwards, then ``convert``."""
+    if observer_non_leaf_module_list:
+        raise NotImplementedError("observers on non-leaf modules are not built")
+    if not inplace:
+        model = copy.deepcopy(model)
+    propagate_qconfig_(model, qconfig_dict)
+    if not any(getattr(m, "qconfig", None) for m in model.modules()):
+        import warnings
+
+        warnings.warn("None of the submodule got qconfig applied. Make sure you passed correct configuration through "
+                      "`qconfig_dict` or by assigning the `.qconfig` attribute directly on submodules")
+    _add_observer_(model, get_default_qconfig_propagation_list())
+    return model
+
+
+def convert(model, mapping=None, inplace=True, remove_qconfig=True):
+    """Swaps the prepared (and calibrated) modules by the static mapping (:360-391)."""
+    if mapping is None:
+        mapping = get_default_static_quant_module_mappings()
+    if not inplace:
+        model = copy.deepcopy(model)
+    _convert(model, mapping)
+    if remove_qconfig:
+        _remove_qconfig(model)
+    return model

@@ -126,6 +126,27 @@ int daxq_quantize_rows_i8(const void* x, int64_t m, int64_t k, int64_t ld_x, con
                           int8_t* q, int64_t ld_q, daxq_stream_t stream);
 int daxq_quantize_rows_e4m3(const void* x, int64_t m, int64_t k, int64_t ld_x, const float* scale,
                             uint8_t* q, int64_t ld_q, daxq_stream_t stream);
+int daxq_quantize_rows_e5m2(const void* x, int64_t m, int64_t k, int64_t ld_x, const float* scale,
+                            uint8_t* q, int64_t ld_q, daxq_stream_t stream);
+
+/*
+ * Per-tensor schemes (the block of dax/quant/qscheme.py:10-26 is the whole tensor).  The GEMM and the leaf
+ * quantisers above take a scale per row / per channel; a per-tensor scale is handed to them written out as a
+ * vector, which gives the same arithmetic per element.  These entry points keep that on the device.
+ *
+ * daxq_tensor_scale: dynamic per-tensor scale from per-row statistics (daxq_row_minmax):
+ *   a = max_i max(-row_min[i], row_max[i]);  scale1[0] = max( round(a / qmax), 2^-23 ), round = bf16 RNE when
+ *   round_bf16 != 0 (the activation rule, dax/quant/nn/dynamic/functional.py:124-129) or none (observer rule,
+ *   dax/quant/quantization/observer.py:97-134); expand[0..n_expand) receives the same value.
+ * daxq_tensor_minmax_update: running min / max of a calibration observer,
+ *   dax/quant/quantization/observer.py:200-214:  min_inout[0] = min(min_inout[0], min_i row_min[i]), same for max.
+ * daxq_broadcast_f32: dst[0..n) = src[0]; how dax/quant/nn/quantized/linear.py:98-100 expands its input scale.
+ */
+int daxq_tensor_scale(const float* row_min, const float* row_max, int64_t m, float qmax, int round_bf16,
+                      float* scale1, float* expand, int64_t n_expand, daxq_stream_t stream);
+int daxq_tensor_minmax_update(const float* row_min, const float* row_max, int64_t m,
+                              float* min_inout, float* max_inout, daxq_stream_t stream);
+int daxq_broadcast_f32(const float* src, float* dst, int64_t n, daxq_stream_t stream);
 
 /*
  * Per-row min and max of a bf16 matrix, in fp32: the statistics of the per-channel weight observer.

@@ -28,6 +28,8 @@ How each function is pinned (see tests/test_oracle_*.py):
   gelu_tanh_bf16           result may differ from an exact evaluation by one ulp
                            at rounding boundaries (floating point: tolerance
                            stated in the tests); gelu checked on every bf16 input
+* act_scale_per_tensor /   reduce to the per-row functions above on the tensor flattened
+  weight_scale_per_tensor  to one row (tests/test_oracle_pins.py)
 * linear_fp8               accumulation order is not fixed by the reference
                            (cuBLASLt fast-accum): "parity unpinned" at bit
                            level, tolerance 2e-2 relative L2; the per-tensor
@@ -265,4 +267,54 @@ def gelu_tanh_bf16(x: torch.Tensor) -> torch.Tensor:
     """``gelu(x, approximate="tanh")`` of a bf16 tensor: evaluated in fp32, rounded once to bf16
     (the activation between the two FFN linears of the DiT)."""
     return torch.nn.functional.gelu(x.float(), approximate="tanh").to(x.dtype)
+
+
+# --------------------------------------------------------------------------- #
+# per-tensor schemes and the static FP8 linear
+# --------------------------------------------------------------------------- #
+def act_scale_per_tensor(x: torch.Tensor, qmax: float) -> torch.Tensor:
+    """Dynamic per-tensor scale, eager dtype chain: the block of dax/quant/qscheme.py:10-26 is the whole
+    tensor, so dax/quant/nn/dynamic/functional.py:124-129 reduces over every dimension.  fp32 [1]."""
+    amax = x.abs().amax()
+    scale = torch.clamp(amax / float(qmax), min=EPS)
+    return scale.to(torch.float32).reshape(1)
+
+
+def weight_scale_per_tensor(w: torch.Tensor, qmax: float) -> torch.Tensor:
+    """MinMaxObserver + _calculate_qparams: dax/quant/quantization/observer.py:200-214 and :97-134, fp32 [1]."""
+    lo, hi = torch.aminmax(w.detach().to(torch.float32))
+    amax = torch.max(-lo, hi)
+    return torch.max(amax / float(qmax), torch.tensor([EPS], dtype=torch.float32)).reshape(1)
+
+
+def linear_int8_schemes(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], act_per_tensor: bool,
+                        weight_per_tensor: bool) -> Dict[str, torch.Tensor]:
+    """INT8 forward for any of the four scheme pairs of dax/quant/nn/dynamic/linear.py:180-228 (the scalar
+    scales broadcast in :214 and :222)."""
+    x2 = x.reshape(-1, x.shape[-1])
+    sw = weight_scale_per_tensor(w, INT8_QMAX) if weight_per_tensor else weight_scale(w, INT8_QMAX)
+    qw = quantize_to_int8(w, sw.reshape(-1, 1))
+    if act_per_tensor:
+        sx = act_scale_per_tensor(x2, INT8_QMAX)
+        xq = quantize_to_int8(x2, sx)
+        sx_rows = sx.expand(x2.shape[0])
+    else:
+        xq, sx = act_quant_int8(x2)
+        sx_rows = sx.reshape(-1)
+    acc = int_mm(xq, qw)
+    out = epilogue_int8(acc, sx_rows, sw.expand(w.shape[0]) if sw.numel() == 1 else sw, bias, x.dtype)
+    return {"xq": xq, "sx": sx, "qw": qw, "sw": sw, "acc": acc, "out": out.view(*x.shape[:-1], w.shape[0])}
+
+
+def static_linear_fp8(x: torch.Tensor, input_scale: torch.Tensor, qweight: torch.Tensor, wscale: torch.Tensor,
+                      bias: Optional[torch.Tensor], act_dtype: torch.dtype = torch.float8_e4m3fn) -> Dict[str, torch.Tensor]:
+    """Static FP8 forward, dax/quant/nn/quantized/linear.py:91-118: leaf quantiser with the stored input scale,
+    then ``_scaled_mm`` emulated in fp32 (accumulation order of the reference unspecified: tolerance)."""
+    x2 = x.reshape(-1, x.shape[-1])
+    xq = quantize_to_fp8(x2, input_scale.reshape(1), act_dtype)
+    acc = xq.to(torch.float32) @ qweight.to(torch.float32).t()
+    o = acc * input_scale.reshape(1) * wscale.reshape(1, -1)
+    if bias is not None:
+        o = o + bias.to(torch.float32)
+    return {"xq": xq, "out": o.to(torch.bfloat16).view(*x.shape[:-1], qweight.shape[0])}
 

@@ -370,3 +370,39 @@ def test_make_inputs_is_seeded_and_has_outliers():
     col_std = x1.float().std(0)
     assert (col_std > 10).sum() == 15  # round(0.01 * 1536) outlier channels, x20
     assert abs(w1.float().std().item() - 0.02) < 2e-3 and abs(b1.float().std().item() - 0.01) < 5e-3
+
+
+def test_per_tensor_scales_reduce_to_the_per_row_functions():
+    """A per-tensor block is the per-row rule applied to the tensor flattened into one row."""
+    g = torch.Generator().manual_seed(9)
+    x = (torch.randn(37, 96, generator=g) * 5).bfloat16()
+    for qmax in (O.INT8_QMAX, O.E4M3_QMAX, O.E5M2_QMAX):
+        assert torch.equal(O.act_scale_per_tensor(x, qmax), O.act_scale(x.reshape(1, -1), qmax).reshape(1))
+        assert torch.equal(O.weight_scale_per_tensor(x, qmax), O.weight_scale(x.reshape(1, -1), qmax).reshape(1))
+    z = torch.zeros(4, 8).bfloat16()
+    assert float(O.act_scale_per_tensor(z, 127)) == 2.0 ** -23 and float(O.weight_scale_per_tensor(z, 127)) == 2.0 ** -23
+    # the four INT8 scheme pairs agree with the per-token / per-channel chain when every row / channel has the same amax
+    x2 = torch.tensor([[1.0, -2.0, 4.0, 0.5]] * 3).bfloat16()
+    w2 = torch.tensor([[0.5, -1.0, 0.25, 1.0]] * 5).bfloat16()
+    b = torch.zeros(5).bfloat16()
+    base = O.linear_int8_schemes(x2, w2, b, False, False)["out"]
+    for ap, wp in ((True, False), (False, True), (True, True)):
+        assert torch.equal(O.linear_int8_schemes(x2, w2, b, ap, wp)["out"], base)
+
+
+def test_static_linear_fp8_matches_the_float_layer():
+    g = torch.Generator().manual_seed(4)
+    x = torch.randn(64, 128, generator=g).bfloat16()
+    w = (torch.randn(32, 128, generator=g) * 0.05).bfloat16()
+    b = (torch.randn(32, generator=g) * 0.01).bfloat16()
+    si = O.weight_scale_per_tensor(x, O.E4M3_QMAX)                 # what a MinMaxObserver calibrated on x gives
+    sw = O.weight_scale_per_tensor(w, O.E4M3_QMAX)
+    qw = O.quantize_to_fp8(w, sw)
+    out = O.static_linear_fp8(x, si, qw, sw, b)["out"]
+    ref = torch.nn.functional.linear(x.float(), w.float(), b.float())
+    assert float((out.float() - ref).norm() / ref.norm()) < 6e-2    # fp8 (3 mantissa bits) quantisation error
+    # per-tensor special case of the library routine on CPU
+    lib = torch._scaled_mm(O.quantize_to_fp8(x, si), qw.t(), scale_a=si.reshape(()), scale_b=sw.reshape(()), bias=b,
+                           out_dtype=torch.bfloat16)
+    assert float((out.float() - lib.float()).norm() / lib.float().norm()) < 4e-3
+
