@@ -354,3 +354,50 @@ def test_block_fusion_host_logic_without_gpu():
     assert qa.shape == (2, 3, 16)
     with pytest.raises(ValueError):
         lin(8, 32, 3)(qa)                                         # K mismatch is reported, not mis-computed
+
+
+def test_prequantised_checkpoint_round_trip_from_a_meta_skeleton(tmp_path):
+    """save_quantized / load_quantized: the file holds the reference's module state; loading builds the
+    quantised modules from the qconfig on a meta skeleton and copies, no kernel involved (runs on the CPU)."""
+    from dax_amd.quant.checkpoint import load_quantized, save_quantized
+    from dax_amd.quant.nn import dynamic, quantized
+    from dax_amd.quant.qscheme import per_channel_symmetric, per_token_symmetric
+    from dax_amd.quant.quantization.qconfig import get_default_fp8_qconfig
+
+    src = Outer()
+    g = torch.Generator().manual_seed(0)
+    q = dynamic.Linear(8, 8, True, None, torch.int8, torch.int8, torch.bfloat16, per_channel_symmetric, per_token_symmetric)
+    q.qweight.copy_(torch.randint(-127, 128, (8, 8), generator=g, dtype=torch.int8))
+    q.weight_scale.copy_(torch.rand(1, 8, generator=g))
+    with torch.no_grad():
+        q.bias.copy_(torch.randn(8, generator=g))
+    src.block.fc = q
+    path = str(tmp_path / "m.safetensors")
+    save_quantized(src, path)
+    with torch.device("meta"):
+        skel = Outer()
+    out = load_quantized(skel, path, {"block": _cfg()}, device="cpu")
+    assert isinstance(out.block.fc, dynamic.Linear) and type(out.embed.fc) is nn.Linear
+    assert not any(p.device.type == "meta" for p in out.parameters())
+    for k, v in src.state_dict().items():
+        assert torch.equal(out.state_dict()[k].view(torch.uint8) if v.dtype == torch.int8 else out.state_dict()[k], 
+                           v.view(torch.uint8) if v.dtype == torch.int8 else v), k
+    assert not any(hasattr(m, "qconfig") for m in out.modules())
+    # a static qconfig gives the static module (fp8 tensors are stored natively in the file)
+    s = Outer()
+    st = quantized.Linear(8, 8, True, None, torch.float8_e4m3fn, torch.float8_e5m2, torch.bfloat16, False)
+    with torch.no_grad():
+        st.qweight.copy_(torch.randn(8, 8, generator=g).to(torch.float8_e4m3fn))
+        st.input_scale.fill_(0.25)
+        st.bias.zero_()
+    s.block.fc = st
+    save_quantized(s, path)
+    with torch.device("meta"):
+        skel2 = Outer()
+    out2 = load_quantized(skel2, path, {"block": get_default_fp8_qconfig()}, device="cpu")
+    assert isinstance(out2.block.fc, quantized.Linear) and float(out2.block.fc.input_scale) == 0.25
+    assert torch.equal(out2.block.fc.qweight.view(torch.uint8), st.qweight.view(torch.uint8))
+    with pytest.raises(RuntimeError):                         # a skeleton that does not match the file is reported
+        with torch.device("meta"):
+            bad = Outer()
+        load_quantized(bad, path, {}, device="cpu")
