@@ -153,7 +153,7 @@ def int_mm(xq: torch.Tensor, wq: torch.Tensor) -> torch.Tensor:
     """int8 [M,K] x int8 [N,K]^T -> int32 [M,N], exact.
 
     dax/quant/nn/dynamic/linear.py:218-220 (out_dtype(aten.mm, int32, ...)).
-    torch._int_mm is the library routine BASELINE names for the CPU path; it is
+    torch._int_mm is the library routine of the CPU path; it is
     exact integer arithmetic, so any summation order gives the same bits.
     """
     return torch._int_mm(xq.contiguous(), wq.t())

@@ -1,4 +1,4 @@
-"""Parity at the exact shapes of the benchmark configurations (BASELINE.json configs 0, 1, 2/3, 4),
+"""Parity at the exact shapes of the five benchmark configurations (config 0: M=4096, K=N=1536; 1: Wan 1.3B 480p; 2 / 3: Wan 14B 720p INT8 / FP8; 4: the 40-layer set),
 through the swapped module.  Rows of a per-token-quantised linear are independent, so at the large M a
 sample of rows (first / last rows of the first / last tiles plus random ones) is compared with the
 oracle bit for bit (INT8) or within 2e-2 relative L2 (FP8), and the whole output is tied to it by
