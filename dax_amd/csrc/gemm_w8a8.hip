@@ -270,11 +270,11 @@ static int launch_gemm(const void* xq, int64_t ld_xq, const float* sx, const voi
     a.gm = g_gm;
     switch (g_variant) {
         case 0: {
-            // library default: the five-stage 256x256 kernel once its tiles fill at least half of the
-            // 256 CUs, otherwise 128x128 tiles (4x as many workgroups; measured cross-over between
-            // M = 1024 and M = 2048 at N = K = 5120)
+            // library default: the five-stage 256x256 kernel once its tiles fill about a third of the
+            // 256 CUs, otherwise 128x128 tiles (4x as many workgroups; measured cross-over at
+            // N = K = 5120: M = 512 -> 642 against 533 T-op/s, M = 1024 -> 948 against 1012)
             const int64_t tiles256 = ((m + 255) / 256) * ((n + 255) / 256);
-            if (tile256_applies(a) && tiles256 >= 128) return launch_tile256s5<FP8>(a, x_e5m2, st);
+            if (tile256_applies(a) && tiles256 >= 80) return launch_tile256s5<FP8>(a, x_e5m2, st);
             if constexpr (FP8) {
                 if (x_e5m2) return launch_cfg<true, 128, 128, 128, 2, 2, true, true>(a, st);
             }
