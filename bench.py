@@ -23,8 +23,9 @@ SHAPES = [("qkv", 5120, 15360), ("out", 5120, 5120), ("ffn_up", 5120, 13824), ("
 PEAK_TOPS = {"int8": 5000.0, "fp8": 5000.0}  # MI355X dense 8-bit MFMA peak
 # Bytes that left L2 towards the fabric per GEMM launch (average of the four shapes), from the rocprofv3
 # FETCH_SIZE / WRITE_SIZE passes over this same command, scaled by the 1 GiB copy in the same run
-# (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0): (8403372 + 1456260) KiB.  Includes Infinity Cache hits.
-GEMM_TRAFFIC_BYTES = {"int8": (8403372 + 1456260) * 1024, "fp8": None}
+# (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0): int8 (8403372 + 1456260) KiB, fp8 (8555857 + 1456106) KiB.  Includes
+# Infinity Cache hits.
+GEMM_TRAFFIC_BYTES = {"int8": (8403372 + 1456260) * 1024, "fp8": (8555857 + 1456106) * 1024}
 
 
 def cpu_baseline(dtype: str, rows: int):
