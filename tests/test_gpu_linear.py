@@ -153,6 +153,37 @@ def test_linear_rejects_unaligned_k(ops):
         ops.linear_i8(xq, torch.ones(8, device="cuda"), wq, torch.ones(8, device="cuda"), None)
 
 
+@pytest.mark.parametrize("variant", [0, 5, 6, 8])
+def test_linear_leading_dimensions_through_the_c_abi(ops, variant):
+    """Operands and output as column slices of wider buffers (ld > logical width), straight through the C ABI:
+    what a caller does that writes q | k | v into one [M, 3N] tensor with three launches."""
+    from dax_amd import _capi
+
+    _capi.set_gemm_variant(variant)
+    m, n, k = 600, 520, 384
+    x, w, b = O.make_inputs(m, k, n, seed=77)
+    qw, sw = O.weight_quant_int8(w)
+    ref = O.linear_int8(x, qw, sw, b)
+    xq_wide = torch.full((m, k + 128), 7, dtype=torch.int8, device="cuda")
+    xq_wide[:, :k] = dev(ref["xq"])
+    wq_wide = torch.full((n, k + 256), -3, dtype=torch.int8, device="cuda")
+    wq_wide[:, :k] = dev(qw)
+    out_wide = torch.full((m, 3 * n + 8), 1.0, dtype=torch.bfloat16, device="cuda")
+    acc_wide = torch.zeros((m, n + 4), dtype=torch.int32, device="cuda")
+    sx, swd, bd = dev(ref["sx"].reshape(-1).contiguous()), dev(sw.reshape(-1).contiguous()), dev(b)
+    col0 = n + 8                                                    # 16-byte aligned column offset
+    rc = _capi.lib().daxq_linear_i8(xq_wide.data_ptr(), k + 128, sx.data_ptr(), wq_wide.data_ptr(), k + 256, swd.data_ptr(),
+                                    bd.data_ptr(), out_wide.data_ptr() + 2 * col0, 3 * n + 8, acc_wide.data_ptr(), n + 4,
+                                    m, n, k, torch.cuda.current_stream().cuda_stream)
+    _capi.check(rc, "linear_i8")
+    torch.cuda.synchronize()
+    assert torch.equal(out_wide[:, col0:col0 + n].cpu().view(torch.int16), ref["out"].view(torch.int16))
+    assert torch.equal(acc_wide[:, :n].cpu(), ref["acc"])
+    assert bool((out_wide[:, :col0] == 1).all()) and bool((out_wide[:, col0 + n:] == 1).all())   # nothing outside the slice
+    assert bool((acc_wide[:, n:] == 0).all())
+    _capi.set_gemm_variant(0)
+
+
 # --------------------------------------------------------------------------- the swapped module
 class ToyBlock(nn.Module):
     def __init__(self, d=256, f=520):
