@@ -22,12 +22,6 @@ namespace daxq {
 
 enum { PRE_LN = 1, PRE_GELU = 2 };
 
-__device__ __forceinline__ float wave_sum_f32(float v) {
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off, 64);
-    return v;
-}
-
 __device__ __forceinline__ void unpack8(const uint4& v, float (&f)[8]) {
     const uint32_t w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll

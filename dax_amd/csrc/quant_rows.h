@@ -24,13 +24,43 @@ __device__ __forceinline__ float scale_from_amax_bits(uint32_t amax_bits, float 
     return fmaxf(s, kEps);
 }
 
+// Wavefront-wide reductions with DPP (data-parallel primitives: the partner lane's value is an operand
+// modifier of the VALU instruction, no trip through the LDS crossbar as with ds_bpermute): four steps
+// give every lane the result of its row of 16 lanes, the four row results are then read as scalars.
+#define DAXQ_DPP_QUAD_SWAP1 0xB1   /* quad_perm [1,0,3,2] */
+#define DAXQ_DPP_QUAD_SWAP2 0x4E   /* quad_perm [2,3,0,1] */
+#define DAXQ_DPP_HALF_MIRROR 0x141 /* lane i <-> 7 - i within 8 */
+#define DAXQ_DPP_ROW_MIRROR 0x140  /* lane i <-> 15 - i within 16 */
+
+template <int CTRL>
+__device__ __forceinline__ uint32_t dpp_u32(uint32_t v) {
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xf, 0xf, true);
+}
+
 __device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) {
-        uint32_t o = (uint32_t)__shfl_xor((int)v, off, 64);
-        v = v > o ? v : o;
-    }
-    return v;
+    uint32_t o;
+    o = dpp_u32<DAXQ_DPP_QUAD_SWAP1>(v); v = v > o ? v : o;
+    o = dpp_u32<DAXQ_DPP_QUAD_SWAP2>(v); v = v > o ? v : o;
+    o = dpp_u32<DAXQ_DPP_HALF_MIRROR>(v); v = v > o ? v : o;
+    o = dpp_u32<DAXQ_DPP_ROW_MIRROR>(v); v = v > o ? v : o;
+    const uint32_t r0 = (uint32_t)__builtin_amdgcn_readlane((int)v, 0), r1 = (uint32_t)__builtin_amdgcn_readlane((int)v, 16);
+    const uint32_t r2 = (uint32_t)__builtin_amdgcn_readlane((int)v, 32), r3 = (uint32_t)__builtin_amdgcn_readlane((int)v, 48);
+    const uint32_t a = r0 > r1 ? r0 : r1, b = r2 > r3 ? r2 : r3;
+    return a > b ? a : b;
+}
+
+// fp32 sum over the wavefront, the same value in every lane (fixed order: deterministic)
+__device__ __forceinline__ float wave_sum_f32(float x) {
+    uint32_t v = __float_as_uint(x);
+    v = __float_as_uint(__uint_as_float(v) + __uint_as_float(dpp_u32<DAXQ_DPP_QUAD_SWAP1>(v)));
+    v = __float_as_uint(__uint_as_float(v) + __uint_as_float(dpp_u32<DAXQ_DPP_QUAD_SWAP2>(v)));
+    v = __float_as_uint(__uint_as_float(v) + __uint_as_float(dpp_u32<DAXQ_DPP_HALF_MIRROR>(v)));
+    v = __float_as_uint(__uint_as_float(v) + __uint_as_float(dpp_u32<DAXQ_DPP_ROW_MIRROR>(v)));
+    const float r0 = __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)v, 0));
+    const float r1 = __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)v, 16));
+    const float r2 = __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)v, 32));
+    const float r3 = __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)v, 48));
+    return (r0 + r1) + (r2 + r3);
 }
 
 __device__ __forceinline__ int q_i8(float x, float inv) {
