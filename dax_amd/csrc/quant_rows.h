@@ -70,10 +70,22 @@ __device__ __forceinline__ int q_i8(float x, float inv) {
 }
 
 // FMT: 0 = int8, 1 = OCP e4m3fn (max 448), 2 = OCP e5m2 (max 57344)
-template <int FMT>
-__device__ __forceinline__ float q_f8_pre(float x, float s) {
+// x / s, correctly rounded, from the correctly rounded reciprocal inv = RN(1 / s) of the row: one multiply,
+// the exact residual by fma, one correction (Markstein's sequence; it yields RN(x / s) unless the
+// significand of s is all ones, which a scale whose low 16 bits are zero never has).  The reference's
+// true division costs about ten instructions per element when spelled x / s.
+// TRUE_DIV: spell the division out (leaf quantiser with an arbitrary fp32 scale, used once per weight).
+template <int FMT, bool TRUE_DIV>
+__device__ __forceinline__ float q_f8_pre(float x, float s, float inv) {
     constexpr float kMax = FMT == 2 ? 57344.0f : 448.0f;
-    float v = x / s;  // IEEE division per element
+    float v;
+    if constexpr (TRUE_DIV) {
+        v = x / s;  // IEEE division
+    } else {
+        const float q0 = x * inv;
+        const float e = __builtin_fmaf(-q0, s, x);
+        v = __builtin_copysignf(__builtin_fmaf(e, inv, q0), x);  // s > 0; keeps -0 for x = -0 (0 + -0 is +0 in the fma)
+    }
     return fminf(fmaxf(v, -kMax), kMax);
 }
 
@@ -86,7 +98,7 @@ __device__ __forceinline__ int cvt_pk_f8(float a, float b, int old, bool hi) {
 }
 
 // 8 bf16 (one 16-byte chunk) -> 8 quantised bytes
-template <int FMT>
+template <int FMT, bool TRUE_DIV = false>
 __device__ __forceinline__ uint2 quant_chunk(const uint4& v, float s, float inv) {
     const uint32_t w[4] = {v.x, v.y, v.z, v.w};
     uint32_t o[2];
@@ -97,8 +109,8 @@ __device__ __forceinline__ uint2 quant_chunk(const uint4& v, float s, float inv)
         float f2 = __uint_as_float(w[2 * h + 1] << 16);
         float f3 = __uint_as_float(w[2 * h + 1] & 0xffff0000u);
         if (FMT != 0) {
-            int p = cvt_pk_f8<FMT>(q_f8_pre<FMT>(f0, s), q_f8_pre<FMT>(f1, s), 0, false);
-            p = cvt_pk_f8<FMT>(q_f8_pre<FMT>(f2, s), q_f8_pre<FMT>(f3, s), p, true);
+            int p = cvt_pk_f8<FMT>(q_f8_pre<FMT, TRUE_DIV>(f0, s, inv), q_f8_pre<FMT, TRUE_DIV>(f1, s, inv), 0, false);
+            p = cvt_pk_f8<FMT>(q_f8_pre<FMT, TRUE_DIV>(f2, s, inv), q_f8_pre<FMT, TRUE_DIV>(f3, s, inv), p, true);
             o[h] = (uint32_t)p;
         } else {
             uint32_t b0 = (uint32_t)q_i8(f0, inv) & 0xffu;

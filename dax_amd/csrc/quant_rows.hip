@@ -67,7 +67,7 @@ __global__ __launch_bounds__(256) void quant_rows_wave(const uint16_t* __restric
     for (int i = 0; i < NCH; ++i) {
         const int c = i * 64 + lane;
         if (c < nch) {
-            qr[c] = quant_chunk<FMT>(v[i], s, inv);
+            qr[c] = quant_chunk<FMT, SCALE_IN>(v[i], s, inv);
         } else if (c < npad) {
             qr[c] = make_uint2(0, 0);
         }
@@ -108,7 +108,7 @@ __global__ __launch_bounds__(256) void quant_rows_block(const uint16_t* __restri
         if (c < k) {
             float f = bf16_bits_to_f32(xr[c]);
             if (FMT != 0) {
-                o = (uint8_t)(cvt_pk_f8<FMT>(q_f8_pre<FMT>(f, s), 0.0f, 0, false) & 0xff);
+                o = (uint8_t)(cvt_pk_f8<FMT>(q_f8_pre<FMT, SCALE_IN>(f, s, inv), 0.0f, 0, false) & 0xff);
             } else {
                 o = (uint8_t)(q_i8(f, inv) & 0xff);
             }

@@ -122,6 +122,37 @@ def test_act_scale_exhaustive_every_bf16_amax(ops, fp8):
     np.testing.assert_array_equal(q[:, :64].cpu().numpy(), qo_b)
 
 
+@pytest.mark.parametrize("fmt", ["e4m3", "e5m2"])
+def test_dynamic_fp8_division_every_bf16_value_under_sampled_abs_max(ops, fmt):
+    """The dynamic FP8 quantiser divides through the row's reciprocal with an exact fma correction instead of a
+    spelled-out division: every finite bf16 value that fits under a row abs-max, for 640 abs-max values spread over
+    all exponents (both signs), must still give the bytes of the reference's true division."""
+    rng = np.random.default_rng(11)
+    amax_bits = np.unique(np.concatenate([rng.choice(ALL_POS_FINITE[1:], 600, replace=False),
+                                          ALL_POS_FINITE[-20:], ALL_POS_FINITE[1:21]]))
+    allv = from_bits(FINITE_BF16)                                   # 65280 values
+    chunks = allv.view(-1, 16320)                                   # 4 x 16320
+    rows = []
+    for ab in amax_bits:
+        a = from_bits(np.array([ab], dtype=np.uint16))
+        body = torch.where(chunks.float().abs() <= a.float(), chunks, torch.zeros_like(chunks))
+        head = torch.zeros(4, 8, dtype=torch.bfloat16)
+        head[:, 0] = a if ab % 2 == 0 else -a
+        rows.append(torch.cat([head, body], 1))                     # 4 rows of 16328 (wave kernel: row in registers)
+    x = torch.cat(rows)
+    fn, ofn = (ops.act_quant_e4m3, O.act_quant_e4m3) if fmt == "e4m3" else (ops.act_quant_e5m2, O.act_quant_e5m2)
+    q, s = fn(dev(x))
+    qo, so = ofn(x)
+    np.testing.assert_array_equal(s.cpu().numpy().view(np.uint32), so.view(-1).numpy().view(np.uint32))
+    bad = int((q[:, :x.shape[1]].cpu() != qo.view(torch.uint8)).sum())
+    assert bad == 0, f"{bad} of {x.numel()} bytes differ"
+    # the general (one block per row) kernel takes the same formula: rows too long for the register kernel
+    xl = x.view(-1, 4 * 16328)[:40].contiguous()
+    q2, s2 = fn(dev(xl))
+    qo2, so2 = ofn(xl)
+    assert torch.equal(q2[:, :xl.shape[1]].cpu(), qo2.view(torch.uint8)) and torch.equal(s2.cpu(), so2.view(-1))
+
+
 def _sampled_scales(qmax, n_act, n_f32, seed):
     x = from_bits(ALL_POS_FINITE).view(-1, 1)
     reach = np.unique(O.act_scale(x, qmax).view(-1).numpy())
