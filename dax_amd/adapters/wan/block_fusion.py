@@ -26,6 +26,7 @@ quantiser behind it.  The reference leaves those fusions to ``torch.compile``
 from __future__ import annotations
 
 import types
+import weakref
 from typing import Optional, Sequence
 
 import torch
@@ -66,19 +67,22 @@ def gelu_tanh_quant(x: Tensor, like: Linear) -> QuantizedActivation:
 
 
 class _SharedQuant:
-    """Remembers the quantised form of the last tensor seen, keyed by identity and version."""
+    """Remembers the quantised form of the last tensor seen.  A hit needs the same tensor object (held
+    through a weak reference, so a new tensor that reuses a freed address cannot match) at the same
+    version counter (any in-place write since then misses)."""
 
     def __init__(self):
-        self.key, self.qa = None, None
+        self.ref, self.version, self.dtype, self.qa = None, None, None, None
 
     def get(self, lin: Linear, x: Tensor) -> QuantizedActivation:
-        key = (x.data_ptr(), x._version, tuple(x.shape), tuple(x.stride()), lin.input_dtype)
-        if key != self.key:
-            self.qa, self.key = lin.quantize_activation(x), key
+        hit = self.ref is not None and self.ref() is x and self.version == x._version and self.dtype == lin.input_dtype
+        if not hit:
+            self.qa = lin.quantize_activation(x)
+            self.ref, self.version, self.dtype = weakref.ref(x), x._version, lin.input_dtype
         return self.qa
 
     def clear(self):
-        self.key, self.qa = None, None
+        self.ref, self.version, self.dtype, self.qa = None, None, None, None
 
 
 def share_input_quant(linears: Sequence[Linear]) -> _SharedQuant:

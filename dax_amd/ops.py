@@ -19,6 +19,13 @@ def pad_k(k: int) -> int:
     return (k + K_ALIGN - 1) // K_ALIGN * K_ALIGN
 
 
+def is_tracing(t: torch.Tensor) -> bool:
+    """True while a graph is being traced over ``t``: it has no storage address to key a cache on."""
+    from torch._subclasses.fake_tensor import FakeTensor
+
+    return torch.compiler.is_compiling() or isinstance(t, FakeTensor)
+
+
 def _stream(t: torch.Tensor) -> int:
     return torch.cuda.current_stream(t.device).cuda_stream
 

@@ -137,6 +137,9 @@ class Linear(nn.Module):
         kp = ops.pad_k(k)
         if kp == k and qw.is_contiguous():
             return qw
+        if ops.is_tracing(qw):
+            # a traced graph cannot key a cache on the storage address: pad inside the graph
+            return torch.nn.functional.pad(qw, (0, kp - k)).contiguous()
         key = (self.qweight.data_ptr(), self.qweight._version, str(qw.device))
         if self._packed is None or self._packed[0] != key:
             buf = torch.zeros((qw.shape[0], kp), dtype=qw.dtype, device=qw.device)
@@ -150,6 +153,8 @@ class Linear(nn.Module):
         ws = self.weight_scale
         if ws.numel() != 1:
             return ws.view(-1)
+        if ops.is_tracing(ws):
+            return ops.broadcast_f32(ws.reshape(1).contiguous(), self.out_features)
         key = (ws.data_ptr(), ws._version, str(ws.device))
         if self._sw_vec is None or self._sw_vec[0] != key:
             self._sw_vec = (key, ops.broadcast_f32(ws.reshape(1).contiguous(), self.out_features))
@@ -177,12 +182,14 @@ class Linear(nn.Module):
                              f"({self.input_dtype}, K={self.in_features})")
         wq = self._gemm_weight()
         sw = self._weight_scale_vector()
+        # the kernels are inference-only (no autograd formula): the bias enters as a plain tensor
+        bias = None if self.bias is None else self.bias.detach()
         if self.compute_dtype == "FP8" and self.input_dtype == torch.float8_e5m2:
-            out = ops.linear_e5m2_e4m3(qa.xq, qa.sx, wq, sw, self.bias)
+            out = ops.linear_e5m2_e4m3(qa.xq, qa.sx, wq, sw, bias)
         elif self.compute_dtype == "FP8":
-            out = ops.linear_e4m3(qa.xq, qa.sx, wq, sw, self.bias)
+            out = ops.linear_e4m3(qa.xq, qa.sx, wq, sw, bias)
         else:
-            out = ops.linear_i8(qa.xq, qa.sx, wq, sw, self.bias)
+            out = ops.linear_i8(qa.xq, qa.sx, wq, sw, bias)
         out = out.view(*qa.prev_dims, self.out_features)
         if out.dtype != self.out_dtype:
             out = out.to(self.out_dtype)

@@ -66,6 +66,8 @@ class Linear(nn.Module):
         kp = ops.pad_k(k)
         if kp == k and qw.is_contiguous():
             return qw
+        if ops.is_tracing(qw):  # no cache keyed on a storage address inside a traced graph
+            return torch.nn.functional.pad(qw, (0, kp - k)).contiguous()
         key = (self.qweight.data_ptr(), self.qweight._version, str(qw.device))
         if self._packed is None or self._packed[0] != key:
             buf = torch.zeros((qw.shape[0], kp), dtype=qw.dtype, device=qw.device)
@@ -77,6 +79,8 @@ class Linear(nn.Module):
         ws = self.weight_scale
         if ws.numel() != 1:
             return ws.view(-1)
+        if ops.is_tracing(ws):
+            return ops.broadcast_f32(ws.reshape(1).contiguous(), self.out_features)
         key = (ws.data_ptr(), ws._version, str(ws.device))
         if self._sw_vec is None or self._sw_vec[0] != key:
             self._sw_vec = (key, ops.broadcast_f32(ws.reshape(1).contiguous(), self.out_features))
@@ -86,12 +90,13 @@ class Linear(nn.Module):
         prev_dims = input.shape[:-1]
         flat = input.view(-1, self.in_features)
         sx = ops.broadcast_f32(self.input_scale.reshape(1), flat.shape[0])
+        bias = None if self.bias is None else self.bias.detach()  # inference-only kernels
         if self.input_dtype == torch.float8_e5m2:
             xq = ops.quantize_rows_e5m2(flat, sx, True)
-            out = ops.linear_e5m2_e4m3(xq, sx, self._gemm_weight(), self._weight_scale_vector(), self.bias)
+            out = ops.linear_e5m2_e4m3(xq, sx, self._gemm_weight(), self._weight_scale_vector(), bias)
         else:
             xq = ops.quantize_rows_e4m3(flat, sx, True)
-            out = ops.linear_e4m3(xq, sx, self._gemm_weight(), self._weight_scale_vector(), self.bias)
+            out = ops.linear_e4m3(xq, sx, self._gemm_weight(), self._weight_scale_vector(), bias)
         out = out.view(*prev_dims, self.out_features)
         if out.dtype != self.out_dtype:
             out = out.to(self.out_dtype)

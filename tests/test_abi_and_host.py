@@ -401,3 +401,23 @@ def test_prequantised_checkpoint_round_trip_from_a_meta_skeleton(tmp_path):
         with torch.device("meta"):
             bad = Outer()
         load_quantized(bad, path, {}, device="cpu")
+
+
+@pytest.mark.parametrize("k", [384, 392])
+@pytest.mark.parametrize("dtype", [torch.int8, torch.float8_e4m3fn])
+def test_module_forward_traces_with_fake_tensors(dtype, k):
+    """Shape and dtype propagation through the fake kernels, as a tracer sees the module: no device, no
+    kernel call.  Also the per-tensor forms, whose scale vectors come from further ops."""
+    from torch._subclasses.fake_tensor import FakeTensorMode
+
+    from dax_amd.quant.nn.dynamic.linear import Linear
+    from dax_amd.quant.qscheme import per_channel_symmetric, per_tensor_symmetric, per_token_symmetric
+
+    for in_s, w_s in [(per_token_symmetric, per_channel_symmetric), (per_tensor_symmetric, per_tensor_symmetric)]:
+        with FakeTensorMode():
+            lin = Linear(k, 520, device="cuda", weight_dtype=dtype, input_dtype=dtype, weight_qscheme=w_s,
+                         input_qscheme=in_s)
+            qa = lin.quantize_activation(torch.empty(2, 300, k, dtype=torch.bfloat16, device="cuda"))
+            assert qa.xq.shape == (600, (k + 127) // 128 * 128) and qa.sx.shape == (600,) and qa.sx.dtype == torch.float32
+            y = lin(torch.empty(2, 300, k, dtype=torch.bfloat16, device="cuda"))
+            assert y.shape == (2, 300, 520) and y.dtype == torch.bfloat16 and y.device.type == "cuda"

@@ -55,7 +55,15 @@ def test_share_input_quant_and_fuse_linears_are_bit_identical():
         x.add_(1)                                                # in-place change: must not reuse the stale form
         attn.to_q(x)
         assert len(calls) == 2
+        y = x.clone()                                            # equal contents, another tensor: a miss
+        attn.to_k(y)
+        assert len(calls) == 3
+        del y
+        z = torch.empty_like(x).copy_(x).mul_(2)                 # may reuse the freed address of y
+        out_z = attn.to_v(z)
         cache.clear()
+        type(attn.to_q).quantize_activation = orig
+        assert torch.equal(out_z, attn.to_v(z))                  # not the stale quantised form of y
     finally:
         type(attn.to_q).quantize_activation = orig
 

@@ -1,0 +1,118 @@
+"""How the swapped module sits in a caller's runtime: inside a traced graph, on a stream that is not
+the default one, and inside a captured HIP graph that is replayed.
+
+The reference module is used under ``torch.compile`` (functional.py:33-36) and runs on whatever stream
+is current while a communication stream is busy (attn_adapter.py:102-160).  Each test compares the
+result with the same module called eagerly on the default stream, bit for bit (same kernels, same inputs).
+"""
+import pytest
+import torch
+from torch import nn
+
+from tests.util import bf16_bits
+
+pytestmark = pytest.mark.gpu
+
+
+def _mlp(k, n, fp8, seed):
+    from dax_amd.quant.quantization import quantize_dynamic
+    from dax_amd.quant.quantization.qconfig import (get_dynamic_fp8_per_token_act_per_channel_weight_qconfig,
+                                                    get_dynamic_int8_per_token_act_per_channel_weight_qconfig)
+
+    torch.manual_seed(seed)
+    model = nn.Sequential(nn.Linear(k, n), nn.GELU(approximate="tanh"), nn.Linear(n, k)).bfloat16().to("cuda")
+    cfg = (get_dynamic_fp8_per_token_act_per_channel_weight_qconfig(activation_dtype=torch.float8_e4m3fn)
+           if fp8 else get_dynamic_int8_per_token_act_per_channel_weight_qconfig())
+    quantize_dynamic(model, {"": cfg})
+    return model
+
+
+def _input(m, k, seed):
+    g = torch.Generator("cpu").manual_seed(seed)
+    return torch.randn(2, m, k, generator=g).bfloat16().to("cuda")
+
+
+def _same(a, b):
+    return (bf16_bits(a) == bf16_bits(b)).all()
+
+
+@pytest.mark.parametrize("k", [384, 392])  # 392: the weight is zero-padded to 512 columns inside the graph
+@pytest.mark.parametrize("fp8", [False, True])
+def test_traced_graph_matches_eager(fp8, k):
+    """One graph without breaks: every op has a fake kernel, so the tracer sees shapes and dtypes only."""
+    model = _mlp(k, 520, fp8, seed=1)
+    x = _input(300, k, seed=2)
+    ref = model(x)
+    traced = torch.compile(model, backend="aot_eager", fullgraph=True)
+    out = traced(x)
+    assert out.shape == ref.shape and out.dtype == torch.bfloat16
+    assert _same(out, ref)
+    x2 = _input(300, k, seed=3)
+    assert _same(traced(x2), model(x2))
+
+
+@pytest.mark.parametrize("fp8", [False, True])
+def test_side_stream_runs_beside_a_busy_default_stream(fp8):
+    """The kernels go to the stream that is current for the input's device, not to the default one: the
+    result is ready while a long spin kernel still holds the default stream."""
+    model = _mlp(512, 768, fp8, seed=4)
+    x = _input(700, 512, seed=5)
+    ref = model(x)
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    blocker_done, side_done = torch.cuda.Event(), torch.cuda.Event()
+    # a spin kernel of about half a second on the default stream; its counter's rate is measured first
+    t0, t1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0.record()
+    torch.cuda._sleep(1_000_000)
+    t1.record()
+    t1.synchronize()
+    ticks_per_ms = 1_000_000 / max(t0.elapsed_time(t1), 1e-3)
+    torch.cuda._sleep(int(min(500 * ticks_per_ms, 4e9)))
+    blocker_done.record()
+    with torch.cuda.stream(side):
+        out = model(x)
+        side_done.record()
+    side_done.synchronize()
+    finished_first = not blocker_done.query()
+    torch.cuda.synchronize()
+    assert _same(out, ref)
+    assert finished_first, "the linear waited for the default stream"
+
+
+@pytest.mark.parametrize("fp8", [False, True])
+def test_captured_graph_replays_match_eager(fp8):
+    """Capture the two linears (and a LayerNorm + quantiser launch in front) once, replay with new input
+    contents, with eager work and synchronisations between the replays; every replay must equal eager."""
+    import dax_amd.ops as ops
+
+    k, n, m = 640, 1024, 520
+    model = _mlp(k, n, fp8, seed=6)
+    lin0 = model[0]
+    ln_quant = ops.layernorm_act_quant_e4m3 if fp8 else ops.layernorm_act_quant_i8
+    from dax_amd.quant.nn.dynamic.linear import QuantizedActivation
+
+    def run(x):
+        q, s, _ = ln_quant(x.view(-1, k), None, None, x.numel() // k, 1e-6, False)
+        y = lin0(QuantizedActivation(q, s, x.shape[:-1], k, lin0.input_dtype))
+        return model[2](model[1](y))
+
+    static_x = _input(m, k, seed=7)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):  # first calls set kernel attributes: keep them outside the capture
+        for _ in range(2):
+            run(static_x)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        static_out = run(static_x)
+    for seed in (8, 9, 10, 11):
+        new_x = _input(m, k, seed=seed)
+        eager = run(new_x)
+        torch.cuda.synchronize()
+        static_x.copy_(new_x)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert _same(static_out, eager), f"replay with seed {seed} differs from eager"
