@@ -233,6 +233,81 @@ __device__ __forceinline__ void tile256_epilogue(const GemmArgs& p, typename Acc
     }
 }
 
+// The same epilogue for INT8 accumulators held as 8 x 8 blocks of 16x16 (v_mfma_i32_16x16x64_i8).
+// In a block a lane owns output row m = l%16 and the columns n = 4*(l/16) + {0..3}.  One
+// v_permlane16_swap per word over two neighbouring blocks gives each lane 8 consecutive columns of one
+// of them: lanes 0-15 block 2jp columns 0-7, lanes 16-31 block 2jp+1 columns 0-7, lanes 32-47 block
+// 2jp columns 8-15, lanes 48-63 block 2jp+1 columns 8-15.
+template <bool DUMP>
+__device__ __forceinline__ void tile256_epilogue16(const GemmArgs& p, v4i (&acc)[8][8], uint8_t* smem, int m0, int n0, int t,
+                                                   int wm, int wn, int l15, int g4, float pre_sx, float pre_sw,
+                                                   float pre_bias) {
+    float* s_sx = reinterpret_cast<float*>(smem);
+    float* s_sw = s_sx + 256;
+    float* s_bias = s_sw + 256;
+    s_sx[t] = pre_sx;
+    s_sw[t] = pre_sw;
+    s_bias[t] = pre_bias;
+    __syncthreads();
+
+    if constexpr (DUMP) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int64_t m = m0 + wm * 128 + i * 16 + l15;
+#pragma unroll
+                for (int v = 0; v < 4; ++v)
+                    static_cast<int32_t*>(p.acc)[m * p.ldacc + n0 + wn * 128 + j * 16 + 4 * g4 + v] = acc[j][i][v];
+            }
+    }
+
+    float sxr[8];
+    float4 swr[8], br[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) sxr[i] = s_sx[wm * 128 + i * 16 + l15];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const int nl = wn * 128 + j * 16 + 4 * g4;
+        swr[j] = *reinterpret_cast<const float4*>(s_sw + nl);
+        br[j] = *reinterpret_cast<const float4*>(s_bias + nl);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const int ml = wm * 128 + i * 16 + l15;
+        const float sxv = sxr[i];
+        uint16_t* orow = p.out + (int64_t)(m0 + ml) * p.ldo + n0 + wn * 128 + (g4 & 1) * 16 + (g4 >> 1) * 8;
+#pragma unroll
+        for (int jp = 0; jp < 4; ++jp) {
+            uint32_t pk[2][2];
+#pragma unroll
+            for (int jj = 0; jj < 2; ++jj) {
+                const int j = 2 * jp + jj;
+                const float sws[4] = {swr[j].x, swr[j].y, swr[j].z, swr[j].w};
+                const float bs[4] = {br[j].x, br[j].y, br[j].z, br[j].w};
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    const int r = 2 * h;
+                    float y0 = (float)acc[j][i][r];  // v_cvt_f32_i32, round to nearest even
+                    float y1 = (float)acc[j][i][r + 1];
+                    y0 = y0 * sxv;
+                    y1 = y1 * sxv;
+                    y0 = y0 * sws[r];
+                    y1 = y1 * sws[r + 1];
+                    const uint32_t o1 = pack_bf16_rne(y0, y1);
+                    // second rounding: the bias is added to the bf16 value
+                    pk[jj][h] = pack_bf16_rne(__uint_as_float(o1 << 16) + bs[r], __uint_as_float(o1 & 0xffff0000u) + bs[r + 1]);
+                }
+            }
+            v2u s0 = __builtin_amdgcn_permlane16_swap(pk[0][0], pk[1][0], false, false);
+            v2u s1 = __builtin_amdgcn_permlane16_swap(pk[0][1], pk[1][1], false, false);
+            *reinterpret_cast<uint4*>(orow + jp * 32) = make_uint4(s0.x, s1.x, s0.y, s1.y);
+        }
+    }
+}
+
 // DUMP: also write the raw accumulators to p.acc (tests); a separate instantiation so that the
 // production kernel carries none of that code.
 // EXP:  timing experiments with wrong results by construction: 1 = no HBM loads in the steady
@@ -489,14 +564,29 @@ constexpr int SMEM = NST * STAGE;                        // 163840
 constexpr int PAIR_LOADS = 16;                           // per thread and pair of slices
 }  // namespace t5
 
-template <bool FP8, bool DUMP, bool XE5>
+// accumulators of a wavefront's 128 x 128 outputs
+template <bool FP8, bool N16>
+struct TileAcc {
+    typedef typename AccT<FP8>::type type;  // 32x32 blocks
+};
+template <>
+struct TileAcc<false, true> {
+    typedef v4i type;  // 16x16 blocks
+};
+
+// N16 (INT8 only): the slice is one v_mfma_i32_16x16x64_i8 per 16x16 block (64 per wave and slice) instead
+// of two v_mfma_i32_32x32x32_i8 per 32x32 block (32).  Same LDS bytes, fragment registers and MFMA
+// cycles; the narrow shape moves fewer accumulator bytes per operation and sustains a higher clock
+// under the board's power limit.
+template <bool FP8, bool DUMP, bool XE5, bool N16 = false>
 __global__ __launch_bounds__(256) void gemm_tile256s5_kernel(const GemmArgs p) {
     using namespace t5;
-    typedef typename AccT<FP8>::type acc_t;
+    static_assert(!(FP8 && N16), "the 16x16 form exists for INT8 only");
     typedef typename Frag<FP8>::type frag_t;
-    constexpr int STEPS = FP8 ? 1 : 2;               // MFMA steps per 64-byte slice
-    constexpr int NREG = 16 * STEPS;                 // MFMAs = scheduling regions per slice
+    constexpr int STEPS = FP8 ? 1 : 2;               // MFMA steps per 64-byte slice (32x32 form)
+    constexpr int NREG = N16 ? 64 : 16 * STEPS;      // MFMAs = scheduling regions per slice
     constexpr int DMA_EVERY = NREG / (PAIR_LOADS / 2);  // regions per DMA load
+    constexpr int READ_EVERY = 3;                    // N16: regions per fragment read (16 reads)
 
     extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
 
@@ -532,12 +622,20 @@ __global__ __launch_bounds__(256) void gemm_tile256s5_kernel(const GemmArgs p) {
     };
 
     // ---- LDS side: row (w*128 + i*32 + l%32), chunk c of the slice at (c ^ g) * 16, g = (l%32 >> 2) & 3
+    //      N16: row (w*128 + i*16 + l%16), the lane's K chunk is l/16
     const int l31 = lane & 31, hi = lane >> 5;
-    const int gq = (l31 >> 2) & 3;
-    const uint8_t* a_rd = smem + (wm * 128 + l31) * BKS;
-    const uint8_t* b_rd = smem + A_BYTES + (wn * 128 + l31) * BKS;
+    const int lr = N16 ? (lane & 15) : l31;  // row of the lane inside an MFMA block
+    const int gq = (lr >> 2) & 3;
+    const uint8_t* a_rd = smem + (wm * 128 + lr) * BKS;
+    const uint8_t* b_rd = smem + A_BYTES + (wn * 128 + lr) * BKS;
     // one fragment: f = 0..3 A block f, 4..7 B block f-4; step ks of the slice in the stage at offset o
+    // (N16: ks selects the upper four of the eight 16-row blocks; every fragment spans the whole slice)
     auto read_frag = [&](uint32_t o, int ks, int f, frag_t (&af)[4], frag_t (&bf)[4]) {
+        if constexpr (N16) {
+            const uint8_t* pr = (f < 4 ? a_rd : b_rd) + o + (ks * 4 + (f & 3)) * 16 * BKS;
+            (f < 4 ? af[f & 3] : bf[f & 3]) = *reinterpret_cast<const v4i*>(pr + (((lane >> 4) ^ gq) << 4));
+            return;
+        }
         const uint8_t* pr = (f < 4 ? a_rd : b_rd) + o + (f & 3) * 32 * BKS;
         if constexpr (!FP8) {
             const int xo = ((ks * 2 + hi) ^ gq) << 4;
@@ -550,15 +648,15 @@ __global__ __launch_bounds__(256) void gemm_tile256s5_kernel(const GemmArgs p) {
         }
     };
 
-    acc_t acc[4][4];
+    typename TileAcc<FP8, N16>::type acc[N16 ? 8 : 4][N16 ? 8 : 4];
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+    for (int j = 0; j < (N16 ? 8 : 4); ++j)
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
+        for (int i = 0; i < (N16 ? 8 : 4); ++i)
 #pragma unroll
-            for (int v = 0; v < 16; ++v) acc[j][i][v] = 0;
+            for (int v = 0; v < (N16 ? 4 : 16); ++v) acc[j][i][v] = 0;
 
-    // fragment sets: [slice parity][MFMA step]
+    // fragment sets: [slice parity][MFMA step] (N16: [slice parity][blocks 0-3 / 4-7])
     frag_t fa00[4] = {}, fb00[4] = {}, fa01[4] = {}, fb01[4] = {}, fa10[4] = {}, fb10[4] = {}, fa11[4] = {}, fb11[4] = {};
 
     const int S = p.k / BKS;  // slices; even because K is a multiple of 128
@@ -581,7 +679,18 @@ __global__ __launch_bounds__(256) void gemm_tile256s5_kernel(const GemmArgs p) {
             if constexpr (ISSUE.value) {
                 if (g % DMA_EVERY == 0) issue_one(o_ld0, o_ld1, g / DMA_EVERY + (ODD.value ? PAIR_LOADS / 2 : 0));
             }
-            if constexpr (NEXT.value) {
+            if constexpr (NEXT.value && N16) {  // 16 reads, one every READ_EVERY regions
+                if (g % READ_EVERY == 0 && g / READ_EVERY < 16) {
+                    const int idx = g / READ_EVERY;
+                    if constexpr (ODD.value) {
+                        if (idx < 8) read_frag(o_next, 0, idx, fa00, fb00);
+                        else read_frag(o_next, 1, idx - 8, fa01, fb01);
+                    } else {
+                        if (idx < 8) read_frag(o_next, 0, idx, fa10, fb10);
+                        else read_frag(o_next, 1, idx - 8, fa11, fb11);
+                    }
+                }
+            } else if constexpr (NEXT.value) {
                 if constexpr (!FP8) {  // 16 reads: step 0 set in regions 0..7, step 1 set in regions 8..15
                     if (g < 8) {
                         if constexpr (ODD.value) read_frag(o_next, 0, g, fa00, fb00);
@@ -597,7 +706,14 @@ __global__ __launch_bounds__(256) void gemm_tile256s5_kernel(const GemmArgs p) {
                     }
                 }
             }
-            if constexpr (!FP8) {
+            if constexpr (N16) {
+                const int j = g >> 3, i = g & 7;  // B block j, A block i
+                const v4i bfr = ODD.value ? (j < 4 ? fb10[j & 3] : fb11[j & 3]) : (j < 4 ? fb00[j & 3] : fb01[j & 3]);
+                const v4i afr = ODD.value ? (i < 4 ? fa10[i & 3] : fa11[i & 3]) : (i < 4 ? fa00[i & 3] : fa01[i & 3]);
+                // accumulator tied in place in AGPRs: left to the register allocator, the 64 four-register
+                // accumulators rotate through one another with copies in the loop
+                asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+a"(acc[j][i]) : "v"(bfr), "v"(afr));
+            } else if constexpr (!FP8) {
                 if constexpr (ODD.value) {
                     if (g < 16) mfma_one<FP8, XE5>(acc, g, fa10, fb10);
                     else mfma_one<FP8, XE5>(acc, g - 16, fa11, fb11);
@@ -657,14 +773,18 @@ __global__ __launch_bounds__(256) void gemm_tile256s5_kernel(const GemmArgs p) {
     if (Q >= 2) pair(No{}, Yes{}, Yes{}, Int<3>{});
     pair(No{}, No{}, No{}, Int<3>{});
 
-    tile256_epilogue<FP8, DUMP>(p, acc, smem, m0, n0, t, wm, wn, l31, hi, pre_sx, pre_sw,
-                                p.bias ? bf16_bits_to_f32(pre_b) : -0.0f);
+    if constexpr (N16)
+        tile256_epilogue16<DUMP>(p, acc, smem, m0, n0, t, wm, wn, lr, lane >> 4, pre_sx, pre_sw,
+                                 p.bias ? bf16_bits_to_f32(pre_b) : -0.0f);
+    else
+        tile256_epilogue<FP8, DUMP>(p, acc, smem, m0, n0, t, wm, wn, l31, hi, pre_sx, pre_sw,
+                                    p.bias ? bf16_bits_to_f32(pre_b) : -0.0f);
 }
 
-template <bool FP8, bool DUMP, bool XE5>
+template <bool FP8, bool DUMP, bool XE5, bool N16 = false>
 static int launch_tile256s5_impl(const GemmArgs& a, hipStream_t st) {
     using namespace t5;
-    auto kern = gemm_tile256s5_kernel<FP8, DUMP, XE5>;
+    auto kern = gemm_tile256s5_kernel<FP8, DUMP, XE5, N16>;
     static bool attr_done = false;
     if (!attr_done) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, SMEM);
@@ -677,19 +797,23 @@ static int launch_tile256s5_impl(const GemmArgs& a, hipStream_t st) {
     return check_launch("gemm_tile256s5");
 }
 
+// wide: INT8 with 32x32x32 MFMAs instead of the 16x16x64 form (kept for the tests and for comparisons)
 template <bool FP8>
-int launch_tile256s5(const GemmArgs& a0, bool x_e5m2, hipStream_t st) {
+int launch_tile256s5(const GemmArgs& a0, bool x_e5m2, bool wide, hipStream_t st) {
     GemmArgs a = a0;
     a.tiles_m = (a.m + 255) / 256;
     a.tiles_n = (a.n + 255) / 256;
     if constexpr (FP8) {
         if (x_e5m2) return a.acc ? launch_tile256s5_impl<true, true, true>(a, st) : launch_tile256s5_impl<true, false, true>(a, st);
+        return a.acc ? launch_tile256s5_impl<true, true, false>(a, st) : launch_tile256s5_impl<true, false, false>(a, st);
+    } else {
+        if (wide) return a.acc ? launch_tile256s5_impl<false, true, false>(a, st) : launch_tile256s5_impl<false, false, false>(a, st);
+        return a.acc ? launch_tile256s5_impl<false, true, false, true>(a, st) : launch_tile256s5_impl<false, false, false, true>(a, st);
     }
-    return a.acc ? launch_tile256s5_impl<FP8, true, false>(a, st) : launch_tile256s5_impl<FP8, false, false>(a, st);
 }
 
-template int launch_tile256s5<false>(const GemmArgs&, bool, hipStream_t);
-template int launch_tile256s5<true>(const GemmArgs&, bool, hipStream_t);
+template int launch_tile256s5<false>(const GemmArgs&, bool, bool, hipStream_t);
+template int launch_tile256s5<true>(const GemmArgs&, bool, bool, hipStream_t);
 
 // timing experiments (INT8 only): exp 1 = no HBM loads in the steady state, 2 = loads only
 int launch_tile256_experiment(const GemmArgs& a0, int exp, hipStream_t st) {

@@ -216,7 +216,7 @@ int launch_tile256(const GemmArgs& a, bool x_e5m2, hipStream_t st);
 bool tile256_applies(const GemmArgs& a);
 int launch_tile256_experiment(const GemmArgs& a, int exp, hipStream_t st);
 template <bool FP8>
-int launch_tile256s5(const GemmArgs& a, bool x_e5m2, hipStream_t st);
+int launch_tile256s5(const GemmArgs& a, bool x_e5m2, bool wide, hipStream_t st);
 
 template <bool FP8, int BM, int BN, int BK, int WM, int WN, bool DIRECT, bool XE5 = false>
 static int launch_cfg(const GemmArgs& a0, hipStream_t st) {
@@ -274,7 +274,7 @@ static int launch_gemm(const void* xq, int64_t ld_xq, const float* sx, const voi
             // 256 CUs, otherwise 128x128 tiles (4x as many workgroups; measured cross-over at
             // N = K = 5120: M = 512 -> 642 against 533 T-op/s, M = 1024 -> 948 against 1012)
             const int64_t tiles256 = ((m + 255) / 256) * ((n + 255) / 256);
-            if (tile256_applies(a) && tiles256 >= 80) return launch_tile256s5<FP8>(a, x_e5m2, st);
+            if (tile256_applies(a) && tiles256 >= 80) return launch_tile256s5<FP8>(a, x_e5m2, false, st);
             if constexpr (FP8) {
                 if (x_e5m2) return launch_cfg<true, 128, 128, 128, 2, 2, true, true>(a, st);
             }
@@ -292,8 +292,9 @@ static int launch_gemm(const void* xq, int64_t ld_xq, const float* sx, const voi
             if (!tile256_applies(a)) return fail(DAXQ_ERR_ARG, "linear: the 256x256 kernel needs m, n >= 256");
             return launch_tile256<FP8>(a, x_e5m2, st);
         case 8:
+        case 9:  // 9: INT8 with 32x32x32 MFMAs
             if (!tile256_applies(a)) return fail(DAXQ_ERR_ARG, "linear: the 256x256 kernel needs m, n >= 256");
-            return launch_tile256s5<FP8>(a, x_e5m2, st);
+            return launch_tile256s5<FP8>(a, x_e5m2, g_variant == 9, st);
         case 101:
         case 102:
         case 103: return launch_tile256_experiment(a, g_variant - 100, st);
@@ -310,7 +311,7 @@ int daxq_set_gemm_variant(int variant) {
         daxq::g_gm = variant - 1000 > 0 ? variant - 1000 : 4;
         return DAXQ_OK;
     }
-    if (variant != 0 && variant != 2 && variant != 5 && variant != 6 && variant != 8 && variant != 101 && variant != 102 && variant != 103)
+    if (variant != 0 && variant != 2 && variant != 5 && variant != 6 && variant != 8 && variant != 9 && variant != 101 && variant != 102 && variant != 103)
         return daxq::fail(DAXQ_ERR_ARG, "unknown gemm variant %d", variant);
     daxq::g_variant = variant;
     return DAXQ_OK;

@@ -14,11 +14,11 @@ from tests.util import bf16_bits, rel_l2
 
 pytestmark = pytest.mark.gpu
 
-VARIANTS = [0, 2, 5, 6, 8]  # 0 = library default, 2 / 5 = generic kernels, 6 / 8 = 256x256 kernels (m, n >= 256)
+VARIANTS = [0, 2, 5, 6, 8, 9]  # 0 = library default, 2 / 5 = generic kernels, 6 = two-stage 256x256, 8 / 9 = five-stage 256x256 (9: INT8 with 32x32 MFMAs)
 
 
 def _skip_if_too_small(variant, m, n):
-    if variant in (6, 8) and (m < 256 or n < 256):
+    if variant in (6, 8, 9) and (m < 256 or n < 256):
         pytest.skip("the 256x256 kernel needs m, n >= 256")
 FP8_TOL = 2e-2
 
