@@ -604,21 +604,26 @@ __global__ __launch_bounds__(256) void gemm_tile256s5_kernel(const GemmArgs p) {
     const uint32_t gsw = (uint32_t)(((t & 3) ^ ((t >> 4) & 3)) << 4);
     uint32_t voff_a = (uint32_t)(t >> 2) * (uint32_t)p.lda + gsw;
     uint32_t voff_b = (uint32_t)(t >> 2) * (uint32_t)p.ldb + gsw;
+    uint32_t voff_a1 = voff_a + BKS, voff_b1 = voff_b + BKS;  // second half of the 128-byte line
     const uint8_t* abase = p.a + (int64_t)m0 * p.lda;
     const uint8_t* bbase = p.b + (int64_t)n0 * p.ldb;
     const int64_t a_step = 64 * p.lda, b_step = 64 * p.ldb;
     const uint32_t lds0 = (uint32_t)(uintptr_t)(DAXQ_LDS uint8_t*)smem;
     const uint32_t wave_lds = lds0 + (uint32_t)__builtin_amdgcn_readfirstlane(wave * 1024);
-    // load g = 0..15 of a pair: operand g/8 (0 = A), row block (g/2)%4, half g%2 -> stage o0 / o1
+    // load g = 0..15 of a pair: operand g/8 (0 = A), row block (g/2)%4, half g%2 -> stage o0 / o1.
+    // Address = uniform row-block base (SGPR pair) + per-lane 32-bit offset: no VALU work per load.
     auto issue_one = [&](uint32_t o0, uint32_t o1, int g) {
         const int opnd = g >> 3, j = (g >> 1) & 3, half = g & 1;
-        const uint8_t* src = (opnd ? bbase + j * b_step : abase + j * a_step) + half * BKS;
+        const uint8_t* src = opnd ? bbase + j * b_step : abase + j * a_step;
+        const uint32_t voff = opnd ? (half ? voff_b1 : voff_b) : (half ? voff_a1 : voff_a);
         const uint32_t dst = wave_lds + (half ? o1 : o0) + opnd * A_BYTES + j * 4096;
-        __builtin_amdgcn_global_load_lds((const DAXQ_GLOBAL void*)(src + (opnd ? voff_b : voff_a)), (DAXQ_LDS void*)(uintptr_t)dst, 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((const DAXQ_GLOBAL void*)(src + voff), (DAXQ_LDS void*)(uintptr_t)dst, 16, 0, 0);
     };
     auto advance = [&]() {
         voff_a += 2 * BKS;
         voff_b += 2 * BKS;
+        voff_a1 += 2 * BKS;
+        voff_b1 += 2 * BKS;
     };
 
     // ---- LDS side: row (w*128 + i*32 + l%32), chunk c of the slice at (c ^ g) * 16, g = (l%32 >> 2) & 3
