@@ -619,11 +619,17 @@ __global__ __launch_bounds__(256) void gemm_tile256s5_kernel(const GemmArgs p) {
         const uint32_t dst = wave_lds + (half ? o1 : o0) + opnd * A_BYTES + j * 4096;
         __builtin_amdgcn_global_load_lds((const DAXQ_GLOBAL void*)(src + voff), (DAXQ_LDS void*)(uintptr_t)dst, 16, 0, 0);
     };
-    auto advance = [&]() {
+    auto advance_a = [&]() {
         voff_a += 2 * BKS;
-        voff_b += 2 * BKS;
         voff_a1 += 2 * BKS;
+    };
+    auto advance_b = [&]() {
+        voff_b += 2 * BKS;
         voff_b1 += 2 * BKS;
+    };
+    auto advance = [&]() {
+        advance_a();
+        advance_b();
     };
 
     // ---- LDS side: row (w*128 + i*32 + l%32), chunk c of the slice at (c ^ g) * 16, g = (l%32 >> 2) & 3
@@ -730,20 +736,33 @@ __global__ __launch_bounds__(256) void gemm_tile256s5_kernel(const GemmArgs p) {
                 if constexpr (ODD.value) mfma_one<FP8, XE5>(acc, g, fa10, fb10);
                 else mfma_one<FP8, XE5>(acc, g, fa00, fb00);
             }
+            // loop bookkeeping inside the last regions, in the issue slots an MFMA leaves free, instead of
+            // in a block of its own behind the slice: lane offsets of the operand this slice loaded, and
+            // (odd slice) the rotation of the stage offsets by one pair
+            if constexpr (ISSUE.value) {
+                if (g == NREG - 2) {
+                    if constexpr (ODD.value) advance_b();
+                    else advance_a();
+                }
+            }
+            if constexpr (ODD.value) {
+                if (g == NREG - 1) {
+                    const uint32_t r0 = st0, r1 = st1;
+                    st0 = st2;
+                    st1 = st3;
+                    st2 = st4;
+                    st3 = r0;
+                    st4 = r1;
+                }
+            }
             __builtin_amdgcn_sched_barrier(0);
         }
-        if constexpr (ISSUE.value && ODD.value) advance();
     };
-    // a pair of slices (s, s+1), s even; YOUNG of the odd slice equals ISSUE (the pair this one started)
+    // a pair of slices (s, s+1), s even; YOUNG of the odd slice equals ISSUE (the pair this one started).
+    // The stage offsets are passed by value: the odd slice rotates them in its last region.
     auto pair = [&](auto ISSUE, auto YOUNG_E, auto NEXT_O, auto EXTRA) {
         slice(No{}, ISSUE, Yes{}, YOUNG_E, EXTRA, st1, st4, st0);
         slice(Yes{}, ISSUE, NEXT_O, ISSUE, EXTRA, st2, st4, st0);
-        const uint32_t r0 = st0, r1 = st1;
-        st0 = st2;
-        st1 = st3;
-        st2 = st4;
-        st3 = r0;
-        st4 = r1;
     };
 
     // ---- prologue: pairs 0 and 1 in flight, pair 0 landed, fragments of slice 0 in set 0
