@@ -556,7 +556,8 @@ int launch_tile256(const GemmArgs& a0, bool x_e5m2, hipStream_t st) {
 //     have landed at the barrier of slice 2q+3;
 //   * fragments of slice s+1 are read during slice s into the other of two register sets.
 // LDS layout of an operand part: [256 rows][64 B], 16-byte chunk c of row r stored at chunk
-// c ^ ((r >> 2) & 3): 16 consecutive lanes (rows) of a ds_read_b128 then cover all 64 banks once.
+// c ^ ((r >> 2) & 3) (32x32 MFMA forms) or c ^ ((r >> 1) & 3) (16x16 form): the ds_read_b128 of either form
+// then runs at the full LDS rate.
 namespace t5 {
 constexpr int BKS = 64, NST = 5, T = 256;
 constexpr int A_BYTES = 256 * BKS, STAGE = 2 * A_BYTES;  // 16 KB, 32 KB
@@ -601,7 +602,9 @@ __global__ __launch_bounds__(256) void gemm_tile256s5_kernel(const GemmArgs p) {
     // ---- HBM side.  One wave instruction fills 1 KB of LDS = 16 rows x 64 B: lane l -> row l/4,
     //      stored chunk l%4, i.e. global chunk (l%4) ^ ((row>>2)&3).  Instruction j of a thread
     //      covers tile rows j*64 + t/4.
-    const uint32_t gsw = (uint32_t)(((t & 3) ^ ((t >> 4) & 3)) << 4);
+    //      N16 swizzles with (row>>1)&3 instead: its fragment reads (16 rows x 4 chunks per instruction) are
+    //      conflict free with that one and lose a fifth of the LDS rate with (row>>2)&3 (measured).
+    const uint32_t gsw = (uint32_t)(((t & 3) ^ ((N16 ? t >> 3 : t >> 4) & 3)) << 4);
     uint32_t voff_a = (uint32_t)(t >> 2) * (uint32_t)p.lda + gsw;
     uint32_t voff_b = (uint32_t)(t >> 2) * (uint32_t)p.ldb + gsw;
     uint32_t voff_a1 = voff_a + BKS, voff_b1 = voff_b + BKS;  // second half of the 128-byte line
@@ -636,7 +639,7 @@ __global__ __launch_bounds__(256) void gemm_tile256s5_kernel(const GemmArgs p) {
     //      N16: row (w*128 + i*16 + l%16), the lane's K chunk is l/16
     const int l31 = lane & 31, hi = lane >> 5;
     const int lr = N16 ? (lane & 15) : l31;  // row of the lane inside an MFMA block
-    const int gq = (lr >> 2) & 3;
+    const int gq = ((N16 ? lr >> 1 : lr >> 2)) & 3;
     const uint8_t* a_rd = smem + (wm * 128 + lr) * BKS;
     const uint8_t* b_rd = smem + A_BYTES + (wn * 128 + lr) * BKS;
     // one fragment: f = 0..3 A block f, 4..7 B block f-4; step ks of the slice in the stage at offset o
