@@ -32,7 +32,10 @@ typedef float v16f __attribute__((ext_vector_type(16)));
         }                                                                      \
     } while (0)
 
-// a, b: 8 operand sets per lane (256 lanes per block share the pattern across blocks)
+// a, b: 8 operand sets per lane (256 lanes per block share the pattern across blocks).  The loop is the GEMM's
+// own MFMA sequence for one 64-byte K slice of a wavefront's 128 x 128 outputs, with every memory instruction
+// removed: INT8 8 x 8 blocks of v_mfma_i32_16x16x64_i8, FP8 4 x 4 blocks of v_mfma_f32_32x32x64_f8f6f4, 256
+// accumulator registers, one operand held over a row of blocks, one wavefront per SIMD.
 template <bool FP8>
 __global__ __launch_bounds__(256) void spin(const int* __restrict__ a_src, const int* __restrict__ b_src, int iters, int* out) {
     constexpr int W = FP8 ? 8 : 4;
@@ -43,43 +46,50 @@ __global__ __launch_bounds__(256) void spin(const int* __restrict__ a_src, const
             b[s][w] = b_src[(s * W + w) * 256 + threadIdx.x];
         }
     if constexpr (!FP8) {
-        v16i c[8];
-        for (int s = 0; s < 8; ++s)
-            for (int v = 0; v < 16; ++v) c[s][v] = 0;
+        v4i c[8][8];
+        for (int j = 0; j < 8; ++j)
+            for (int i = 0; i < 8; ++i)
+                for (int v = 0; v < 4; ++v) c[j][i][v] = 0;
         v4i av[8], bv[8];
 #pragma unroll
         for (int s = 0; s < 8; ++s) {
             av[s] = v4i{a[s][0], a[s][1], a[s][2], a[s][3]};
             bv[s] = v4i{b[s][0], b[s][1], b[s][2], b[s][3]};
         }
-        for (int it = 0; it < iters; it += 8) {
+        for (int it = 0; it < iters; ++it) {
 #pragma unroll
-            for (int u = 0; u < 8; ++u)  // static operand rotation: every accumulator sees every B set
+            for (int j = 0; j < 8; ++j)
 #pragma unroll
-                for (int s = 0; s < 8; ++s) c[s] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av[s], bv[(s + u) & 7], c[s], 0, 0, 0);
+                for (int i = 0; i < 8; ++i)  // accumulator tied in place, as in the GEMM
+                    asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+a"(c[j][i]) : "v"(bv[j]), "v"(av[i]));
         }
         int r = 0;
-        for (int s = 0; s < 8; ++s) r += c[s][0];
+        for (int j = 0; j < 8; ++j)
+            for (int i = 0; i < 8; ++i) r += c[j][i][0];
         out[blockIdx.x * 256 + threadIdx.x] = r;
     } else {
-        v16f c[8];
-        for (int s = 0; s < 8; ++s)
-            for (int v = 0; v < 16; ++v) c[s][v] = 0;
+        v16f c[4][4];
+        for (int j = 0; j < 4; ++j)
+            for (int i = 0; i < 4; ++i)
+                for (int v = 0; v < 16; ++v) c[j][i][v] = 0;
         v8i av[8], bv[8];
 #pragma unroll
         for (int s = 0; s < 8; ++s) {
             av[s] = v8i{a[s][0], a[s][1], a[s][2], a[s][3], a[s][4], a[s][5], a[s][6], a[s][7]};
             bv[s] = v8i{b[s][0], b[s][1], b[s][2], b[s][3], b[s][4], b[s][5], b[s][6], b[s][7]};
         }
-        for (int it = 0; it < iters; it += 8) {
+        for (int it = 0; it < iters; it += 2) {
 #pragma unroll
-            for (int u = 0; u < 8; ++u)
+            for (int h = 0; h < 2; ++h)  // two slices: operand sets 0-3 and 4-7
 #pragma unroll
-                for (int s = 0; s < 8; ++s)
-                    c[s] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av[s], bv[(s + u) & 7], c[s], 0, 0, 0, 0, 0, 0);
+                for (int j = 0; j < 4; ++j)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                        c[j][i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bv[4 * h + j], av[4 * h + i], c[j][i], 0, 0, 0, 0, 0, 0);
         }
         float r = 0;
-        for (int s = 0; s < 8; ++s) r += c[s][0];
+        for (int j = 0; j < 4; ++j)
+            for (int i = 0; i < 4; ++i) r += c[j][i][0];
         out[blockIdx.x * 256 + threadIdx.x] = (int)r;
     }
 }
@@ -104,7 +114,7 @@ static uint8_t to_e4m3(float v) {  // nearest e4m3fn by search over the 254 fini
 int main() {
     hipDeviceProp_t prop;
     CHECK(hipGetDeviceProperties(&prop, 0));
-    const int blocks = 2 * prop.multiProcessorCount;  // two workgroups of 4 waves per CU: 2 waves per SIMD
+    const int blocks = prop.multiProcessorCount;  // one workgroup of 4 waves per CU, like the GEMM
     int *da, *db, *dout;
     const size_t words = 8 * 8 * 256;
     CHECK(hipMalloc(&da, words * 4));
@@ -140,8 +150,8 @@ int main() {
             }
             CHECK(hipMemcpy(da, ha.data(), ha.size(), hipMemcpyHostToDevice));
             CHECK(hipMemcpy(db, hb.data(), hb.size(), hipMemcpyHostToDevice));
-            const int iters = fp8 ? 100000 : 200000;  // ~50-100 ms per launch
-            const double ops_per_mfma = fp8 ? 2.0 * 32 * 32 * 64 : 2.0 * 32 * 32 * 32;
+            const int iters = 60000;  // slices per wavefront, ~70 ms per launch
+            const double ops_per_slice = 2.0 * 128 * 128 * 64;
             double best = 0, last = 0;
             for (int rep = 0; rep < 3; ++rep) {
                 CHECK(hipEventRecord(e0));
@@ -153,7 +163,7 @@ int main() {
                 CHECK(hipEventSynchronize(e1));
                 float ms;
                 CHECK(hipEventElapsedTime(&ms, e0, e1));
-                last = (double)blocks * 4 * iters * 8 * ops_per_mfma / ms / 1e9;
+                last = (double)blocks * 4 * iters * ops_per_slice / ms / 1e9;
                 if (last > best) best = last;
             }
             // the last repetition is the one at thermal / power steady state
