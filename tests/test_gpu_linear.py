@@ -88,9 +88,13 @@ def test_linear_i8_adversarial_extremes(ops, variant):
     np.testing.assert_array_equal(bf16_bits(out), bf16_bits(O.epilogue_int8(want, sx.view(-1, 1), sw.view(1, -1), None)))
 
 
-def test_linear_i8_one_hot_layout(ops):
+@pytest.mark.parametrize("variant", [0, 6, 8, 9])
+def test_linear_i8_one_hot_layout(ops, variant):
     # a single non-zero in each operand lands in exactly one accumulator: catches any
     # row/column or operand transposition inside the MFMA tiling
+    from dax_amd import _capi
+
+    _capi.set_gemm_variant(variant)
     m, n, k = 300, 300, 256
     rng = np.random.default_rng(0)
     for _ in range(6):
@@ -153,7 +157,7 @@ def test_linear_rejects_unaligned_k(ops):
         ops.linear_i8(xq, torch.ones(8, device="cuda"), wq, torch.ones(8, device="cuda"), None)
 
 
-@pytest.mark.parametrize("variant", [0, 5, 6, 8])
+@pytest.mark.parametrize("variant", [0, 5, 6, 8, 9])
 def test_linear_leading_dimensions_through_the_c_abi(ops, variant):
     """Operands and output as column slices of wider buffers (ld > logical width), straight through the C ABI:
     what a caller does that writes q | k | v into one [M, 3N] tensor with three launches."""
