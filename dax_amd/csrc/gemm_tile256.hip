@@ -113,14 +113,17 @@ __device__ __forceinline__ void load_one_frag(const FragAddr& fa, int stage, int
     }
 }
 
-template <bool FP8, bool XE5>
+// ZERO: the block's first MFMA of a tile, which starts from zero instead of the accumulator
+template <bool FP8, bool XE5, bool ZERO = false>
 __device__ __forceinline__ void mfma_one(typename AccT<FP8>::type (&acc)[4][4], int g, const typename Frag<FP8>::type (&af)[4],
                                          const typename Frag<FP8>::type (&bf)[4]) {
     const int j = g >> 2, i = g & 3;
+    typename AccT<FP8>::type c = {};
+    if constexpr (!ZERO) c = acc[j][i];
     if constexpr (!FP8)
-        acc[j][i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[j], af[i], acc[j][i], 0, 0, 0);
+        acc[j][i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[j], af[i], c, 0, 0, 0);
     else
-        acc[j][i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bf[j], af[i], acc[j][i], 0, XE5 ? 1 : 0, 0, 0, 0, 0);
+        acc[j][i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bf[j], af[i], c, 0, XE5 ? 1 : 0, 0, 0, 0, 0);
 }
 
 // acc[j][i]: 32x32 block with rows = n (W rows, MFMA "A" operand) and columns = m (X rows, "B"
@@ -663,12 +666,6 @@ __global__ __launch_bounds__(256) void gemm_tile256s5_kernel(const GemmArgs p) {
     };
 
     typename TileAcc<FP8, N16>::type acc[N16 ? 8 : 4][N16 ? 8 : 4];
-#pragma unroll
-    for (int j = 0; j < (N16 ? 8 : 4); ++j)
-#pragma unroll
-        for (int i = 0; i < (N16 ? 8 : 4); ++i)
-#pragma unroll
-            for (int v = 0; v < (N16 ? 4 : 16); ++v) acc[j][i][v] = 0;
 
     // fragment sets: [slice parity][MFMA step] (N16: [slice parity][blocks 0-3 / 4-7])
     frag_t fa00[4] = {}, fb00[4] = {}, fa01[4] = {}, fb01[4] = {}, fa10[4] = {}, fb10[4] = {}, fa11[4] = {}, fb11[4] = {};
@@ -685,7 +682,9 @@ __global__ __launch_bounds__(256) void gemm_tile256s5_kernel(const GemmArgs p) {
     //   YOUNG  loads issued after those of slice s+1 exist and may stay in flight: a whole pair at
     //          an even slice, the A half of the newest pair at an odd one (vmcnt retires in order)
     //   EXTRA  younger loads that are not tile loads (the epilogue's scales) and may stay in flight
-    auto slice = [&](auto ODD, auto ISSUE, auto NEXT, auto YOUNG, auto EXTRA, uint32_t o_next, uint32_t o_ld0, uint32_t o_ld1) {
+    //   FIRST  slice 0 of the tile: its MFMAs start from zero, the accumulators need no clearing
+    auto slice = [&](auto ODD, auto ISSUE, auto NEXT, auto YOUNG, auto EXTRA, auto FIRST, uint32_t o_next, uint32_t o_ld0, uint32_t o_ld1)
+                     __attribute__((always_inline)) {
         __builtin_amdgcn_s_waitcnt(vmcnt_imm((YOUNG.value ? (ODD.value ? PAIR_LOADS / 2 : PAIR_LOADS) : 0) + EXTRA.value) & lgkmcnt0_mask());
         __builtin_amdgcn_s_barrier();
 #pragma unroll
@@ -726,18 +725,21 @@ __global__ __launch_bounds__(256) void gemm_tile256s5_kernel(const GemmArgs p) {
                 const v4i afr = ODD.value ? (i < 4 ? fa10[i & 3] : fa11[i & 3]) : (i < 4 ? fa00[i & 3] : fa01[i & 3]);
                 // accumulator tied in place in AGPRs: left to the register allocator, the 64 four-register
                 // accumulators rotate through one another with copies in the loop
-                asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+a"(acc[j][i]) : "v"(bfr), "v"(afr));
+                if constexpr (FIRST.value)
+                    asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, 0" : "=a"(acc[j][i]) : "v"(bfr), "v"(afr));
+                else
+                    asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+a"(acc[j][i]) : "v"(bfr), "v"(afr));
             } else if constexpr (!FP8) {
                 if constexpr (ODD.value) {
                     if (g < 16) mfma_one<FP8, XE5>(acc, g, fa10, fb10);
                     else mfma_one<FP8, XE5>(acc, g - 16, fa11, fb11);
                 } else {
-                    if (g < 16) mfma_one<FP8, XE5>(acc, g, fa00, fb00);
+                    if (g < 16) mfma_one<FP8, XE5, FIRST.value>(acc, g, fa00, fb00);
                     else mfma_one<FP8, XE5>(acc, g - 16, fa01, fb01);
                 }
             } else {
                 if constexpr (ODD.value) mfma_one<FP8, XE5>(acc, g, fa10, fb10);
-                else mfma_one<FP8, XE5>(acc, g, fa00, fb00);
+                else mfma_one<FP8, XE5, FIRST.value>(acc, g, fa00, fb00);
             }
             // loop bookkeeping inside the last regions, in the issue slots an MFMA leaves free, instead of
             // in a block of its own behind the slice: lane offsets of the operand this slice loaded, and
@@ -763,9 +765,9 @@ __global__ __launch_bounds__(256) void gemm_tile256s5_kernel(const GemmArgs p) {
     };
     // a pair of slices (s, s+1), s even; YOUNG of the odd slice equals ISSUE (the pair this one started).
     // The stage offsets are passed by value: the odd slice rotates them in its last region.
-    auto pair = [&](auto ISSUE, auto YOUNG_E, auto NEXT_O, auto EXTRA) {
-        slice(No{}, ISSUE, Yes{}, YOUNG_E, EXTRA, st1, st4, st0);
-        slice(Yes{}, ISSUE, NEXT_O, ISSUE, EXTRA, st2, st4, st0);
+    auto pair = [&](auto ISSUE, auto YOUNG_E, auto NEXT_O, auto EXTRA, auto FIRST) __attribute__((always_inline)) {
+        slice(No{}, ISSUE, Yes{}, YOUNG_E, EXTRA, FIRST, st1, st4, st0);
+        slice(Yes{}, ISSUE, NEXT_O, ISSUE, EXTRA, No{}, st2, st4, st0);
     };
 
     // ---- prologue: pairs 0 and 1 in flight, pair 0 landed, fragments of slice 0 in set 0
@@ -788,7 +790,15 @@ __global__ __launch_bounds__(256) void gemm_tile256s5_kernel(const GemmArgs p) {
     }
 
     const int Q = S >> 1;  // pairs
-    for (int q = 0; q + 2 < Q; ++q) pair(Yes{}, Yes{}, Yes{}, Int<0>{});
+    if (Q >= 3) {
+        pair(Yes{}, Yes{}, Yes{}, Int<0>{}, Yes{});
+    } else {  // short K: no pair to peel, clear the accumulators instead
+#pragma unroll
+        for (int j = 0; j < (N16 ? 8 : 4); ++j)
+#pragma unroll
+            for (int i = 0; i < (N16 ? 8 : 4); ++i) acc[j][i] = typename TileAcc<FP8, N16>::type{};
+    }
+    for (int q = 1; q + 2 < Q; ++q) pair(Yes{}, Yes{}, Yes{}, Int<0>{}, No{});
 
     // The epilogue's scales and bias are requested here, behind the last tile loads, so that their
     // latency is covered by the remaining two pairs of slices.  Always three loads (a missing bias
@@ -797,8 +807,8 @@ __global__ __launch_bounds__(256) void gemm_tile256s5_kernel(const GemmArgs p) {
     const uint16_t pre_b = (p.bias ? p.bias : reinterpret_cast<const uint16_t*>(p.sw))[n0 + t];
     __builtin_amdgcn_sched_barrier(0);
 
-    if (Q >= 2) pair(No{}, Yes{}, Yes{}, Int<3>{});
-    pair(No{}, No{}, No{}, Int<3>{});
+    if (Q >= 2) pair(No{}, Yes{}, Yes{}, Int<3>{}, No{});
+    pair(No{}, No{}, No{}, Int<3>{}, No{});
 
     if constexpr (N16)
         tile256_epilogue16<DUMP>(p, acc, smem, m0, n0, t, wm, wn, lr, lane >> 4, pre_sx, pre_sw,
