@@ -313,9 +313,7 @@ __device__ __forceinline__ void tile256_epilogue16(const GemmArgs& p, v4i (&acc)
 
 // DUMP: also write the raw accumulators to p.acc (tests); a separate instantiation so that the
 // production kernel carries none of that code.
-// EXP:  timing experiments with wrong results by construction: 1 = no HBM loads in the steady
-//       state, 2 = loads only (no LDS reads, no MFMA), 3 = all tiles load tile (0,0)'s panels (L2 hits).
-template <bool FP8, bool DUMP, int EXP = 0, bool XE5 = false>
+template <bool FP8, bool DUMP, bool XE5 = false>
 __global__ __launch_bounds__(256) void gemm_tile256_kernel(const GemmArgs p) {
     using namespace t256;
     typedef typename AccT<FP8>::type acc_t;
@@ -338,9 +336,8 @@ __global__ __launch_bounds__(256) void gemm_tile256_kernel(const GemmArgs p) {
     const uint32_t chunk = (uint32_t)((slot ^ swz(r8)) << 4);
     uint32_t voff_a = (uint32_t)r8 * (uint32_t)p.lda + chunk;
     uint32_t voff_b = (uint32_t)r8 * (uint32_t)p.ldb + chunk;
-    // EXP 3: every tile loads the panels of tile (0, 0), so that all loads hit L2
-    const uint8_t* abase = p.a + (EXP == 3 ? 0 : (int64_t)m0 * p.lda);
-    const uint8_t* bbase = p.b + (EXP == 3 ? 0 : (int64_t)n0 * p.ldb);
+    const uint8_t* abase = p.a + (int64_t)m0 * p.lda;
+    const uint8_t* bbase = p.b + (int64_t)n0 * p.ldb;
     const int64_t a_step = 32 * p.lda, b_step = 32 * p.ldb;
 
     // ---- LDS side
@@ -364,7 +361,6 @@ __global__ __launch_bounds__(256) void gemm_tile256_kernel(const GemmArgs p) {
 
     // MFMA steps 0 .. n-2 of a slice, each overlapped with the fragment reads of the next step
     auto steps_but_last = [&](int cur) {
-        if constexpr (EXP == 2) return;
         if constexpr (!FP8) {
             load_frags<FP8>(fa, cur, 1, fa1, fb1);
             mfma_step<FP8, XE5>(acc, fa0, fb0);
@@ -398,7 +394,7 @@ __global__ __launch_bounds__(256) void gemm_tile256_kernel(const GemmArgs p) {
         }
     };
     auto next_frags = [&](int nxt) {
-        if constexpr (EXP != 2) load_frags<FP8>(fa, nxt, 0, fa0, fb0);
+        load_frags<FP8>(fa, nxt, 0, fa0, fb0);
     };
 
     {
@@ -406,7 +402,6 @@ __global__ __launch_bounds__(256) void gemm_tile256_kernel(const GemmArgs p) {
         const uint32_t lds0 = (uint32_t)(uintptr_t)(DAXQ_LDS uint8_t*)smem;
         const uint32_t wave_lds = lds0 + (uint32_t)__builtin_amdgcn_readfirstlane(wave * 1024);
         auto issue_one = [&](int stage, int g) {  // g = 0..7: A rows g*32.., g = 8..15: B rows (g-8)*32..
-            if constexpr (EXP == 1) return;
             if (g < 8)
                 __builtin_amdgcn_global_load_lds((const DAXQ_GLOBAL void*)(abase + g * a_step + voff_a),
                                                  (DAXQ_LDS void*)(uintptr_t)(wave_lds + stage * STAGE + g * 4096), 16, 0, 0);
@@ -443,14 +438,14 @@ __global__ __launch_bounds__(256) void gemm_tile256_kernel(const GemmArgs p) {
 #pragma unroll
                 for (int g = 0; g < 16; ++g) {
                     if constexpr (ISSUE.value) issue_one(cur, g);
-                    if constexpr (NEXT.value && EXP != 2)
+                    if constexpr (NEXT.value)
                         if (g < 8) load_one_frag<FP8>(fa, cur ^ 1, g, fa0, fb0);
-                    if constexpr (EXP != 2) mfma_one<FP8, XE5>(acc, g, fa1, fb1);
+                    mfma_one<FP8, XE5>(acc, g, fa1, fb1);
                     __builtin_amdgcn_sched_barrier(0);
                 }
                 if constexpr (ISSUE.value) advance();
             } else {
-                if constexpr (EXP != 2) {
+                {
                     load_frags<FP8>(fa, cur, 2, fa2, fb2);
                     mfma_step<FP8, XE5>(acc, fa0, fb0);
 #pragma unroll
@@ -472,13 +467,13 @@ __global__ __launch_bounds__(256) void gemm_tile256_kernel(const GemmArgs p) {
 #pragma unroll
                 for (int g = 0; g < 16; ++g) {
                     if constexpr (ISSUE.value) issue_one(cur, g);
-                    if constexpr (NEXT.value && EXP != 2)
+                    if constexpr (NEXT.value)
                         if (g < 8) load_one_frag<FP8>(fa, cur ^ 1, g, fa0, fb0);
-                    if constexpr (EXP != 2) mfma_one<FP8, XE5>(acc, g, fa2, fb2);
+                    mfma_one<FP8, XE5>(acc, g, fa2, fb2);
                     __builtin_amdgcn_sched_barrier(0);
                 }
                 if constexpr (ISSUE.value) advance();
-                if constexpr (EXP != 2) {
+                {
                     if constexpr (NEXT.value) load_frags<FP8>(fa, cur ^ 1, 1, fa1, fb1);
                     mfma_step<FP8, XE5>(acc, fa3, fb3);
                     if constexpr (NEXT.value) {
@@ -500,7 +495,7 @@ __global__ __launch_bounds__(256) void gemm_tile256_kernel(const GemmArgs p) {
         }
         __builtin_amdgcn_s_barrier();
         next_frags(0);
-        if constexpr (!FP8 && EXP != 2) load_frags<FP8>(fa, 0, 1, fa1, fb1);
+        if constexpr (!FP8) load_frags<FP8>(fa, 0, 1, fa1, fb1);
         int kt = 0;
         for (; kt + 2 < KT; ++kt) slice(kt & 1, Yes{}, Yes{});
         if (kt + 1 < KT) {
@@ -516,10 +511,10 @@ __global__ __launch_bounds__(256) void gemm_tile256_kernel(const GemmArgs p) {
                                 p.bias ? bf16_bits_to_f32(p.bias[n0 + t]) : -0.0f);
 }
 
-template <bool FP8, bool DUMP, int EXP = 0, bool XE5 = false>
+template <bool FP8, bool DUMP, bool XE5 = false>
 static int launch_tile256_impl(const GemmArgs& a, hipStream_t st) {
     using namespace t256;
-    auto kern = gemm_tile256_kernel<FP8, DUMP, EXP, XE5>;
+    auto kern = gemm_tile256_kernel<FP8, DUMP, XE5>;
     static bool attr_done = false;
     if (!attr_done) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, SMEM);
@@ -540,7 +535,7 @@ int launch_tile256(const GemmArgs& a0, bool x_e5m2, hipStream_t st) {
     a.tiles_n = (a.n + BN - 1) / BN;
     if constexpr (FP8) {
         if (x_e5m2)
-            return a.acc ? launch_tile256_impl<true, true, 0, true>(a, st) : launch_tile256_impl<true, false, 0, true>(a, st);
+            return a.acc ? launch_tile256_impl<true, true, true>(a, st) : launch_tile256_impl<true, false, true>(a, st);
     }
     return a.acc ? launch_tile256_impl<FP8, true>(a, st) : launch_tile256_impl<FP8, false>(a, st);
 }
@@ -851,16 +846,6 @@ int launch_tile256s5(const GemmArgs& a0, bool x_e5m2, bool wide, hipStream_t st)
 
 template int launch_tile256s5<false>(const GemmArgs&, bool, bool, hipStream_t);
 template int launch_tile256s5<true>(const GemmArgs&, bool, bool, hipStream_t);
-
-// timing experiments (INT8 only): exp 1 = no HBM loads in the steady state, 2 = loads only
-int launch_tile256_experiment(const GemmArgs& a0, int exp, hipStream_t st) {
-    using namespace t256;
-    GemmArgs a = a0;
-    a.tiles_m = (a.m + BM - 1) / BM;
-    a.tiles_n = (a.n + BN - 1) / BN;
-    if (exp == 3) return launch_tile256_impl<false, false, 3>(a, st);
-    return exp == 1 ? launch_tile256_impl<false, false, 1>(a, st) : launch_tile256_impl<false, false, 2>(a, st);
-}
 
 // the kernel applies: both dimensions hold a whole tile and the 32-bit row offsets cannot overflow
 bool tile256_applies(const GemmArgs& a) {

@@ -214,7 +214,6 @@ static int g_gm = 4;
 template <bool FP8>
 int launch_tile256(const GemmArgs& a, bool x_e5m2, hipStream_t st);
 bool tile256_applies(const GemmArgs& a);
-int launch_tile256_experiment(const GemmArgs& a, int exp, hipStream_t st);
 template <bool FP8>
 int launch_tile256s5(const GemmArgs& a, bool x_e5m2, bool wide, hipStream_t st);
 
@@ -295,9 +294,6 @@ static int launch_gemm(const void* xq, int64_t ld_xq, const float* sx, const voi
         case 9:  // 9: INT8 with 32x32x32 MFMAs
             if (!tile256_applies(a)) return fail(DAXQ_ERR_ARG, "linear: the 256x256 kernel needs m, n >= 256");
             return launch_tile256s5<FP8>(a, x_e5m2, g_variant == 9, st);
-        case 101:
-        case 102:
-        case 103: return launch_tile256_experiment(a, g_variant - 100, st);
         default: return fail(DAXQ_ERR_ARG, "linear: unknown gemm variant %d", g_variant);
     }
 }
@@ -311,7 +307,7 @@ int daxq_set_gemm_variant(int variant) {
         daxq::g_gm = variant - 1000 > 0 ? variant - 1000 : 4;
         return DAXQ_OK;
     }
-    if (variant != 0 && variant != 2 && variant != 5 && variant != 6 && variant != 8 && variant != 9 && variant != 101 && variant != 102 && variant != 103)
+    if (variant != 0 && variant != 2 && variant != 5 && variant != 6 && variant != 8 && variant != 9)
         return daxq::fail(DAXQ_ERR_ARG, "unknown gemm variant %d", variant);
     daxq::g_variant = variant;
     return DAXQ_OK;

@@ -199,8 +199,10 @@ int daxq_linear_e5m2_e4m3(const uint8_t* xq, int64_t ld_xq, const float* sx,
                           float* acc, int64_t ld_acc,
                           int64_t m, int64_t n, int64_t k, daxq_stream_t stream);
 
-/* Selects a GEMM kernel variant for tuning and tests (0 = library default).
- * Process-wide; not part of the reference interface. */
+/* Selects a GEMM kernel for tests and comparisons; every choice computes the same results.
+ * 0 = library default (by shape), 2 / 5 = generic 256x256 / 128x128 tiles, 6 = two-stage 256x256 kernel,
+ * 8 = five-stage 256x256 kernel, 9 = the same with 32x32x32 INT8 MFMAs; 1000 + d sets the depth d of the
+ * tile-order groups.  Process-wide; not part of the reference interface. */
 int daxq_set_gemm_variant(int variant);
 
 #ifdef __cplusplus
