@@ -3,13 +3,14 @@
 // Two forms of the same tile live here.  gemm_tile256s5_kernel (second half of the file, K in
 // 64-byte slices through five 32 KB LDS stages) is the one the library launches;
 // gemm_tile256_kernel (K in 128-byte slices, two 64 KB stages) came first and stays as a second
-// implementation for the tests and for timing experiments.  They share everything but the main loop.
+// implementation for the tests.  They share everything but the main loop.
 //
 // Work decomposition
 //   workgroup  256 x 256 outputs, 4 wavefronts (one per SIMD) in a 2 x 2 grid
-//   wavefront  128 x 128 outputs = 4 x 4 MFMA 32x32 blocks, 256 accumulator registers (AGPRs)
+//   wavefront  128 x 128 outputs in 256 accumulator registers (AGPRs): 4 x 4 MFMA blocks of 32x32
+//              (FP8, and INT8 in the older forms) or 8 x 8 blocks of 16x16 (INT8 in the five-stage kernel)
 // A 2 x 2 wave grid is what minimises LDS reads per MFMA for a square tile: 128 bytes of K are
-// read (2 + 2) * 256 * 128 B = 128 KB per workgroup against 128 MFMAs of 32 cycles per wave.
+// read (2 + 2) * 256 * 128 B = 128 KB per workgroup against 4096 MFMA cycles per wave.
 //
 // Data movement of the two-stage form
 //   HBM/L2 -> LDS   global_load_lds_dwordx4 (no VGPR staging): 16 per thread and slice.  The 16-byte
