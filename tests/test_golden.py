@@ -6,7 +6,6 @@ import json
 import os
 
 import pytest
-import torch
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 FIX = json.load(open(os.path.join(HERE, "golden", "config0_int8.json")))

@@ -7,7 +7,7 @@ import pytest
 import torch
 
 from oracle import daxq_oracle as O
-from tests.util import ALL_POS_FINITE, FINITE_BF16, bf16_bits, from_bits
+from tests.util import ALL_POS_FINITE, FINITE_BF16, from_bits
 
 pytestmark = pytest.mark.gpu
 
