@@ -806,6 +806,12 @@ __global__ __launch_bounds__(256) void gemm_tile256s5_kernel(const GemmArgs p) {
     if (Q >= 2) pair(No{}, Yes{}, Yes{}, Int<3>{}, No{});
     pair(No{}, No{}, No{}, Int<3>{}, No{});
 
+    if constexpr (N16) {
+        // the 16x16 MFMAs are inline asm, so the compiler cannot count the wait states between the last one
+        // and the first read of its result; the epilogue starts with an LDS write and a barrier, and these
+        // 24 idle cycles keep that distance whatever is scheduled in between
+        asm volatile("s_nop 15\n\ts_nop 7" ::: "memory");
+    }
     if constexpr (N16)
         tile256_epilogue16<DUMP>(p, acc, smem, m0, n0, t, wm, wn, lr, lane >> 4, pre_sx, pre_sw,
                                  p.bias ? bf16_bits_to_f32(pre_b) : -0.0f);
