@@ -223,11 +223,19 @@ static int launch_fused_rows(const char* what, const void* x, int64_t m, int64_t
     if (nchunks <= N) {                                                                                                  \
         int64_t want = quads;                                                                                            \
         if (PRE == PRE_LN) {                                                                                             \
-            int per_cu = 0;                                                                                              \
-            hipError_t oe = yp ? hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, fused_rows_wave<N, FMT, PRE, true>, 256, lds) \
-                               : hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, fused_rows_wave<N, FMT, PRE, false>, 256, lds); \
-            if (oe != hipSuccess || per_cu <= 0) return fail(DAXQ_ERR_LAUNCH, "%s: occupancy query failed", what);       \
-            want = (int64_t)cus * per_cu;                                                                                \
+            /* asked once per kernel and LDS size (k); a race between two threads stores the same value twice */         \
+            static int cached_per_cu[2] = {0, 0};                                                                        \
+            static int64_t cached_k[2] = {0, 0};                                                                         \
+            const int slot = yp ? 1 : 0;                                                                                 \
+            if (cached_per_cu[slot] <= 0 || cached_k[slot] != k) {                                                       \
+                int per_cu = 0;                                                                                          \
+                hipError_t oe = yp ? hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, fused_rows_wave<N, FMT, PRE, true>, 256, lds) \
+                                   : hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, fused_rows_wave<N, FMT, PRE, false>, 256, lds); \
+                if (oe != hipSuccess || per_cu <= 0) return fail(DAXQ_ERR_LAUNCH, "%s: occupancy query failed", what);   \
+                cached_k[slot] = k;                                                                                      \
+                cached_per_cu[slot] = per_cu;                                                                            \
+            }                                                                                                            \
+            want = (int64_t)cus * cached_per_cu[slot];                                                                   \
         }                                                                                                                \
         const dim3 grid((unsigned)(quads < want ? quads : want));                                                        \
         if (yp)                                                                                                          \
