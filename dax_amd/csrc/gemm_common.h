@@ -37,6 +37,19 @@ struct GemmArgs {
     int gm;  // depth (in tile rows) of the groups the tile order walks through
 };
 
+// Raises a kernel's dynamic LDS limit once per device.  `done` is the caller's per-kernel bit mask of the devices
+// already set up (a race between two threads sets the same attribute twice).
+inline int ensure_dynamic_lds(const void* kern, int bytes, uint64_t& done) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return fail(DAXQ_ERR_LAUNCH, "hipGetDevice failed");
+    const uint64_t bit = dev < 64 ? (uint64_t)1 << dev : 0;
+    if (done & bit) return DAXQ_OK;
+    hipError_t e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (e != hipSuccess) return fail(DAXQ_ERR_LAUNCH, "hipFuncSetAttribute(%d bytes LDS): %s", bytes, hipGetErrorString(e));
+    done |= bit;
+    return DAXQ_OK;
+}
+
 // s_waitcnt immediate that waits for vmcnt <= n only (gfx9 encoding: vmcnt in bits 3:0 and 15:14,
 // expcnt 6:4 and lgkmcnt 11:8 left at their maxima)
 constexpr int vmcnt_imm(int n) { return (n & 15) | ((n >> 4) << 14) | 0x0070 | 0x0f00; }

@@ -516,12 +516,8 @@ template <bool FP8, bool DUMP, bool XE5 = false>
 static int launch_tile256_impl(const GemmArgs& a, hipStream_t st) {
     using namespace t256;
     auto kern = gemm_tile256_kernel<FP8, DUMP, XE5>;
-    static bool attr_done = false;
-    if (!attr_done) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, SMEM);
-        if (e != hipSuccess) return fail(DAXQ_ERR_LAUNCH, "hipFuncSetAttribute(%d bytes LDS): %s", SMEM, hipGetErrorString(e));
-        attr_done = true;
-    }
+    static uint64_t lds_set = 0;  // per instantiation
+    if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), SMEM, lds_set)) return rc;
     const int64_t nt = (int64_t)a.tiles_m * a.tiles_n;
     if (nt > 0x7fffffff) return fail(DAXQ_ERR_ARG, "gemm: too many tiles");
     hipLaunchKernelGGL(kern, dim3((unsigned)nt), dim3(T), SMEM, st, a);
@@ -824,12 +820,8 @@ template <bool FP8, bool DUMP, bool XE5, bool N16 = false>
 static int launch_tile256s5_impl(const GemmArgs& a, hipStream_t st) {
     using namespace t5;
     auto kern = gemm_tile256s5_kernel<FP8, DUMP, XE5, N16>;
-    static bool attr_done = false;
-    if (!attr_done) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, SMEM);
-        if (e != hipSuccess) return fail(DAXQ_ERR_LAUNCH, "hipFuncSetAttribute(%d bytes LDS): %s", SMEM, hipGetErrorString(e));
-        attr_done = true;
-    }
+    static uint64_t lds_set = 0;  // per instantiation
+    if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), SMEM, lds_set)) return rc;
     const int64_t nt = (int64_t)a.tiles_m * a.tiles_n;
     if (nt > 0x7fffffff) return fail(DAXQ_ERR_ARG, "gemm: too many tiles");
     hipLaunchKernelGGL(kern, dim3((unsigned)nt), dim3(T), SMEM, st, a);

@@ -224,12 +224,8 @@ static int launch_cfg(const GemmArgs& a0, hipStream_t st) {
     a.tiles_n = (a.n + BN - 1) / BN;
     constexpr int smem = 2 * (BM + BN) * BK;
     auto kern = gemm_w8a8_kernel<FP8, BM, BN, BK, WM, WN, DIRECT, XE5>;
-    static bool attr_done = false;  // per instantiation; benign if two threads race to set the same value
-    if (!attr_done) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, smem);
-        if (e != hipSuccess) return fail(DAXQ_ERR_LAUNCH, "hipFuncSetAttribute(%d bytes LDS): %s", smem, hipGetErrorString(e));
-        attr_done = true;
-    }
+    static uint64_t lds_set = 0;  // per instantiation
+    if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), smem, lds_set)) return rc;
     const int64_t nt = (int64_t)a.tiles_m * a.tiles_n;
     if (nt > 0x7fffffff) return fail(DAXQ_ERR_ARG, "gemm: too many tiles");
     hipLaunchKernelGGL(kern, dim3((unsigned)nt), dim3(WM * WN * 64), smem, st, a);
