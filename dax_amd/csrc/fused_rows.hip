@@ -86,7 +86,7 @@ __global__ __launch_bounds__(256) void fused_rows_wave(const uint16_t* __restric
 #pragma unroll
         for (int i = 0; i < NCH; ++i) {
             const int c = i * 64 + lane;
-            v[i] = c < nch ? xr[c] : make_uint4(0, 0, 0, 0);
+            v[i] = c < nch ? load_stream_16(xr + c) : make_uint4(0, 0, 0, 0);
         }
 
         if constexpr (PRE == PRE_LN) {
@@ -181,9 +181,9 @@ __global__ __launch_bounds__(256) void fused_rows_wave(const uint16_t* __restric
         for (int i = 0; i < NCH; ++i) {
             const int c = i * 64 + lane;
             if (c < nch) {
-                qr[c] = quant_chunk<FMT>(v[i], s, inv);
+                store_stream_8(qr + c, quant_chunk<FMT>(v[i], s, inv));
             } else if (c < npad) {
-                qr[c] = make_uint2(0, 0);
+                store_stream_8(qr + c, make_uint2(0, 0));
             }
         }
     }

@@ -39,7 +39,7 @@ __global__ __launch_bounds__(256) void quant_rows_wave(const uint16_t* __restric
     for (int i = 0; i < NCH; ++i) {
         const int c = i * 64 + lane;
         if (c < nch) {
-            v[i] = xr[c];
+            v[i] = load_stream_16(xr + c);
         } else {
             v[i] = make_uint4(0, 0, 0, 0);
         }
@@ -67,9 +67,9 @@ __global__ __launch_bounds__(256) void quant_rows_wave(const uint16_t* __restric
     for (int i = 0; i < NCH; ++i) {
         const int c = i * 64 + lane;
         if (c < nch) {
-            qr[c] = quant_chunk<FMT, SCALE_IN>(v[i], s, inv);
+            store_stream_8(qr + c, quant_chunk<FMT, SCALE_IN>(v[i], s, inv));
         } else if (c < npad) {
-            qr[c] = make_uint2(0, 0);
+            store_stream_8(qr + c, make_uint2(0, 0));
         }
     }
 }
