@@ -39,11 +39,12 @@ __device__ __forceinline__ uint4 pack8(const float (&f)[8]) {
 // gelu(x, approximate="tanh") = 0.5 x (1 + tanh(u)), u = sqrt(2/pi) (x + 0.044715 x^3), evaluated as
 // x / (1 + exp(-2u)): the same function without the cancellation in 1 + tanh(u) for negative x.
 __device__ __forceinline__ float gelu_tanh_f32(float x) {
-    constexpr float kBeta = 0.7978845608028654f, kKappa = 0.044715f, kLog2e = 1.4426950408889634f;
-    const float x2 = x * x;
-    const float u = kBeta * (x + kKappa * x2 * x);
-    const float e = __builtin_amdgcn_exp2f(-2.0f * kLog2e * u);  // exp(-2u); +inf for very negative x
-    return x * __builtin_amdgcn_rcpf(1.0f + e);                  // x * 0 = -0 there, as the limit
+    // exp(-2u) = exp2(x * (c1 + c2 x^2)) with c1 = -2 log2(e) sqrt(2/pi), c2 = 0.044715 c1: three operations in
+    // front of the v_exp_f32 instead of six
+    constexpr float kC1 = -2.0f * 1.4426950408889634f * 0.7978845608028654f, kC2 = kC1 * 0.044715f;
+    const float t = x * __builtin_fmaf(x * x, kC2, kC1);
+    const float e = __builtin_amdgcn_exp2f(t);   // exp(-2u); +inf for very negative x
+    return x * __builtin_amdgcn_rcpf(1.0f + e);  // x * 0 = -0 there, as the limit
 }
 
 // One wavefront per row, 4 rows per workgroup pass, grid-stride over row quads.
