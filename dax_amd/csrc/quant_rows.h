@@ -63,10 +63,13 @@ __device__ __forceinline__ float wave_sum_f32(float x) {
     return (r0 + r1) + (r2 + r3);
 }
 
-__device__ __forceinline__ int q_i8(float x, float inv) {
-    float r = rintf(x * inv);  // v_rndne_f32: round half to even
+// clamp(rint(x * inv), -128, 127) as the low byte of a float: the product is clamped first (same result, the
+// bounds are integers) and 1.5 * 2^23 is added, which rounds it to an integer, half to even, in the low mantissa
+// bits; those bits are the two's-complement value.  Two operations fewer than round + convert.
+__device__ __forceinline__ uint32_t q_i8_bits(float x, float inv) {
+    float r = x * inv;
     r = fminf(fmaxf(r, -128.0f), 127.0f);
-    return (int)r;
+    return __float_as_uint(r + 12582912.0f);
 }
 
 // FMT: 0 = int8, 1 = OCP e4m3fn (max 448), 2 = OCP e5m2 (max 57344)
@@ -113,11 +116,10 @@ __device__ __forceinline__ uint2 quant_chunk(const uint4& v, float s, float inv)
             p = cvt_pk_f8<FMT>(q_f8_pre<FMT, TRUE_DIV>(f2, s, inv), q_f8_pre<FMT, TRUE_DIV>(f3, s, inv), p, true);
             o[h] = (uint32_t)p;
         } else {
-            uint32_t b0 = (uint32_t)q_i8(f0, inv) & 0xffu;
-            uint32_t b1 = (uint32_t)q_i8(f1, inv) & 0xffu;
-            uint32_t b2 = (uint32_t)q_i8(f2, inv) & 0xffu;
-            uint32_t b3 = (uint32_t)q_i8(f3, inv) & 0xffu;
-            o[h] = b0 | (b1 << 8) | (b2 << 16) | (b3 << 24);
+            // byte 0 of each of the four words: three v_perm_b32
+            const uint32_t p01 = __builtin_amdgcn_perm(q_i8_bits(f1, inv), q_i8_bits(f0, inv), 0x0c0c0400u);
+            const uint32_t p23 = __builtin_amdgcn_perm(q_i8_bits(f3, inv), q_i8_bits(f2, inv), 0x0c0c0400u);
+            o[h] = __builtin_amdgcn_perm(p23, p01, 0x05040100u);
         }
     }
     return make_uint2(o[0], o[1]);

@@ -110,7 +110,7 @@ __global__ __launch_bounds__(256) void quant_rows_block(const uint16_t* __restri
             if (FMT != 0) {
                 o = (uint8_t)(cvt_pk_f8<FMT>(q_f8_pre<FMT, SCALE_IN>(f, s, inv), 0.0f, 0, false) & 0xff);
             } else {
-                o = (uint8_t)(q_i8(f, inv) & 0xff);
+                o = (uint8_t)(q_i8_bits(f, inv) & 0xffu);
             }
         }
         qr[c] = o;
