@@ -68,6 +68,50 @@ def test_linear_i8_bit_exact(ops, variant, m, n, k):
     np.testing.assert_array_equal(bf16_bits(out2), bf16_bits(ref2))
 
 
+def _random_shapes(count, seed):
+    rng = np.random.default_rng(seed)
+    shapes = []
+    for _ in range(count):
+        m = int(rng.integers(256, 1400))
+        n = int(rng.integers(32, 160)) * 8           # any multiple of 8 from 256 up
+        k = int(rng.integers(1, 13)) * 128
+        shapes.append((m, n, k, int(rng.integers(0, 3)) * 128, int(rng.integers(0, 5)) * 8))
+    return shapes
+
+
+@pytest.mark.parametrize("variant", [8, 9, 6])
+@pytest.mark.parametrize("m,n,k,pad_k,pad_n", _random_shapes(14, seed=2024))
+def test_linear_i8_random_shapes_and_strides_bit_exact(ops, variant, m, n, k, pad_k, pad_n):
+    """Seeded random M, N, K (edge tiles shifted inwards in both directions, short and long K) with padded leading
+    dimensions, raw int8 operands straight through the C ABI: accumulators and outputs against the integer oracle."""
+    from dax_amd import _capi
+
+    _capi.set_gemm_variant(variant)
+    g = torch.Generator("cpu").manual_seed(m * 7 + n * 3 + k)
+    xq = torch.randint(-127, 128, (m, k), generator=g, dtype=torch.int32).to(torch.int8)
+    wq = torch.randint(-127, 128, (n, k), generator=g, dtype=torch.int32).to(torch.int8)
+    sx = (torch.rand(m, generator=g) * 0.02 + 1e-3).float()
+    sw = (torch.rand(n, generator=g) * 0.002 + 1e-4).float()
+    b = (torch.randn(n, generator=g) * 0.5).bfloat16()
+    want_acc = O.int_mm(xq, wq)
+    want_out = O.epilogue_int8(want_acc, sx.view(-1, 1), sw.view(1, -1), b)
+    xq_wide = torch.full((m, k + pad_k), 5, dtype=torch.int8, device="cuda")
+    xq_wide[:, :k] = dev(xq)
+    wq_wide = torch.full((n, k + pad_k), -7, dtype=torch.int8, device="cuda")
+    wq_wide[:, :k] = dev(wq)
+    out_wide = torch.full((m, n + pad_n), 3.0, dtype=torch.bfloat16, device="cuda")
+    acc_wide = torch.full((m, n + pad_n), -1, dtype=torch.int32, device="cuda")
+    sxd, swd, bd = dev(sx), dev(sw), dev(b)
+    rc = _capi.lib().daxq_linear_i8(xq_wide.data_ptr(), k + pad_k, sxd.data_ptr(), wq_wide.data_ptr(), k + pad_k,
+                                    swd.data_ptr(), bd.data_ptr(), out_wide.data_ptr(), n + pad_n, acc_wide.data_ptr(),
+                                    n + pad_n, m, n, k, torch.cuda.current_stream().cuda_stream)
+    _capi.check(rc, "linear_i8")
+    torch.cuda.synchronize()
+    assert torch.equal(acc_wide[:, :n].cpu(), want_acc)
+    np.testing.assert_array_equal(bf16_bits(out_wide[:, :n]), bf16_bits(want_out))
+    assert bool((out_wide[:, n:] == 3.0).all()) and bool((acc_wide[:, n:] == -1).all())   # nothing outside
+
+
 @pytest.mark.parametrize("variant", VARIANTS)
 def test_linear_i8_adversarial_extremes(ops, variant):
     from dax_amd import _capi
