@@ -174,6 +174,41 @@ def test_linear_e4m3_within_tolerance(ops, variant, m, n, k):
     assert r < 3e-3, r                          # what fp32 accumulation actually delivers
 
 
+@pytest.mark.parametrize("variant", [8, 6])
+@pytest.mark.parametrize("e5m2", [False, True])
+@pytest.mark.parametrize("m,n,k,pad_k,pad_n", _random_shapes(8, seed=77))
+def test_linear_fp8_random_shapes_accumulators(ops, variant, e5m2, m, n, k, pad_k, pad_n):
+    """Seeded random shapes with padded leading dimensions and raw fp8 bytes through the C ABI: the fp32 accumulators
+    against the exact sum of the decoded products (float64), element by element."""
+    from dax_amd import _capi
+
+    _capi.set_gemm_variant(variant)
+    g = torch.Generator("cpu").manual_seed(m + 5 * n + 11 * k)
+    act_dtype = torch.float8_e5m2 if e5m2 else torch.float8_e4m3fn
+    xf = (torch.randn(m, k, generator=g) * 3).to(act_dtype)
+    wf = (torch.randn(n, k, generator=g) * 0.5).to(torch.float8_e4m3fn)
+    want = xf.double() @ wf.double().t()
+    bound = xf.double().abs() @ wf.double().abs().t()          # sum of |products|: the scale of the rounding error
+    xq_wide = torch.zeros((m, k + pad_k), dtype=torch.uint8, device="cuda")
+    xq_wide[:, :k] = dev(xf.view(torch.uint8))
+    wq_wide = torch.zeros((n, k + pad_k), dtype=torch.uint8, device="cuda")
+    wq_wide[:, :k] = dev(wf.view(torch.uint8))
+    out_wide = torch.zeros((m, n + pad_n), dtype=torch.bfloat16, device="cuda")
+    acc_wide = torch.full((m, n + pad_n), -1.0, dtype=torch.float32, device="cuda")
+    ones_m, ones_n = torch.ones(m, device="cuda"), torch.ones(n, device="cuda")
+    fn = _capi.lib().daxq_linear_e5m2_e4m3 if e5m2 else _capi.lib().daxq_linear_e4m3
+    rc = fn(xq_wide.data_ptr(), k + pad_k, ones_m.data_ptr(), wq_wide.data_ptr(), k + pad_k, ones_n.data_ptr(), None,
+            out_wide.data_ptr(), n + pad_n, acc_wide.data_ptr(), n + pad_n, m, n, k,
+            torch.cuda.current_stream().cuda_stream)
+    _capi.check(rc, "linear fp8")
+    torch.cuda.synchronize()
+    got = acc_wide[:, :n].cpu().double()
+    err = ((got - want).abs() / bound.clamp_min(1e-30)).max().item()
+    assert err < 2e-5, err        # fp32 accumulation of K products: a few 2^-24 of the sum of magnitudes
+    assert bool((acc_wide[:, n:] == -1.0).all())
+    assert torch.equal(out_wide[:, :n].cpu(), acc_wide[:, :n].cpu().bfloat16())   # unit scales, no bias: out = bf16(acc)
+
+
 @pytest.mark.parametrize("variant", [0, 5, 6])
 @pytest.mark.parametrize("m,n,k", [(300, 520, 256), (17, 24, 384), (512, 1536, 1536), (4096, 1536, 1536)])
 def test_linear_e5m2_activations_within_tolerance(ops, variant, m, n, k):
