@@ -23,8 +23,9 @@
 //   fragments of slice kt+1 are spread over its MFMAs.
 //
 // Tiles at the M / N edge are shifted inwards (origin min(tile*256, dim-256)) instead of being
-// predicated: the overlap rows are computed twice with identical results.  Shapes with
-// M < 256 or N < 256 take the generic kernel in gemm_w8a8.hip.
+// predicated: the overlap rows are computed twice with identical results.  The five-stage kernel
+// also exists on 128x128 tiles (launches with too few 256-tiles to fill the CUs); shapes with
+// M < 128 or N < 128 take the generic kernel in gemm_w8a8.hip.
 #include "gemm_common.h"
 
 namespace daxq {
@@ -115,10 +116,10 @@ __device__ __forceinline__ void load_one_frag(const FragAddr& fa, int stage, int
 }
 
 // ZERO: the block's first MFMA of a tile, which starts from zero instead of the accumulator
-template <bool FP8, bool XE5, bool ZERO = false>
-__device__ __forceinline__ void mfma_one(typename AccT<FP8>::type (&acc)[4][4], int g, const typename Frag<FP8>::type (&af)[4],
+template <bool FP8, bool XE5, bool ZERO = false, int NB = 4>
+__device__ __forceinline__ void mfma_one(typename AccT<FP8>::type (&acc)[NB][NB], int g, const typename Frag<FP8>::type (&af)[4],
                                          const typename Frag<FP8>::type (&bf)[4]) {
-    const int j = g >> 2, i = g & 3;
+    const int j = g / NB, i = g % NB;
     typename AccT<FP8>::type c = {};
     if constexpr (!ZERO) c = acc[j][i];
     if constexpr (!FP8)
@@ -148,27 +149,31 @@ __device__ __forceinline__ void mfma_step(typename AccT<FP8>::type (&acc)[4][4],
 // columns n = 8q + 4*(l/32) + {0..3}.  Two v_permlane32_swap per pair of q give each lane 8
 // consecutive columns, stored as one 16-byte write.  The tile's scales and bias are staged in LDS.
 // pre_*: this thread's element (index t) of the tile's sx / sw / bias, already loaded by the caller.
-template <bool FP8, bool DUMP>
-__device__ __forceinline__ void tile256_epilogue(const GemmArgs& p, typename AccT<FP8>::type (&acc)[4][4], uint8_t* smem,
+// NB: 32x32 blocks per operand and wavefront (4: 256x256 tile, 2: 128x128 tile); the tile edge is 64 * NB.
+template <bool FP8, bool DUMP, int NB = 4>
+__device__ __forceinline__ void tile256_epilogue(const GemmArgs& p, typename AccT<FP8>::type (&acc)[NB][NB], uint8_t* smem,
                                                  int m0, int n0, int t, int wm, int wn, int l31, int hi, float pre_sx,
                                                  float pre_sw, float pre_bias) {
+    constexpr int BT = 64 * NB, WT = 32 * NB;
     float* s_sx = reinterpret_cast<float*>(smem);
-    float* s_sw = s_sx + 256;
-    float* s_bias = s_sw + 256;
-    s_sx[t] = pre_sx;
-    s_sw[t] = pre_sw;
-    s_bias[t] = pre_bias;
+    float* s_sw = s_sx + BT;
+    float* s_bias = s_sw + BT;
+    if (BT == 256 || t < BT) {
+        s_sx[t] = pre_sx;
+        s_sw[t] = pre_sw;
+        s_bias[t] = pre_bias;
+    }
     __syncthreads();
 
     if constexpr (DUMP) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+        for (int j = 0; j < NB; ++j)
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int64_t m = m0 + wm * 128 + i * 32 + l31;
+            for (int i = 0; i < NB; ++i) {
+                const int64_t m = m0 + wm * WT + i * 32 + l31;
 #pragma unroll
                 for (int v = 0; v < 16; ++v) {
-                    const int n = n0 + wn * 128 + j * 32 + 8 * (v >> 2) + 4 * hi + (v & 3);
+                    const int n = n0 + wn * WT + j * 32 + 8 * (v >> 2) + 4 * hi + (v & 3);
                     if constexpr (!FP8)
                         static_cast<int32_t*>(p.acc)[m * p.ldacc + n] = acc[j][i][v];
                     else
@@ -179,27 +184,27 @@ __device__ __forceinline__ void tile256_epilogue(const GemmArgs& p, typename Acc
 
     // every scale and bias value this lane needs goes into registers in one burst of LDS reads
     // (the fragment registers of the main loop are free now): 4 x sx, 16 x 4 sw, 16 x 4 bias
-    float sxr[4];
-    float4 swr[4][4], br[4][4];
+    float sxr[NB];
+    float4 swr[NB][4], br[NB][4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) sxr[i] = s_sx[wm * 128 + i * 32 + l31];
+    for (int i = 0; i < NB; ++i) sxr[i] = s_sx[wm * WT + i * 32 + l31];
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+    for (int j = 0; j < NB; ++j)
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-            const int nl = wn * 128 + j * 32 + 8 * q + 4 * hi;
+            const int nl = wn * WT + j * 32 + 8 * q + 4 * hi;
             swr[j][q] = *reinterpret_cast<const float4*>(s_sw + nl);
             br[j][q] = *reinterpret_cast<const float4*>(s_bias + nl);
         }
     __builtin_amdgcn_sched_barrier(0);
 
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int ml = wm * 128 + i * 32 + l31;
+    for (int i = 0; i < NB; ++i) {
+        const int ml = wm * WT + i * 32 + l31;
         const float sxv = sxr[i];
-        uint16_t* orow = p.out + (int64_t)(m0 + ml) * p.ldo + n0 + wn * 128 + 8 * hi;
+        uint16_t* orow = p.out + (int64_t)(m0 + ml) * p.ldo + n0 + wn * WT + 8 * hi;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
+        for (int j = 0; j < NB; ++j) {
             uint32_t pk[4][2];
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
@@ -242,49 +247,53 @@ __device__ __forceinline__ void tile256_epilogue(const GemmArgs& p, typename Acc
 // v_permlane16_swap per word over two neighbouring blocks gives each lane 8 consecutive columns of one
 // of them: lanes 0-15 block 2jp columns 0-7, lanes 16-31 block 2jp+1 columns 0-7, lanes 32-47 block
 // 2jp columns 8-15, lanes 48-63 block 2jp+1 columns 8-15.
-template <bool DUMP>
-__device__ __forceinline__ void tile256_epilogue16(const GemmArgs& p, v4i (&acc)[8][8], uint8_t* smem, int m0, int n0, int t,
+// NB: 16x16 blocks per operand and wavefront (8: 256x256 tile, 4: 128x128 tile); the tile edge is 32 * NB.
+template <bool DUMP, int NB = 8>
+__device__ __forceinline__ void tile256_epilogue16(const GemmArgs& p, v4i (&acc)[NB][NB], uint8_t* smem, int m0, int n0, int t,
                                                    int wm, int wn, int l15, int g4, float pre_sx, float pre_sw,
                                                    float pre_bias) {
+    constexpr int BT = 32 * NB, WT = 16 * NB;
     float* s_sx = reinterpret_cast<float*>(smem);
-    float* s_sw = s_sx + 256;
-    float* s_bias = s_sw + 256;
-    s_sx[t] = pre_sx;
-    s_sw[t] = pre_sw;
-    s_bias[t] = pre_bias;
+    float* s_sw = s_sx + BT;
+    float* s_bias = s_sw + BT;
+    if (BT == 256 || t < BT) {
+        s_sx[t] = pre_sx;
+        s_sw[t] = pre_sw;
+        s_bias[t] = pre_bias;
+    }
     __syncthreads();
 
     if constexpr (DUMP) {
 #pragma unroll
-        for (int j = 0; j < 8; ++j)
+        for (int j = 0; j < NB; ++j)
 #pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                const int64_t m = m0 + wm * 128 + i * 16 + l15;
+            for (int i = 0; i < NB; ++i) {
+                const int64_t m = m0 + wm * WT + i * 16 + l15;
 #pragma unroll
                 for (int v = 0; v < 4; ++v)
-                    static_cast<int32_t*>(p.acc)[m * p.ldacc + n0 + wn * 128 + j * 16 + 4 * g4 + v] = acc[j][i][v];
+                    static_cast<int32_t*>(p.acc)[m * p.ldacc + n0 + wn * WT + j * 16 + 4 * g4 + v] = acc[j][i][v];
             }
     }
 
-    float sxr[8];
-    float4 swr[8], br[8];
+    float sxr[NB];
+    float4 swr[NB], br[NB];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) sxr[i] = s_sx[wm * 128 + i * 16 + l15];
+    for (int i = 0; i < NB; ++i) sxr[i] = s_sx[wm * WT + i * 16 + l15];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-        const int nl = wn * 128 + j * 16 + 4 * g4;
+    for (int j = 0; j < NB; ++j) {
+        const int nl = wn * WT + j * 16 + 4 * g4;
         swr[j] = *reinterpret_cast<const float4*>(s_sw + nl);
         br[j] = *reinterpret_cast<const float4*>(s_bias + nl);
     }
     __builtin_amdgcn_sched_barrier(0);
 
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        const int ml = wm * 128 + i * 16 + l15;
+    for (int i = 0; i < NB; ++i) {
+        const int ml = wm * WT + i * 16 + l15;
         const float sxv = sxr[i];
-        uint16_t* orow = p.out + (int64_t)(m0 + ml) * p.ldo + n0 + wn * 128 + (g4 & 1) * 16 + (g4 >> 1) * 8;
+        uint16_t* orow = p.out + (int64_t)(m0 + ml) * p.ldo + n0 + wn * WT + (g4 & 1) * 16 + (g4 >> 1) * 8;
 #pragma unroll
-        for (int jp = 0; jp < 4; ++jp) {
+        for (int jp = 0; jp < NB / 2; ++jp) {
             uint32_t pk[2][2];
 #pragma unroll
             for (int jj = 0; jj < 2; ++jj) {
@@ -553,11 +562,11 @@ int launch_tile256(const GemmArgs& a0, bool x_e5m2, hipStream_t st) {
 // LDS layout of an operand part: [256 rows][64 B], 16-byte chunk c of row r stored at chunk
 // c ^ ((r >> 2) & 3) (32x32 MFMA forms) or c ^ ((r >> 1) & 3) (16x16 form): the ds_read_b128 of either form
 // then runs at the full LDS rate.
+//
+// BT: tile edge.  256 is the form described above; 128 (wavefronts of 64 x 64, five 16 KB stages, two workgroups
+// per CU) is the same pipeline for launches with too few 256-tiles to fill the CUs.
 namespace t5 {
 constexpr int BKS = 64, NST = 5, T = 256;
-constexpr int A_BYTES = 256 * BKS, STAGE = 2 * A_BYTES;  // 16 KB, 32 KB
-constexpr int SMEM = NST * STAGE;                        // 163840
-constexpr int PAIR_LOADS = 16;                           // per thread and pair of slices
 }  // namespace t5
 
 // accumulators of a wavefront's 128 x 128 outputs
@@ -574,15 +583,21 @@ struct TileAcc<false, true> {
 // of two v_mfma_i32_32x32x32_i8 per 32x32 block (32).  Same LDS bytes, fragment registers and MFMA
 // cycles; the narrow shape moves fewer accumulator bytes per operation and sustains a higher clock
 // under the board's power limit.
-template <bool FP8, bool DUMP, bool XE5, bool N16 = false>
+template <bool FP8, bool DUMP, bool XE5, bool N16 = false, int BT = 256>
 __global__ __launch_bounds__(256) void gemm_tile256s5_kernel(const GemmArgs p) {
     using namespace t5;
     static_assert(!(FP8 && N16), "the 16x16 form exists for INT8 only");
+    static_assert(BT == 256 || BT == 128, "tile edge");
     typedef typename Frag<FP8>::type frag_t;
+    constexpr int WT = BT / 2;                        // edge of a wavefront's outputs
+    constexpr int NB = WT / (N16 ? 16 : 32);          // MFMA blocks per operand and wavefront: 8 / 4 (256), 4 / 2 (128)
+    constexpr int A_BYTES = BT * BKS, STAGE = 2 * A_BYTES;
+    constexpr int PAIR_LOADS = BT / 16;               // DMA loads per thread and pair of slices
+    constexpr int JB = BT / 64;                       // 64-row blocks of an operand part (one DMA instruction each)
     constexpr int STEPS = FP8 ? 1 : 2;               // MFMA steps per 64-byte slice (32x32 form)
-    constexpr int NREG = N16 ? 64 : 16 * STEPS;      // MFMAs = scheduling regions per slice
-    constexpr int DMA_EVERY = NREG / (PAIR_LOADS / 2);  // regions per DMA load
-    constexpr int READ_EVERY = 3;                    // N16: regions per fragment read (16 reads)
+    constexpr int NREG = N16 ? NB * NB : NB * NB * STEPS;  // MFMAs = scheduling regions per slice
+    constexpr int DMA_EVERY = NREG / (PAIR_LOADS / 2);     // regions per DMA load
+    constexpr int READ_EVERY = NREG >= 48 ? 3 : NREG / (2 * NB);  // N16: regions per fragment read (2 * NB reads)
 
     extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
 
@@ -590,9 +605,9 @@ __global__ __launch_bounds__(256) void gemm_tile256s5_kernel(const GemmArgs p) {
     const int wm = wave >> 1, wn = wave & 1;
     int tm, tn;
     tile_of_block(p.gm, blockIdx.x, p.tiles_m, p.tiles_n, tm, tn);
-    int m0 = tm * 256, n0 = tn * 256;
-    m0 = m0 + 256 <= p.m ? m0 : p.m - 256;
-    n0 = n0 + 256 <= p.n ? n0 : p.n - 256;
+    int m0 = tm * BT, n0 = tn * BT;
+    m0 = m0 + BT <= p.m ? m0 : p.m - BT;
+    n0 = n0 + BT <= p.n ? n0 : p.n - BT;
 
     // ---- HBM side.  One wave instruction fills 1 KB of LDS = 16 rows x 64 B: lane l -> row l/4,
     //      stored chunk l%4, i.e. global chunk (l%4) ^ ((row>>2)&3).  Instruction j of a thread
@@ -608,10 +623,10 @@ __global__ __launch_bounds__(256) void gemm_tile256s5_kernel(const GemmArgs p) {
     const int64_t a_step = 64 * p.lda, b_step = 64 * p.ldb;
     const uint32_t lds0 = (uint32_t)(uintptr_t)(DAXQ_LDS uint8_t*)smem;
     const uint32_t wave_lds = lds0 + (uint32_t)__builtin_amdgcn_readfirstlane(wave * 1024);
-    // load g = 0..15 of a pair: operand g/8 (0 = A), row block (g/2)%4, half g%2 -> stage o0 / o1.
+    // load g of a pair (16 for a 256 tile): first half of them operand A, row block (g/2) % JB, half g%2 -> stage o0 / o1.
     // Address = uniform row-block base (SGPR pair) + per-lane 32-bit offset: no VALU work per load.
     auto issue_one = [&](uint32_t o0, uint32_t o1, int g) {
-        const int opnd = g >> 3, j = (g >> 1) & 3, half = g & 1;
+        const int opnd = g / (PAIR_LOADS / 2), j = (g >> 1) % JB, half = g & 1;
         const uint8_t* src = opnd ? bbase + j * b_step : abase + j * a_step;
         const uint32_t voff = opnd ? (half ? voff_b1 : voff_b) : (half ? voff_a1 : voff_a);
         const uint32_t dst = wave_lds + (half ? o1 : o0) + opnd * A_BYTES + j * 4096;
@@ -635,8 +650,8 @@ __global__ __launch_bounds__(256) void gemm_tile256s5_kernel(const GemmArgs p) {
     const int l31 = lane & 31, hi = lane >> 5;
     const int lr = N16 ? (lane & 15) : l31;  // row of the lane inside an MFMA block
     const int gq = ((N16 ? lr >> 1 : lr >> 2)) & 3;
-    const uint8_t* a_rd = smem + (wm * 128 + lr) * BKS;
-    const uint8_t* b_rd = smem + A_BYTES + (wn * 128 + lr) * BKS;
+    const uint8_t* a_rd = smem + (wm * WT + lr) * BKS;
+    const uint8_t* b_rd = smem + A_BYTES + (wn * WT + lr) * BKS;
     // one fragment: f = 0..3 A block f, 4..7 B block f-4; step ks of the slice in the stage at offset o
     // (N16: ks selects the upper four of the eight 16-row blocks; every fragment spans the whole slice)
     auto read_frag = [&](uint32_t o, int ks, int f, frag_t (&af)[4], frag_t (&bf)[4]) {
@@ -645,6 +660,7 @@ __global__ __launch_bounds__(256) void gemm_tile256s5_kernel(const GemmArgs p) {
             (f < 4 ? af[f & 3] : bf[f & 3]) = *reinterpret_cast<const v4i*>(pr + (((lane >> 4) ^ gq) << 4));
             return;
         }
+        if ((f & 3) >= NB) return;  // 128 tile: two 32-row blocks per operand
         const uint8_t* pr = (f < 4 ? a_rd : b_rd) + o + (f & 3) * 32 * BKS;
         if constexpr (!FP8) {
             const int xo = ((ks * 2 + hi) ^ gq) << 4;
@@ -657,7 +673,7 @@ __global__ __launch_bounds__(256) void gemm_tile256s5_kernel(const GemmArgs p) {
         }
     };
 
-    typename TileAcc<FP8, N16>::type acc[N16 ? 8 : 4][N16 ? 8 : 4];
+    typename TileAcc<FP8, N16>::type acc[NB][NB];
 
     // fragment sets: [slice parity][MFMA step] (N16: [slice parity][blocks 0-3 / 4-7])
     frag_t fa00[4] = {}, fb00[4] = {}, fa01[4] = {}, fb01[4] = {}, fa10[4] = {}, fb10[4] = {}, fa11[4] = {}, fb11[4] = {};
@@ -684,9 +700,10 @@ __global__ __launch_bounds__(256) void gemm_tile256s5_kernel(const GemmArgs p) {
             if constexpr (ISSUE.value) {
                 if (g % DMA_EVERY == 0) issue_one(o_ld0, o_ld1, g / DMA_EVERY + (ODD.value ? PAIR_LOADS / 2 : 0));
             }
-            if constexpr (NEXT.value && N16) {  // 16 reads, one every READ_EVERY regions
-                if (g % READ_EVERY == 0 && g / READ_EVERY < 16) {
-                    const int idx = g / READ_EVERY;
+            if constexpr (NEXT.value && N16) {  // 2 * NB reads, one every READ_EVERY regions
+                if (g % READ_EVERY == 0 && g / READ_EVERY < 2 * NB) {
+                    // NB = 8: blocks 0-3 of A and B, then blocks 4-7; NB = 4: blocks 0-3 of A and B
+                    const int idx = NB == 8 ? g / READ_EVERY : (g / READ_EVERY < NB ? g / READ_EVERY : 4 + g / READ_EVERY - NB);
                     if constexpr (ODD.value) {
                         if (idx < 8) read_frag(o_next, 0, idx, fa00, fb00);
                         else read_frag(o_next, 1, idx - 8, fa01, fb01);
@@ -696,23 +713,28 @@ __global__ __launch_bounds__(256) void gemm_tile256s5_kernel(const GemmArgs p) {
                     }
                 }
             } else if constexpr (NEXT.value) {
-                if constexpr (!FP8) {  // 16 reads: step 0 set in regions 0..7, step 1 set in regions 8..15
-                    if (g < 8) {
-                        if constexpr (ODD.value) read_frag(o_next, 0, g, fa00, fb00);
-                        else read_frag(o_next, 0, g, fa10, fb10);
-                    } else if (g < 16) {
-                        if constexpr (ODD.value) read_frag(o_next, 1, g - 8, fa01, fb01);
-                        else read_frag(o_next, 1, g - 8, fa11, fb11);
+                // fragment fi of a step: the NB blocks of A, then the NB blocks of B (slot 4 + block in read_frag)
+                if constexpr (!FP8) {  // 2 * NB reads of step 0 in the first regions, then those of step 1
+                    if (g < 4 * NB) {
+                        const int fi = g % (2 * NB), f = fi < NB ? fi : 4 + fi - NB;
+                        if (g < 2 * NB) {
+                            if constexpr (ODD.value) read_frag(o_next, 0, f, fa00, fb00);
+                            else read_frag(o_next, 0, f, fa10, fb10);
+                        } else {
+                            if constexpr (ODD.value) read_frag(o_next, 1, f, fa01, fb01);
+                            else read_frag(o_next, 1, f, fa11, fb11);
+                        }
                     }
                 } else {
-                    if (g < 8) {
-                        if constexpr (ODD.value) read_frag(o_next, 0, g, fa00, fb00);
-                        else read_frag(o_next, 0, g, fa10, fb10);
+                    if (g < 2 * NB) {
+                        const int f = g < NB ? g : 4 + g - NB;
+                        if constexpr (ODD.value) read_frag(o_next, 0, f, fa00, fb00);
+                        else read_frag(o_next, 0, f, fa10, fb10);
                     }
                 }
             }
             if constexpr (N16) {
-                const int j = g >> 3, i = g & 7;  // B block j, A block i
+                const int j = g / NB, i = g % NB;  // B block j, A block i
                 const v4i bfr = ODD.value ? (j < 4 ? fb10[j & 3] : fb11[j & 3]) : (j < 4 ? fb00[j & 3] : fb01[j & 3]);
                 const v4i afr = ODD.value ? (i < 4 ? fa10[i & 3] : fa11[i & 3]) : (i < 4 ? fa00[i & 3] : fa01[i & 3]);
                 // accumulator tied in place in AGPRs: left to the register allocator, the 64 four-register
@@ -723,21 +745,22 @@ __global__ __launch_bounds__(256) void gemm_tile256s5_kernel(const GemmArgs p) {
                     asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+a"(acc[j][i]) : "v"(bfr), "v"(afr));
             } else if constexpr (!FP8) {
                 if constexpr (ODD.value) {
-                    if (g < 16) mfma_one<FP8, XE5>(acc, g, fa10, fb10);
-                    else mfma_one<FP8, XE5>(acc, g - 16, fa11, fb11);
+                    if (g < NB * NB) mfma_one<FP8, XE5, false, NB>(acc, g, fa10, fb10);
+                    else mfma_one<FP8, XE5, false, NB>(acc, g - NB * NB, fa11, fb11);
                 } else {
-                    if (g < 16) mfma_one<FP8, XE5, FIRST.value>(acc, g, fa00, fb00);
-                    else mfma_one<FP8, XE5>(acc, g - 16, fa01, fb01);
+                    if (g < NB * NB) mfma_one<FP8, XE5, FIRST.value, NB>(acc, g, fa00, fb00);
+                    else mfma_one<FP8, XE5, false, NB>(acc, g - NB * NB, fa01, fb01);
                 }
             } else {
-                if constexpr (ODD.value) mfma_one<FP8, XE5>(acc, g, fa10, fb10);
-                else mfma_one<FP8, XE5, FIRST.value>(acc, g, fa00, fb00);
+                if constexpr (ODD.value) mfma_one<FP8, XE5, false, NB>(acc, g, fa10, fb10);
+                else mfma_one<FP8, XE5, FIRST.value, NB>(acc, g, fa00, fb00);
             }
             // loop bookkeeping inside the last regions, in the issue slots an MFMA leaves free, instead of
             // in a block of its own behind the slice: lane offsets of the operand this slice loaded, and
             // (odd slice) the rotation of the stage offsets by one pair
             if constexpr (ISSUE.value) {
-                if (g == NREG - 2) {
+                // behind the slice's last load (with a load in every region that is the last region)
+                if (g == (DMA_EVERY == 1 ? NREG - 1 : NREG - 2)) {
                     if constexpr (ODD.value) advance_b();
                     else advance_a();
                 }
@@ -778,7 +801,7 @@ __global__ __launch_bounds__(256) void gemm_tile256s5_kernel(const GemmArgs p) {
 #pragma unroll
     for (int f = 0; f < 8; ++f) {
         read_frag(0, 0, f, fa00, fb00);
-        if constexpr (!FP8) read_frag(0, 1, f, fa01, fb01);
+        if constexpr (!FP8 && !(N16 && NB == 4)) read_frag(0, 1, f, fa01, fb01);  // 16x16 form: blocks 4-7 exist for NB = 8
     }
 
     const int Q = S >> 1;  // pairs
@@ -786,40 +809,58 @@ __global__ __launch_bounds__(256) void gemm_tile256s5_kernel(const GemmArgs p) {
         pair(Yes{}, Yes{}, Yes{}, Int<0>{}, Yes{});
     } else {  // short K: no pair to peel, clear the accumulators instead
 #pragma unroll
-        for (int j = 0; j < (N16 ? 8 : 4); ++j)
+        for (int j = 0; j < NB; ++j)
 #pragma unroll
-            for (int i = 0; i < (N16 ? 8 : 4); ++i) acc[j][i] = typename TileAcc<FP8, N16>::type{};
+            for (int i = 0; i < NB; ++i) acc[j][i] = typename TileAcc<FP8, N16>::type{};
     }
     for (int q = 1; q + 2 < Q; ++q) pair(Yes{}, Yes{}, Yes{}, Int<0>{}, No{});
 
     // The epilogue's scales and bias are requested here, behind the last tile loads, so that their
     // latency is covered by the remaining two pairs of slices.  Always three loads (a missing bias
     // reads a scale instead and is replaced by -0.0: x + (-0.0) == x bit for bit).
-    const float pre_sx = p.sx[m0 + t], pre_sw = p.sw[n0 + t];
-    const uint16_t pre_b = (p.bias ? p.bias : reinterpret_cast<const uint16_t*>(p.sw))[n0 + t];
+    // (every wavefront issues them, so that the counts the waits are written for hold: with a 128 tile the upper
+    // two wavefronts repeat the loads of the lower two and drop the values)
+    const int tt = t & (BT - 1);
+    const float pre_sx = p.sx[m0 + tt], pre_sw = p.sw[n0 + tt];
+    const uint16_t pre_b = (p.bias ? p.bias : reinterpret_cast<const uint16_t*>(p.sw))[n0 + tt];
     __builtin_amdgcn_sched_barrier(0);
 
     if (Q >= 2) pair(No{}, Yes{}, Yes{}, Int<3>{}, No{});
     pair(No{}, No{}, No{}, Int<3>{}, No{});
 
     if constexpr (N16) {
-        // the 16x16 MFMAs are inline asm, so the compiler cannot count the wait states between the last one
-        // and the first read of its result; the epilogue starts with an LDS write and a barrier, and these
-        // 24 idle cycles keep that distance whatever is scheduled in between
-        asm volatile("s_nop 15\n\ts_nop 7" ::: "memory");
+        // The 16x16 MFMAs are inline asm, so the compiler cannot count the wait states between one of them and a
+        // VALU read of its result, and it places such reads right behind the MFMA if nothing stops it.  Volatile
+        // asm statements keep their order: 24 idle cycles first, then every accumulator is passed through an empty
+        // statement, which no read of it can move above.
+        asm volatile("s_nop 15\n\ts_nop 7");
+#pragma unroll
+        for (int j = 0; j < NB; j += 2) {
+            if constexpr (NB == 8) {
+                asm volatile(""
+                             : "+a"(acc[j][0]), "+a"(acc[j][1]), "+a"(acc[j][2]), "+a"(acc[j][3]), "+a"(acc[j][4]), "+a"(acc[j][5]),
+                               "+a"(acc[j][6]), "+a"(acc[j][7]), "+a"(acc[j + 1][0]), "+a"(acc[j + 1][1]), "+a"(acc[j + 1][2]),
+                               "+a"(acc[j + 1][3]), "+a"(acc[j + 1][4]), "+a"(acc[j + 1][5]), "+a"(acc[j + 1][6]), "+a"(acc[j + 1][7]));
+            } else {
+                asm volatile(""
+                             : "+a"(acc[j][0]), "+a"(acc[j][1]), "+a"(acc[j][2]), "+a"(acc[j][3]), "+a"(acc[j + 1][0]),
+                               "+a"(acc[j + 1][1]), "+a"(acc[j + 1][2]), "+a"(acc[j + 1][3]));
+            }
+        }
     }
     if constexpr (N16)
-        tile256_epilogue16<DUMP>(p, acc, smem, m0, n0, t, wm, wn, lr, lane >> 4, pre_sx, pre_sw,
-                                 p.bias ? bf16_bits_to_f32(pre_b) : -0.0f);
+        tile256_epilogue16<DUMP, NB>(p, acc, smem, m0, n0, t, wm, wn, lr, lane >> 4, pre_sx, pre_sw,
+                                     p.bias ? bf16_bits_to_f32(pre_b) : -0.0f);
     else
-        tile256_epilogue<FP8, DUMP>(p, acc, smem, m0, n0, t, wm, wn, l31, hi, pre_sx, pre_sw,
-                                    p.bias ? bf16_bits_to_f32(pre_b) : -0.0f);
+        tile256_epilogue<FP8, DUMP, NB>(p, acc, smem, m0, n0, t, wm, wn, l31, hi, pre_sx, pre_sw,
+                                        p.bias ? bf16_bits_to_f32(pre_b) : -0.0f);
 }
 
-template <bool FP8, bool DUMP, bool XE5, bool N16 = false>
+template <bool FP8, bool DUMP, bool XE5, bool N16 = false, int BT = 256>
 static int launch_tile256s5_impl(const GemmArgs& a, hipStream_t st) {
     using namespace t5;
-    auto kern = gemm_tile256s5_kernel<FP8, DUMP, XE5, N16>;
+    constexpr int SMEM = NST * 2 * BT * BKS;  // 160 KB (256 tile), 80 KB (128 tile)
+    auto kern = gemm_tile256s5_kernel<FP8, DUMP, XE5, N16, BT>;
     static uint64_t lds_set = 0;  // per instantiation
     if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), SMEM, lds_set)) return rc;
     const int64_t nt = (int64_t)a.tiles_m * a.tiles_n;
@@ -828,23 +869,30 @@ static int launch_tile256s5_impl(const GemmArgs& a, hipStream_t st) {
     return check_launch("gemm_tile256s5");
 }
 
-// wide: INT8 with 32x32x32 MFMAs instead of the 16x16x64 form (kept for the tests and for comparisons)
+// wide:  INT8 with 32x32x32 MFMAs instead of the 16x16x64 form (256 tile only; kept for the tests and for comparisons)
+// small: 128x128 tiles (needs m, n >= 128)
 template <bool FP8>
-int launch_tile256s5(const GemmArgs& a0, bool x_e5m2, bool wide, hipStream_t st) {
+int launch_tile256s5(const GemmArgs& a0, bool x_e5m2, bool wide, bool small, hipStream_t st) {
     GemmArgs a = a0;
-    a.tiles_m = (a.m + 255) / 256;
-    a.tiles_n = (a.n + 255) / 256;
+    const int bt = small ? 128 : 256;
+    a.tiles_m = (a.m + bt - 1) / bt;
+    a.tiles_n = (a.n + bt - 1) / bt;
     if constexpr (FP8) {
+        if (small) {
+            if (x_e5m2) return a.acc ? launch_tile256s5_impl<true, true, true, false, 128>(a, st) : launch_tile256s5_impl<true, false, true, false, 128>(a, st);
+            return a.acc ? launch_tile256s5_impl<true, true, false, false, 128>(a, st) : launch_tile256s5_impl<true, false, false, false, 128>(a, st);
+        }
         if (x_e5m2) return a.acc ? launch_tile256s5_impl<true, true, true>(a, st) : launch_tile256s5_impl<true, false, true>(a, st);
         return a.acc ? launch_tile256s5_impl<true, true, false>(a, st) : launch_tile256s5_impl<true, false, false>(a, st);
     } else {
+        if (small) return a.acc ? launch_tile256s5_impl<false, true, false, true, 128>(a, st) : launch_tile256s5_impl<false, false, false, true, 128>(a, st);
         if (wide) return a.acc ? launch_tile256s5_impl<false, true, false>(a, st) : launch_tile256s5_impl<false, false, false>(a, st);
         return a.acc ? launch_tile256s5_impl<false, true, false, true>(a, st) : launch_tile256s5_impl<false, false, false, true>(a, st);
     }
 }
 
-template int launch_tile256s5<false>(const GemmArgs&, bool, bool, hipStream_t);
-template int launch_tile256s5<true>(const GemmArgs&, bool, bool, hipStream_t);
+template int launch_tile256s5<false>(const GemmArgs&, bool, bool, bool, hipStream_t);
+template int launch_tile256s5<true>(const GemmArgs&, bool, bool, bool, hipStream_t);
 
 // the kernel applies: both dimensions hold a whole tile and the 32-bit row offsets cannot overflow
 bool tile256_applies(const GemmArgs& a) {

@@ -215,7 +215,7 @@ template <bool FP8>
 int launch_tile256(const GemmArgs& a, bool x_e5m2, hipStream_t st);
 bool tile256_applies(const GemmArgs& a);
 template <bool FP8>
-int launch_tile256s5(const GemmArgs& a, bool x_e5m2, bool wide, hipStream_t st);
+int launch_tile256s5(const GemmArgs& a, bool x_e5m2, bool wide, bool small, hipStream_t st);
 
 template <bool FP8, int BM, int BN, int BK, int WM, int WN, bool DIRECT, bool XE5 = false>
 static int launch_cfg(const GemmArgs& a0, hipStream_t st) {
@@ -265,11 +265,14 @@ static int launch_gemm(const void* xq, int64_t ld_xq, const float* sx, const voi
     a.gm = g_gm;
     switch (g_variant) {
         case 0: {
-            // library default: the five-stage 256x256 kernel once its tiles fill about a third of the
-            // 256 CUs, otherwise 128x128 tiles (4x as many workgroups; measured cross-over at
-            // N = K = 5120: M = 512 -> 642 against 533 T-op/s, M = 1024 -> 948 against 1012)
+            // library default: the five-stage kernel on 256x256 tiles once there is one for every second CU, on
+            // 128x128 tiles (4x as many workgroups, two per CU) below that, and the generic kernel for operands
+            // smaller than one such tile.  Measured at N = K = 5120 (INT8, T-op/s, 128 / 256 tiles):
+            // M = 512 -> 1127 / 551, M = 1024 (80 large tiles) -> 1275 / 1055, M = 2048 (160) -> 1542 / 1817;
+            // 4096 x 1536 x 1536 (96) -> 1182 / 895, 8192 x 1536 x 1536 (192) -> 1517 / 1587.
             const int64_t tiles256 = ((m + 255) / 256) * ((n + 255) / 256);
-            if (tile256_applies(a) && tiles256 >= 80) return launch_tile256s5<FP8>(a, x_e5m2, false, st);
+            if (tile256_applies(a) && tiles256 >= 128) return launch_tile256s5<FP8>(a, x_e5m2, false, false, st);
+            if (m >= 128 && n >= 128 && a.lda < (1 << 26) && a.ldb < (1 << 26)) return launch_tile256s5<FP8>(a, x_e5m2, false, true, st);
             if constexpr (FP8) {
                 if (x_e5m2) return launch_cfg<true, 128, 128, 128, 2, 2, true, true>(a, st);
             }
@@ -289,7 +292,10 @@ static int launch_gemm(const void* xq, int64_t ld_xq, const float* sx, const voi
         case 8:
         case 9:  // 9: INT8 with 32x32x32 MFMAs
             if (!tile256_applies(a)) return fail(DAXQ_ERR_ARG, "linear: the 256x256 kernel needs m, n >= 256");
-            return launch_tile256s5<FP8>(a, x_e5m2, g_variant == 9, st);
+            return launch_tile256s5<FP8>(a, x_e5m2, g_variant == 9, false, st);
+        case 11:  // the five-stage kernel on 128x128 tiles
+            if (m < 128 || n < 128 || a.lda >= (1 << 26) || a.ldb >= (1 << 26)) return fail(DAXQ_ERR_ARG, "linear: the 128x128 kernel needs m, n >= 128");
+            return launch_tile256s5<FP8>(a, x_e5m2, false, true, st);
         default: return fail(DAXQ_ERR_ARG, "linear: unknown gemm variant %d", g_variant);
     }
 }
@@ -303,7 +309,7 @@ int daxq_set_gemm_variant(int variant) {
         daxq::g_gm = variant - 1000 > 0 ? variant - 1000 : 4;
         return DAXQ_OK;
     }
-    if (variant != 0 && variant != 2 && variant != 5 && variant != 6 && variant != 8 && variant != 9)
+    if (variant != 0 && variant != 2 && variant != 5 && variant != 6 && variant != 8 && variant != 9 && variant != 11)
         return daxq::fail(DAXQ_ERR_ARG, "unknown gemm variant %d", variant);
     daxq::g_variant = variant;
     return DAXQ_OK;

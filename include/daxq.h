@@ -201,7 +201,8 @@ int daxq_linear_e5m2_e4m3(const uint8_t* xq, int64_t ld_xq, const float* sx,
 
 /* Selects a GEMM kernel for tests and comparisons; every choice computes the same results.
  * 0 = library default (by shape), 2 / 5 = generic 256x256 / 128x128 tiles, 6 = two-stage 256x256 kernel,
- * 8 = five-stage 256x256 kernel, 9 = the same with 32x32x32 INT8 MFMAs; 1000 + d sets the depth d of the
+ * 8 = five-stage 256x256 kernel, 9 = the same with 32x32x32 INT8 MFMAs, 11 = the same on 128x128 tiles;
+ * 1000 + d sets the depth d of the
  * tile-order groups.  Process-wide; not part of the reference interface. */
 int daxq_set_gemm_variant(int variant);
 

@@ -14,12 +14,14 @@ from tests.util import bf16_bits, rel_l2
 
 pytestmark = pytest.mark.gpu
 
-VARIANTS = [0, 2, 5, 6, 8, 9]  # 0 = library default, 2 / 5 = generic kernels, 6 = two-stage 256x256, 8 / 9 = five-stage 256x256 (9: INT8 with 32x32 MFMAs)
+VARIANTS = [0, 2, 5, 6, 8, 9, 11]  # 0 = library default, 2 / 5 = generic kernels, 6 = two-stage 256x256, 8 / 9 = five-stage 256x256 (9: INT8 with 32x32 MFMAs), 11 = five-stage 128x128
 
 
 def _skip_if_too_small(variant, m, n):
     if variant in (6, 8, 9) and (m < 256 or n < 256):
         pytest.skip("the 256x256 kernel needs m, n >= 256")
+    if variant == 11 and (m < 128 or n < 128):
+        pytest.skip("the 128x128 kernel needs m, n >= 128")
 FP8_TOL = 2e-2
 
 
@@ -79,7 +81,7 @@ def _random_shapes(count, seed):
     return shapes
 
 
-@pytest.mark.parametrize("variant", [8, 9, 6])
+@pytest.mark.parametrize("variant", [8, 9, 6, 11])
 @pytest.mark.parametrize("m,n,k,pad_k,pad_n", _random_shapes(14, seed=2024))
 def test_linear_i8_random_shapes_and_strides_bit_exact(ops, variant, m, n, k, pad_k, pad_n):
     """Seeded random M, N, K (edge tiles shifted inwards in both directions, short and long K) with padded leading
@@ -132,7 +134,7 @@ def test_linear_i8_adversarial_extremes(ops, variant):
     np.testing.assert_array_equal(bf16_bits(out), bf16_bits(O.epilogue_int8(want, sx.view(-1, 1), sw.view(1, -1), None)))
 
 
-@pytest.mark.parametrize("variant", [0, 6, 8, 9])
+@pytest.mark.parametrize("variant", [0, 6, 8, 9, 11])
 def test_linear_i8_one_hot_layout(ops, variant):
     # a single non-zero in each operand lands in exactly one accumulator: catches any
     # row/column or operand transposition inside the MFMA tiling
@@ -174,7 +176,7 @@ def test_linear_e4m3_within_tolerance(ops, variant, m, n, k):
     assert r < 3e-3, r                          # what fp32 accumulation actually delivers
 
 
-@pytest.mark.parametrize("variant", [8, 6])
+@pytest.mark.parametrize("variant", [8, 6, 11])
 @pytest.mark.parametrize("e5m2", [False, True])
 @pytest.mark.parametrize("m,n,k,pad_k,pad_n", _random_shapes(8, seed=77))
 def test_linear_fp8_random_shapes_accumulators(ops, variant, e5m2, m, n, k, pad_k, pad_n):
@@ -236,7 +238,7 @@ def test_linear_rejects_unaligned_k(ops):
         ops.linear_i8(xq, torch.ones(8, device="cuda"), wq, torch.ones(8, device="cuda"), None)
 
 
-@pytest.mark.parametrize("variant", [0, 5, 6, 8, 9])
+@pytest.mark.parametrize("variant", [0, 5, 6, 8, 9, 11])
 def test_linear_leading_dimensions_through_the_c_abi(ops, variant):
     """Operands and output as column slices of wider buffers (ld > logical width), straight through the C ABI:
     what a caller does that writes q | k | v into one [M, 3N] tensor with three launches."""
