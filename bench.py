@@ -25,7 +25,7 @@ PEAK_TOPS = {"int8": 5000.0, "fp8": 5000.0}  # MI355X dense 8-bit MFMA peak
 # FETCH_SIZE / WRITE_SIZE passes over this same command, scaled by the 1 GiB copy in the same run
 # (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0): int8 (8403372 + 1456260) KiB, fp8 (8555857 + 1456106) KiB.  Includes
 # Infinity Cache hits.
-GEMM_TRAFFIC_BYTES = {"int8": (8630435 + 1456275) * 1024, "fp8": (8718503 + 1456168) * 1024}
+GEMM_TRAFFIC_BYTES = {"int8": (8704018 + 1456303) * 1024, "fp8": (8801768 + 1456150) * 1024}
 
 
 def cpu_baseline(dtype: str, rows: int):
