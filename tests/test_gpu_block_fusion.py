@@ -97,3 +97,18 @@ def test_unquantised_blocks_are_left_alone():
 
     model = Transformer().to(torch.bfloat16).to("cuda")
     assert fuse_transformer_blocks(model) == 0
+
+
+@pytest.mark.parametrize("fp8", [False, True])
+def test_quantised_transformer_under_torch_compile(fp8):
+    """The reference's deployment: the whole transformer with swapped linears inside torch.compile
+    (dax/adapters/wan/functional.py:33-36).  The code generator re-fuses the fp32 LayerNorm / modulation / attention
+    code around the daxq ops, so the comparison with eager is a tolerance, not bit equality."""
+    pytest.importorskip("triton")
+    model = _model(fp8)
+    x, ctx, t = _inputs(model)
+    with torch.no_grad():
+        ref = model(x, ctx, t)
+        out = torch.compile(model)(x, ctx, t)
+    assert out.shape == ref.shape and out.dtype == ref.dtype
+    assert rel_l2(out, ref) < 2e-2
