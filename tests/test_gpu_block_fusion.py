@@ -99,13 +99,18 @@ def test_unquantised_blocks_are_left_alone():
     assert fuse_transformer_blocks(model) == 0
 
 
+@pytest.mark.parametrize("fused", [False, True])
 @pytest.mark.parametrize("fp8", [False, True])
-def test_quantised_transformer_under_torch_compile(fp8):
+def test_quantised_transformer_under_torch_compile(fp8, fused):
     """The reference's deployment: the whole transformer with swapped linears inside torch.compile
     (dax/adapters/wan/functional.py:33-36).  The code generator re-fuses the fp32 LayerNorm / modulation / attention
     code around the daxq ops, so the comparison with eager is a tolerance, not bit equality."""
     pytest.importorskip("triton")
     model = _model(fp8)
+    if fused:  # the explicit producer + quantiser fusions trace as well
+        from dax_amd.adapters.wan import fuse_transformer_blocks
+
+        fuse_transformer_blocks(model)
     x, ctx, t = _inputs(model)
     with torch.no_grad():
         ref = model(x, ctx, t)
