@@ -421,3 +421,17 @@ def test_module_forward_traces_with_fake_tensors(dtype, k):
             assert qa.xq.shape == (600, (k + 127) // 128 * 128) and qa.sx.shape == (600,) and qa.sx.dtype == torch.float32
             y = lin(torch.empty(2, 300, k, dtype=torch.bfloat16, device="cuda"))
             assert y.shape == (2, 300, 520) and y.dtype == torch.bfloat16 and y.device.type == "cuda"
+
+
+def test_product_never_touches_the_oracle_or_a_cpu_path():
+    """The oracle is test infrastructure: no file of the package names it, and every custom op is registered for
+    the GPU only."""
+    pkg = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "dax_amd")
+    for root, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".h", ".c", ".cpp")):
+                text = open(os.path.join(root, f), errors="ignore").read()
+                assert not re.search(r"\boracle\b", text), f"{os.path.join(root, f)} mentions the oracle"
+    ops_src = open(os.path.join(pkg, "ops.py")).read()
+    decls = [line for line in ops_src.splitlines() if line.startswith("@torch.library.custom_op(")]
+    assert decls and all('device_types="cuda"' in d for d in decls)
