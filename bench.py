@@ -20,15 +20,19 @@ if ROOT not in sys.path:
 
 M_TOKENS = 75600
 SHAPES = [("qkv", 5120, 15360), ("out", 5120, 5120), ("ffn_up", 5120, 13824), ("ffn_down", 13824, 5120)]
+# The other linear set the reference is quoted on (Wan2.1-1.3B at 480p, 21*30*52 tokens): --model 1.3b.  Not the
+# headline workload; its K = N = 1536 linear sits below the MFMA/HBM ridge, so HBM GB/s is reported beside T-op/s.
+MODELS = {"14b": ("Wan2.1-14B 720p", "wan2.1_14b_720p", M_TOKENS, SHAPES),
+          "1.3b": ("Wan2.1-1.3B 480p", "wan2.1_1.3b_480p", 32760,
+                   [("qkv", 1536, 4608), ("out", 1536, 1536), ("ffn_up", 1536, 8960), ("ffn_down", 8960, 1536)])}
 PEAK_TOPS = {"int8": 5000.0, "fp8": 5000.0}  # MI355X dense 8-bit MFMA peak
 # Bytes that left L2 towards the fabric per GEMM launch (average of the four shapes), from the rocprofv3
 # FETCH_SIZE / WRITE_SIZE passes over this same command, scaled by the 1 GiB copy in the same run
-# (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0): int8 (8403372 + 1456260) KiB, fp8 (8555857 + 1456106) KiB.  Includes
-# Infinity Cache hits.
-GEMM_TRAFFIC_BYTES = {"int8": (8704018 + 1456303) * 1024, "fp8": (8801768 + 1456150) * 1024}
+# (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0); KiB read + KiB written below.  Includes Infinity Cache hits.
+GEMM_TRAFFIC_BYTES = {"int8": (8645383 + 1456310) * 1024, "fp8": (8771832 + 1456134) * 1024}
 
 
-def cpu_baseline(dtype: str, rows: int):
+def cpu_baseline(dtype: str, rows: int, shapes=SHAPES, m_tokens=M_TOKENS):
     """The reference's CPU path (oracle: eager quantiser + torch._int_mm / fp32-emulated fp8
     matmul + epilogue) on a bounded sample of `rows` tokens of the same four shapes."""
     import torch
@@ -36,7 +40,7 @@ def cpu_baseline(dtype: str, rows: int):
     from oracle import daxq_oracle as O
 
     ops_done, t_total = 0.0, 0.0
-    for i, (_, k, n) in enumerate(SHAPES):
+    for i, (_, k, n) in enumerate(shapes):
         x, w, b = O.make_inputs(rows, k, n, seed=i)
         if dtype == "int8":
             qw, sw = O.weight_quant_int8(w)
@@ -49,7 +53,7 @@ def cpu_baseline(dtype: str, rows: int):
         t_total += time.perf_counter() - t0
         ops_done += 2.0 * rows * n * k
     return {"value": ops_done / t_total / 1e12, "unit": "TOPS", "cores": torch.get_num_threads(), "kind": "port",
-            "sample": f"first {rows} of {M_TOKENS} tokens of each of the 4 shapes, {t_total:.1f} s, "
+            "sample": f"first {rows} of {m_tokens} tokens of each of the 4 shapes, {t_total:.1f} s, "
                       f"os.cpu_count()={os.cpu_count()}"}
 
 
@@ -80,7 +84,9 @@ def main():
     ap.add_argument("--workload", choices=["block", "model40"], default="block",
                     help="block: the four linears of one DiT block (the headline workload); model40: 40 layers x "
                          "{QKV, out, cross-q, cross-k, cross-v (512 text tokens), FFN up, FFN down} with distinct weights")
-    ap.add_argument("--m", type=int, default=M_TOKENS)
+    ap.add_argument("--model", choices=sorted(MODELS), default="14b",
+                    help="which linear set: 14b (the headline workload) or 1.3b (M = 32760, hidden 1536, FFN 8960)")
+    ap.add_argument("--m", type=int, default=0, help="tokens (0 = the model's own count)")
     ap.add_argument("--cpu-rows", type=int, default=0, help="tokens in the CPU-baseline sample (0 = pick for 10-30 s)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-mfma-ceiling", action="store_true")
@@ -103,20 +109,24 @@ def main():
         _capi.set_gemm_variant(1000 + args.tile_group)
     dev = torch.device("cuda:0")
     fp8 = args.dtype == "fp8"
-    m = args.m
+    model_name, model_tag, m_model, shapes = MODELS[args.model]
+    if args.workload == "model40" and args.model != "14b":
+        sys.exit("bench.py: the 40-layer workload is defined for --model 14b only")
+    m = args.m or m_model
+    hidden, ffn = shapes[0][1], shapes[3][1]
 
     # ---- synthetic inputs, resident in HBM
     g = torch.Generator(device="cpu").manual_seed(0)
     layers = []
     xs = {}
-    for k in (5120, 13824):
+    for k in (hidden, ffn):
         x = torch.randn(m, k, device=dev, dtype=torch.bfloat16)
         idx = torch.randperm(k, generator=g)[: max(1, round(0.01 * k))].to(dev)
         x[:, idx] *= 20
         xs[k] = x
     text = torch.randn(512, 5120, device=dev, dtype=torch.bfloat16)
     if args.workload == "block":
-        plan = [(name, k, n, xs[k]) for name, k, n in SHAPES]
+        plan = [(name, k, n, xs[k]) for name, k, n in shapes]
     else:
         one = [("qkv", 5120, 15360, xs[5120]), ("out", 5120, 5120, xs[5120]), ("cross_q", 5120, 5120, xs[5120]),
                ("cross_k", 5120, 5120, text), ("cross_v", 5120, 5120, text), ("ffn_up", 5120, 13824, xs[5120]),
@@ -182,13 +192,16 @@ def main():
         rows, k, n, cnt = e["rows"], e["k"], e["n"], e["launches"]
         e["gemm_tops"] = round(cnt * 2.0 * rows * n * k / (e["gemm_ms"] * 1e-3) / 1e12, 1)
         e["quant_gbps"] = round(cnt * (3.0 * rows * k + 4.0 * rows) / (e["quant_ms"] * 1e-3) / 1e9, 1)
+        # algorithmic bytes of the GEMM launch: both operands, scales, bias, the bf16 output
+        e["gemm_gbps"] = round(cnt * (rows * k + 4.0 * rows + n * k + 6.0 * n + 2.0 * rows * n)
+                               / (e["gemm_ms"] * 1e-3) / 1e9, 1)
         e["quant_ms"], e["gemm_ms"] = round(e["quant_ms"], 4), round(e["gemm_ms"], 4)
     achieved = total_ops / (gemm_ms_sum * 1e-3) / 1e12
     peak = PEAK_TOPS[args.dtype]
 
     info = _capi.device_info(0)
     res = {
-        "metric": f"w8a8_linear_tops_wan2.1_14b_720p_{args.dtype}" + ("" if args.workload == "block" else "_40_layers"),
+        "metric": f"w8a8_linear_tops_{model_tag}_{args.dtype}" + ("" if args.workload == "block" else "_40_layers"),
         "value": round(value, 2),
         "unit": "TOPS",
         "n_gpus": 1,
@@ -200,8 +213,8 @@ def main():
         "vs_baseline": None,
         "dtype": "int8" if not fp8 else "fp8_e4m3fn",
         "data": "synthetic",
-        "config": {"workload": (f"Wan2.1-14B 720p linear set, {args.dtype.upper()} W8A8, M={m} tokens: "
-                                "QKV 5120->15360, out 5120->5120, FFN 5120->13824, FFN 13824->5120; "
+        "config": {"workload": (f"{model_name} linear set, {args.dtype.upper()} W8A8, M={m} tokens: "
+                                + ", ".join(f"{nm} {k}->{n}" for nm, k, n in shapes) + "; "
                                 "per linear: per-token act quant + MFMA GEMM + fused scale/bias/bf16 epilogue")
                    if args.workload == "block" else
                    (f"Wan2.1-14B 720p, 40 layers x (QKV 5120->15360, out, cross-q 5120->5120 at M={m}; cross-k, cross-v "
@@ -210,7 +223,7 @@ def main():
                    "gemm_variant": args.variant},
         "pct_of_mfma_peak": round(100.0 * value / peak, 2),
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": peak, "unit": "TFLOP/s",
-                     "frac": round(achieved / peak, 4), "traffic": GEMM_TRAFFIC_BYTES[args.dtype] if (m == M_TOKENS and args.workload == "block") else None,
+                     "frac": round(achieved / peak, 4), "traffic": GEMM_TRAFFIC_BYTES[args.dtype] if (m == M_TOKENS and args.workload == "block" and args.model == "14b") else None,
                      "kernel": "gemm_tile256s5_kernel, average launch over the four shapes; 8-bit ops counted as 2*M*N*K"
                      if args.workload == "block" else "all GEMM launches of the step (the 512-token ones run gemm_w8a8_kernel)",
                      "gemm_ms_per_step": round(gemm_ms_sum, 4), "quant_ms_per_step": round(quant_ms_sum, 4)},
@@ -230,13 +243,13 @@ def main():
         return a.elapsed_time(b2) / reps
 
     fmt = "e4m3" if fp8 else "i8"
-    mul = 1 + 0.1 * torch.randn(1, 5120, device=dev)
-    add = 0.1 * torch.randn(1, 5120, device=dev)
-    ln_ms = timed(lambda: getattr(ops, "layernorm_act_quant_" + fmt)(xs[5120], mul, add, m, 1e-6))
-    ge_ms = timed(lambda: getattr(ops, "gelu_tanh_act_quant_" + fmt)(xs[13824]))
+    mul = 1 + 0.1 * torch.randn(1, hidden, device=dev)
+    add = 0.1 * torch.randn(1, hidden, device=dev)
+    ln_ms = timed(lambda: getattr(ops, "layernorm_act_quant_" + fmt)(xs[hidden], mul, add, m, 1e-6))
+    ge_ms = timed(lambda: getattr(ops, "gelu_tanh_act_quant_" + fmt)(xs[ffn]))
     res["fused_producers"] = {
-        "layernorm_modulate_quant_k5120": {"ms": round(ln_ms, 4), "gbps": round(3.0 * m * 5120 / (ln_ms * 1e-3) / 1e9, 1)},
-        "gelu_tanh_quant_k13824": {"ms": round(ge_ms, 4), "gbps": round(3.0 * m * 13824 / (ge_ms * 1e-3) / 1e9, 1)},
+        f"layernorm_modulate_quant_k{hidden}": {"ms": round(ln_ms, 4), "gbps": round(3.0 * m * hidden / (ln_ms * 1e-3) / 1e9, 1)},
+        f"gelu_tanh_quant_k{ffn}": {"ms": round(ge_ms, 4), "gbps": round(3.0 * m * ffn / (ge_ms * 1e-3) / 1e9, 1)},
         "hbm_peak_gbps": 8000.0}
     if not args.no_mfma_ceiling:
         sus = mfma_sustained(args.dtype)
@@ -248,7 +261,7 @@ def main():
                 "gemm_frac_of_workload_ceiling": round(achieved / sus["workload"], 4)}
     if not args.no_cpu_baseline:
         rows = args.cpu_rows or (49152 if not fp8 else 24576)
-        res["cpu_baseline"] = cpu_baseline(args.dtype, min(rows, m))
+        res["cpu_baseline"] = cpu_baseline(args.dtype, min(rows, m), shapes, m)
     print(json.dumps(res), flush=True)
 
 

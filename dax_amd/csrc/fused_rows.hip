@@ -36,6 +36,15 @@ __device__ __forceinline__ uint4 pack8(const float (&f)[8]) {
                       pack_bf16_rne(f[6], f[7]));
 }
 
+// The row stays packed (bf16 pairs) between the passes over it.  Without this the compiler keeps the unpacked
+// fp32 copies of one pass alive for the next one, three times the registers, and the kernel loses half of its
+// wavefronts per SIMD.
+template <int N>
+__device__ __forceinline__ void forget_values(uint4 (&v)[N]) {
+#pragma unroll
+    for (int i = 0; i < N; ++i) asm volatile("" : "+v"(v[i].x), "+v"(v[i].y), "+v"(v[i].z), "+v"(v[i].w));
+}
+
 // gelu(x, approximate="tanh") = 0.5 x (1 + tanh(u)), u = sqrt(2/pi) (x + 0.044715 x^3), evaluated as
 // x / (1 + exp(-2u)): the same function without the cancellation in 1 + tanh(u) for negative x.
 __device__ __forceinline__ float gelu_tanh_f32(float x) {
@@ -52,17 +61,36 @@ __device__ __forceinline__ float gelu_tanh_f32(float x) {
 //         vectors of the workgroup's current group are staged in LDS (mul / add may be null: 1 / 0).
 // PRE_GELU: y = bf16( gelu_tanh(x) ).
 // Requires k % 8 == 0, 16-byte aligned rows of x (and y), 8-byte aligned rows of q, ld_q/8 <= NCH*64.
+// The quantise-only LayerNorm form for rows of up to 12 x 64 chunks holds two rows (the current and the requested
+// next one) and is kept at three wavefronts per SIMD (170 registers).
 template <int NCH, int FMT, int PRE, bool WRITE_Y>
-__global__ __launch_bounds__(256) void fused_rows_wave(const uint16_t* __restrict__ x, int64_t m, int k, int64_t ld_x,
-                                                       const float* __restrict__ mul, const float* __restrict__ add,
-                                                       int64_t rows_per_group, float eps, uint16_t* __restrict__ y,
-                                                       int64_t ld_y, uint8_t* __restrict__ q, int64_t ld_q,
-                                                       float* __restrict__ scale, float qmax) {
-    extern __shared__ __attribute__((aligned(16))) float s_vec[];  // PRE_LN: mul[k] then add[k]
+__global__ __launch_bounds__(256, (PRE == PRE_LN && NCH <= 12 && !WRITE_Y) ? 3 : 1) void fused_rows_wave(
+    const uint16_t* __restrict__ x, int64_t m, int k, int64_t ld_x, const float* __restrict__ mul,
+    const float* __restrict__ add, int64_t rows_per_group, float eps, uint16_t* __restrict__ y, int64_t ld_y,
+    uint8_t* __restrict__ q, int64_t ld_q, float* __restrict__ scale, float qmax) {
+    // PRE_LN: mul then add, each in the order the lanes read them: per 64 chunks of 8 elements, the first halves of
+    // the 64 chunks, then the second halves, so that one 16-byte read per lane covers 1 KB without a gap (the plain
+    // order makes the lanes read 16 bytes every 32 and half of the banks collide)
+    extern __shared__ __attribute__((aligned(16))) float s_vec[];
+    const int kpad = ((k + 511) >> 9) << 9;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int nch = k >> 3;
     const int npad = (int)(ld_q >> 3);
     int64_t staged = -1;
+    // The resident LayerNorm form requests the wavefront's next row before it works on the current one.
+    constexpr bool AHEAD = PRE == PRE_LN && NCH <= 12;
+    auto load_row = [&](int64_t r, uint4 (&dst)[NCH]) {
+        const uint4* xr = reinterpret_cast<const uint4*>(x + r * ld_x);
+#pragma unroll
+        for (int i = 0; i < NCH; ++i) {
+            const int c = i * 64 + lane;
+            dst[i] = c < nch ? load_stream_16(xr + c) : make_uint4(0, 0, 0, 0);
+        }
+    };
+    uint4 v[NCH], nv[AHEAD ? NCH : 1];
+    if constexpr (AHEAD) {
+        if ((int64_t)blockIdx.x * 4 + wave < m) load_row((int64_t)blockIdx.x * 4 + wave, v);
+    }
 
     for (int64_t row0 = (int64_t)blockIdx.x * 4; row0 < m; row0 += (int64_t)gridDim.x * 4) {
         const int64_t row = row0 + wave;
@@ -72,9 +100,11 @@ __global__ __launch_bounds__(256) void fused_rows_wave(const uint16_t* __restric
             const int64_t g0 = row0 / rows_per_group;
             if (g0 != staged) {
                 __syncthreads();  // everyone is done with the previous group's vectors
-                for (int c = threadIdx.x; c < k; c += 256) {
-                    s_vec[c] = mul ? mul[g0 * k + c] : 1.0f;
-                    s_vec[k + c] = add ? add[g0 * k + c] : 0.0f;
+                for (int e = threadIdx.x; e < k; e += 256) {
+                    const int c = e >> 3;
+                    const int pos = (((((c >> 6) << 1) + ((e >> 2) & 1)) * 64 + (c & 63)) << 2) | (e & 3);
+                    s_vec[pos] = mul ? mul[g0 * k + e] : 1.0f;
+                    s_vec[kpad + pos] = add ? add[g0 * k + e] : 0.0f;
                 }
                 staged = g0;
                 __syncthreads();
@@ -82,12 +112,11 @@ __global__ __launch_bounds__(256) void fused_rows_wave(const uint16_t* __restric
         }
         if (row >= m) continue;
 
-        const uint4* xr = reinterpret_cast<const uint4*>(x + row * ld_x);
-        uint4 v[NCH];
-#pragma unroll
-        for (int i = 0; i < NCH; ++i) {
-            const int c = i * 64 + lane;
-            v[i] = c < nch ? load_stream_16(xr + c) : make_uint4(0, 0, 0, 0);
+        if constexpr (AHEAD) {
+            const int64_t next = row + (int64_t)gridDim.x * 4;
+            if (next < m) load_row(next, nv);
+        } else {
+            load_row(row, v);
         }
 
         if constexpr (PRE == PRE_LN) {
@@ -100,6 +129,7 @@ __global__ __launch_bounds__(256) void fused_rows_wave(const uint16_t* __restric
                 sum += ((f[0] + f[1]) + (f[2] + f[3])) + ((f[4] + f[5]) + (f[6] + f[7]));
             }
             const float mean = wave_sum_f32(sum) / (float)k;
+            forget_values(v);
             float ssq = 0.0f;
 #pragma unroll
             for (int i = 0; i < NCH; ++i) {
@@ -114,6 +144,7 @@ __global__ __launch_bounds__(256) void fused_rows_wave(const uint16_t* __restric
                 }
             }
             const float var = wave_sum_f32(ssq) / (float)k;
+            forget_values(v);
             const float rstd = 1.0f / sqrtf(var + eps);  // IEEE sqrt and division
             const int64_t g = row / rows_per_group;
             const bool in_lds = g == staged;
@@ -124,10 +155,11 @@ __global__ __launch_bounds__(256) void fused_rows_wave(const uint16_t* __restric
                     float f[8], a[8], b[8];
                     unpack8(v[i], f);
                     if (in_lds) {
-                        const float4 a0 = *reinterpret_cast<const float4*>(s_vec + c * 8);
-                        const float4 a1 = *reinterpret_cast<const float4*>(s_vec + c * 8 + 4);
-                        const float4 b0 = *reinterpret_cast<const float4*>(s_vec + k + c * 8);
-                        const float4 b1 = *reinterpret_cast<const float4*>(s_vec + k + c * 8 + 4);
+                        const float* sv = s_vec + (i * 128 + lane) * 4;
+                        const float4 a0 = *reinterpret_cast<const float4*>(sv);
+                        const float4 a1 = *reinterpret_cast<const float4*>(sv + 256);
+                        const float4 b0 = *reinterpret_cast<const float4*>(sv + kpad);
+                        const float4 b1 = *reinterpret_cast<const float4*>(sv + kpad + 256);
                         a[0] = a0.x, a[1] = a0.y, a[2] = a0.z, a[3] = a0.w, a[4] = a1.x, a[5] = a1.y, a[6] = a1.z, a[7] = a1.w;
                         b[0] = b0.x, b[1] = b0.y, b[2] = b0.z, b[3] = b0.w, b[4] = b1.x, b[5] = b1.y, b[6] = b1.z, b[7] = b1.w;
                     } else {
@@ -187,6 +219,10 @@ __global__ __launch_bounds__(256) void fused_rows_wave(const uint16_t* __restric
                 store_stream_8(qr + c, make_uint2(0, 0));
             }
         }
+        if constexpr (AHEAD) {
+#pragma unroll
+            for (int i = 0; i < NCH; ++i) v[i] = nv[i];
+        }
     }
 }
 
@@ -218,7 +254,7 @@ static int launch_fused_rows(const char* what, const void* x, int64_t m, int64_t
     // number against 0.355 / 0.49 ms with twice / half as many) -- so that the staged vectors are reused over
     // many rows; the GELU form has nothing to reuse and takes one quad of rows per workgroup
     const int64_t quads = (m + 3) / 4;
-    const size_t lds = PRE == PRE_LN ? (size_t)k * 8 : 0;
+    const size_t lds = PRE == PRE_LN ? (size_t)((k + 511) / 512) * 512 * 8 : 0;  // two vectors, padded to whole 64-chunk groups
     const dim3 block(256);
 #define DAXQ_F_CASE(N)                                                                                                   \
     if (nchunks <= N) {                                                                                                  \
