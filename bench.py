@@ -6,7 +6,8 @@ per linear, the per-token activation quantiser and the MFMA GEMM with the fused 
 Inputs (bf16 activations, pre-quantised weights, scales, bias) are resident in HBM before the
 timed region.  Prints one JSON line.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--dtype int8|fp8] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--dtype int8|fp8|fp8_e5m2] [--model 14b|1.3b]
+                    [--workload block|model40] [--no-cpu-baseline]
 """
 import argparse
 import json
@@ -25,7 +26,7 @@ SHAPES = [("qkv", 5120, 15360), ("out", 5120, 5120), ("ffn_up", 5120, 13824), ("
 MODELS = {"14b": ("Wan2.1-14B 720p", "wan2.1_14b_720p", M_TOKENS, SHAPES),
           "1.3b": ("Wan2.1-1.3B 480p", "wan2.1_1.3b_480p", 32760,
                    [("qkv", 1536, 4608), ("out", 1536, 1536), ("ffn_up", 1536, 8960), ("ffn_down", 8960, 1536)])}
-PEAK_TOPS = {"int8": 5000.0, "fp8": 5000.0}  # MI355X dense 8-bit MFMA peak
+PEAK_TOPS = {"int8": 5000.0, "fp8": 5000.0, "fp8_e5m2": 5000.0}  # MI355X dense 8-bit MFMA peak
 # Bytes that left L2 towards the fabric per GEMM launch (average of the four shapes), from the rocprofv3
 # FETCH_SIZE / WRITE_SIZE passes over this same command, scaled by the 1 GiB copy in the same run
 # (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0); KiB read + KiB written below.  Includes Infinity Cache hits.
@@ -49,7 +50,7 @@ def cpu_baseline(dtype: str, rows: int, shapes=SHAPES, m_tokens=M_TOKENS):
         else:
             qw, sw = O.weight_quant_e4m3(w)
             t0 = time.perf_counter()
-            O.linear_e4m3(x, qw, sw, b)
+            O.linear_e4m3(x, qw, sw, b, **({"act_dtype": torch.float8_e5m2} if dtype == "fp8_e5m2" else {}))
         t_total += time.perf_counter() - t0
         ops_done += 2.0 * rows * n * k
     return {"value": ops_done / t_total / 1e12, "unit": "TOPS", "cores": torch.get_num_threads(), "kind": "port",
@@ -78,7 +79,9 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--dtype", choices=["int8", "fp8"], default="int8")
+    ap.add_argument("--dtype", choices=["int8", "fp8", "fp8_e5m2"], default="int8",
+                    help="fp8: e4m3fn activations and weights (the quoted FP8 configuration); fp8_e5m2: e5m2 activations "
+                         "against e4m3fn weights, the default of the reference's FP8 qconfig factory")
     ap.add_argument("--variant", type=int, default=0)
     ap.add_argument("--tile-group", type=int, default=0, help="tile-order group depth (0 = library default)")
     ap.add_argument("--workload", choices=["block", "model40"], default="block",
@@ -108,7 +111,8 @@ def main():
     if args.tile_group:
         _capi.set_gemm_variant(1000 + args.tile_group)
     dev = torch.device("cuda:0")
-    fp8 = args.dtype == "fp8"
+    fp8 = args.dtype != "int8"
+    e5m2 = args.dtype == "fp8_e5m2"
     model_name, model_tag, m_model, shapes = MODELS[args.model]
     if args.workload == "model40" and args.model != "14b":
         sys.exit("bench.py: the 40-layer workload is defined for --model 14b only")
@@ -140,8 +144,8 @@ def main():
         qw = (ops.quantize_rows_e4m3 if fp8 else ops.quantize_rows_i8)(w, sw, True)
         layers.append((name, k, n, x, qw, sw, b))
         del w
-    act_quant = ops.act_quant_e4m3 if fp8 else ops.act_quant_i8
-    linear = ops.linear_e4m3 if fp8 else ops.linear_i8
+    act_quant = ops.act_quant_e5m2 if e5m2 else ops.act_quant_e4m3 if fp8 else ops.act_quant_i8
+    linear = ops.linear_e5m2_e4m3 if e5m2 else ops.linear_e4m3 if fp8 else ops.linear_i8
 
     def step(ev=None):
         for li, (name, k, n, x, qw, sw, b) in enumerate(layers):
@@ -211,7 +215,7 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "int8" if not fp8 else "fp8_e4m3fn",
+        "dtype": "int8" if not fp8 else "fp8_e5m2_x_e4m3fn" if e5m2 else "fp8_e4m3fn",
         "data": "synthetic",
         "config": {"workload": (f"{model_name} linear set, {args.dtype.upper()} W8A8, M={m} tokens: "
                                 + ", ".join(f"{nm} {k}->{n}" for nm, k, n in shapes) + "; "
@@ -223,7 +227,7 @@ def main():
                    "gemm_variant": args.variant},
         "pct_of_mfma_peak": round(100.0 * value / peak, 2),
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": peak, "unit": "TFLOP/s",
-                     "frac": round(achieved / peak, 4), "traffic": GEMM_TRAFFIC_BYTES[args.dtype] if (m == M_TOKENS and args.workload == "block" and args.model == "14b") else None,
+                     "frac": round(achieved / peak, 4), "traffic": GEMM_TRAFFIC_BYTES.get(args.dtype) if (m == M_TOKENS and args.workload == "block" and args.model == "14b") else None,
                      "kernel": "gemm_tile256s5_kernel, average launch over the four shapes; 8-bit ops counted as 2*M*N*K"
                      if args.workload == "block" else "all GEMM launches of the step (the 512-token ones run gemm_w8a8_kernel)",
                      "gemm_ms_per_step": round(gemm_ms_sum, 4), "quant_ms_per_step": round(quant_ms_sum, 4)},
@@ -242,7 +246,7 @@ def main():
         torch.cuda.synchronize()
         return a.elapsed_time(b2) / reps
 
-    fmt = "e4m3" if fp8 else "i8"
+    fmt = "e5m2" if e5m2 else "e4m3" if fp8 else "i8"
     mul = 1 + 0.1 * torch.randn(1, hidden, device=dev)
     add = 0.1 * torch.randn(1, hidden, device=dev)
     ln_ms = timed(lambda: getattr(ops, "layernorm_act_quant_" + fmt)(xs[hidden], mul, add, m, 1e-6))
