@@ -25,7 +25,9 @@ SHAPES = [("qkv", 5120, 15360), ("out", 5120, 5120), ("ffn_up", 5120, 13824), ("
 # headline workload; its K = N = 1536 linear sits below the MFMA/HBM ridge, so HBM GB/s is reported beside T-op/s.
 MODELS = {"14b": ("Wan2.1-14B 720p", "wan2.1_14b_720p", M_TOKENS, SHAPES),
           "1.3b": ("Wan2.1-1.3B 480p", "wan2.1_1.3b_480p", 32760,
-                   [("qkv", 1536, 4608), ("out", 1536, 1536), ("ffn_up", 1536, 8960), ("ffn_down", 8960, 1536)])}
+                   [("qkv", 1536, 4608), ("out", 1536, 1536), ("ffn_up", 1536, 8960), ("ffn_down", 8960, 1536)]),
+          # the single linear the reference's CPU path is quoted on
+          "config0": ("single linear 4096 x 1536 -> 1536", "single_4096x1536x1536", 4096, [("linear", 1536, 1536)])}
 PEAK_TOPS = {"int8": 5000.0, "fp8": 5000.0, "fp8_e5m2": 5000.0}  # MI355X dense 8-bit MFMA peak
 # Bytes that left L2 towards the fabric per GEMM launch (average of the four shapes), from the rocprofv3
 # FETCH_SIZE / WRITE_SIZE passes over this same command, scaled by the 1 GiB copy in the same run
@@ -54,7 +56,7 @@ def cpu_baseline(dtype: str, rows: int, shapes=SHAPES, m_tokens=M_TOKENS):
         t_total += time.perf_counter() - t0
         ops_done += 2.0 * rows * n * k
     return {"value": ops_done / t_total / 1e12, "unit": "TOPS", "cores": torch.get_num_threads(), "kind": "port",
-            "sample": f"first {rows} of {m_tokens} tokens of each of the 4 shapes, {t_total:.1f} s, "
+            "sample": f"first {rows} of {m_tokens} tokens of each of the {len(shapes)} shapes, {t_total:.1f} s, "
                       f"os.cpu_count()={os.cpu_count()}"}
 
 
@@ -88,7 +90,8 @@ def main():
                     help="block: the four linears of one DiT block (the headline workload); model40: 40 layers x "
                          "{QKV, out, cross-q, cross-k, cross-v (512 text tokens), FFN up, FFN down} with distinct weights")
     ap.add_argument("--model", choices=sorted(MODELS), default="14b",
-                    help="which linear set: 14b (the headline workload) or 1.3b (M = 32760, hidden 1536, FFN 8960)")
+                    help="which linear set: 14b (the headline workload), 1.3b (M = 32760, hidden 1536, FFN 8960) or "
+                         "config0 (one linear, M = 4096, K = N = 1536)")
     ap.add_argument("--m", type=int, default=0, help="tokens (0 = the model's own count)")
     ap.add_argument("--cpu-rows", type=int, default=0, help="tokens in the CPU-baseline sample (0 = pick for 10-30 s)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -117,13 +120,13 @@ def main():
     if args.workload == "model40" and args.model != "14b":
         sys.exit("bench.py: the 40-layer workload is defined for --model 14b only")
     m = args.m or m_model
-    hidden, ffn = shapes[0][1], shapes[3][1]
+    hidden, ffn = shapes[0][1], shapes[-1][1]
 
     # ---- synthetic inputs, resident in HBM
     g = torch.Generator(device="cpu").manual_seed(0)
     layers = []
     xs = {}
-    for k in (hidden, ffn):
+    for k in sorted({hidden, ffn}):
         x = torch.randn(m, k, device=dev, dtype=torch.bfloat16)
         idx = torch.randperm(k, generator=g)[: max(1, round(0.01 * k))].to(dev)
         x[:, idx] *= 20
@@ -228,7 +231,7 @@ def main():
         "pct_of_mfma_peak": round(100.0 * value / peak, 2),
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": peak, "unit": "TFLOP/s",
                      "frac": round(achieved / peak, 4), "traffic": GEMM_TRAFFIC_BYTES.get(args.dtype) if (m == M_TOKENS and args.workload == "block" and args.model == "14b") else None,
-                     "kernel": "gemm_tile256s5_kernel, average launch over the four shapes; 8-bit ops counted as 2*M*N*K"
+                     "kernel": f"gemm_tile256s5_kernel, average launch over the {len(shapes)} shape(s); 8-bit ops counted as 2*M*N*K"
                      if args.workload == "block" else "all GEMM launches of the step (the 512-token ones run gemm_w8a8_kernel)",
                      "gemm_ms_per_step": round(gemm_ms_sum, 4), "quant_ms_per_step": round(quant_ms_sum, 4)},
         "per_linear": per_layer,
