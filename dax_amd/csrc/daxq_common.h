@@ -19,6 +19,11 @@ constexpr float kEps = 1.1920928955078125e-07f;  // 2^-23 = torch.finfo(float32)
 
 __device__ __forceinline__ float bf16_bits_to_f32(uint32_t b) { return __uint_as_float(b << 16); }
 
+// max / min that give NaN when either operand is NaN, like torch.max / torch.min / torch.clamp on tensors
+// (fmaxf and fminf drop a NaN operand, which would turn a poisoned row into finite garbage)
+__device__ __forceinline__ float max_nan(float a, float b) { return (a != a || a > b) ? a : b; }
+__device__ __forceinline__ float min_nan(float a, float b) { return (a != a || a < b) ? a : b; }
+
 // f32 -> bf16 bits, round to nearest even (finite inputs)
 __device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
     uint32_t u = __float_as_uint(f);

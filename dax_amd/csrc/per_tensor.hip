@@ -20,8 +20,8 @@ constexpr int kRedThreads = 1024;
 __device__ __forceinline__ void block_minmax(float& lo, float& hi, float* s_lo, float* s_hi) {
 #pragma unroll
     for (int off = 32; off >= 1; off >>= 1) {
-        lo = fminf(lo, __shfl_xor(lo, off, 64));
-        hi = fmaxf(hi, __shfl_xor(hi, off, 64));
+        lo = min_nan(lo, __shfl_xor(lo, off, 64));
+        hi = max_nan(hi, __shfl_xor(hi, off, 64));
     }
     const int wave = threadIdx.x >> 6;
     if ((threadIdx.x & 63) == 0) {
@@ -32,8 +32,8 @@ __device__ __forceinline__ void block_minmax(float& lo, float& hi, float* s_lo, 
     lo = s_lo[0];
     hi = s_hi[0];
     for (int w = 1; w < kRedThreads / 64; ++w) {
-        lo = fminf(lo, s_lo[w]);
-        hi = fmaxf(hi, s_hi[w]);
+        lo = min_nan(lo, s_lo[w]);
+        hi = max_nan(hi, s_hi[w]);
     }
 }
 
@@ -44,14 +44,14 @@ __global__ __launch_bounds__(kRedThreads) void tensor_scale_kernel(const float* 
     __shared__ float s_lo[kRedThreads / 64], s_hi[kRedThreads / 64];
     float lo = __builtin_inff(), hi = -__builtin_inff();
     for (int64_t i = threadIdx.x; i < m; i += kRedThreads) {
-        lo = fminf(lo, mn[i]);
-        hi = fmaxf(hi, mx[i]);
+        lo = min_nan(lo, mn[i]);
+        hi = max_nan(hi, mx[i]);
     }
     block_minmax(lo, hi, s_lo, s_hi);
-    const float amax = fmaxf(-lo, hi);  // = max |x|: exact, the inputs are bf16 values
+    const float amax = max_nan(-lo, hi);  // = max |x|: exact, the inputs are bf16 values
     float s = amax / qmax;              // IEEE division
     if (round_bf16) s = bf16_bits_to_f32(f32_to_bf16_bits(s));
-    s = fmaxf(s, kEps);
+    s = max_nan(s, kEps);
     if (threadIdx.x == 0) scale1[0] = s;
     for (int64_t i = threadIdx.x; i < n_expand; i += kRedThreads) expand[i] = s;
 }
@@ -62,13 +62,13 @@ __global__ __launch_bounds__(kRedThreads) void tensor_minmax_kernel(const float*
     __shared__ float s_lo[kRedThreads / 64], s_hi[kRedThreads / 64];
     float lo = __builtin_inff(), hi = -__builtin_inff();
     for (int64_t i = threadIdx.x; i < m; i += kRedThreads) {
-        lo = fminf(lo, mn[i]);
-        hi = fmaxf(hi, mx[i]);
+        lo = min_nan(lo, mn[i]);
+        hi = max_nan(hi, mx[i]);
     }
     block_minmax(lo, hi, s_lo, s_hi);
     if (threadIdx.x == 0) {
-        min_inout[0] = fminf(min_inout[0], lo);
-        max_inout[0] = fmaxf(max_inout[0], hi);
+        min_inout[0] = min_nan(min_inout[0], lo);
+        max_inout[0] = max_nan(max_inout[0], hi);
     }
 }
 

@@ -21,7 +21,7 @@ __device__ __forceinline__ float scale_from_amax_bits(uint32_t amax_bits, float 
     float a = bf16_bits_to_f32(amax_bits);
     float s = a / qmax;  // IEEE binary32 division (hipcc default: correctly rounded)
     if (ROUND_BF16) s = bf16_bits_to_f32(f32_to_bf16_bits(s));
-    return fmaxf(s, kEps);
+    return max_nan(s, kEps);  // clamp(min=eps): a NaN abs-max (a NaN anywhere in the row) stays NaN
 }
 
 // Wavefront-wide reductions with DPP (data-parallel primitives: the partner lane's value is an operand
@@ -89,6 +89,9 @@ __device__ __forceinline__ float q_f8_pre(float x, float s, float inv) {
         const float e = __builtin_fmaf(-q0, s, x);
         v = __builtin_copysignf(__builtin_fmaf(e, inv, q0), x);  // s > 0; keeps -0 for x = -0 (0 + -0 is +0 in the fma)
     }
+    // With a scale from the caller a NaN element must stay NaN through the clamp, as in the reference, and become
+    // the format's NaN byte; with the row's own scale a NaN element has already made that scale NaN.
+    if constexpr (TRUE_DIV) return min_nan(max_nan(v, -kMax), kMax);
     return fminf(fmaxf(v, -kMax), kMax);
 }
 

@@ -163,13 +163,13 @@ __global__ __launch_bounds__(256) void row_minmax_kernel(const uint16_t* __restr
     float lo = __builtin_inff(), hi = -__builtin_inff();
     for (int64_t c = threadIdx.x; c < k; c += 256) {
         float f = bf16_bits_to_f32(xr[c]);
-        lo = fminf(lo, f);
-        hi = fmaxf(hi, f);
+        lo = min_nan(lo, f);
+        hi = max_nan(hi, f);
     }
 #pragma unroll
     for (int off = 32; off >= 1; off >>= 1) {
-        lo = fminf(lo, __shfl_xor(lo, off, 64));
-        hi = fmaxf(hi, __shfl_xor(hi, off, 64));
+        lo = min_nan(lo, __shfl_xor(lo, off, 64));
+        hi = max_nan(hi, __shfl_xor(hi, off, 64));
     }
     if ((threadIdx.x & 63) == 0) {
         rlo[threadIdx.x >> 6] = lo;
@@ -177,8 +177,8 @@ __global__ __launch_bounds__(256) void row_minmax_kernel(const uint16_t* __restr
     }
     __syncthreads();
     if (threadIdx.x == 0) {
-        mn[row] = fminf(fminf(rlo[0], rlo[1]), fminf(rlo[2], rlo[3]));
-        mx[row] = fmaxf(fmaxf(rhi[0], rhi[1]), fmaxf(rhi[2], rhi[3]));
+        mn[row] = min_nan(min_nan(rlo[0], rlo[1]), min_nan(rlo[2], rlo[3]));
+        mx[row] = max_nan(max_nan(rhi[0], rhi[1]), max_nan(rhi[2], rhi[3]));
     }
 }
 
@@ -187,8 +187,8 @@ __global__ void scale_from_minmax_kernel(const float* __restrict__ mn, const flo
                                          float qmax, float* __restrict__ scale) {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n) {
-        const float a = fmaxf(-mn[i], mx[i]);
-        scale[i] = fmaxf(a / qmax, kEps);
+        const float a = max_nan(-mn[i], mx[i]);
+        scale[i] = max_nan(a / qmax, kEps);
     }
 }
 
