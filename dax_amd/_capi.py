@@ -24,6 +24,7 @@ SIGNATURES = {
     "daxq_abi_version": [],
     "daxq_last_error": [],
     "daxq_device_info": [_INT, C.POINTER(_INT), C.POINTER(_INT), C.POINTER(_INT), C.c_char_p, _INT],
+    "daxq_init": [],
     "daxq_act_quant_i8": [_P, _I64, _I64, _I64, _P, _I64, _P, _P],
     "daxq_act_quant_e4m3": [_P, _I64, _I64, _I64, _P, _I64, _P, _P],
     "daxq_act_quant_e5m2": [_P, _I64, _I64, _I64, _P, _I64, _P, _P],
@@ -92,12 +93,17 @@ def device_info(device: int = 0) -> dict:
 
 
 def require_gfx950(device: int) -> None:
-    """Raises unless `device` is a gfx950 (checked once per device)."""
+    """Raises unless `device` is a gfx950 (checked once per device); on the first check the library's kernels are
+    prepared on that device (daxq_init), so that even the first op call may sit inside a stream capture."""
     if device in _checked_devices:
         return
     info = device_info(device)
     if info["status"] != 0:
         raise RuntimeError(f"daxq needs an MI355X (gfx950) device: {last_error()}")
+    import torch
+
+    with torch.cuda.device(device):
+        check(lib().daxq_init(), "daxq_init")
     _checked_devices.add(device)
 
 

@@ -521,12 +521,18 @@ __global__ __launch_bounds__(256) void gemm_tile256_kernel(const GemmArgs p) {
                                 p.bias ? bf16_bits_to_f32(p.bias[n0 + t]) : -0.0f);
 }
 
+// raises the kernel's dynamic LDS limit on the current device (once per device)
+template <bool FP8, bool DUMP, bool XE5 = false>
+static int prepare_tile256() {
+    static uint64_t lds_set = 0;  // per instantiation
+    return ensure_dynamic_lds(reinterpret_cast<const void*>(gemm_tile256_kernel<FP8, DUMP, XE5>), t256::SMEM, lds_set);
+}
+
 template <bool FP8, bool DUMP, bool XE5 = false>
 static int launch_tile256_impl(const GemmArgs& a, hipStream_t st) {
     using namespace t256;
     auto kern = gemm_tile256_kernel<FP8, DUMP, XE5>;
-    static uint64_t lds_set = 0;  // per instantiation
-    if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), SMEM, lds_set)) return rc;
+    if (int rc = prepare_tile256<FP8, DUMP, XE5>()) return rc;
     const int64_t nt = (int64_t)a.tiles_m * a.tiles_n;
     if (nt > 0x7fffffff) return fail(DAXQ_ERR_ARG, "gemm: too many tiles");
     hipLaunchKernelGGL(kern, dim3((unsigned)nt), dim3(T), SMEM, st, a);
@@ -857,12 +863,18 @@ __global__ __launch_bounds__(256) void gemm_tile256s5_kernel(const GemmArgs p) {
 }
 
 template <bool FP8, bool DUMP, bool XE5, bool N16 = false, int BT = 256>
+static int prepare_tile256s5() {
+    static uint64_t lds_set = 0;  // per instantiation
+    return ensure_dynamic_lds(reinterpret_cast<const void*>(gemm_tile256s5_kernel<FP8, DUMP, XE5, N16, BT>),
+                              t5::NST * 2 * BT * t5::BKS, lds_set);
+}
+
+template <bool FP8, bool DUMP, bool XE5, bool N16 = false, int BT = 256>
 static int launch_tile256s5_impl(const GemmArgs& a, hipStream_t st) {
     using namespace t5;
     constexpr int SMEM = NST * 2 * BT * BKS;  // 160 KB (256 tile), 80 KB (128 tile)
     auto kern = gemm_tile256s5_kernel<FP8, DUMP, XE5, N16, BT>;
-    static uint64_t lds_set = 0;  // per instantiation
-    if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), SMEM, lds_set)) return rc;
+    if (int rc = prepare_tile256s5<FP8, DUMP, XE5, N16, BT>()) return rc;
     const int64_t nt = (int64_t)a.tiles_m * a.tiles_n;
     if (nt > 0x7fffffff) return fail(DAXQ_ERR_ARG, "gemm: too many tiles");
     hipLaunchKernelGGL(kern, dim3((unsigned)nt), dim3(T), SMEM, st, a);
@@ -893,6 +905,35 @@ int launch_tile256s5(const GemmArgs& a0, bool x_e5m2, bool wide, bool small, hip
 
 template int launch_tile256s5<false>(const GemmArgs&, bool, bool, bool, hipStream_t);
 template int launch_tile256s5<true>(const GemmArgs&, bool, bool, bool, hipStream_t);
+
+// Every instantiation the launchers above can pick, prepared on the current device: afterwards no launch changes a
+// kernel attribute any more, so the first launch may already sit inside a stream capture.
+int prepare_tile256_kernels() {
+    int rc = 0;
+#define DAXQ_PREP(...) if (!rc) rc = __VA_ARGS__()
+    DAXQ_PREP(prepare_tile256<false, false>);
+    DAXQ_PREP(prepare_tile256<false, true>);
+    DAXQ_PREP(prepare_tile256<true, false>);
+    DAXQ_PREP(prepare_tile256<true, true>);
+    DAXQ_PREP(prepare_tile256<true, false, true>);
+    DAXQ_PREP(prepare_tile256<true, true, true>);
+    DAXQ_PREP(prepare_tile256s5<false, false, false, true, 256>);
+    DAXQ_PREP(prepare_tile256s5<false, true, false, true, 256>);
+    DAXQ_PREP(prepare_tile256s5<false, false, false, false, 256>);
+    DAXQ_PREP(prepare_tile256s5<false, true, false, false, 256>);
+    DAXQ_PREP(prepare_tile256s5<false, false, false, true, 128>);
+    DAXQ_PREP(prepare_tile256s5<false, true, false, true, 128>);
+    DAXQ_PREP(prepare_tile256s5<true, false, false, false, 256>);
+    DAXQ_PREP(prepare_tile256s5<true, true, false, false, 256>);
+    DAXQ_PREP(prepare_tile256s5<true, false, true, false, 256>);
+    DAXQ_PREP(prepare_tile256s5<true, true, true, false, 256>);
+    DAXQ_PREP(prepare_tile256s5<true, false, false, false, 128>);
+    DAXQ_PREP(prepare_tile256s5<true, true, false, false, 128>);
+    DAXQ_PREP(prepare_tile256s5<true, false, true, false, 128>);
+    DAXQ_PREP(prepare_tile256s5<true, true, true, false, 128>);
+#undef DAXQ_PREP
+    return rc;
+}
 
 // the kernel applies: both dimensions hold a whole tile and the 32-bit row offsets cannot overflow
 bool tile256_applies(const GemmArgs& a) {

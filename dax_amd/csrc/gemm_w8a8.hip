@@ -217,6 +217,15 @@ bool tile256_applies(const GemmArgs& a);
 template <bool FP8>
 int launch_tile256s5(const GemmArgs& a, bool x_e5m2, bool wide, bool small, hipStream_t st);
 
+int prepare_tile256_kernels();
+
+template <bool FP8, int BM, int BN, int BK, int WM, int WN, bool DIRECT, bool XE5 = false>
+static int prepare_cfg() {
+    static uint64_t lds_set = 0;  // per instantiation
+    return ensure_dynamic_lds(reinterpret_cast<const void*>(gemm_w8a8_kernel<FP8, BM, BN, BK, WM, WN, DIRECT, XE5>),
+                              2 * (BM + BN) * BK, lds_set);
+}
+
 template <bool FP8, int BM, int BN, int BK, int WM, int WN, bool DIRECT, bool XE5 = false>
 static int launch_cfg(const GemmArgs& a0, hipStream_t st) {
     GemmArgs a = a0;
@@ -224,8 +233,7 @@ static int launch_cfg(const GemmArgs& a0, hipStream_t st) {
     a.tiles_n = (a.n + BN - 1) / BN;
     constexpr int smem = 2 * (BM + BN) * BK;
     auto kern = gemm_w8a8_kernel<FP8, BM, BN, BK, WM, WN, DIRECT, XE5>;
-    static uint64_t lds_set = 0;  // per instantiation
-    if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), smem, lds_set)) return rc;
+    if (int rc = prepare_cfg<FP8, BM, BN, BK, WM, WN, DIRECT, XE5>()) return rc;
     const int64_t nt = (int64_t)a.tiles_m * a.tiles_n;
     if (nt > 0x7fffffff) return fail(DAXQ_ERR_ARG, "gemm: too many tiles");
     hipLaunchKernelGGL(kern, dim3((unsigned)nt), dim3(WM * WN * 64), smem, st, a);
@@ -303,6 +311,17 @@ static int launch_gemm(const void* xq, int64_t ld_xq, const float* sx, const voi
 }  // namespace daxq
 
 extern "C" {
+
+int daxq_init(void) {
+    using namespace daxq;
+    int rc = prepare_tile256_kernels();
+    if (!rc) rc = prepare_cfg<false, 128, 128, 128, 2, 2, true>();
+    if (!rc) rc = prepare_cfg<true, 128, 128, 128, 2, 2, true>();
+    if (!rc) rc = prepare_cfg<true, 128, 128, 128, 2, 2, true, true>();
+    if (!rc) rc = prepare_cfg<false, 256, 256, 128, 2, 4, true>();
+    if (!rc) rc = prepare_cfg<true, 256, 256, 128, 2, 4, true>();
+    return rc;
+}
 
 int daxq_set_gemm_variant(int variant) {
     if (variant >= 1000 && variant < 1064) {  // tuning hook: 1000 + depth of the tile-order groups

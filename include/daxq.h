@@ -46,6 +46,12 @@ const char* daxq_last_error(void);
  * Replaces the CUDA-version guards of dax/quant/nn/dynamic/linear.py:44-57. */
 int daxq_device_info(int device, int* cu_count, int* clock_khz, int* lds_bytes, char* arch, int arch_len);
 
+/* Optional set-up for the current HIP device: raises the dynamic LDS limit of every GEMM kernel now instead of at a
+ * kernel's first launch (a kernel attribute cannot be changed while a stream is being captured, so without this call
+ * the first launch of each kernel has to happen outside a capture).  Idempotent, cheap after the first call, launches
+ * nothing.  No counterpart in the reference, whose kernels come from torch. */
+int daxq_init(void);
+
 /*
  * Dynamic per-token symmetric activation quantisation, INT8.
  * Replaces dynamic_quantize_to_int8 / _dynamic_quantize_func / quantize_to_int8

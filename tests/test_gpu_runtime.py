@@ -121,3 +121,44 @@ def test_captured_graph_replays_match_eager(fp8):
         graph.replay()
         torch.cuda.synchronize()
         assert _same(static_out, eager), f"replay with seed {seed} differs from eager"
+
+
+_FIRST_LAUNCH_IN_CAPTURE = r"""
+import sys
+import torch
+from torch import nn
+sys.path.insert(0, sys.argv[1])
+from dax_amd.quant.quantization import quantize_dynamic
+from dax_amd.quant.quantization.qconfig import (get_dynamic_fp8_per_token_act_per_channel_weight_qconfig,
+                                                get_dynamic_int8_per_token_act_per_channel_weight_qconfig)
+for fp8 in (False, True):
+    torch.manual_seed(0)
+    model = nn.Sequential(nn.Linear(640, 1024), nn.GELU(approximate="tanh"), nn.Linear(1024, 640)).bfloat16().cuda()
+    cfg = (get_dynamic_fp8_per_token_act_per_channel_weight_qconfig(activation_dtype=torch.float8_e4m3fn)
+           if fp8 else get_dynamic_int8_per_token_act_per_channel_weight_qconfig())
+    quantize_dynamic(model, {"": cfg})
+    x = torch.randn(2, 520, 640, device="cuda").bfloat16()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):      # no forward has run yet in this process
+        y = model(x)
+    graph.replay()
+    torch.cuda.synchronize()
+    captured = y.clone()
+    eager = model(x)
+    torch.cuda.synchronize()
+    assert torch.equal(captured.view(torch.int16), eager.view(torch.int16)), "fp8" if fp8 else "int8"
+print("first-launch-in-capture ok")
+"""
+
+
+def test_first_forward_of_a_process_inside_a_capture():
+    """The library prepares its kernels (daxq_init) when a device is first used, so nothing has to be launched
+    before a capture: a fresh process captures its very first forward and the replay equals eager."""
+    import os
+    import subprocess
+    import sys
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, "-c", _FIRST_LAUNCH_IN_CAPTURE, root], capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0 and "first-launch-in-capture ok" in r.stdout, r.stdout[-2000:] + r.stderr[-2000:]
