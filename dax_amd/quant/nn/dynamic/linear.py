@@ -164,6 +164,8 @@ class Linear(nn.Module):
         """Dynamic quantisation of ``input`` [..., K] in this module's activation dtype and scheme
         (:204-208, :146-150): one scale per token, or one for the whole tensor written out per token."""
         flat = input.view(-1, self.in_features)
+        if flat.stride(-1) != 1:  # a view with strided columns: the reference's torch ops take it, the kernels want rows
+            flat = flat.contiguous()
         if self.input_qscheme == per_token_symmetric:
             xq, sx = getattr(ops, _ACT_QUANT[self.input_dtype])(flat)
         else:

@@ -328,6 +328,33 @@ def test_quantize_dynamic_int8_module_matches_oracle(home):
     np.testing.assert_array_equal(bf16_bits(z.view(-1, 64)), bf16_bits(h))
 
 
+def test_module_takes_the_input_shapes_of_nn_linear():
+    """[..., K] -> [..., N] for any leading shape the reference's view(-1, K) accepts (dynamic/linear.py:181-183,
+    :224-226): no token at all, a single vector, several leading dimensions, a view with strided columns."""
+    from dax_amd.quant.quantization import quantize_dynamic
+    from dax_amd.quant.quantization.qconfig import get_dynamic_int8_per_token_act_per_channel_weight_qconfig as cfg
+
+    model = _toy(4).to("cuda")
+    w, b = model.to_q.weight.detach().cpu().clone(), model.to_q.bias.detach().cpu().clone()
+    quantize_dynamic(model, {"": cfg(), "proj_out": None})
+    qw, sw = O.weight_quant_int8(w)
+    lin = model.to_q
+    for shape in [(0, 256), (2, 0, 256), (256,), (1, 256), (2, 3, 5, 256)]:
+        g = torch.Generator("cpu").manual_seed(len(shape))
+        x = torch.randn(*shape, generator=g).bfloat16()
+        y = lin(x.to("cuda"))
+        assert y.shape == shape[:-1] + (256,) and y.dtype == torch.bfloat16
+        if x.numel():
+            ref = O.linear_int8(x.reshape(-1, 256), qw, sw, b)["out"]
+            np.testing.assert_array_equal(bf16_bits(y.reshape(-1, 256)), bf16_bits(ref))
+    wide = torch.randn(10, 512, generator=torch.Generator("cpu").manual_seed(9)).bfloat16()
+    y = lin(wide.to("cuda")[:, ::2])                      # every second column: a view, not contiguous rows
+    ref = O.linear_int8(wide[:, ::2].contiguous(), qw, sw, b)["out"]
+    np.testing.assert_array_equal(bf16_bits(y), bf16_bits(ref))
+    with pytest.raises(RuntimeError):                      # not flattenable by view: the reference raises as well
+        lin(torch.randn(2, 5, 256, device="cuda").bfloat16().transpose(0, 1))
+
+
 def test_quantize_dynamic_fp8_module_matches_oracle():
     from dax_amd.quant.nn.dynamic import Linear as QLinear
     from dax_amd.quant.quantization import quantize_dynamic
