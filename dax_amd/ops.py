@@ -26,8 +26,32 @@ def is_tracing(t: torch.Tensor) -> bool:
     return torch.compiler.is_compiling() or isinstance(t, FakeTensor)
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream(t: torch.Tensor) -> int:
+    """The HIP stream that is current for the tensor's device, as an integer handle."""
+    idx = t.device.index
+    if _raw_stream is not None and idx is not None:
+        return _raw_stream(idx)  # the same handle without building a Stream object (a tenth of the host time)
     return torch.cuda.current_stream(t.device).cuda_stream
+
+
+class _NoGuard:
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *exc):
+        return False
+
+
+_NO_GUARD = _NoGuard()
+
+
+def _on_device(t: torch.Tensor):
+    """Context that makes the tensor's device current for the allocations and the launch; with a single GPU it is
+    current already and the guard (several microseconds per call) is left out."""
+    return torch.cuda.device(t.device) if torch.cuda.device_count() > 1 else _NO_GUARD
 
 
 def _need_gpu(t: torch.Tensor, what: str) -> None:
@@ -52,7 +76,7 @@ def _act_quant(x: torch.Tensor, fp8, e5m2: bool = False) -> Tuple[torch.Tensor, 
     _rows_bf16(x, name)
     m, k = x.shape
     kp = pad_k(k)
-    with torch.cuda.device(x.device):
+    with _on_device(x):
         q = torch.empty((m, kp), dtype=torch.uint8 if fp8 else torch.int8, device=x.device)
         s = torch.empty((m,), dtype=torch.float32, device=x.device)
         if m:
@@ -116,7 +140,7 @@ def _layernorm_act_quant(fmt: str, x, mul, add, rows_per_group: int, eps: float,
     if rows_per_group <= 0:
         raise ValueError(f"daxq::{name}: rows_per_group must be positive")
     groups = max(1, -(-m // rows_per_group))
-    with torch.cuda.device(x.device):
+    with _on_device(x):
         q, s, y = _fused_out(x, fmt, want_y)
         if m:
             fn = getattr(_capi.lib(), "daxq_" + name)
@@ -131,7 +155,7 @@ def _gelu_tanh_act_quant(fmt: str, x, want_y: bool):
     name = "gelu_tanh_act_quant_" + fmt
     _rows_bf16(x, name)
     m, k = x.shape
-    with torch.cuda.device(x.device):
+    with _on_device(x):
         q, s, y = _fused_out(x, fmt, want_y)
         if m:
             fn = getattr(_capi.lib(), "daxq_" + name)
@@ -203,7 +227,7 @@ def _quantize_rows(x: torch.Tensor, scale: torch.Tensor, fmt: str, padded: bool)
         raise ValueError(f"daxq::{name}: scale must be fp32 with one value per row on {x.device}")
     scale = scale.reshape(-1).contiguous()
     ld_q = pad_k(k) if padded else k
-    with torch.cuda.device(x.device):
+    with _on_device(x):
         q = torch.empty((m, ld_q), dtype=torch.int8 if fmt == "i8" else torch.uint8, device=x.device)
         if m:
             fn = getattr(_capi.lib(), "daxq_" + name)
@@ -241,7 +265,7 @@ def row_minmax(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
     """Per-row (min, max) of a bf16 matrix in fp32."""
     _rows_bf16(x, "row_minmax")
     m, k = x.shape
-    with torch.cuda.device(x.device):
+    with _on_device(x):
         lo = torch.empty((m,), dtype=torch.float32, device=x.device)
         hi = torch.empty((m,), dtype=torch.float32, device=x.device)
         if m:
@@ -262,7 +286,7 @@ def scale_from_minmax(min_val: torch.Tensor, max_val: torch.Tensor, qmax: float)
     if min_val.dtype != torch.float32 or max_val.dtype != torch.float32 or min_val.shape != max_val.shape:
         raise ValueError("daxq::scale_from_minmax: min/max must be fp32 tensors of one shape")
     lo, hi = min_val.contiguous(), max_val.contiguous()
-    with torch.cuda.device(lo.device):
+    with _on_device(lo):
         s = torch.empty_like(lo)
         _capi.check(_capi.lib().daxq_scale_from_minmax(lo.data_ptr(), hi.data_ptr(), lo.numel(), float(qmax),
                                                        s.data_ptr(), _stream(lo)), "scale_from_minmax")
@@ -291,7 +315,7 @@ def _linear(xq, sx, wq, sw, bias, fp8: bool, want_acc: bool, x_e5m2: bool = Fals
     sx = sx.reshape(-1).contiguous()
     sw = sw.reshape(-1).contiguous()
     bias_c = bias.contiguous() if bias is not None else None
-    with torch.cuda.device(xq.device):
+    with _on_device(xq):
         out = torch.empty((m, n), dtype=torch.bfloat16, device=xq.device)
         acc = torch.empty((m, n), dtype=torch.float32 if fp8 else torch.int32, device=xq.device) if want_acc else None
         if m and n:
@@ -359,6 +383,42 @@ linear_e4m3_acc.register_fake(lambda xq, sx, wq, sw, bias: (
     _lin_fake(xq, sx, wq, sw, bias), xq.new_empty((xq.shape[0], wq.shape[0]), dtype=torch.float32)))
 
 
+# ----------------------------------------------------------------------------- quantiser + GEMM behind one dispatch
+def _dynamic_linear(x, wq, sw, bias, fmt: str):
+    """Per-token quantiser and GEMM of one linear, the same two launches as act_quant_* + linear_*; one op call
+    instead of two halves the host time per forward, which is what a small linear costs."""
+    fp8 = fmt != "i8"
+    xq, sx = _act_quant(x, fp8, fmt == "e5m2")
+    if xq.shape[1] != wq.shape[1]:
+        raise ValueError(f"daxq::dynamic_linear_{fmt}: x has K={x.shape[1]} (padded {xq.shape[1]}), the weight {wq.shape[1]}")
+    return _linear(xq, sx, wq, sw, bias, fp8, False, fmt == "e5m2")[0]
+
+
+@torch.library.custom_op("daxq::dynamic_linear_i8", mutates_args=(), device_types="cuda")
+def dynamic_linear_i8(x: torch.Tensor, wq: torch.Tensor, sw: torch.Tensor, bias: Optional[torch.Tensor]) -> torch.Tensor:
+    """bf16 [M,K] -> per-token int8 -> x int8 [N, pad128(K)]^T with the fused epilogue -> bf16 [M,N]."""
+    return _dynamic_linear(x, wq, sw, bias, "i8")
+
+
+@torch.library.custom_op("daxq::dynamic_linear_e4m3", mutates_args=(), device_types="cuda")
+def dynamic_linear_e4m3(x: torch.Tensor, wq: torch.Tensor, sw: torch.Tensor, bias: Optional[torch.Tensor]) -> torch.Tensor:
+    return _dynamic_linear(x, wq, sw, bias, "e4m3")
+
+
+@torch.library.custom_op("daxq::dynamic_linear_e5m2_e4m3", mutates_args=(), device_types="cuda")
+def dynamic_linear_e5m2_e4m3(x: torch.Tensor, wq: torch.Tensor, sw: torch.Tensor, bias: Optional[torch.Tensor]) -> torch.Tensor:
+    return _dynamic_linear(x, wq, sw, bias, "e5m2")
+
+
+def _dyn_fake(x, wq, sw, bias):
+    return x.new_empty((x.shape[0], wq.shape[0]), dtype=torch.bfloat16)
+
+
+dynamic_linear_i8.register_fake(_dyn_fake)
+dynamic_linear_e4m3.register_fake(_dyn_fake)
+dynamic_linear_e5m2_e4m3.register_fake(_dyn_fake)
+
+
 # ----------------------------------------------------------------------------- per-tensor scales
 @torch.library.custom_op("daxq::tensor_scale", mutates_args=(), device_types="cuda")
 def tensor_scale(row_min: torch.Tensor, row_max: torch.Tensor, qmax: float, round_bf16: bool,
@@ -368,7 +428,7 @@ def tensor_scale(row_min: torch.Tensor, row_max: torch.Tensor, qmax: float, roun
     if row_min.dtype != torch.float32 or row_max.dtype != torch.float32 or row_min.shape != row_max.shape or row_min.numel() == 0:
         raise ValueError("daxq::tensor_scale: row_min / row_max must be non-empty fp32 tensors of one shape")
     lo, hi = row_min.contiguous(), row_max.contiguous()
-    with torch.cuda.device(lo.device):
+    with _on_device(lo):
         s1 = torch.empty((1,), dtype=torch.float32, device=lo.device)
         ex = torch.empty((n_expand,), dtype=torch.float32, device=lo.device)
         _capi.check(_capi.lib().daxq_tensor_scale(lo.data_ptr(), hi.data_ptr(), lo.numel(), float(qmax), int(round_bf16),
@@ -391,7 +451,7 @@ def tensor_minmax_update(row_min: torch.Tensor, row_max: torch.Tensor, min_inout
             raise ValueError("daxq::tensor_minmax_update: contiguous fp32 tensors on one device expected")
     if min_inout.numel() != 1 or max_inout.numel() != 1 or row_min.numel() == 0 or row_min.numel() != row_max.numel():
         raise ValueError("daxq::tensor_minmax_update: bad shapes")
-    with torch.cuda.device(row_min.device):
+    with _on_device(row_min):
         _capi.check(_capi.lib().daxq_tensor_minmax_update(row_min.data_ptr(), row_max.data_ptr(), row_min.numel(),
                                                           min_inout.data_ptr(), max_inout.data_ptr(), _stream(row_min)),
                     "tensor_minmax_update")
@@ -406,7 +466,7 @@ def broadcast_f32(src: torch.Tensor, n: int) -> torch.Tensor:
     _need_gpu(src, "broadcast_f32")
     if src.dtype != torch.float32 or src.numel() != 1:
         raise ValueError("daxq::broadcast_f32: src must hold one fp32 value")
-    with torch.cuda.device(src.device):
+    with _on_device(src):
         dst = torch.empty((n,), dtype=torch.float32, device=src.device)
         _capi.check(_capi.lib().daxq_broadcast_f32(src.data_ptr(), dst.data_ptr(), n, _stream(src)), "broadcast_f32")
     return dst

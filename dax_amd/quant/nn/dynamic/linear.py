@@ -49,6 +49,8 @@ class QuantizedActivation:
 
 
 _ACT_QUANT = {torch.int8: "act_quant_i8", torch.float8_e4m3fn: "act_quant_e4m3", torch.float8_e5m2: "act_quant_e5m2"}
+_DYNAMIC_LINEAR = {torch.int8: "dynamic_linear_i8", torch.float8_e4m3fn: "dynamic_linear_e4m3",
+                   torch.float8_e5m2: "dynamic_linear_e5m2_e4m3"}
 
 
 class Linear(nn.Module):
@@ -178,6 +180,15 @@ class Linear(nn.Module):
         return QuantizedActivation(xq, sx, input.shape[:-1], self.in_features, self.input_dtype)
 
     def forward(self, input) -> Tensor:
+        if not isinstance(input, QuantizedActivation) and self.input_qscheme == per_token_symmetric:
+            # the common case: quantiser and GEMM behind one op call
+            flat = input.view(-1, self.in_features)
+            if flat.stride(-1) != 1:
+                flat = flat.contiguous()
+            bias = None if self.bias is None else self.bias.detach()
+            out = getattr(ops, _DYNAMIC_LINEAR[self.input_dtype])(flat, self._gemm_weight(), self._weight_scale_vector(), bias)
+            out = out.view(*input.shape[:-1], self.out_features)
+            return out if out.dtype == self.out_dtype else out.to(self.out_dtype)
         qa = input if isinstance(input, QuantizedActivation) else self.quantize_activation(input)
         if qa.dtype != self.input_dtype or qa.in_features != self.in_features:
             raise ValueError(f"quantised activation ({qa.dtype}, K={qa.in_features}) does not fit this linear "
