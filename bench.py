@@ -32,7 +32,7 @@ PEAK_TOPS = {"int8": 5000.0, "fp8": 5000.0, "fp8_e5m2": 5000.0}  # MI355X dense 
 # Bytes that left L2 towards the fabric per GEMM launch (average of the four shapes), from the rocprofv3
 # FETCH_SIZE / WRITE_SIZE passes over this same command, scaled by the 1 GiB copy in the same run
 # (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0); KiB read + KiB written below.  Includes Infinity Cache hits.
-GEMM_TRAFFIC_BYTES = {"int8": (8645383 + 1456310) * 1024, "fp8": (8771832 + 1456134) * 1024}
+GEMM_TRAFFIC_BYTES = {"int8": (8609732 + 1456238) * 1024, "fp8": (8771425 + 1456117) * 1024}
 
 
 def cpu_baseline(dtype: str, rows: int, shapes=SHAPES, m_tokens=M_TOKENS):
