@@ -57,6 +57,21 @@ def test_traced_graph_matches_eager(fp8, k, backend):
 
 
 @pytest.mark.parametrize("fp8", [False, True])
+def test_compiled_with_graph_replay_matches_eager(fp8):
+    """torch.compile(mode="reduce-overhead"): the generated code and the daxq ops are captured into a HIP graph by
+    the compiler's runtime and replayed from the third call on; every call equals eager."""
+    pytest.importorskip("triton")
+    model = _mlp(384, 520, fp8, seed=12)
+    compiled = torch.compile(model, mode="reduce-overhead", fullgraph=True)
+    for seed in (13, 14, 15, 16, 17):
+        x = _input(300, 384, seed=seed)
+        ref = model(x)
+        out = compiled(x).clone()   # the replayed graph owns its output buffer
+        torch.cuda.synchronize()
+        assert _same(out, ref), f"call with seed {seed} differs from eager"
+
+
+@pytest.mark.parametrize("fp8", [False, True])
 def test_side_stream_runs_beside_a_busy_default_stream(fp8):
     """The kernels go to the stream that is current for the input's device, not to the default one: the
     result is ready while a long spin kernel still holds the default stream."""
