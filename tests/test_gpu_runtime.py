@@ -177,3 +177,10 @@ def test_first_forward_of_a_process_inside_a_capture():
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
     r = subprocess.run([sys.executable, "-c", _FIRST_LAUNCH_IN_CAPTURE, root], capture_output=True, text=True, timeout=300)
     assert r.returncode == 0 and "first-launch-in-capture ok" in r.stdout, r.stdout[-2000:] + r.stderr[-2000:]
+
+
+def test_init_is_idempotent():
+    from dax_amd import _capi
+
+    for _ in range(3):
+        assert _capi.lib().daxq_init() == 0, _capi.last_error()
