@@ -14,6 +14,14 @@ from tests.util import bf16_bits
 pytestmark = pytest.mark.gpu
 
 
+@pytest.fixture(autouse=True)
+def _fresh_compiler_cache():
+    """Every test here compiles the same Sequential.forward code object for another module; the compiler keeps at
+    most eight specialisations per code object and refuses the ninth under fullgraph=True."""
+    torch._dynamo.reset()
+    yield
+
+
 def _mlp(k, n, fp8, seed):
     from dax_amd.quant.quantization import quantize_dynamic
     from dax_amd.quant.quantization.qconfig import (get_dynamic_fp8_per_token_act_per_channel_weight_qconfig,
