@@ -30,10 +30,20 @@ How each function is pinned (see tests/test_oracle_*.py):
                            stated in the tests); gelu checked on every bf16 input
 * act_scale_per_tensor /   reduce to the per-row functions above on the tensor flattened
   weight_scale_per_tensor  to one row (tests/test_oracle_pins.py)
-* linear_fp8               accumulation order is not fixed by the reference
-                           (cuBLASLt fast-accum): "parity unpinned" at bit
-                           level, tolerance 2e-2 relative L2; the per-tensor
-                           special case is checked against torch._scaled_mm CPU
+* linear_fp8 /             float64 evaluation from the decoded bytes with one final rounding
+  static_linear_fp8 /      (tests/test_oracle_pins.py: all four e4m3fn / e5m2 operand pairs, per-row and
+  scaled_mm_fp32           per-column scales, a bias as large as the outputs): at most one bf16 step
+                           apart on < 1 % of the outputs, which a dropped bias, a second rounding or
+                           the other format's decoding all break; uniform scales reduce to the library
+                           routine torch._scaled_mm on CPU, called on the oracle's own operands.  The
+                           summation order of the reference's GPU matmul (cuBLASLt fast-accum) is not
+                           fixed, so GPU comparisons against it use the 2e-2 relative-L2 tolerance
+* dynamic_quantize         every block of every scheme equals the per-row rule on the block flattened
+                           to one row (brute force over blocks); fp16 scales exhaustive over every
+                           finite fp16 abs-max against numpy; fp32 / fp16 inputs against numpy fp32
+                           arithmetic and the C fp8 encoders
+* linear_int8_float_       float64 matmul on the bf16 de-quantised weight (tolerance: the float
+  fallback                 matmul's summation order is the library's)
 """
 
 from __future__ import annotations
@@ -113,6 +123,45 @@ def act_quant_e5m2(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
     return quantize_to_fp8(x2, s, torch.float8_e5m2), s
 
 
+def get_reduction_params(block_size, input_size):
+    """View shape and reduced dims of a block scheme.  dax/quant/nn/dynamic/functional.py:13-51: a dim that is
+    split into several blocks becomes (n_blocks, block) with the second reduced; a dim the block spans is
+    reduced in place; block 1 keeps the dim."""
+    assert len(block_size) == len(input_size)
+    view, dims = [], []
+    for blk, size in zip(block_size, input_size):
+        if blk != size and blk > 1:
+            assert size % blk == 0
+            view += [size // blk, blk]
+            dims.append(len(view) - 1)
+        else:
+            view.append(size)
+            if blk != 1:
+                dims.append(len(view) - 1)
+    return view, dims
+
+
+def dynamic_quantize(x: torch.Tensor, block_size, target_dtype: torch.dtype) -> Tuple[torch.Tensor, torch.Tensor]:
+    """``_dynamic_quantize_func`` for any block shape and any of the input dtypes it accepts (fp32 / fp16 / bf16),
+    as its two wrappers call it (quant_max of the target dtype, eps = float32 eps, fp32 scales).
+    dax/quant/nn/dynamic/functional.py:54-148, :152-206.  Returns (values in x's shape, scales with every
+    reduced dim kept as 1, in the view shape of get_reduction_params)."""
+    qmax = INT8_QMAX if target_dtype == torch.int8 else torch.finfo(target_dtype).max
+    view, dims = get_reduction_params(tuple(block_size), tuple(x.shape))
+    xv = x.view(view)  # :121
+    amax = xv.abs().amax(dim=dims, keepdim=False) if dims else xv.abs()  # :124
+    scale = torch.clamp(amax / float(qmax), min=EPS)  # :126-127, in x's dtype
+    if scale.dtype != torch.float32:  # :128-129
+        scale = scale.to(torch.float32)
+    after = list(view)
+    for i in dims:  # :131-135
+        after[i] = 1
+    scale = scale.view(after)
+    if target_dtype == torch.int8:  # :137-148
+        return quantize_to_int8(xv, scale).view(x.shape), scale
+    return quantize_to_fp8(xv, scale, target_dtype).view(x.shape), scale
+
+
 # --------------------------------------------------------------------------- #
 # weight quantisation (per output channel, one time)
 # --------------------------------------------------------------------------- #
@@ -135,10 +184,14 @@ def weight_quant_int8(w: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
     return quantize_to_int8(w, s.view(-1, 1)), s.view(1, -1)
 
 
+def weight_quant_fp8(w: torch.Tensor, dtype: torch.dtype = torch.float8_e4m3fn) -> Tuple[torch.Tensor, torch.Tensor]:
+    """dax/quant/nn/dynamic/linear.py:276-299 with the fp8 leaf quantiser (either of FP8_ALLOWED_DTYPES)."""
+    s = weight_scale(w, torch.finfo(dtype).max)
+    return quantize_to_fp8(w, s.view(-1, 1), dtype), s.view(1, -1)
+
+
 def weight_quant_e4m3(w: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
-    """dax/quant/nn/dynamic/linear.py:276-299 with the fp8 leaf quantiser."""
-    s = weight_scale(w, E4M3_QMAX)
-    return quantize_to_fp8(w, s.view(-1, 1)), s.view(1, -1)
+    return weight_quant_fp8(w, torch.float8_e4m3fn)
 
 
 def dequant_weight(qweight: torch.Tensor, wscale: torch.Tensor, out_dtype=torch.bfloat16) -> torch.Tensor:
@@ -200,31 +253,76 @@ def linear_int8(x: torch.Tensor, qweight: torch.Tensor, wscale: torch.Tensor,
     return res
 
 
+def scaled_mm_fp32(xq: torch.Tensor, qweight: torch.Tensor, scale_a: torch.Tensor, scale_b: torch.Tensor,
+                   bias: Optional[torch.Tensor], out_dtype: torch.dtype, row_chunk: int = 8192) -> torch.Tensor:
+    """``torch._scaled_mm(xq, qweight.T, scale_a, scale_b, bias, out_dtype)`` restated in fp32.
+
+    dax/quant/nn/dynamic/linear.py:155-173 and dax/quant/nn/quantized/linear.py:105-113 call it with
+    row-wise scales ([M,1] x [1,N], CUDA only) or per-tensor scales (one element each, the case the CPU
+    routine implements).  Semantics: out_dtype( (sum_k a*b in fp32) * scale_a * scale_b + bias ), one
+    rounding.  The summation order of the reference (cuBLASLt, use_fast_accum=True) is not specified.
+    """
+    wf = qweight.to(torch.float32)
+    sa = scale_a.to(torch.float32).reshape(-1, 1)
+    sb = scale_b.to(torch.float32).reshape(1, -1)
+    outs = []
+    for r0 in range(0, xq.shape[0], row_chunk):
+        acc = xq[r0:r0 + row_chunk].to(torch.float32) @ wf.t()
+        o = acc * (sa[r0:r0 + row_chunk] if sa.shape[0] > 1 else sa) * sb
+        if bias is not None:
+            o = o + bias.to(torch.float32)
+        outs.append(o.to(out_dtype))
+    return torch.cat(outs, 0)
+
+
+def linear_fp8(x: torch.Tensor, qweight: torch.Tensor, wscale: torch.Tensor, bias: Optional[torch.Tensor],
+               act_dtype: torch.dtype = torch.float8_e4m3fn, per_tensor: bool = False,
+               out_dtype: Optional[torch.dtype] = None, row_chunk: int = 8192) -> Dict[str, torch.Tensor]:
+    """Whole FP8 forward of the dynamic module.  dax/quant/nn/dynamic/linear.py:145-178.
+
+    ``qweight`` is float8_e4m3fn or float8_e5m2 [N,K]; ``act_dtype`` the activation format (the FP8 qconfig's
+    default is float8_e5m2, qconfig.py:85-87).  per-token + per-channel: scale_a [M,1], scale_b [1,N], the matmul
+    writes bf16 with a bf16 bias (:111-116, :166-170) and the result is cast to the module's out_dtype afterwards
+    (:177-178).  per-tensor + per-tensor: one-element scales and the matmul writes out_dtype directly.
+    ``out_dtype`` defaults to x's dtype (the module takes it from the float weight, :263).
+    """
+    out_dtype = out_dtype or x.dtype
+    prev = x.shape[:-1]
+    x2 = x.reshape(-1, x.shape[-1])
+    qmax = torch.finfo(act_dtype).max
+    if per_tensor:
+        sx = act_scale_per_tensor(x2, qmax)
+        mm_dtype = out_dtype
+    else:
+        sx = act_scale(x2, qmax)
+        mm_dtype = torch.bfloat16
+    xq = quantize_to_fp8(x2, sx, act_dtype)
+    out = scaled_mm_fp32(xq, qweight, sx, wscale, None if bias is None else bias.to(mm_dtype), mm_dtype, row_chunk)
+    if out.dtype != out_dtype:
+        out = out.to(out_dtype)
+    return {"xq": xq, "sx": sx, "out": out.view(*prev, qweight.shape[0])}
+
+
 def linear_e4m3(x: torch.Tensor, qweight: torch.Tensor, wscale: torch.Tensor,
                 bias: Optional[torch.Tensor], row_chunk: int = 8192,
                 act_dtype: torch.dtype = torch.float8_e4m3fn) -> Dict[str, torch.Tensor]:
-    """Whole FP8 forward.  dax/quant/nn/dynamic/linear.py:145-178.
+    """The per-token / per-channel FP8 forward of a bf16 module (the benchmark's FP8 configuration)."""
+    return linear_fp8(x, qweight, wscale, bias, act_dtype=act_dtype, row_chunk=row_chunk)
 
-    torch._scaled_mm with row-wise scales is CUDA-only, so the matmul is
-    emulated in fp32: bf16( (Xq . Wq^T in fp32) * sx * sw + bias ), one rounding.
-    The summation order of the reference (cuBLASLt, use_fast_accum=True) is not
-    specified; comparisons against this function use a tolerance.  ``act_dtype``
-    float8_e5m2 gives the reference's default FP8 pairing (e5m2 activations against
-    e4m3fn weights).
-    """
-    prev = x.shape[:-1]
-    x2 = x.reshape(-1, x.shape[-1])
-    xq, sx = act_quant_e4m3(x2) if act_dtype == torch.float8_e4m3fn else act_quant_e5m2(x2)
-    wf = qweight.to(torch.float32)
-    outs = []
-    for r0 in range(0, x2.shape[0], row_chunk):
-        acc = xq[r0:r0 + row_chunk].to(torch.float32) @ wf.t()
-        o = acc * sx[r0:r0 + row_chunk] * wscale.reshape(1, -1)
-        if bias is not None:
-            o = o + bias.to(torch.float32)
-        outs.append(o.to(torch.bfloat16))
-    out = torch.cat(outs, 0).view(*prev, qweight.shape[0])
-    return {"xq": xq, "sx": sx, "out": out}
+
+def takes_float_fallback(m: int, k: int, n: int) -> bool:
+    """The shapes the reference's INT8 forward hands to a float matmul when it runs un-compiled:
+    M <= 16, or K or N not a positive multiple of 8.  dax/quant/nn/dynamic/linear.py:186-194."""
+    return not (m > 16 and k % 8 == 0 and k > 0 and n % 8 == 0 and n > 0)
+
+
+def linear_int8_float_fallback(x: torch.Tensor, qweight: torch.Tensor, wscale: torch.Tensor,
+                               bias: Optional[torch.Tensor]) -> torch.Tensor:
+    """``F.linear(input, self.weight, self.bias)`` on the de-quantised weight.  dax/quant/nn/dynamic/linear.py:195-202,
+    taken only outside a compiled graph (``not is_compiling()``).  The matmul is a float one in the module's dtype;
+    its summation order is the library's, so comparisons use a tolerance."""
+    w = dequant_weight(qweight, wscale, x.dtype)
+    return torch.nn.functional.linear(x, w, None if bias is None else bias.to(x.dtype))
 
 
 # --------------------------------------------------------------------------- #
@@ -307,14 +405,16 @@ def linear_int8_schemes(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.T
 
 
 def static_linear_fp8(x: torch.Tensor, input_scale: torch.Tensor, qweight: torch.Tensor, wscale: torch.Tensor,
-                      bias: Optional[torch.Tensor], act_dtype: torch.dtype = torch.float8_e4m3fn) -> Dict[str, torch.Tensor]:
-    """Static FP8 forward, dax/quant/nn/quantized/linear.py:91-118: leaf quantiser with the stored input scale,
-    then ``_scaled_mm`` emulated in fp32 (accumulation order of the reference unspecified: tolerance)."""
+                      bias: Optional[torch.Tensor], act_dtype: torch.dtype = torch.float8_e4m3fn,
+                      out_dtype: Optional[torch.dtype] = None) -> Dict[str, torch.Tensor]:
+    """Static FP8 forward, dax/quant/nn/quantized/linear.py:91-118: leaf quantiser with the stored input scale
+    (one element), then ``_scaled_mm`` restated in fp32 (accumulation order of the reference unspecified: tolerance).
+    With a per-channel weight scale the input scale is expanded to [M,1] and the matmul writes bf16 (:98-104)."""
+    out_dtype = out_dtype or x.dtype
     x2 = x.reshape(-1, x.shape[-1])
     xq = quantize_to_fp8(x2, input_scale.reshape(1), act_dtype)
-    acc = xq.to(torch.float32) @ qweight.to(torch.float32).t()
-    o = acc * input_scale.reshape(1) * wscale.reshape(1, -1)
-    if bias is not None:
-        o = o + bias.to(torch.float32)
-    return {"xq": xq, "out": o.to(torch.bfloat16).view(*x.shape[:-1], qweight.shape[0])}
-
+    mm_dtype = torch.bfloat16 if wscale.numel() > 1 else out_dtype
+    out = scaled_mm_fp32(xq, qweight, input_scale.reshape(1), wscale, None if bias is None else bias.to(mm_dtype), mm_dtype)
+    if out.dtype != out_dtype:
+        out = out.to(out_dtype)
+    return {"xq": xq, "out": out.view(*x.shape[:-1], qweight.shape[0])}

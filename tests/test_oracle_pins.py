@@ -345,22 +345,172 @@ def test_linear_int8_end_to_end_small(closed_form):
 
 
 # ------------------------------------------------------------------ fp8 linear
-def test_linear_e4m3_matches_float_and_per_tensor_scaled_mm():
-    x, w, b = O.make_inputs(64, 256, 48, seed=12)
-    qw, sw = O.weight_quant_e4m3(w)
-    r = O.linear_e4m3(x, qw, sw, b)
+def decode_fp8(bits: np.ndarray, ebits: int) -> np.ndarray:
+    """OCP e4m3fn (ebits 4) / e5m2 (ebits 5) bytes -> float64, from the bit layout alone: sign, biased
+    exponent, mantissa; exponent 0 is subnormal.  e4m3fn has no infinities (S.1111.111 is NaN), e5m2 is IEEE-like."""
+    b = bits.astype(np.int64)
+    mbits = 7 - ebits
+    bias = (1 << (ebits - 1)) - 1
+    sign = np.where(b & 0x80, -1.0, 1.0)
+    e = (b >> mbits) & ((1 << ebits) - 1)
+    m = (b & ((1 << mbits) - 1)).astype(np.float64)
+    val = np.where(e == 0, m * 2.0 ** (1 - bias - mbits), (1.0 + m * 2.0 ** -mbits) * 2.0 ** (e.astype(np.float64) - bias))
+    if ebits == 4:
+        val = np.where((b & 0x7F) == 0x7F, np.nan, val)
+    else:
+        val = np.where(e == 31, np.where(m == 0, np.inf, np.nan), val)
+    return sign * val
+
+
+def f64_to_bf16_bits_rne(y: np.ndarray) -> np.ndarray:
+    """float64 -> bf16 bit pattern with ONE round-to-nearest-even (no intermediate float32 rounding):
+    the two neighbouring bf16 values are built by truncating the float32 that lies at or below |y|."""
+    y = np.asarray(y, np.float64)
+    a = np.abs(y)
+    f = a.astype(np.float32)
+    f = np.where(f.astype(np.float64) > a, np.nextafter(f, np.float32(0)), f).astype(np.float32)  # f <= |y|
+    lo = (f.view(np.uint32) >> 16).astype(np.uint32)  # bf16 at or below |y|
+    lo_v = (lo << 16).astype(np.uint32).view(np.float32).astype(np.float64)
+    hi_v = ((lo + 1) << 16).astype(np.uint32).view(np.float32).astype(np.float64)
+    up = (a - lo_v > hi_v - a) | ((a - lo_v == hi_v - a) & ((lo & 1) == 1))
+    mag = (lo + up.astype(np.uint32)).astype(np.uint16)
+    return np.where(np.signbit(y), mag | 0x8000, mag).astype(np.uint16)
+
+
+def ulps_apart(a_bits: np.ndarray, b_bits: np.ndarray) -> np.ndarray:
+    def key(u):
+        u = u.astype(np.int32)
+        return np.where(u & 0x8000, -(u & 0x7FFF), u)
+    return np.abs(key(a_bits) - key(b_bits))
+
+
+def scaled_mm_exact(xq_bits, x_ebits, wq_bits, w_ebits, sa, sb, bias_bits):
+    """bf16( sum_k dec(xq) dec(wq) * sa * sb + bias ) with every step in float64 and one final rounding."""
+    acc = decode_fp8(xq_bits, x_ebits) @ decode_fp8(wq_bits, w_ebits).T
+    y = acc * sa.astype(np.float64).reshape(-1, 1) * sb.astype(np.float64).reshape(1, -1)
+    if bias_bits is not None:
+        y = y + (bias_bits.astype(np.uint32) << 16).view(np.float32).astype(np.float64).reshape(1, -1)
+    return f64_to_bf16_bits_rne(y)
+
+
+def test_decode_and_rounding_helpers(closed_form):
+    allb = np.arange(256, dtype=np.uint8)
+    for ebits, table in ((4, closed_form.e4m3fn_table()), (5, closed_form.e5m2_table())):
+        d = decode_fp8(allb, ebits)
+        ok = ~np.isnan(table)
+        np.testing.assert_array_equal(d[ok], table[ok].astype(np.float64))
+        assert np.isnan(d[~ok]).all()
+    # one rounding: a value just above a bf16 tie that float32 would first round onto the tie
+    tie = np.float64(1.0) + 2.0 ** -8  # midway between bf16 1.0 and 1.0078125
+    assert f64_to_bf16_bits_rne(np.array([tie]))[0] == 0x3F80  # tie -> even
+    assert f64_to_bf16_bits_rne(np.array([tie + 2.0 ** -40]))[0] == 0x3F81  # float32 would see the tie
+    assert f64_to_bf16_bits_rne(np.array([-tie - 2.0 ** -40]))[0] == 0xBF81
+    v = np.random.default_rng(0).standard_normal(4096).astype(np.float32)
+    np.testing.assert_array_equal(f64_to_bf16_bits_rne(v.astype(np.float64)), bf16_bits(torch.from_numpy(v).bfloat16()))
+
+
+def _fp8_case(seed, m=96, k=384, n=80):
+    """Rows / channels with scales spread over two decades and a bias as large as the outputs, so that a dropped
+    bias, a dropped scale, a transposed scale or a second rounding each move many outputs."""
+    x, w, _ = O.make_inputs(m, k, n, seed=seed)
+    g = torch.Generator().manual_seed(seed + 100)
+    x = (x.float() * torch.logspace(-1, 1, m).view(-1, 1)).bfloat16()
+    w = (w.float() * torch.logspace(-1, 1, n).view(-1, 1)).bfloat16()
+    b = (torch.randn(n, generator=g) * torch.nn.functional.linear(x.float(), w.float()).std()).bfloat16()
+    return x, w, b
+
+
+@pytest.mark.parametrize("act_dtype,w_dtype", [(torch.float8_e4m3fn, torch.float8_e4m3fn), (torch.float8_e5m2, torch.float8_e4m3fn),
+                                               (torch.float8_e4m3fn, torch.float8_e5m2), (torch.float8_e5m2, torch.float8_e5m2)])
+def test_linear_fp8_vs_float64_closed_form(act_dtype, w_dtype):
+    """The FP8 forward against an evaluation from the decoded bytes in float64 with a single rounding: the fp32
+    restatement may land on the other side of a bf16 rounding boundary (fp32 accumulation error ~1e-6 relative
+    against the bf16 half-step 2e-3), never further."""
+    x, w, b = _fp8_case(21)
+    qw, sw = O.weight_quant_fp8(w, w_dtype)
+    r = O.linear_fp8(x, qw, sw, b, act_dtype=act_dtype)
+    eb = lambda dt: 4 if dt == torch.float8_e4m3fn else 5
+    want = scaled_mm_exact(r["xq"].view(torch.uint8).numpy(), eb(act_dtype), qw.view(torch.uint8).numpy(), eb(w_dtype),
+                           r["sx"].numpy(), sw.numpy(), bf16_bits(b))
+    got = bf16_bits(r["out"])
+    d = ulps_apart(got, want)
+    assert d.max() <= 1 and (d != 0).mean() < 0.01, (d.max(), (d != 0).mean())
+    # what the check is sensitive to: each of these restatement mistakes fails it
+    acc = decode_fp8(r["xq"].view(torch.uint8).numpy(), eb(act_dtype)) @ decode_fp8(qw.view(torch.uint8).numpy(), eb(w_dtype)).T
+    y = acc * r["sx"].numpy().astype(np.float64) * sw.numpy().astype(np.float64)
+    bias64 = b.float().numpy().astype(np.float64)
+    no_bias = f64_to_bf16_bits_rne(y)
+    twice = f64_to_bf16_bits_rne((f64_to_bf16_bits_rne(y).astype(np.uint32) << 16).view(np.float32).astype(np.float64) + bias64)
+    other = scaled_mm_exact(r["xq"].view(torch.uint8).numpy(), 9 - eb(act_dtype), qw.view(torch.uint8).numpy(), eb(w_dtype),
+                            r["sx"].numpy(), sw.numpy(), bf16_bits(b))
+    for name, wrong in (("no bias", no_bias), ("rounded twice", twice), ("other fp8 decoding", other)):
+        dw = ulps_apart(got, wrong)
+        assert dw.max() > 1 or (dw != 0).mean() >= 0.01, name
+    # and it sits where a quantised layer should: close to the float layer it replaces
     ref = torch.nn.functional.linear(x.float(), w.float(), b.float())
-    rel = (r["out"].float() - ref).norm() / ref.norm()
-    assert rel < 1e-1  # e4m3 has 3 mantissa bits
-    # library special case: per-tensor scales reduce to torch._scaled_mm on CPU
-    xq = r["xq"][:32].contiguous()
-    one = torch.tensor(0.5), torch.tensor(0.25)
-    try:
-        lib = torch._scaled_mm(xq, qw.t(), scale_a=one[0], scale_b=one[1], out_dtype=torch.bfloat16)
-    except (RuntimeError, NotImplementedError) as e:  # pragma: no cover
-        pytest.skip(f"torch._scaled_mm not available on this CPU build: {e}")
-    emu = ((xq.float() @ qw.float().t()) * 0.5 * 0.25).bfloat16()
-    assert ((lib.float() - emu.float()).norm() / emu.float().norm()) < 1e-2
+    assert float((r["out"].float() - ref).norm() / ref.norm()) < (0.2 if torch.float8_e5m2 in (act_dtype, w_dtype) else 0.1)
+
+
+def test_linear_fp8_per_tensor_is_the_library_scaled_mm():
+    """Uniform scales reduce the forward to torch._scaled_mm with per-tensor scales, which the CPU build
+    implements: the oracle function itself is called, with rows of equal abs-max and one weight scale."""
+    x, w, b = _fp8_case(22, m=64, k=256, n=48)
+    x[:, 0] = x.abs().max()  # every row has the same abs-max -> one activation scale
+    for act_dtype in (torch.float8_e4m3fn, torch.float8_e5m2):
+        sw1 = O.weight_scale_per_tensor(w, O.E4M3_QMAX)
+        qw = O.quantize_to_fp8(w, sw1)
+        for per_tensor in (False, True):
+            r = O.linear_fp8(x, qw, sw1.expand(1, w.shape[0]) if not per_tensor else sw1, b, act_dtype=act_dtype,
+                             per_tensor=per_tensor)
+            sx = r["sx"].reshape(-1)
+            assert (sx == sx[0]).all()
+            try:
+                lib = torch._scaled_mm(r["xq"], qw.t(), scale_a=sx[0].reshape(()), scale_b=sw1.reshape(()), bias=b,
+                                       out_dtype=torch.bfloat16)
+            except (RuntimeError, NotImplementedError) as e:  # pragma: no cover
+                pytest.skip(f"torch._scaled_mm not available on this CPU build: {e}")
+            d = ulps_apart(bf16_bits(r["out"]), bf16_bits(lib))
+            assert d.max() <= 1 and (d != 0).mean() < 0.01, (act_dtype, per_tensor, d.max(), (d != 0).mean())
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+def test_linear_fp8_other_module_dtypes(dtype):
+    """fp16 / fp32 modules: per-token rounds to bf16 (bf16 bias) and casts afterwards, per-tensor rounds to the
+    module's dtype directly (dax/quant/nn/dynamic/linear.py:106-118, :166-178)."""
+    x, w, b = _fp8_case(23, m=48, k=256, n=32)
+    x, w, b = x.to(dtype), w.to(dtype), b.to(dtype)
+    qw, sw = O.weight_quant_fp8(w)
+    r = O.linear_fp8(x, qw, sw, b)
+    assert r["out"].dtype == dtype and r["sx"].dtype == torch.float32
+    want = scaled_mm_exact(r["xq"].view(torch.uint8).numpy(), 4, qw.view(torch.uint8).numpy(), 4, r["sx"].numpy(), sw.numpy(),
+                           bf16_bits(b.bfloat16()))
+    d = ulps_apart(bf16_bits(r["out"].bfloat16()), want)  # exact cast back: out holds bf16 values
+    assert torch.equal(r["out"], r["out"].bfloat16().to(dtype)) and d.max() <= 1 and (d != 0).mean() < 0.01
+    sw1 = O.weight_scale_per_tensor(w, O.E4M3_QMAX)
+    qw1 = O.quantize_to_fp8(w, sw1)
+    r1 = O.linear_fp8(x, qw1, sw1, b, per_tensor=True)
+    acc = decode_fp8(r1["xq"].view(torch.uint8).numpy(), 4) @ decode_fp8(qw1.view(torch.uint8).numpy(), 4).T
+    y = acc * float(r1["sx"]) * float(sw1) + b.double().numpy()
+    assert r1["out"].dtype == dtype
+    rel = np.abs(r1["out"].double().numpy() - y).max() / np.abs(y).max()
+    assert rel < (1e-3 if dtype == torch.float16 else 1e-6) and not torch.equal(r1["out"], r1["out"].bfloat16().to(dtype))
+
+
+def test_float_fallback_rule_and_value():
+    """The un-compiled reference hands M <= 16 or K / N not a multiple of 8 to a float matmul on the de-quantised
+    weight (dax/quant/nn/dynamic/linear.py:186-202)."""
+    assert O.takes_float_fallback(16, 64, 64) and not O.takes_float_fallback(17, 64, 64)
+    assert O.takes_float_fallback(64, 60, 64) and O.takes_float_fallback(64, 64, 12) and O.takes_float_fallback(1, 8, 8)
+    x, w, b = O.make_inputs(16, 256, 48, seed=31)
+    qw, sw = O.weight_quant_int8(w)
+    out = O.linear_int8_float_fallback(x, qw, sw, b)
+    wd = (qw.bfloat16() * sw.view(-1, 1).bfloat16()).double()  # the weight property: scale and product rounded to bf16
+    want = x.double() @ wd.t() + b.double()
+    assert out.dtype == torch.bfloat16
+    assert float((out.double() - want).norm() / want.norm()) < 4e-3  # bf16 output rounding
+    # weight-only quantisation error, against the W8A8 result on the same rows
+    q = O.linear_int8(x, qw, sw, b)["out"]
+    assert 1e-4 < float((out.float() - q.float()).norm() / q.float().norm()) < 5e-2
 
 
 def test_make_inputs_is_seeded_and_has_outliers():
@@ -390,19 +540,115 @@ def test_per_tensor_scales_reduce_to_the_per_row_functions():
         assert torch.equal(O.linear_int8_schemes(x2, w2, b, ap, wp)["out"], base)
 
 
-def test_static_linear_fp8_matches_the_float_layer():
+def test_static_linear_fp8_closed_form_and_library():
     g = torch.Generator().manual_seed(4)
     x = torch.randn(64, 128, generator=g).bfloat16()
     w = (torch.randn(32, 128, generator=g) * 0.05).bfloat16()
-    b = (torch.randn(32, generator=g) * 0.01).bfloat16()
+    ref0 = torch.nn.functional.linear(x.float(), w.float())
+    b = (torch.randn(32, generator=g) * ref0.std()).bfloat16()
     si = O.weight_scale_per_tensor(x, O.E4M3_QMAX)                 # what a MinMaxObserver calibrated on x gives
     sw = O.weight_scale_per_tensor(w, O.E4M3_QMAX)
     qw = O.quantize_to_fp8(w, sw)
-    out = O.static_linear_fp8(x, si, qw, sw, b)["out"]
-    ref = torch.nn.functional.linear(x.float(), w.float(), b.float())
-    assert float((out.float() - ref).norm() / ref.norm()) < 6e-2    # fp8 (3 mantissa bits) quantisation error
-    # per-tensor special case of the library routine on CPU
-    lib = torch._scaled_mm(O.quantize_to_fp8(x, si), qw.t(), scale_a=si.reshape(()), scale_b=sw.reshape(()), bias=b,
-                           out_dtype=torch.bfloat16)
-    assert float((out.float() - lib.float()).norm() / lib.float().norm()) < 4e-3
+    for act_dtype, ebits in ((torch.float8_e4m3fn, 4), (torch.float8_e5m2, 5)):
+        si_a = O.weight_scale_per_tensor(x, torch.finfo(act_dtype).max)
+        r = O.static_linear_fp8(x, si_a, qw, sw, b, act_dtype)
+        want = scaled_mm_exact(r["xq"].view(torch.uint8).numpy(), ebits, qw.view(torch.uint8).numpy(), 4,
+                               si_a.numpy().repeat(64), sw.numpy().repeat(32), bf16_bits(b))
+        d = ulps_apart(bf16_bits(r["out"]), want)
+        assert d.max() <= 1 and (d != 0).mean() < 0.01
+        dn = ulps_apart(bf16_bits(O.static_linear_fp8(x, si_a, qw, sw, None, act_dtype)["out"]), want)
+        assert (dn != 0).mean() > 0.5  # the bias matters in this case
+        # per-tensor scales: the library routine on CPU
+        lib = torch._scaled_mm(r["xq"], qw.t(), scale_a=si_a.reshape(()), scale_b=sw.reshape(()), bias=b, out_dtype=torch.bfloat16)
+        dl = ulps_apart(bf16_bits(r["out"]), bf16_bits(lib))
+        assert dl.max() <= 1 and (dl != 0).mean() < 0.01
+    # per-channel weight scale: the same closed form with a scale per column
+    qwc, swc = O.weight_quant_e4m3(w)
+    rc = O.static_linear_fp8(x, si, qwc, swc, b)
+    want = scaled_mm_exact(rc["xq"].view(torch.uint8).numpy(), 4, qwc.view(torch.uint8).numpy(), 4, si.numpy().repeat(64),
+                           swc.numpy().reshape(-1), bf16_bits(b))
+    d = ulps_apart(bf16_bits(rc["out"]), want)
+    assert d.max() <= 1 and (d != 0).mean() < 0.01
+    ref = ref0 + b.float()
+    assert float((rc["out"].float() - ref).norm() / ref.norm()) < 6e-2    # fp8 (3 mantissa bits) quantisation error
 
+
+# ------------------------------------------------------------------ general blocks and input dtypes
+def test_dynamic_quantize_reduces_to_the_per_row_rule_on_each_block():
+    """A block of any shape is the pinned per-row rule applied to the block flattened into one row; the scale
+    tensor keeps every reduced dim as 1 in the view shape of the reduction."""
+    g = torch.Generator().manual_seed(40)
+    x = (torch.randn(2, 6, 8, 12, generator=g) * torch.logspace(-2, 2, 12)).bfloat16()
+    x[0, 1] = 0
+    assert O.get_reduction_params((3, 3, 2, 10), (3, 3, 10, 10)) == ([3, 3, 5, 2, 10], [0, 1, 3, 4])  # the reference's own example
+    cases = {  # block -> scale shape
+        (1, 1, 1, 12): (2, 6, 8, 1), (2, 6, 8, 12): (1, 1, 1, 1), (2, 6, 8, 1): (1, 1, 1, 12), (1, 1, 1, 4): (2, 6, 8, 3, 1),
+        (1, 3, 2, 12): (2, 2, 1, 4, 1, 1), (2, 1, 8, 6): (1, 6, 1, 2, 1), (1, 6, 1, 1): (2, 1, 8, 12)}
+    for target, qmax in ((torch.int8, 127.0), (torch.float8_e4m3fn, 448.0), (torch.float8_e5m2, 57344.0)):
+        for block, sshape in cases.items():
+            q, sc = O.dynamic_quantize(x, block, target)
+            assert q.shape == x.shape and q.dtype == target and sc.dtype == torch.float32 and tuple(sc.shape) == sshape
+            qf = q.view(torch.uint8) if target != torch.int8 else q
+            # brute force over the blocks
+            import itertools
+            steps = [range(0, n, b) for n, b in zip(x.shape, block)]
+            scs = []
+            for origin in itertools.product(*steps):
+                sl = tuple(slice(o, o + b) for o, b in zip(origin, block))
+                row = x[sl].reshape(1, -1)
+                s1 = O.act_scale(row, qmax)
+                want = O.quantize_to_int8(row, s1) if target == torch.int8 else O.quantize_to_fp8(row, s1, target).view(torch.uint8)
+                assert torch.equal(qf[sl].reshape(1, -1), want), (target, block, origin)
+                scs.append(float(s1))
+            assert scs == sc.reshape(-1).tolist()  # row-major over the kept dims
+
+
+def test_act_scale_fp16_and_fp32_inputs_exhaustive():
+    """The scale is computed in the input's dtype (dax/quant/nn/dynamic/functional.py:124-129): fp16 rounds the
+    quotient to fp16 (subnormals included) before the 2^-23 floor; fp32 does not round."""
+    h = np.arange(0, 0x7C00, dtype=np.uint16).view(np.float16)  # every non-negative finite fp16
+    x = torch.from_numpy(h.copy()).view(-1, 1)
+    for qmax in (127.0, 448.0, 57344.0):
+        got = O.act_scale(x, qmax).view(-1).numpy()
+        want = np.maximum((h.astype(np.float32) / np.float32(qmax)).astype(np.float16), np.float16(2.0 ** -23)).astype(np.float32)
+        np.testing.assert_array_equal(got, want)
+        assert got.min() == np.float32(2.0 ** -23)
+    f = (np.random.default_rng(3).standard_normal(5000) * 10.0 ** np.random.default_rng(4).integers(-30, 30, 5000)).astype(np.float32)
+    got = O.act_scale(torch.from_numpy(np.abs(f)).view(-1, 1), 127.0).view(-1).numpy()
+    np.testing.assert_array_equal(got, np.maximum(np.abs(f) / np.float32(127.0), np.float32(2.0 ** -23)))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+def test_quantize_leaf_other_input_dtypes(closed_form, dtype):
+    """x is widened to fp32 exactly before the multiply / divide (fp32 scale), so the closed forms on the fp32
+    value hold for fp16 and fp32 inputs; checked through numpy fp32 arithmetic and the C fp8 encoders."""
+    g = torch.Generator().manual_seed(41)
+    x = (torch.randn(64, 96, generator=g) * torch.logspace(-3, 3, 96)).to(dtype)
+    s = O.act_scale(x, 127.0)
+    q = O.quantize_to_int8(x, s).numpy()
+    inv = (np.float32(1.0) / s.numpy()).astype(np.float32)
+    want = np.clip(np.rint((x.float().numpy() * inv).astype(np.float32)), -128, 127).astype(np.int8)
+    np.testing.assert_array_equal(q, want)
+    for fdt, enc in ((torch.float8_e4m3fn, closed_form.f32_to_e4m3fn), (torch.float8_e5m2, closed_form.f32_to_e5m2)):
+        qmax = torch.finfo(fdt).max
+        s8 = O.act_scale(x, qmax)
+        q8 = O.quantize_to_fp8(x, s8, fdt).view(torch.uint8).numpy()
+        v = np.clip((x.float().numpy() / s8.numpy()).astype(np.float32), -qmax, qmax).astype(np.float32)
+        np.testing.assert_array_equal(q8, enc(v.reshape(-1)).reshape(v.shape))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+def test_linear_int8_other_module_dtypes(closed_form, dtype):
+    """INT8 forward of an fp16 / fp32 module: exact accumulators, fp32 scaling, cast to the module's dtype and a
+    bias add in that dtype (dax/quant/nn/dynamic/linear.py:221-228)."""
+    x, w, b = O.make_inputs(40, 256, 48, seed=42)
+    x, w, b = x.to(dtype), w.to(dtype), b.to(dtype)
+    qw, sw = O.weight_quant_int8(w)
+    r = O.linear_int8(x, qw, sw, b)
+    assert r["out"].dtype == dtype
+    acc = closed_form.gemm_i8(r["xq"].numpy(), qw.numpy())
+    np.testing.assert_array_equal(r["acc"].numpy(), acc)
+    y = (acc.astype(np.float32) * r["sx"].numpy()).astype(np.float32) * sw.numpy()
+    npdt = np.float16 if dtype == torch.float16 else np.float32
+    want = (y.astype(npdt).astype(np.float32) + b.float().numpy()).astype(npdt)
+    np.testing.assert_array_equal(r["out"].numpy(), want)
