@@ -61,6 +61,16 @@ def _need_gpu(t: torch.Tensor, what: str) -> None:
     _capi.require_gfx950(t.device.index if t.device.index is not None else torch.cuda.current_device())
 
 
+def _same_device(what: str, ref: torch.Tensor, **others) -> None:
+    """Raises unless every given tensor lives on ref's device.  A custom op registered for "cuda" is dispatched as
+    soon as one argument is a device tensor, so a module left on the CPU would otherwise hand host addresses to
+    the kernels' loads."""
+    for name, t in others.items():
+        if t is not None and t.device != ref.device:
+            raise ValueError(f"daxq::{what}: expected all tensors to be on the same device, but {name} is on {t.device} "
+                             f"and the first operand on {ref.device}")
+
+
 def _rows_bf16(x: torch.Tensor, what: str) -> None:
     _need_gpu(x, what)
     if x.dtype != torch.bfloat16:
@@ -283,6 +293,7 @@ row_minmax.register_fake(lambda x: (x.new_empty((x.shape[0],), dtype=torch.float
 def scale_from_minmax(min_val: torch.Tensor, max_val: torch.Tensor, qmax: float) -> torch.Tensor:
     """max(max(-min, max) / qmax, 2^-23) element-wise in fp32."""
     _need_gpu(min_val, "scale_from_minmax")
+    _same_device("scale_from_minmax", min_val, max_val=max_val)
     if min_val.dtype != torch.float32 or max_val.dtype != torch.float32 or min_val.shape != max_val.shape:
         raise ValueError("daxq::scale_from_minmax: min/max must be fp32 tensors of one shape")
     lo, hi = min_val.contiguous(), max_val.contiguous()
@@ -300,6 +311,7 @@ scale_from_minmax.register_fake(lambda min_val, max_val, qmax: torch.empty_like(
 def _linear(xq, sx, wq, sw, bias, fp8: bool, want_acc: bool, x_e5m2: bool = False):
     name = "linear_e5m2_e4m3" if x_e5m2 else "linear_e4m3" if fp8 else "linear_i8"
     _need_gpu(xq, name)
+    _same_device(name, xq, sx=sx, wq=wq, sw=sw, bias=bias)
     qdt = torch.uint8 if fp8 else torch.int8
     if xq.dtype != qdt or wq.dtype != qdt:
         raise ValueError(f"daxq::{name}: operands must be {qdt}")
@@ -388,6 +400,7 @@ def _dynamic_linear(x, wq, sw, bias, fmt: str):
     """Per-token quantiser and GEMM of one linear, the same two launches as act_quant_* + linear_*; one op call
     instead of two halves the host time per forward, which is what a small linear costs."""
     fp8 = fmt != "i8"
+    _same_device("dynamic_linear_" + fmt, x, wq=wq, sw=sw, bias=bias)  # before the quantiser is launched
     xq, sx = _act_quant(x, fp8, fmt == "e5m2")
     if xq.shape[1] != wq.shape[1]:
         raise ValueError(f"daxq::dynamic_linear_{fmt}: x has K={x.shape[1]} (padded {xq.shape[1]}), the weight {wq.shape[1]}")
@@ -425,6 +438,7 @@ def tensor_scale(row_min: torch.Tensor, row_max: torch.Tensor, qmax: float, roun
                  n_expand: int) -> Tuple[torch.Tensor, torch.Tensor]:
     """Per-tensor scale from per-row (min, max): (scale fp32 [1], the same value n_expand times)."""
     _need_gpu(row_min, "tensor_scale")
+    _same_device("tensor_scale", row_min, row_max=row_max)
     if row_min.dtype != torch.float32 or row_max.dtype != torch.float32 or row_min.shape != row_max.shape or row_min.numel() == 0:
         raise ValueError("daxq::tensor_scale: row_min / row_max must be non-empty fp32 tensors of one shape")
     lo, hi = row_min.contiguous(), row_max.contiguous()

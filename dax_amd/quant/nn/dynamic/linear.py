@@ -8,10 +8,15 @@ and the same exceptions for invalid dtype / qscheme combinations.
 What differs is where the arithmetic runs: ``forward`` is two HIP launches -- the fused
 per-token quantiser and the MFMA GEMM with the scale / bias / bf16 epilogue -- and the
 conversion in ``get_qlinear`` uses the HIP observer and leaf-quantiser kernels.  Numerics are
-those of the reference's eager op sequence (:180-228 for INT8, :145-178 for FP8).  The
-reference's eager-only escape to a float matmul for M <= 16 or misaligned K/N (:186-202,
-never taken under its own ``torch.compile`` decorator) does not exist here: every shape goes
-through the quantised kernels.
+those of the reference's eager op sequence (:180-228 for INT8, :145-178 for FP8).
+
+Control flow for small INT8 problems: the reference hands M <= 16, or K / N that are not
+multiples of 8, to a float matmul on the de-quantised weight, but only when the forward is NOT
+being compiled (:186-202, ``not is_compiling()``) -- and its forward carries a ``torch.compile``
+decorator (:143), so as shipped every shape is quantised.  That is the default here too.
+``Linear.uncompiled_small_shape_fallback = True`` (class or instance attribute) gives the
+un-compiled behaviour instead: those shapes then run ``F.linear(input, self.weight, self.bias)``,
+a plain library matmul on the cold path.
 """
 from __future__ import annotations
 
@@ -22,6 +27,7 @@ from torch import Tensor, nn
 
 from .... import ops
 from ...qscheme import per_channel_symmetric, per_tensor_symmetric, per_token_symmetric
+from .._derived import DerivedOperands
 from .functional import FP8_ALLOWED_DTYPES
 
 logger = logging.getLogger(__name__)
@@ -53,8 +59,11 @@ _DYNAMIC_LINEAR = {torch.int8: "dynamic_linear_i8", torch.float8_e4m3fn: "dynami
                    torch.float8_e5m2: "dynamic_linear_e5m2_e4m3"}
 
 
-class Linear(nn.Module):
+class Linear(DerivedOperands, nn.Module):
     _FLOAT_MODULE = nn.Linear
+    # False: every shape is quantised, as under the reference's own torch.compile decorator (:143); True: the
+    # un-compiled reference's float matmul for M <= 16 or K / N not multiples of 8 (:186-202)
+    uncompiled_small_shape_fallback = False
 
     def __init__(
         self,
@@ -118,10 +127,7 @@ class Linear(nn.Module):
         self.compute_dtype = compute_dtype
         self.weight_qscheme = weight_qscheme
         self.input_qscheme = input_qscheme
-        # derived, never saved: (key, K-padded byte view of qweight) for the GEMM, and the per-tensor
-        # weight scale written out once per output channel
-        self._packed = None
-        self._sw_vec = None
+        self._init_derived()
 
     # ------------------------------------------------------------------ derived views
     @property
@@ -129,39 +135,7 @@ class Linear(nn.Module):
         """De-quantised weight in out_dtype, [N,K] (:139-141)."""
         return self.qweight.to(self.out_dtype) * self.weight_scale.T.to(self.out_dtype)
 
-    def _gemm_weight(self) -> Tensor:
-        """qweight as the byte matrix [N, pad128(K)] the GEMM reads; a zero-padded copy is
-        kept only when K is not a multiple of 128, and rebuilt when qweight changes."""
-        qw = self.qweight
-        if qw.dtype == torch.float8_e4m3fn:
-            qw = qw.view(torch.uint8)
-        k = qw.shape[1]
-        kp = ops.pad_k(k)
-        if kp == k and qw.is_contiguous():
-            return qw
-        if ops.is_tracing(qw):
-            # a traced graph cannot key a cache on the storage address: pad inside the graph
-            return torch.nn.functional.pad(qw, (0, kp - k)).contiguous()
-        key = (self.qweight.data_ptr(), self.qweight._version, str(qw.device))
-        if self._packed is None or self._packed[0] != key:
-            buf = torch.zeros((qw.shape[0], kp), dtype=qw.dtype, device=qw.device)
-            buf[:, :k] = qw
-            self._packed = (key, buf)
-        return self._packed[1]
-
     # ------------------------------------------------------------------ forward
-    def _weight_scale_vector(self) -> Tensor:
-        """weight_scale as the fp32 [N] vector the GEMM reads."""
-        ws = self.weight_scale
-        if ws.numel() != 1:
-            return ws.view(-1)
-        if ops.is_tracing(ws):
-            return ops.broadcast_f32(ws.reshape(1).contiguous(), self.out_features)
-        key = (ws.data_ptr(), ws._version, str(ws.device))
-        if self._sw_vec is None or self._sw_vec[0] != key:
-            self._sw_vec = (key, ops.broadcast_f32(ws.reshape(1).contiguous(), self.out_features))
-        return self._sw_vec[1]
-
     def quantize_activation(self, input: Tensor) -> QuantizedActivation:
         """Dynamic quantisation of ``input`` [..., K] in this module's activation dtype and scheme
         (:204-208, :146-150): one scale per token, or one for the whole tensor written out per token."""
@@ -179,7 +153,21 @@ class Linear(nn.Module):
                                                  torch.float8_e5m2: "e5m2"}[self.input_dtype])(flat, sx, True)
         return QuantizedActivation(xq, sx, input.shape[:-1], self.in_features, self.input_dtype)
 
+    def _takes_float_fallback(self, input) -> bool:
+        if not self.uncompiled_small_shape_fallback or self.compute_dtype != "INT8" or torch.compiler.is_compiling():
+            return False
+        if isinstance(input, QuantizedActivation):
+            return False
+        m = input.numel() // max(self.in_features, 1)
+        k, n = self.in_features, self.out_features
+        return not (m > 16 and k % 8 == 0 and k > 0 and n % 8 == 0 and n > 0)
+
     def forward(self, input) -> Tensor:
+        self._check_device(input.device)
+        if self._takes_float_fallback(input):
+            logger.warning("int8 matmul not taken for this combination of dimensions, float implementation instead. "
+                           "M: %d, K: %d, N: %d", input.numel() // self.in_features, self.in_features, self.out_features)
+            return torch.nn.functional.linear(input, self.weight, self.bias)
         if not isinstance(input, QuantizedActivation) and self.input_qscheme == per_token_symmetric:
             # the common case: quantiser and GEMM behind one op call
             flat = input.view(-1, self.in_features)
@@ -277,6 +265,7 @@ class Linear(nn.Module):
         if not reserve_float_weight:  # release the float parameters' memory
             del mod.weight
             del mod.bias
+        qlinear.refresh_derived()
         return qlinear
 
     @classmethod

@@ -20,10 +20,11 @@ from torch import Tensor, nn
 
 from .... import ops
 from ...qscheme import per_channel_symmetric
+from .._derived import DerivedOperands
 from .functional import FP8_ALLOWED_DTYPES, quantize_to_fp8
 
 
-class Linear(nn.Module):
+class Linear(DerivedOperands, nn.Module):
     _FLOAT_MODULE = nn.Linear
 
     def __init__(self, in_features: int, out_features: int, bias: bool = True, device=None, weight_dtype=None,
@@ -52,41 +53,15 @@ class Linear(nn.Module):
         self.weight_dtype = weight_dtype or torch.float8_e4m3fn
         self.input_dtype = input_dtype or torch.float8_e4m3fn
         self.row_wise_scale = row_wise_scale
-        self._packed = None
-        self._sw_vec = None
+        self._init_derived()
 
     @property
     def weight(self):
         """De-quantised weight in out_dtype (:87-89)."""
         return self.qweight.to(self.out_dtype) * self.weight_scale.reshape(-1, 1).to(self.out_dtype)
 
-    def _gemm_weight(self) -> Tensor:
-        qw = self.qweight.detach().view(torch.uint8)
-        k = qw.shape[1]
-        kp = ops.pad_k(k)
-        if kp == k and qw.is_contiguous():
-            return qw
-        if ops.is_tracing(qw):  # no cache keyed on a storage address inside a traced graph
-            return torch.nn.functional.pad(qw, (0, kp - k)).contiguous()
-        key = (self.qweight.data_ptr(), self.qweight._version, str(qw.device))
-        if self._packed is None or self._packed[0] != key:
-            buf = torch.zeros((qw.shape[0], kp), dtype=qw.dtype, device=qw.device)
-            buf[:, :k] = qw
-            self._packed = (key, buf)
-        return self._packed[1]
-
-    def _weight_scale_vector(self) -> Tensor:
-        ws = self.weight_scale
-        if ws.numel() != 1:
-            return ws.view(-1)
-        if ops.is_tracing(ws):
-            return ops.broadcast_f32(ws.reshape(1).contiguous(), self.out_features)
-        key = (ws.data_ptr(), ws._version, str(ws.device))
-        if self._sw_vec is None or self._sw_vec[0] != key:
-            self._sw_vec = (key, ops.broadcast_f32(ws.reshape(1).contiguous(), self.out_features))
-        return self._sw_vec[1]
-
     def forward(self, input: Tensor) -> Tensor:
+        self._check_device(input.device)
         prev_dims = input.shape[:-1]
         flat = input.view(-1, self.in_features)
         sx = ops.broadcast_f32(self.input_scale.reshape(1), flat.shape[0])
@@ -153,6 +128,7 @@ class Linear(nn.Module):
         if not reserve_float_weight:  # release the float parameters' memory
             del mod.weight
             del mod.bias
+        qlinear.refresh_derived()
         return qlinear
 
     @classmethod

@@ -98,9 +98,9 @@ class MinMaxObserver(UniformQuantizationObserverBase):
 
     def calculate_qparams(self):
         lo, hi = self.min_val.reshape(1), self.max_val.reshape(1)
-        if bool(torch.isinf(lo).any()) or bool(torch.isinf(hi).any()):
-            return None  # nothing observed yet: a pre-quantised checkpoint supplies the scales (:116-120)
-        return self._calculate_qparams(lo, hi)
+        if bool(lo == float("inf")) and bool(hi == float("-inf")):
+            return None  # the untouched state: nothing observed yet, a pre-quantised checkpoint supplies the scales
+        return self._calculate_qparams(lo, hi)  # a real +-inf in the calibration data gives an infinite scale, as there
 
     def extra_repr(self):
         return f"min_val={self.min_val}, max_val={self.max_val}"

@@ -112,30 +112,40 @@ def quantize_dynamic(model, qconfig_dict=None, mapping=None, inplace=True, remov
     return model
 
 
-def _add_observer_(module, qconfig_propagation_list, device=None):
+def _insert_activation_observer(module, device):
+    """Adds ``activation_post_process`` to `module` and the pre-hook that shows it the module's input (:173-189)."""
+    if getattr(module, "qconfig", None) is None:
+        return
+    observer = module.qconfig.activation()
+    if device is not None:
+        observer.to(device)
+    module.add_module("activation_post_process", observer)
+    module.register_forward_pre_hook(_observer_forward_pre_hook, prepend=True)
+
+
+def _add_observer_(module, qconfig_propagation_list, non_leaf_module_list=None, device=None):
     """Gives every leaf module of a listed type with a qconfig an ``activation_post_process`` observer on
-    the module's device, called first among its forward pre-hooks (:123-247)."""
-    for child in module.children():
-        if isinstance(child, nn.Dropout):
-            continue
-        _add_observer_(child, qconfig_propagation_list, device)
-    is_leaf = not any(True for _ in module.children())
-    if (is_leaf and not isinstance(module, nn.Sequential) and type_before_parametrizations(module) in qconfig_propagation_list
-            and getattr(module, "qconfig", None) is not None):
-        observer = module.qconfig.activation()
+    the module's device, called first among its forward pre-hooks; a child whose type is in
+    ``non_leaf_module_list`` gets one as a whole and is not descended into (:123-247)."""
+    if device is None:
         devices = _module_devices(module)
         assert len(devices) <= 1, f"_add_observer_ only works with cpu or single-device CUDA modules, but got devices {devices}"
-        if devices:
-            observer.to(next(iter(devices)))
-        module.add_module("activation_post_process", observer)
-        module.register_forward_pre_hook(_observer_forward_pre_hook, prepend=True)
+        device = next(iter(devices)) if devices else None
+    for child in module.children():
+        if type_before_parametrizations(child) is nn.Dropout:
+            continue
+        if non_leaf_module_list is not None and type_before_parametrizations(child) in non_leaf_module_list:
+            _insert_activation_observer(child, device)
+        else:
+            _add_observer_(child, qconfig_propagation_list, non_leaf_module_list, device)
+    is_leaf = not any(True for _ in module.children())
+    if is_leaf and not isinstance(module, nn.Sequential) and type_before_parametrizations(module) in qconfig_propagation_list:
+        _insert_activation_observer(module, device)
 
 
 def prepare(model, qconfig_dict=None, inplace=True, observer_non_leaf_module_list=None):
     """Attaches qconfigs and activation observers for calibration (:250-301); run data through the model
     afterwards, then ``convert``."""
-    if observer_non_leaf_module_list:
-        raise NotImplementedError("observers on non-leaf modules are not built")
     if not inplace:
         model = copy.deepcopy(model)
     propagate_qconfig_(model, qconfig_dict)
@@ -144,7 +154,7 @@ def prepare(model, qconfig_dict=None, inplace=True, observer_non_leaf_module_lis
 
         warnings.warn("None of the submodule got qconfig applied. Make sure you passed correct configuration through "
                       "`qconfig_dict` or by assigning the `.qconfig` attribute directly on submodules")
-    _add_observer_(model, get_default_qconfig_propagation_list())
+    _add_observer_(model, get_default_qconfig_propagation_list(), observer_non_leaf_module_list)
     return model
 
 

@@ -187,8 +187,15 @@ def test_default_mappings_and_prepare_convert_flow():
     assert isinstance(m.block.fc, FakeQ) and type(m.embed.fc) is nn.Linear
     assert list(m.block.fc._forward_pre_hooks.values()) == [user_hook]
     assert not any(hasattr(mod, "qconfig") or hasattr(mod, "activation_post_process") for mod in m.modules())
-    with pytest.raises(NotImplementedError):
-        prepare(Outer(), {}, observer_non_leaf_module_list=[nn.Sequential])
+    # observer_non_leaf_module_list: a listed non-leaf child is observed as a whole and not descended into
+    # (dax/quant/quantization/quantize.py:205-210)
+    m = Outer()
+    prepare(m, {"": get_default_fp8_qconfig(), "embed": None}, observer_non_leaf_module_list=[Inner])
+    assert isinstance(m.block.activation_post_process, MinMaxObserver)
+    assert list(m.block._forward_pre_hooks.values())[0] is _observer_forward_pre_hook
+    assert not hasattr(m.block.fc, "activation_post_process")           # not descended into
+    assert not hasattr(m.embed, "activation_post_process")              # its qconfig is None
+    assert isinstance(m.proj_out.activation_post_process, MinMaxObserver)  # leaves elsewhere as before
 
 
 def test_static_linear_state_and_validation():
