@@ -11,7 +11,7 @@ import threading
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "libdaxq.so")
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 _lock = threading.Lock()
 _lib = None
@@ -41,11 +41,19 @@ SIGNATURES = {
     "daxq_tensor_minmax_update": [_P, _P, _I64, _P, _P, _P],
     "daxq_broadcast_f32": [_P, _P, _I64, _P],
     "daxq_row_minmax": [_P, _I64, _I64, _I64, _P, _P, _P],
+    "daxq_row_minmax_t": [_P, _INT, _I64, _I64, _I64, _P, _P, _P],
+    "daxq_act_quant_rows": [_P, _INT, _INT, _I64, _I64, _I64, _P, _I64, _P, _P],
+    "daxq_quantize_rows": [_P, _INT, _INT, _I64, _I64, _I64, _P, _P, _I64, _P],
+    "daxq_block_scale": [_P, _INT, _INT, C.POINTER(_I64), C.POINTER(C.c_int32), _F32, _INT, _P, _P],
+    "daxq_block_quantize": [_P, _INT, _INT, _INT, C.POINTER(_I64), C.POINTER(C.c_int32), _P, _P, _P],
     "daxq_scale_from_minmax": [_P, _P, _I64, _F32, _P, _P],
     "daxq_linear_i8": [_P, _I64, _P, _P, _I64, _P, _P, _P, _I64, _P, _I64, _I64, _I64, _I64, _P],
     "daxq_linear_e4m3": [_P, _I64, _P, _P, _I64, _P, _P, _P, _I64, _P, _I64, _I64, _I64, _I64, _P],
     "daxq_linear_e5m2_e4m3": [_P, _I64, _P, _P, _I64, _P, _P, _P, _I64, _P, _I64, _I64, _I64, _I64, _P],
-    "daxq_set_gemm_variant": [_INT],
+    "daxq_linear_splitk_choice": [_I64, _I64, _I64],
+    "daxq_linear_splitk_workspace_bytes": [_I64, _I64, _INT],
+    "daxq_linear_w8a8_splitk": [_INT, _INT, _P, _I64, _P, _P, _I64, _P, _P, _P, _I64, _I64, _I64, _I64, _INT, _P, _I64, _P],
+    "daxq_linear_w8a8": [_INT, _INT, _INT, _P, _I64, _P, _P, _I64, _P, _P, _P, _I64, _P, _I64, _I64, _I64, _I64, _INT, _P],
 }
 
 
@@ -66,7 +74,8 @@ def lib() -> C.CDLL:
                 for name, args in SIGNATURES.items():
                     fn = getattr(L, name)
                     fn.argtypes = args
-                    fn.restype = C.c_char_p if name == "daxq_last_error" else _INT
+                    fn.restype = (C.c_char_p if name == "daxq_last_error" else
+                                  _I64 if name == "daxq_linear_splitk_workspace_bytes" else _INT)
                 got = L.daxq_abi_version()
                 if got != ABI_VERSION:
                     raise RuntimeError(f"libdaxq ABI {got} != expected {ABI_VERSION}; rebuild the library")
@@ -107,5 +116,28 @@ def require_gfx950(device: int) -> None:
     _checked_devices.add(device)
 
 
-def set_gemm_variant(v: int) -> None:
-    check(lib().daxq_set_gemm_variant(int(v)), "daxq_set_gemm_variant")
+FMT = {"i8": 0, "e4m3": 1, "e5m2": 2}  # DAXQ_FMT_*
+FLOAT_KIND = {"bf16": 0, "f16": 1, "f32": 2}  # DAXQ_BF16 / DAXQ_F16 / DAXQ_F32
+
+
+# ---- test / comparison hook: which GEMM implementation the ops ask for (the `kernel` argument of daxq_linear_w8a8).
+# Host-side only: the library itself keeps no selection, every call names its kernel.
+_kernel_choice = 0
+_tile_group = 0
+
+
+def debug_select_gemm(v: int) -> None:
+    """0 = the library's choice by shape; 2 / 5 / 6 / 8 / 9 / 11 = one implementation (include/daxq.h);
+    1000 + d = depth d of the tile-order groups (1000 = default)."""
+    global _kernel_choice, _tile_group
+    v = int(v)
+    if 1000 <= v < 1064:
+        _tile_group = v - 1000
+    elif v in (0, 2, 5, 6, 8, 9, 11):
+        _kernel_choice = v
+    else:
+        raise DaxqError(f"unknown gemm kernel choice {v}")
+
+
+def kernel_arg() -> int:
+    return _kernel_choice | (_tile_group << 16)

@@ -1,6 +1,8 @@
 // Types and helpers shared by the W8A8 GEMM kernels (gfx950).
 #pragma once
 
+#include <atomic>
+
 #include "daxq_common.h"
 
 namespace daxq {
@@ -35,18 +37,28 @@ struct GemmArgs {
     int m, n, k;
     int tiles_m, tiles_n;
     int gm;  // depth (in tile rows) of the groups the tile order walks through
+    int out_kind;  // element type of out and bias: DAXQ_BF16 / DAXQ_F16 / DAXQ_F32 (the tiled kernels write bf16 only)
+    // split-K launches only: K is cut into `splits` equal ranges, one workgroup each; partial accumulators go to
+    // `partials` ([tile][split][64 KiB]) and the workgroup that arrives last at `counters[tile]` adds them up
+    int splits;
+    int32_t* counters;
+    void* partials;
 };
+
+// FP8 operand formats of a launch as one template parameter: bit 0 = activations are e5m2, bit 1 = weights are e5m2
+// (the format selects of the f8f6f4 MFMA are instruction immediates)
+constexpr int kF8XE5 = 1, kF8WE5 = 2;
 
 // Raises a kernel's dynamic LDS limit once per device.  `done` is the caller's per-kernel bit mask of the devices
 // already set up (a race between two threads sets the same attribute twice).
-inline int ensure_dynamic_lds(const void* kern, int bytes, uint64_t& done) {
+inline int ensure_dynamic_lds(const void* kern, int bytes, std::atomic<uint64_t>& done) {
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess) return fail(DAXQ_ERR_LAUNCH, "hipGetDevice failed");
     const uint64_t bit = dev < 64 ? (uint64_t)1 << dev : 0;
-    if (done & bit) return DAXQ_OK;
+    if (done.load(std::memory_order_acquire) & bit) return DAXQ_OK;
     hipError_t e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
     if (e != hipSuccess) return fail(DAXQ_ERR_LAUNCH, "hipFuncSetAttribute(%d bytes LDS): %s", bytes, hipGetErrorString(e));
-    done |= bit;
+    done.fetch_or(bit, std::memory_order_release);
     return DAXQ_OK;
 }
 

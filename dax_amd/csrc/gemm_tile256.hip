@@ -116,7 +116,8 @@ __device__ __forceinline__ void load_one_frag(const FragAddr& fa, int stage, int
 }
 
 // ZERO: the block's first MFMA of a tile, which starts from zero instead of the accumulator
-template <bool FP8, bool XE5, bool ZERO = false, int NB = 4>
+// F8: FP8 operand formats (kF8XE5 / kF8WE5: e5m2 activation / weight bytes)
+template <bool FP8, int F8, bool ZERO = false, int NB = 4>
 __device__ __forceinline__ void mfma_one(typename AccT<FP8>::type (&acc)[NB][NB], int g, const typename Frag<FP8>::type (&af)[4],
                                          const typename Frag<FP8>::type (&bf)[4]) {
     const int j = g / NB, i = g % NB;
@@ -125,13 +126,13 @@ __device__ __forceinline__ void mfma_one(typename AccT<FP8>::type (&acc)[NB][NB]
     if constexpr (!FP8)
         acc[j][i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[j], af[i], c, 0, 0, 0);
     else
-        acc[j][i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bf[j], af[i], c, 0, XE5 ? 1 : 0, 0, 0, 0, 0);
+        acc[j][i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bf[j], af[i], c, (F8 & kF8WE5) ? 1 : 0, (F8 & kF8XE5) ? 1 : 0, 0, 0, 0, 0);
 }
 
 // acc[j][i]: 32x32 block with rows = n (W rows, MFMA "A" operand) and columns = m (X rows, "B"
 // operand), so that a lane ends up owning one output row m and runs of 4 consecutive n.
-// XE5: the activation bytes are e5m2 instead of e4m3fn (format select of the MFMA "B" operand).
-template <bool FP8, bool XE5>
+// F8: e5m2 instead of e4m3fn bytes (format selects: weights are the MFMA "A" operand, activations the "B" operand).
+template <bool FP8, int F8>
 __device__ __forceinline__ void mfma_step(typename AccT<FP8>::type (&acc)[4][4], const typename Frag<FP8>::type (&af)[4],
                                           const typename Frag<FP8>::type (&bf)[4]) {
 #pragma unroll
@@ -141,7 +142,7 @@ __device__ __forceinline__ void mfma_step(typename AccT<FP8>::type (&acc)[4][4],
             if constexpr (!FP8)
                 acc[j][i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[j], af[i], acc[j][i], 0, 0, 0);
             else
-                acc[j][i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bf[j], af[i], acc[j][i], 0, XE5 ? 1 : 0, 0, 0, 0, 0);
+                acc[j][i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bf[j], af[i], acc[j][i], (F8 & kF8WE5) ? 1 : 0, (F8 & kF8XE5) ? 1 : 0, 0, 0, 0, 0);
         }
 }
 
@@ -524,7 +525,7 @@ __global__ __launch_bounds__(256) void gemm_tile256_kernel(const GemmArgs p) {
 // raises the kernel's dynamic LDS limit on the current device (once per device)
 template <bool FP8, bool DUMP, bool XE5 = false>
 static int prepare_tile256() {
-    static uint64_t lds_set = 0;  // per instantiation
+    static std::atomic<uint64_t> lds_set{0};  // per instantiation
     return ensure_dynamic_lds(reinterpret_cast<const void*>(gemm_tile256_kernel<FP8, DUMP, XE5>), t256::SMEM, lds_set);
 }
 
@@ -589,7 +590,13 @@ struct TileAcc<false, true> {
 // of two v_mfma_i32_32x32x32_i8 per 32x32 block (32).  Same LDS bytes, fragment registers and MFMA
 // cycles; the narrow shape moves fewer accumulator bytes per operation and sustains a higher clock
 // under the board's power limit.
-template <bool FP8, bool DUMP, bool XE5, bool N16 = false, int BT = 256>
+//
+// SPLITK (128 tile): K is cut into p.splits ranges and blockIdx.x = tile * splits + split.  A workgroup accumulates
+// its range, writes the accumulators to the workspace (one 16-byte vector per lane and store instruction), and
+// counts itself in at the tile's counter; the workgroup that arrives last adds the partial results of all ranges
+// in range order (so FP8 sums do not depend on who was last) and runs the epilogue.  No workgroup waits for
+// another.  The last one sets the counter back to zero.
+template <bool FP8, bool DUMP, int F8, bool N16 = false, int BT = 256, bool SPLITK = false>
 __global__ __launch_bounds__(256) void gemm_tile256s5_kernel(const GemmArgs p) {
     using namespace t5;
     static_assert(!(FP8 && N16), "the 16x16 form exists for INT8 only");
@@ -610,7 +617,14 @@ __global__ __launch_bounds__(256) void gemm_tile256s5_kernel(const GemmArgs p) {
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
     const int wm = wave >> 1, wn = wave & 1;
     int tm, tn;
-    tile_of_block(p.gm, blockIdx.x, p.tiles_m, p.tiles_n, tm, tn);
+    int tile_id = blockIdx.x, split = 0, klen = p.k;  // klen: bytes of K this workgroup covers, a multiple of 128
+    if constexpr (SPLITK) {
+        static_assert(BT == 128 && !DUMP, "split-K exists on 128 tiles, without the accumulator dump");
+        tile_id = blockIdx.x / p.splits;
+        split = blockIdx.x - tile_id * p.splits;
+        klen = p.k / p.splits;
+    }
+    tile_of_block(p.gm, tile_id, p.tiles_m, p.tiles_n, tm, tn);
     int m0 = tm * BT, n0 = tn * BT;
     m0 = m0 + BT <= p.m ? m0 : p.m - BT;
     n0 = n0 + BT <= p.n ? n0 : p.n - BT;
@@ -624,8 +638,8 @@ __global__ __launch_bounds__(256) void gemm_tile256s5_kernel(const GemmArgs p) {
     uint32_t voff_a = (uint32_t)(t >> 2) * (uint32_t)p.lda + gsw;
     uint32_t voff_b = (uint32_t)(t >> 2) * (uint32_t)p.ldb + gsw;
     uint32_t voff_a1 = voff_a + BKS, voff_b1 = voff_b + BKS;  // second half of the 128-byte line
-    const uint8_t* abase = p.a + (int64_t)m0 * p.lda;
-    const uint8_t* bbase = p.b + (int64_t)n0 * p.ldb;
+    const uint8_t* abase = p.a + (int64_t)m0 * p.lda + (int64_t)split * klen;
+    const uint8_t* bbase = p.b + (int64_t)n0 * p.ldb + (int64_t)split * klen;
     const int64_t a_step = 64 * p.lda, b_step = 64 * p.ldb;
     const uint32_t lds0 = (uint32_t)(uintptr_t)(DAXQ_LDS uint8_t*)smem;
     const uint32_t wave_lds = lds0 + (uint32_t)__builtin_amdgcn_readfirstlane(wave * 1024);
@@ -684,7 +698,7 @@ __global__ __launch_bounds__(256) void gemm_tile256s5_kernel(const GemmArgs p) {
     // fragment sets: [slice parity][MFMA step] (N16: [slice parity][blocks 0-3 / 4-7])
     frag_t fa00[4] = {}, fb00[4] = {}, fa01[4] = {}, fb01[4] = {}, fa10[4] = {}, fb10[4] = {}, fa11[4] = {}, fb11[4] = {};
 
-    const int S = p.k / BKS;  // slices; even because K is a multiple of 128
+    const int S = klen / BKS;  // slices; even because K (and each split range) is a multiple of 128
     // stage offsets of slices s .. s+4 (s = the even slice of the current pair)
     uint32_t st0 = 0, st1 = STAGE, st2 = 2 * STAGE, st3 = 3 * STAGE, st4 = 4 * STAGE;
 
@@ -751,15 +765,15 @@ __global__ __launch_bounds__(256) void gemm_tile256s5_kernel(const GemmArgs p) {
                     asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+a"(acc[j][i]) : "v"(bfr), "v"(afr));
             } else if constexpr (!FP8) {
                 if constexpr (ODD.value) {
-                    if (g < NB * NB) mfma_one<FP8, XE5, false, NB>(acc, g, fa10, fb10);
-                    else mfma_one<FP8, XE5, false, NB>(acc, g - NB * NB, fa11, fb11);
+                    if (g < NB * NB) mfma_one<FP8, F8, false, NB>(acc, g, fa10, fb10);
+                    else mfma_one<FP8, F8, false, NB>(acc, g - NB * NB, fa11, fb11);
                 } else {
-                    if (g < NB * NB) mfma_one<FP8, XE5, FIRST.value, NB>(acc, g, fa00, fb00);
-                    else mfma_one<FP8, XE5, false, NB>(acc, g - NB * NB, fa01, fb01);
+                    if (g < NB * NB) mfma_one<FP8, F8, FIRST.value, NB>(acc, g, fa00, fb00);
+                    else mfma_one<FP8, F8, false, NB>(acc, g - NB * NB, fa01, fb01);
                 }
             } else {
-                if constexpr (ODD.value) mfma_one<FP8, XE5, false, NB>(acc, g, fa10, fb10);
-                else mfma_one<FP8, XE5, FIRST.value, NB>(acc, g, fa00, fb00);
+                if constexpr (ODD.value) mfma_one<FP8, F8, false, NB>(acc, g, fa10, fb10);
+                else mfma_one<FP8, F8, FIRST.value, NB>(acc, g, fa00, fb00);
             }
             // loop bookkeeping inside the last regions, in the issue slots an MFMA leaves free, instead of
             // in a block of its own behind the slice: lane offsets of the operand this slice loaded, and
@@ -854,6 +868,63 @@ __global__ __launch_bounds__(256) void gemm_tile256s5_kernel(const GemmArgs p) {
             }
         }
     }
+    if constexpr (SPLITK) {
+        // ---- partial accumulators -> workspace; the last workgroup of the tile sums all of them
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));  // the scale / bias loads have landed: the waits above count them
+        constexpr int VPB = N16 ? 1 : 4;           // 16-byte vectors per lane and MFMA block
+        constexpr int NV = NB * NB * VPB;          // per lane: 16 of them = 64 registers either way
+        typedef int v4raw __attribute__((ext_vector_type(4)));
+        v4raw* mine = static_cast<v4raw*>(p.partials) + (int64_t)blockIdx.x * NV * 256 + t;
+#pragma unroll
+        for (int j = 0; j < NB; ++j)
+#pragma unroll
+            for (int i = 0; i < NB; ++i)
+#pragma unroll
+                for (int v = 0; v < VPB; ++v) {
+                    v4raw w;
+                    if constexpr (N16) {
+                        w = acc[j][i];
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) w[e] = __float_as_int(acc[j][i][4 * v + e]);  // (a by-value call: __builtin_bit_cast of a vector element reads element 0)
+                    }
+                    mine[((j * NB + i) * VPB + v) * 256] = w;
+                }
+        __threadfence();  // the partial result is visible device-wide before the counter moves
+        __syncthreads();
+        int* flag = reinterpret_cast<int*>(smem + 2048);  // LDS is free: nobody reads a stage after the last barrier
+        if (t == 0) *flag = atomicAdd(p.counters + tile_id, 1) == p.splits - 1;
+        __syncthreads();
+        if (!*flag) return;
+        __threadfence();  // acquire: the other workgroups' partial results
+        const v4raw* all = static_cast<const v4raw*>(p.partials) + (int64_t)tile_id * p.splits * NV * 256 + t;
+#pragma unroll
+        for (int j = 0; j < NB; ++j)
+#pragma unroll
+            for (int i = 0; i < NB; ++i)
+#pragma unroll
+                for (int v = 0; v < VPB; ++v) {
+                    v4raw sum = all[((j * NB + i) * VPB + v) * 256];
+                    for (int sp = 1; sp < p.splits; ++sp) {
+                        const v4raw w = all[((int64_t)sp * NV + (j * NB + i) * VPB + v) * 256];
+                        if constexpr (FP8) {
+#pragma unroll
+                            for (int e = 0; e < 4; ++e)
+                                sum[e] = __float_as_int(__int_as_float(sum[e]) + __int_as_float(w[e]));
+                        } else {
+                            sum += w;
+                        }
+                    }
+                    if constexpr (N16) {
+                        acc[j][i] = sum;
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) acc[j][i][4 * v + e] = __int_as_float(sum[e]);
+                    }
+                }
+        if (t == 0) p.counters[tile_id] = 0;  // ready for the next launch on this workspace
+        __syncthreads();                      // every thread has read the flag before the epilogue reuses the LDS
+    }
     if constexpr (N16)
         tile256_epilogue16<DUMP, NB>(p, acc, smem, m0, n0, t, wm, wn, lr, lane >> 4, pre_sx, pre_sw,
                                      p.bias ? bf16_bits_to_f32(pre_b) : -0.0f);
@@ -862,19 +933,52 @@ __global__ __launch_bounds__(256) void gemm_tile256s5_kernel(const GemmArgs p) {
                                         p.bias ? bf16_bits_to_f32(pre_b) : -0.0f);
 }
 
-template <bool FP8, bool DUMP, bool XE5, bool N16 = false, int BT = 256>
+template <bool FP8, bool DUMP, int F8, bool N16 = false, int BT = 256, bool SPLITK = false>
 static int prepare_tile256s5() {
-    static uint64_t lds_set = 0;  // per instantiation
-    return ensure_dynamic_lds(reinterpret_cast<const void*>(gemm_tile256s5_kernel<FP8, DUMP, XE5, N16, BT>),
+    static std::atomic<uint64_t> lds_set{0};  // per instantiation
+    return ensure_dynamic_lds(reinterpret_cast<const void*>(gemm_tile256s5_kernel<FP8, DUMP, F8, N16, BT, SPLITK>),
                               t5::NST * 2 * BT * t5::BKS, lds_set);
 }
 
-template <bool FP8, bool DUMP, bool XE5, bool N16 = false, int BT = 256>
+// split-K launch on 128 tiles: a.splits ranges of K, a.counters zero, a.partials large enough (checked by the caller)
+template <bool FP8, int F8>
+static int launch_splitk_impl(const GemmArgs& a, hipStream_t st) {
+    using namespace t5;
+    constexpr int SMEM = NST * 2 * 128 * BKS;
+    auto kern = gemm_tile256s5_kernel<FP8, false, F8, !FP8, 128, true>;
+    if (int rc = prepare_tile256s5<FP8, false, F8, !FP8, 128, true>()) return rc;
+    const int64_t nt = (int64_t)a.tiles_m * a.tiles_n * a.splits;
+    if (nt > 0x7fffffff) return fail(DAXQ_ERR_ARG, "gemm: too many workgroups");
+    hipLaunchKernelGGL(kern, dim3((unsigned)nt), dim3(T), SMEM, st, a);
+    return check_launch("gemm_tile128_splitk");
+}
+
+template <bool FP8>
+int launch_tile128_splitk(const GemmArgs& a0, int f8, hipStream_t st) {
+    GemmArgs a = a0;
+    a.tiles_m = (a.m + 127) / 128;
+    a.tiles_n = (a.n + 127) / 128;
+    if constexpr (FP8) {
+        switch (f8) {
+            case 1: return launch_splitk_impl<true, 1>(a, st);
+            case 2: return launch_splitk_impl<true, 2>(a, st);
+            case 3: return launch_splitk_impl<true, 3>(a, st);
+            default: return launch_splitk_impl<true, 0>(a, st);
+        }
+    } else {
+        return launch_splitk_impl<false, 0>(a, st);
+    }
+}
+
+template int launch_tile128_splitk<false>(const GemmArgs&, int, hipStream_t);
+template int launch_tile128_splitk<true>(const GemmArgs&, int, hipStream_t);
+
+template <bool FP8, bool DUMP, int F8, bool N16 = false, int BT = 256>
 static int launch_tile256s5_impl(const GemmArgs& a, hipStream_t st) {
     using namespace t5;
     constexpr int SMEM = NST * 2 * BT * BKS;  // 160 KB (256 tile), 80 KB (128 tile)
-    auto kern = gemm_tile256s5_kernel<FP8, DUMP, XE5, N16, BT>;
-    if (int rc = prepare_tile256s5<FP8, DUMP, XE5, N16, BT>()) return rc;
+    auto kern = gemm_tile256s5_kernel<FP8, DUMP, F8, N16, BT>;
+    if (int rc = prepare_tile256s5<FP8, DUMP, F8, N16, BT>()) return rc;
     const int64_t nt = (int64_t)a.tiles_m * a.tiles_n;
     if (nt > 0x7fffffff) return fail(DAXQ_ERR_ARG, "gemm: too many tiles");
     hipLaunchKernelGGL(kern, dim3((unsigned)nt), dim3(T), SMEM, st, a);
@@ -883,28 +987,35 @@ static int launch_tile256s5_impl(const GemmArgs& a, hipStream_t st) {
 
 // wide:  INT8 with 32x32x32 MFMAs instead of the 16x16x64 form (256 tile only; kept for the tests and for comparisons)
 // small: 128x128 tiles (needs m, n >= 128)
+// f8:    FP8 operand formats (kF8XE5 | kF8WE5)
+template <bool FP8, int F8>
+static int launch_tile256s5_f8(const GemmArgs& a, bool small, hipStream_t st) {
+    if (small) return a.acc ? launch_tile256s5_impl<true, true, F8, false, 128>(a, st) : launch_tile256s5_impl<true, false, F8, false, 128>(a, st);
+    return a.acc ? launch_tile256s5_impl<true, true, F8>(a, st) : launch_tile256s5_impl<true, false, F8>(a, st);
+}
+
 template <bool FP8>
-int launch_tile256s5(const GemmArgs& a0, bool x_e5m2, bool wide, bool small, hipStream_t st) {
+int launch_tile256s5(const GemmArgs& a0, int f8, bool wide, bool small, hipStream_t st) {
     GemmArgs a = a0;
     const int bt = small ? 128 : 256;
     a.tiles_m = (a.m + bt - 1) / bt;
     a.tiles_n = (a.n + bt - 1) / bt;
     if constexpr (FP8) {
-        if (small) {
-            if (x_e5m2) return a.acc ? launch_tile256s5_impl<true, true, true, false, 128>(a, st) : launch_tile256s5_impl<true, false, true, false, 128>(a, st);
-            return a.acc ? launch_tile256s5_impl<true, true, false, false, 128>(a, st) : launch_tile256s5_impl<true, false, false, false, 128>(a, st);
+        switch (f8) {
+            case 1: return launch_tile256s5_f8<true, 1>(a, small, st);
+            case 2: return launch_tile256s5_f8<true, 2>(a, small, st);
+            case 3: return launch_tile256s5_f8<true, 3>(a, small, st);
+            default: return launch_tile256s5_f8<true, 0>(a, small, st);
         }
-        if (x_e5m2) return a.acc ? launch_tile256s5_impl<true, true, true>(a, st) : launch_tile256s5_impl<true, false, true>(a, st);
-        return a.acc ? launch_tile256s5_impl<true, true, false>(a, st) : launch_tile256s5_impl<true, false, false>(a, st);
     } else {
-        if (small) return a.acc ? launch_tile256s5_impl<false, true, false, true, 128>(a, st) : launch_tile256s5_impl<false, false, false, true, 128>(a, st);
-        if (wide) return a.acc ? launch_tile256s5_impl<false, true, false>(a, st) : launch_tile256s5_impl<false, false, false>(a, st);
-        return a.acc ? launch_tile256s5_impl<false, true, false, true>(a, st) : launch_tile256s5_impl<false, false, false, true>(a, st);
+        if (small) return a.acc ? launch_tile256s5_impl<false, true, 0, true, 128>(a, st) : launch_tile256s5_impl<false, false, 0, true, 128>(a, st);
+        if (wide) return a.acc ? launch_tile256s5_impl<false, true, 0>(a, st) : launch_tile256s5_impl<false, false, 0>(a, st);
+        return a.acc ? launch_tile256s5_impl<false, true, 0, true>(a, st) : launch_tile256s5_impl<false, false, 0, true>(a, st);
     }
 }
 
-template int launch_tile256s5<false>(const GemmArgs&, bool, bool, bool, hipStream_t);
-template int launch_tile256s5<true>(const GemmArgs&, bool, bool, bool, hipStream_t);
+template int launch_tile256s5<false>(const GemmArgs&, int, bool, bool, hipStream_t);
+template int launch_tile256s5<true>(const GemmArgs&, int, bool, bool, hipStream_t);
 
 // Every instantiation the launchers above can pick, prepared on the current device: afterwards no launch changes a
 // kernel attribute any more, so the first launch may already sit inside a stream capture.
@@ -917,20 +1028,24 @@ int prepare_tile256_kernels() {
     DAXQ_PREP(prepare_tile256<true, true>);
     DAXQ_PREP(prepare_tile256<true, false, true>);
     DAXQ_PREP(prepare_tile256<true, true, true>);
-    DAXQ_PREP(prepare_tile256s5<false, false, false, true, 256>);
-    DAXQ_PREP(prepare_tile256s5<false, true, false, true, 256>);
-    DAXQ_PREP(prepare_tile256s5<false, false, false, false, 256>);
-    DAXQ_PREP(prepare_tile256s5<false, true, false, false, 256>);
-    DAXQ_PREP(prepare_tile256s5<false, false, false, true, 128>);
-    DAXQ_PREP(prepare_tile256s5<false, true, false, true, 128>);
-    DAXQ_PREP(prepare_tile256s5<true, false, false, false, 256>);
-    DAXQ_PREP(prepare_tile256s5<true, true, false, false, 256>);
-    DAXQ_PREP(prepare_tile256s5<true, false, true, false, 256>);
-    DAXQ_PREP(prepare_tile256s5<true, true, true, false, 256>);
-    DAXQ_PREP(prepare_tile256s5<true, false, false, false, 128>);
-    DAXQ_PREP(prepare_tile256s5<true, true, false, false, 128>);
-    DAXQ_PREP(prepare_tile256s5<true, false, true, false, 128>);
-    DAXQ_PREP(prepare_tile256s5<true, true, true, false, 128>);
+    DAXQ_PREP(prepare_tile256s5<false, false, 0, true, 256>);
+    DAXQ_PREP(prepare_tile256s5<false, true, 0, true, 256>);
+    DAXQ_PREP(prepare_tile256s5<false, false, 0, false, 256>);
+    DAXQ_PREP(prepare_tile256s5<false, true, 0, false, 256>);
+    DAXQ_PREP(prepare_tile256s5<false, false, 0, true, 128>);
+    DAXQ_PREP(prepare_tile256s5<false, true, 0, true, 128>);
+    DAXQ_PREP(prepare_tile256s5<false, false, 0, true, 128, true>);
+#define DAXQ_PREP_F8(F8)                                         \
+    DAXQ_PREP(prepare_tile256s5<true, false, F8, false, 128, true>); \
+    DAXQ_PREP(prepare_tile256s5<true, false, F8, false, 256>);   \
+    DAXQ_PREP(prepare_tile256s5<true, true, F8, false, 256>);    \
+    DAXQ_PREP(prepare_tile256s5<true, false, F8, false, 128>);   \
+    DAXQ_PREP(prepare_tile256s5<true, true, F8, false, 128>)
+    DAXQ_PREP_F8(0);
+    DAXQ_PREP_F8(1);
+    DAXQ_PREP_F8(2);
+    DAXQ_PREP_F8(3);
+#undef DAXQ_PREP_F8
 #undef DAXQ_PREP
     return rc;
 }

@@ -1,4 +1,5 @@
-// W8A8 GEMM on gfx950 MFMA with the fused scale / bias / bf16 epilogue.
+// W8A8 GEMM on gfx950 MFMA with the fused scale / bias / cast epilogue: the generic kernel (any shape, any
+// FP8 operand pairing, bf16 / fp16 / fp32 outputs) and the dispatcher behind the daxq_linear_* entry points.
 //
 //   INT8: acc[i,j] = sum_k xq[i,k] * wq[j,k]  (int32, exact)   v_mfma_i32_32x32x32_i8
 //         out = bf16( f32( bf16( f32_rne(acc) * sx[i] * sw[j] ) ) + f32(bias[j]) )
@@ -17,12 +18,14 @@
 // that the ds_read_b128 of 16 consecutive rows at one K offset hits 16 different bank
 // groups.  Workgroup ids are remapped so that the tiles resident on one XCD (ids
 // congruent mod 8) form a compact patch of the output and share A/B panels in that XCD's L2.
+#include <type_traits>
+
 #include "gemm_common.h"
 
 namespace daxq {
 
-// XE5: the activation bytes (MFMA "A" operand here) are e5m2 instead of e4m3fn
-template <bool FP8, int BM, int BN, int BK, int WM, int WN, bool DIRECT, bool XE5 = false>
+// F8: FP8 operand formats (kF8XE5: the activation bytes, MFMA "A" operand here, are e5m2; kF8WE5: the weight bytes)
+template <bool FP8, int BM, int BN, int BK, int WM, int WN, bool DIRECT, int F8 = 0>
 __global__ __launch_bounds__(WM* WN * 64) void gemm_w8a8_kernel(const GemmArgs p) {
     constexpr int T = WM * WN * 64;
     constexpr int TM = BM / WM, TN = BN / WN;  // wave tile
@@ -118,7 +121,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_w8a8_kernel(const GemmArgs p
                 for (int i = 0; i < MB; ++i)
 #pragma unroll
                     for (int j = 0; j < NB; ++j)
-                        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(af[i], bf[j], acc[i][j], XE5 ? 1 : 0, 0, 0, 0, 0, 0);
+                        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(af[i], bf[j], acc[i][j], (F8 & kF8XE5) ? 1 : 0, (F8 & kF8WE5) ? 1 : 0, 0, 0, 0, 0);
             }
         }
     };
@@ -173,86 +176,135 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_w8a8_kernel(const GemmArgs p
     }
 
     // ---- epilogue: lane owns column n = l%32 of each 32x32 block, register v owns row
-    //      8*(v/4) + 4*(l/32) + v%4
+    //      8*(v/4) + 4*(l/32) + v%4.  The element type of out / bias is a run-time choice here (this kernel is the
+    //      one that serves fp16 / fp32 modules): INT8 rounds to that type, then adds the bias in it (a second
+    //      rounding, dax/quant/nn/dynamic/linear.py:225-228); FP8 adds the bias in fp32 and rounds once (_scaled_mm).
+    auto epilogue = [&](auto KIND) {
+        constexpr int OK = decltype(KIND)::value;
+        auto round_out = [](float y) -> float {  // y rounded to the output type, as a float
+            if constexpr (OK == DAXQ_BF16) {
+                return bf16_bits_to_f32(f32_to_bf16_bits(y));
+            } else if constexpr (OK == DAXQ_F16) {
+                // The empty statement hides where y comes from.  Without it the instruction selector folds the fp32
+                // multiply (or add) that produced y and this conversion into one mixed-precision fma
+                // (v_fma_mixlo_f16), which rounds the exact product ONCE to fp16: on products whose fp32 rounding
+                // lands on an fp16 tie that is a different result from the two roundings the op sequence asks for.
+                asm volatile("" : "+v"(y));
+                return (float)(_Float16)y;
+            } else {
+                return y;
+            }
+        };
 #pragma unroll
-    for (int j = 0; j < NB; ++j) {
-        const int n = n0 + wn * TN + j * 32 + l31;
-        const bool n_ok = n < p.n;
-        const int nc = n_ok ? n : p.n - 1;
-        const float swv = p.sw[nc];
-        const float bv = p.bias ? bf16_bits_to_f32(p.bias[nc]) : 0.0f;
+        for (int j = 0; j < NB; ++j) {
+            const int n = n0 + wn * TN + j * 32 + l31;
+            const bool n_ok = n < p.n;
+            const int nc = n_ok ? n : p.n - 1;
+            const float swv = p.sw[nc];
+            float bv = 0.0f;
+            if (p.bias) {
+                if constexpr (OK == DAXQ_BF16) bv = bf16_bits_to_f32(p.bias[nc]);
+                else if constexpr (OK == DAXQ_F16) bv = (float)reinterpret_cast<const _Float16*>(p.bias)[nc];
+                else bv = reinterpret_cast<const float*>(p.bias)[nc];
+            }
 #pragma unroll
-        for (int i = 0; i < MB; ++i) {
+            for (int i = 0; i < MB; ++i) {
 #pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const int m = m0 + wm * TM + i * 32 + 8 * (v >> 2) + 4 * hi + (v & 3);
-                if (m < p.m && n_ok) {
-                    const float sxv = p.sx[m];
-                    uint32_t o;
-                    if constexpr (!FP8) {
-                        float y = (float)acc[i][j][v];  // v_cvt_f32_i32, round to nearest even
-                        y = y * sxv;
-                        y = y * swv;
-                        o = f32_to_bf16_bits(y);
-                        if (p.bias) o = f32_to_bf16_bits(bf16_bits_to_f32(o) + bv);
-                        if (p.acc) static_cast<int32_t*>(p.acc)[(int64_t)m * p.ldacc + n] = acc[i][j][v];
-                    } else {
-                        float y = acc[i][j][v] * sxv * swv + bv;
-                        o = f32_to_bf16_bits(y);
-                        if (p.acc) static_cast<float*>(p.acc)[(int64_t)m * p.ldacc + n] = acc[i][j][v];
+                for (int v = 0; v < 16; ++v) {
+                    const int m = m0 + wm * TM + i * 32 + 8 * (v >> 2) + 4 * hi + (v & 3);
+                    if (m < p.m && n_ok) {
+                        const float sxv = p.sx[m];
+                        float o;
+                        if constexpr (!FP8) {
+                            float y = (float)acc[i][j][v];  // v_cvt_f32_i32, round to nearest even
+                            y = y * sxv;
+                            y = y * swv;
+                            o = round_out(y);
+                            if (p.bias) o = round_out(o + bv);
+                            if (p.acc) static_cast<int32_t*>(p.acc)[(int64_t)m * p.ldacc + n] = acc[i][j][v];
+                        } else {
+                            o = round_out(acc[i][j][v] * sxv * swv + bv);
+                            if (p.acc) static_cast<float*>(p.acc)[(int64_t)m * p.ldacc + n] = acc[i][j][v];
+                        }
+                        const int64_t at = (int64_t)m * p.ldo + n;
+                        if constexpr (OK == DAXQ_BF16) p.out[at] = (uint16_t)(__float_as_uint(o) >> 16);
+                        else if constexpr (OK == DAXQ_F16) reinterpret_cast<_Float16*>(p.out)[at] = (_Float16)o;
+                        else reinterpret_cast<float*>(p.out)[at] = o;
                     }
-                    p.out[(int64_t)m * p.ldo + n] = (uint16_t)o;
                 }
             }
         }
-    }
+    };
+    if (p.out_kind == DAXQ_BF16) epilogue(std::integral_constant<int, DAXQ_BF16>{});
+    else if (p.out_kind == DAXQ_F16) epilogue(std::integral_constant<int, DAXQ_F16>{});
+    else epilogue(std::integral_constant<int, DAXQ_F32>{});
 }
-
-static int g_variant = 0;
-static int g_gm = 4;
 
 template <bool FP8>
 int launch_tile256(const GemmArgs& a, bool x_e5m2, hipStream_t st);
 bool tile256_applies(const GemmArgs& a);
 template <bool FP8>
-int launch_tile256s5(const GemmArgs& a, bool x_e5m2, bool wide, bool small, hipStream_t st);
+int launch_tile256s5(const GemmArgs& a, int f8, bool wide, bool small, hipStream_t st);
+template <bool FP8>
+int launch_tile128_splitk(const GemmArgs& a, int f8, hipStream_t st);
 
 int prepare_tile256_kernels();
 
-template <bool FP8, int BM, int BN, int BK, int WM, int WN, bool DIRECT, bool XE5 = false>
+template <bool FP8, int BM, int BN, int BK, int WM, int WN, bool DIRECT, int F8 = 0>
 static int prepare_cfg() {
-    static uint64_t lds_set = 0;  // per instantiation
-    return ensure_dynamic_lds(reinterpret_cast<const void*>(gemm_w8a8_kernel<FP8, BM, BN, BK, WM, WN, DIRECT, XE5>),
+    static std::atomic<uint64_t> lds_set{0};  // per instantiation
+    return ensure_dynamic_lds(reinterpret_cast<const void*>(gemm_w8a8_kernel<FP8, BM, BN, BK, WM, WN, DIRECT, F8>),
                               2 * (BM + BN) * BK, lds_set);
 }
 
-template <bool FP8, int BM, int BN, int BK, int WM, int WN, bool DIRECT, bool XE5 = false>
+template <bool FP8, int BM, int BN, int BK, int WM, int WN, bool DIRECT, int F8 = 0>
 static int launch_cfg(const GemmArgs& a0, hipStream_t st) {
     GemmArgs a = a0;
     a.tiles_m = (a.m + BM - 1) / BM;
     a.tiles_n = (a.n + BN - 1) / BN;
     constexpr int smem = 2 * (BM + BN) * BK;
-    auto kern = gemm_w8a8_kernel<FP8, BM, BN, BK, WM, WN, DIRECT, XE5>;
-    if (int rc = prepare_cfg<FP8, BM, BN, BK, WM, WN, DIRECT, XE5>()) return rc;
+    auto kern = gemm_w8a8_kernel<FP8, BM, BN, BK, WM, WN, DIRECT, F8>;
+    if (int rc = prepare_cfg<FP8, BM, BN, BK, WM, WN, DIRECT, F8>()) return rc;
     const int64_t nt = (int64_t)a.tiles_m * a.tiles_n;
     if (nt > 0x7fffffff) return fail(DAXQ_ERR_ARG, "gemm: too many tiles");
     hipLaunchKernelGGL(kern, dim3((unsigned)nt), dim3(WM * WN * 64), smem, st, a);
     return check_launch("gemm_w8a8");
 }
 
+// the generic kernel on BT x BT tiles for any FP8 operand pairing
+template <bool FP8, int BT>
+static int launch_generic(const GemmArgs& a, int f8, hipStream_t st) {
+    constexpr int WN = BT == 256 ? 4 : 2;
+    if constexpr (FP8) {
+        switch (f8) {
+            case 1: return launch_cfg<true, BT, BT, 128, 2, WN, true, 1>(a, st);
+            case 2: return launch_cfg<true, BT, BT, 128, 2, WN, true, 2>(a, st);
+            case 3: return launch_cfg<true, BT, BT, 128, 2, WN, true, 3>(a, st);
+            default: break;
+        }
+    }
+    return launch_cfg<FP8, BT, BT, 128, 2, WN, true, 0>(a, st);
+}
+
+// Kernel choices of the `kernel` argument (daxq_linear_w8a8): low 16 bits pick the implementation, bits 16-23 the
+// depth of the tile-order groups (0 = 4 tile rows).
+enum { K_DEFAULT = 0, K_GENERIC256 = 2, K_GENERIC128 = 5, K_TWO_STAGE = 6, K_FIVE_STAGE = 8, K_FIVE_STAGE_WIDE = 9, K_FIVE_STAGE_128 = 11 };
+
 template <bool FP8>
 static int launch_gemm(const void* xq, int64_t ld_xq, const float* sx, const void* wq, int64_t ld_wq, const float* sw,
                        const void* bias, void* out, int64_t ld_out, void* acc, int64_t ld_acc, int64_t m, int64_t n,
-                       int64_t k, hipStream_t st, bool x_e5m2 = false) {
+                       int64_t k, hipStream_t st, int f8 = 0, int out_kind = DAXQ_BF16, int kernel = 0) {
     if (m < 0 || n < 0 || k <= 0 || ld_xq < k || ld_wq < k || ld_out < n || (acc && ld_acc < n))
         return fail(DAXQ_ERR_ARG, "linear: bad shape m=%lld n=%lld k=%lld", (long long)m, (long long)n, (long long)k);
+    if (out_kind != DAXQ_BF16 && out_kind != DAXQ_F16 && out_kind != DAXQ_F32) return fail(DAXQ_ERR_ARG, "linear: unknown output type %d", out_kind);
     if (m == 0 || n == 0) return DAXQ_OK;
     if (!xq || !sx || !wq || !sw || !out) return fail(DAXQ_ERR_ARG, "linear: null pointer");
     if (m > 0x7fffffff || n > 0x7fffffff || k > 0x7fffffff) return fail(DAXQ_ERR_ARG, "linear: dimension exceeds int32");
     if (k % DAXQ_K_ALIGN != 0) return fail(DAXQ_ERR_ALIGN, "linear: k=%lld is not a multiple of %d (zero-pad the operands)", (long long)k, DAXQ_K_ALIGN);
     if (((uintptr_t)xq & 15) || ((uintptr_t)wq & 15) || (ld_xq & 15) || (ld_wq & 15))
         return fail(DAXQ_ERR_ALIGN, "linear: xq/wq must be 16-byte aligned with leading dimensions that are multiples of 16");
-    if (((uintptr_t)out & 1) || ((uintptr_t)sx & 3) || ((uintptr_t)sw & 3) || ((uintptr_t)bias & 1) || ((uintptr_t)acc & 3))
+    const uintptr_t oa = out_kind == DAXQ_F32 ? 3 : 1;
+    if (((uintptr_t)out & oa) || ((uintptr_t)sx & 3) || ((uintptr_t)sw & 3) || ((uintptr_t)bias & oa) || ((uintptr_t)acc & 3))
         return fail(DAXQ_ERR_ALIGN, "linear: misaligned out/scale/bias/acc pointer");
     GemmArgs a;
     a.a = static_cast<const uint8_t*>(xq);
@@ -270,68 +322,190 @@ static int launch_gemm(const void* xq, int64_t ld_xq, const float* sx, const voi
     a.n = (int)n;
     a.k = (int)k;
     a.tiles_m = a.tiles_n = 0;
-    a.gm = g_gm;
-    switch (g_variant) {
-        case 0: {
+    a.gm = (kernel >> 16) & 0xff ? (kernel >> 16) & 0xff : 4;
+    a.out_kind = out_kind;
+    a.splits = 1;
+    a.counters = nullptr;
+    a.partials = nullptr;
+    const int which = kernel & 0xffff;
+    const bool fits32 = a.lda < (1 << 26) && a.ldb < (1 << 26);  // 32-bit row offsets of the tiled kernels
+    if (out_kind != DAXQ_BF16 && which != K_DEFAULT && which != K_GENERIC256 && which != K_GENERIC128)
+        return fail(DAXQ_ERR_ARG, "linear: kernel %d writes bf16 only", which);
+    switch (which) {
+        case K_DEFAULT: {
+            // fp16 / fp32 outputs (modules that are not bf16): the generic kernel, which rounds to any of the three
+            if (out_kind != DAXQ_BF16)
+                return (m >= 256 && n >= 256) ? launch_generic<FP8, 256>(a, f8, st) : launch_generic<FP8, 128>(a, f8, st);
             // library default: the five-stage kernel on 256x256 tiles once there is one for every second CU, on
             // 128x128 tiles (4x as many workgroups, two per CU) below that, and the generic kernel for operands
             // smaller than one such tile.  Measured at N = K = 5120 (INT8, T-op/s, 128 / 256 tiles):
             // M = 512 -> 1127 / 551, M = 1024 (80 large tiles) -> 1275 / 1055, M = 2048 (160) -> 1542 / 1817;
             // 4096 x 1536 x 1536 (96) -> 1182 / 895, 8192 x 1536 x 1536 (192) -> 1517 / 1587.
             const int64_t tiles256 = ((m + 255) / 256) * ((n + 255) / 256);
-            if (tile256_applies(a) && tiles256 >= 128) return launch_tile256s5<FP8>(a, x_e5m2, false, false, st);
-            if (m >= 128 && n >= 128 && a.lda < (1 << 26) && a.ldb < (1 << 26)) return launch_tile256s5<FP8>(a, x_e5m2, false, true, st);
-            if constexpr (FP8) {
-                if (x_e5m2) return launch_cfg<true, 128, 128, 128, 2, 2, true, true>(a, st);
-            }
-            return launch_cfg<FP8, 128, 128, 128, 2, 2, true>(a, st);
+            if (tile256_applies(a) && tiles256 >= 128) return launch_tile256s5<FP8>(a, f8, false, false, st);
+            if (m >= 128 && n >= 128 && fits32) return launch_tile256s5<FP8>(a, f8, false, true, st);
+            return launch_generic<FP8, 128>(a, f8, st);
         }
-        case 2:
-            if (x_e5m2) return fail(DAXQ_ERR_ARG, "linear: gemm variant 2 has no e5m2 form");
-            return launch_cfg<FP8, 256, 256, 128, 2, 4, true>(a, st);
-        case 5:
-            if constexpr (FP8) {
-                if (x_e5m2) return launch_cfg<true, 128, 128, 128, 2, 2, true, true>(a, st);
-            }
-            return launch_cfg<FP8, 128, 128, 128, 2, 2, true>(a, st);
-        case 6:
+        case K_GENERIC256: return launch_generic<FP8, 256>(a, f8, st);
+        case K_GENERIC128: return launch_generic<FP8, 128>(a, f8, st);
+        case K_TWO_STAGE:
             if (!tile256_applies(a)) return fail(DAXQ_ERR_ARG, "linear: the 256x256 kernel needs m, n >= 256");
-            return launch_tile256<FP8>(a, x_e5m2, st);
-        case 8:
-        case 9:  // 9: INT8 with 32x32x32 MFMAs
+            if (f8 & kF8WE5) return fail(DAXQ_ERR_ARG, "linear: the two-stage kernel has no e5m2-weight form");
+            return launch_tile256<FP8>(a, f8 & kF8XE5, st);
+        case K_FIVE_STAGE:
+        case K_FIVE_STAGE_WIDE:  // INT8 with 32x32x32 MFMAs
             if (!tile256_applies(a)) return fail(DAXQ_ERR_ARG, "linear: the 256x256 kernel needs m, n >= 256");
-            return launch_tile256s5<FP8>(a, x_e5m2, g_variant == 9, false, st);
-        case 11:  // the five-stage kernel on 128x128 tiles
-            if (m < 128 || n < 128 || a.lda >= (1 << 26) || a.ldb >= (1 << 26)) return fail(DAXQ_ERR_ARG, "linear: the 128x128 kernel needs m, n >= 128");
-            return launch_tile256s5<FP8>(a, x_e5m2, false, true, st);
-        default: return fail(DAXQ_ERR_ARG, "linear: unknown gemm variant %d", g_variant);
+            return launch_tile256s5<FP8>(a, f8, which == K_FIVE_STAGE_WIDE, false, st);
+        case K_FIVE_STAGE_128:
+            if (m < 128 || n < 128 || !fits32) return fail(DAXQ_ERR_ARG, "linear: the 128x128 kernel needs m, n >= 128");
+            return launch_tile256s5<FP8>(a, f8, false, true, st);
+        default: return fail(DAXQ_ERR_ARG, "linear: unknown kernel choice %d", which);
     }
+}
+
+// ---- split-K: launches with too few 128x128 tiles to fill the CUs cut K into ranges ------------------------------
+constexpr int64_t kPartialBytes = 128 * 128 * 4;  // one workgroup's accumulators: 64 registers x 256 lanes
+
+static int64_t splitk_tiles(int64_t m, int64_t n) { return ((m + 127) / 128) * ((n + 127) / 128); }
+// The head of a workspace holds the tile counters.  Its size is fixed, not derived from the problem: a workspace is
+// reused by launches of different shapes, and the counters must stay zero between them, so no launch may ever put
+// partial results where another one keeps counters.
+constexpr int64_t kCounterBytes = 16384;
+constexpr int64_t kMaxSplitTiles = kCounterBytes / 4;
+
+// How many ranges pay: as many as keep every range at least 512 bytes of K deep, divide K / 128 evenly and do not put
+// more than two workgroups on a CU (two is what the LDS holds); 1 = no split.
+static int splitk_choice(int64_t m, int64_t n, int64_t k) {
+    if (m < 128 || n < 128 || k % DAXQ_K_ALIGN) return 1;
+    const int64_t tiles = splitk_tiles(m, n), units = k / DAXQ_K_ALIGN;
+    int best = 1;
+    for (int s = 2; s <= 8; ++s)
+        if (units % s == 0 && k / s >= 512 && tiles * s <= 512) best = s;
+    return tiles >= 256 ? 1 : best;
+}
+
+template <bool FP8>
+static int launch_gemm_splitk(const void* xq, int64_t ld_xq, const float* sx, const void* wq, int64_t ld_wq,
+                              const float* sw, const void* bias, void* out, int64_t ld_out, int64_t m, int64_t n, int64_t k,
+                              int splits, void* workspace, int64_t workspace_bytes, hipStream_t st, int f8) {
+    if (splits == 0) splits = splitk_choice(m, n, k);
+    if (splits <= 1)  // nothing to split (or not worth it): the plain launch, which needs no workspace
+        return launch_gemm<FP8>(xq, ld_xq, sx, wq, ld_wq, sw, bias, out, ld_out, nullptr, 0, m, n, k, st, f8);
+    if (m < 128 || n < 128) return fail(DAXQ_ERR_ARG, "linear_splitk: needs m, n >= 128 (got %lld, %lld)", (long long)m, (long long)n);
+    if (m > 0x7fffffff || n > 0x7fffffff || k <= 0 || k > 0x7fffffff || ld_xq < k || ld_wq < k || ld_out < n)
+        return fail(DAXQ_ERR_ARG, "linear_splitk: bad shape m=%lld n=%lld k=%lld", (long long)m, (long long)n, (long long)k);
+    if (k % DAXQ_K_ALIGN != 0 || (k / DAXQ_K_ALIGN) % splits != 0)
+        return fail(DAXQ_ERR_ALIGN, "linear_splitk: k=%lld does not divide into %d ranges that are multiples of %d", (long long)k, splits, DAXQ_K_ALIGN);
+    if (!xq || !sx || !wq || !sw || !out) return fail(DAXQ_ERR_ARG, "linear_splitk: null pointer");
+    if (((uintptr_t)xq & 15) || ((uintptr_t)wq & 15) || (ld_xq & 15) || (ld_wq & 15) || ld_xq >= (1 << 26) || ld_wq >= (1 << 26))
+        return fail(DAXQ_ERR_ALIGN, "linear_splitk: xq/wq must be 16-byte aligned with leading dimensions that are multiples of 16 below 2^26");
+    if (((uintptr_t)out & 1) || ((uintptr_t)sx & 3) || ((uintptr_t)sw & 3) || ((uintptr_t)bias & 1))
+        return fail(DAXQ_ERR_ALIGN, "linear_splitk: misaligned out/scale/bias pointer");
+    const int64_t tiles = splitk_tiles(m, n), cbytes = kCounterBytes;
+    if (tiles > kMaxSplitTiles) return fail(DAXQ_ERR_ARG, "linear_splitk: %lld output tiles, at most %lld (split-K is for launches with few tiles)", (long long)tiles, (long long)kMaxSplitTiles);
+    const int64_t need = cbytes + tiles * splits * kPartialBytes;
+    if (!workspace || ((uintptr_t)workspace & 255)) return fail(DAXQ_ERR_ALIGN, "linear_splitk: the workspace must be 256-byte aligned");
+    if (workspace_bytes < need)
+        return fail(DAXQ_ERR_ARG, "linear_splitk: workspace of %lld bytes, %lld needed for m=%lld n=%lld in %d ranges", (long long)workspace_bytes,
+                    (long long)need, (long long)m, (long long)n, splits);
+    GemmArgs a;
+    a.a = static_cast<const uint8_t*>(xq);
+    a.b = static_cast<const uint8_t*>(wq);
+    a.sx = sx;
+    a.sw = sw;
+    a.bias = static_cast<const uint16_t*>(bias);
+    a.out = static_cast<uint16_t*>(out);
+    a.acc = nullptr;
+    a.lda = ld_xq;
+    a.ldb = ld_wq;
+    a.ldo = ld_out;
+    a.ldacc = 0;
+    a.m = (int)m;
+    a.n = (int)n;
+    a.k = (int)k;
+    a.tiles_m = a.tiles_n = 0;
+    a.gm = 4;
+    a.out_kind = DAXQ_BF16;
+    a.splits = splits;
+    a.counters = static_cast<int32_t*>(workspace);
+    a.partials = static_cast<uint8_t*>(workspace) + cbytes;
+    return launch_tile128_splitk<FP8>(a, f8, st);
+}
+
+static int splitk_formats(int x_fmt, int w_fmt, bool& fp8, int& f8) {
+    const bool x8 = x_fmt == DAXQ_FMT_E4M3 || x_fmt == DAXQ_FMT_E5M2, w8 = w_fmt == DAXQ_FMT_E4M3 || w_fmt == DAXQ_FMT_E5M2;
+    if (x_fmt == DAXQ_FMT_I8 && w_fmt == DAXQ_FMT_I8) {
+        fp8 = false;
+        f8 = 0;
+        return DAXQ_OK;
+    }
+    if (x8 && w8) {
+        fp8 = true;
+        f8 = (x_fmt == DAXQ_FMT_E5M2 ? kF8XE5 : 0) | (w_fmt == DAXQ_FMT_E5M2 ? kF8WE5 : 0);
+        return DAXQ_OK;
+    }
+    return fail(DAXQ_ERR_ARG, "linear: unsupported operand formats x=%d w=%d (int8 x int8, or fp8 x fp8)", x_fmt, w_fmt);
 }
 
 }  // namespace daxq
 
 extern "C" {
 
+int daxq_linear_splitk_choice(int64_t m, int64_t n, int64_t k) { return daxq::splitk_choice(m, n, k); }
+
+int64_t daxq_linear_splitk_workspace_bytes(int64_t m, int64_t n, int splits) {
+    using namespace daxq;
+    if (m <= 0 || n <= 0 || splits <= 1) return 0;
+    return kCounterBytes + splitk_tiles(m, n) * splits * kPartialBytes;
+}
+
+int daxq_linear_w8a8_splitk(int x_fmt, int w_fmt, const void* xq, int64_t ld_xq, const float* sx, const void* wq,
+                            int64_t ld_wq, const float* sw, const void* bias, void* out, int64_t ld_out, int64_t m,
+                            int64_t n, int64_t k, int splits, void* workspace, int64_t workspace_bytes,
+                            daxq_stream_t stream) {
+    using namespace daxq;
+    bool fp8;
+    int f8;
+    if (int rc = splitk_formats(x_fmt, w_fmt, fp8, f8)) return rc;
+    if (splits < 0 || splits > 64) return fail(DAXQ_ERR_ARG, "linear_splitk: splits must be 0 (library's choice) to 64");
+    return fp8 ? launch_gemm_splitk<true>(xq, ld_xq, sx, wq, ld_wq, sw, bias, out, ld_out, m, n, k, splits, workspace,
+                                          workspace_bytes, (hipStream_t)stream, f8)
+               : launch_gemm_splitk<false>(xq, ld_xq, sx, wq, ld_wq, sw, bias, out, ld_out, m, n, k, splits, workspace,
+                                           workspace_bytes, (hipStream_t)stream, 0);
+}
+
 int daxq_init(void) {
     using namespace daxq;
     int rc = prepare_tile256_kernels();
-    if (!rc) rc = prepare_cfg<false, 128, 128, 128, 2, 2, true>();
-    if (!rc) rc = prepare_cfg<true, 128, 128, 128, 2, 2, true>();
-    if (!rc) rc = prepare_cfg<true, 128, 128, 128, 2, 2, true, true>();
-    if (!rc) rc = prepare_cfg<false, 256, 256, 128, 2, 4, true>();
-    if (!rc) rc = prepare_cfg<true, 256, 256, 128, 2, 4, true>();
+#define DAXQ_PREP_ALL(FP8, BT, WN)                                        \
+    if (!rc) rc = prepare_cfg<FP8, BT, BT, 128, 2, WN, true, 0>();
+    DAXQ_PREP_ALL(false, 128, 2)
+    DAXQ_PREP_ALL(false, 256, 4)
+    DAXQ_PREP_ALL(true, 128, 2)
+    DAXQ_PREP_ALL(true, 256, 4)
+#undef DAXQ_PREP_ALL
+#define DAXQ_PREP_F8(F8)                                                  \
+    if (!rc) rc = prepare_cfg<true, 128, 128, 128, 2, 2, true, F8>();      \
+    if (!rc) rc = prepare_cfg<true, 256, 256, 128, 2, 4, true, F8>();
+    DAXQ_PREP_F8(1)
+    DAXQ_PREP_F8(2)
+    DAXQ_PREP_F8(3)
+#undef DAXQ_PREP_F8
     return rc;
 }
 
-int daxq_set_gemm_variant(int variant) {
-    if (variant >= 1000 && variant < 1064) {  // tuning hook: 1000 + depth of the tile-order groups
-        daxq::g_gm = variant - 1000 > 0 ? variant - 1000 : 4;
-        return DAXQ_OK;
-    }
-    if (variant != 0 && variant != 2 && variant != 5 && variant != 6 && variant != 8 && variant != 9 && variant != 11)
-        return daxq::fail(DAXQ_ERR_ARG, "unknown gemm variant %d", variant);
-    daxq::g_variant = variant;
-    return DAXQ_OK;
+int daxq_linear_w8a8(int x_fmt, int w_fmt, int out_dtype, const void* xq, int64_t ld_xq, const float* sx, const void* wq,
+                     int64_t ld_wq, const float* sw, const void* bias, void* out, int64_t ld_out, void* acc,
+                     int64_t ld_acc, int64_t m, int64_t n, int64_t k, int kernel, daxq_stream_t stream) {
+    using namespace daxq;
+    const bool x8 = x_fmt == DAXQ_FMT_E4M3 || x_fmt == DAXQ_FMT_E5M2, w8 = w_fmt == DAXQ_FMT_E4M3 || w_fmt == DAXQ_FMT_E5M2;
+    if (x_fmt == DAXQ_FMT_I8 && w_fmt == DAXQ_FMT_I8)
+        return launch_gemm<false>(xq, ld_xq, sx, wq, ld_wq, sw, bias, out, ld_out, acc, ld_acc, m, n, k, (hipStream_t)stream, 0,
+                                  out_dtype, kernel);
+    if (x8 && w8)
+        return launch_gemm<true>(xq, ld_xq, sx, wq, ld_wq, sw, bias, out, ld_out, acc, ld_acc, m, n, k, (hipStream_t)stream,
+                                 (x_fmt == DAXQ_FMT_E5M2 ? kF8XE5 : 0) | (w_fmt == DAXQ_FMT_E5M2 ? kF8WE5 : 0), out_dtype, kernel);
+    return fail(DAXQ_ERR_ARG, "linear: unsupported operand formats x=%d w=%d (int8 x int8, or fp8 x fp8)", x_fmt, w_fmt);
 }
 
 int daxq_linear_i8(const int8_t* xq, int64_t ld_xq, const float* sx, const int8_t* wq, int64_t ld_wq, const float* sw,
@@ -348,12 +522,11 @@ int daxq_linear_e4m3(const uint8_t* xq, int64_t ld_xq, const float* sx, const ui
                                    (hipStream_t)stream);
 }
 
-
 int daxq_linear_e5m2_e4m3(const uint8_t* xq, int64_t ld_xq, const float* sx, const uint8_t* wq, int64_t ld_wq,
                           const float* sw, const void* bias, void* out, int64_t ld_out, float* acc, int64_t ld_acc,
                           int64_t m, int64_t n, int64_t k, daxq_stream_t stream) {
     return daxq::launch_gemm<true>(xq, ld_xq, sx, wq, ld_wq, sw, bias, out, ld_out, acc, ld_acc, m, n, k,
-                                   (hipStream_t)stream, true);
+                                   (hipStream_t)stream, daxq::kF8XE5);
 }
 
 }  // extern "C"

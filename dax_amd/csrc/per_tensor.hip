@@ -48,9 +48,10 @@ __global__ __launch_bounds__(kRedThreads) void tensor_scale_kernel(const float* 
         hi = max_nan(hi, mx[i]);
     }
     block_minmax(lo, hi, s_lo, s_hi);
-    const float amax = max_nan(-lo, hi);  // = max |x|: exact, the inputs are bf16 values
+    const float amax = max_nan(-lo, hi);  // = max |x|: exact, the statistics are the tensor's own values
     float s = amax / qmax;              // IEEE division
-    if (round_bf16) s = bf16_bits_to_f32(f32_to_bf16_bits(s));
+    if (round_bf16 == 1) s = round_to_x<DAXQ_BF16>(s);  // the quotient is rounded to the tensor's own element type
+    else if (round_bf16 == 2) s = round_to_x<DAXQ_F16>(s);
     s = max_nan(s, kEps);
     if (threadIdx.x == 0) scale1[0] = s;
     for (int64_t i = threadIdx.x; i < n_expand; i += kRedThreads) expand[i] = s;

@@ -15,12 +15,37 @@ __device__ __forceinline__ uint32_t pk_max_u16(uint32_t a, uint32_t b) {
     return __builtin_bit_cast(uint32_t, r);
 }
 
-// abs-max bits (sign cleared) of a row -> fp32 scale, exactly as the reference rounds it
-template <bool ROUND_BF16>
+// Element type of the tensor being quantised: XT = DAXQ_BF16 / DAXQ_F16 (two per 32-bit word) / DAXQ_F32.
+// The bit pattern of a non-negative value orders like the value in all three, NaN above infinity.
+template <int XT>
+__device__ __forceinline__ float x_bits_to_f32(uint32_t b) {
+    if constexpr (XT == DAXQ_BF16) return __uint_as_float(b << 16);
+    else if constexpr (XT == DAXQ_F16) return (float)__builtin_bit_cast(_Float16, (uint16_t)b);
+    else return __uint_as_float(b);
+}
+
+// f32 rounded to the element type (round to nearest even, subnormals of fp16 included), as a float
+template <int XT>
+__device__ __forceinline__ float round_to_x(float s) {
+    if constexpr (XT == DAXQ_BF16) {
+        if (s != s) return s;
+        return bf16_bits_to_f32(f32_to_bf16_bits(s));
+    } else if constexpr (XT == DAXQ_F16) {
+        asm volatile("" : "+v"(s));  // keeps the conversion a conversion (no fold with the operation that produced s)
+        return (float)(_Float16)s;
+    } else {
+        return s;
+    }
+}
+
+// abs-max bits (sign cleared) of a block -> fp32 scale, exactly as the reference rounds it: the quotient is
+// computed and floored in the tensor's own dtype when ROUND (dynamic activations,
+// dax/quant/nn/dynamic/functional.py:124-129), in fp32 otherwise (weight observer).
+template <bool ROUND, int XT = DAXQ_BF16>
 __device__ __forceinline__ float scale_from_amax_bits(uint32_t amax_bits, float qmax) {
-    float a = bf16_bits_to_f32(amax_bits);
+    float a = x_bits_to_f32<XT>(amax_bits);
     float s = a / qmax;  // IEEE binary32 division (hipcc default: correctly rounded)
-    if (ROUND_BF16) s = bf16_bits_to_f32(f32_to_bf16_bits(s));
+    if (ROUND) s = round_to_x<XT>(s);
     return max_nan(s, kEps);  // clamp(min=eps): a NaN abs-max (a NaN anywhere in the row) stays NaN
 }
 
@@ -103,17 +128,25 @@ __device__ __forceinline__ int cvt_pk_f8(float a, float b, int old, bool hi) {
         return hi ? __builtin_amdgcn_cvt_pk_fp8_f32(a, b, old, true) : __builtin_amdgcn_cvt_pk_fp8_f32(a, b, old, false);
 }
 
-// 8 bf16 (one 16-byte chunk) -> 8 quantised bytes
-template <int FMT, bool TRUE_DIV = false>
+// 8 bf16 / fp16 values (one 16-byte chunk) -> 8 quantised bytes
+template <int FMT, bool TRUE_DIV = false, int XT = DAXQ_BF16>
 __device__ __forceinline__ uint2 quant_chunk(const uint4& v, float s, float inv) {
     const uint32_t w[4] = {v.x, v.y, v.z, v.w};
     uint32_t o[2];
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
-        float f0 = __uint_as_float(w[2 * h] << 16);
-        float f1 = __uint_as_float(w[2 * h] & 0xffff0000u);
-        float f2 = __uint_as_float(w[2 * h + 1] << 16);
-        float f3 = __uint_as_float(w[2 * h + 1] & 0xffff0000u);
+        float f0, f1, f2, f3;
+        if constexpr (XT == DAXQ_BF16) {
+            f0 = __uint_as_float(w[2 * h] << 16);
+            f1 = __uint_as_float(w[2 * h] & 0xffff0000u);
+            f2 = __uint_as_float(w[2 * h + 1] << 16);
+            f3 = __uint_as_float(w[2 * h + 1] & 0xffff0000u);
+        } else {
+            f0 = x_bits_to_f32<XT>(w[2 * h] & 0xffffu);
+            f1 = x_bits_to_f32<XT>(w[2 * h] >> 16);
+            f2 = x_bits_to_f32<XT>(w[2 * h + 1] & 0xffffu);
+            f3 = x_bits_to_f32<XT>(w[2 * h + 1] >> 16);
+        }
         if (FMT != 0) {
             int p = cvt_pk_f8<FMT>(q_f8_pre<FMT, TRUE_DIV>(f0, s, inv), q_f8_pre<FMT, TRUE_DIV>(f1, s, inv), 0, false);
             p = cvt_pk_f8<FMT>(q_f8_pre<FMT, TRUE_DIV>(f2, s, inv), q_f8_pre<FMT, TRUE_DIV>(f3, s, inv), p, true);

@@ -1,4 +1,4 @@
-// Row-wise symmetric quantisation of a bf16 matrix to int8 or OCP e4m3fn.
+// Row-wise symmetric quantisation of a bf16 / fp16 / fp32 matrix to int8, OCP e4m3fn or OCP e5m2.
 //
 // One launch covers both uses on the path:
 //   * dynamic per-token activation quantisation (scale rounded to bf16 first, as
@@ -22,7 +22,8 @@ namespace daxq {
 // Requires k % 8 == 0, ld_x % 8 == 0, ld_q % 8 == 0, 16-byte aligned x, 8-byte aligned q,
 // and ld_q / 8 <= NCH * 64.
 // SCALE_IN: the per-row scale is an input (leaf quantiser) instead of being derived from the row.
-template <int NCH, int FMT, bool ROUND_BF16, bool SCALE_IN>
+// XT: element type of x, DAXQ_BF16 or DAXQ_F16 (8 elements per 16-byte chunk either way).
+template <int NCH, int FMT, bool ROUND_BF16, bool SCALE_IN, int XT = DAXQ_BF16>
 __global__ __launch_bounds__(256) void quant_rows_wave(const uint16_t* __restrict__ x, int64_t m, int k,
                                                        int64_t ld_x, uint8_t* __restrict__ q, int64_t ld_q,
                                                        float* __restrict__ scale, float qmax) {
@@ -57,7 +58,7 @@ __global__ __launch_bounds__(256) void quant_rows_wave(const uint16_t* __restric
         }
         uint32_t amax = (mx & 0xffffu) > (mx >> 16) ? (mx & 0xffffu) : (mx >> 16);
         amax = wave_max_u32(amax);
-        s = scale_from_amax_bits<ROUND_BF16>(amax, qmax);
+        s = scale_from_amax_bits<ROUND_BF16, XT>(amax, qmax);
         if (lane == 0) scale[row] = s;
     }
     const float inv = 1.0f / s;  // IEEE division, not v_rcp_f32
@@ -67,28 +68,40 @@ __global__ __launch_bounds__(256) void quant_rows_wave(const uint16_t* __restric
     for (int i = 0; i < NCH; ++i) {
         const int c = i * 64 + lane;
         if (c < nch) {
-            store_stream_8(qr + c, quant_chunk<FMT, SCALE_IN>(v[i], s, inv));
+            // the reciprocal sequence of the FP8 forms is verified exhaustively for bf16 elements; fp16 rows divide
+            store_stream_8(qr + c, quant_chunk<FMT, SCALE_IN || XT != DAXQ_BF16, XT>(v[i], s, inv));
         } else if (c < npad) {
             store_stream_8(qr + c, make_uint2(0, 0));
         }
     }
 }
 
-// General path: any k / alignment / row length; one 256-thread block per row, two passes.
-template <int FMT, bool ROUND_BF16, bool SCALE_IN>
-__global__ __launch_bounds__(256) void quant_rows_block(const uint16_t* __restrict__ x, int64_t m, int64_t k,
+// General path: any k / alignment / row length / element type; one 256-thread block per row, two passes.
+template <int XT>
+struct XWord {
+    typedef uint16_t type;
+};
+template <>
+struct XWord<DAXQ_F32> {
+    typedef uint32_t type;
+};
+
+template <int FMT, bool ROUND_BF16, bool SCALE_IN, int XT = DAXQ_BF16>
+__global__ __launch_bounds__(256) void quant_rows_block(const void* __restrict__ xv, int64_t m, int64_t k,
                                                         int64_t ld_x, uint8_t* __restrict__ q, int64_t ld_q,
                                                         float* __restrict__ scale, float qmax) {
+    typedef typename XWord<XT>::type word_t;
+    constexpr uint32_t kAbs = XT == DAXQ_F32 ? 0x7fffffffu : 0x7fffu;
     __shared__ uint32_t red[4];
     const int64_t row = blockIdx.x;
-    const uint16_t* xr = x + row * ld_x;
+    const word_t* xr = static_cast<const word_t*>(xv) + row * ld_x;
     float s;
     if constexpr (SCALE_IN) {
         s = scale[row];
     } else {
         uint32_t mx = 0;
         for (int64_t c = threadIdx.x; c < k; c += 256) {
-            uint32_t a = xr[c] & 0x7fffu;
+            uint32_t a = xr[c] & kAbs;
             mx = a > mx ? a : mx;
         }
         mx = wave_max_u32(mx);
@@ -98,7 +111,7 @@ __global__ __launch_bounds__(256) void quant_rows_block(const uint16_t* __restri
         amax = red[1] > amax ? red[1] : amax;
         amax = red[2] > amax ? red[2] : amax;
         amax = red[3] > amax ? red[3] : amax;
-        s = scale_from_amax_bits<ROUND_BF16>(amax, qmax);
+        s = scale_from_amax_bits<ROUND_BF16, XT>(amax, qmax);
         if (threadIdx.x == 0) scale[row] = s;
     }
     const float inv = 1.0f / s;
@@ -106,9 +119,10 @@ __global__ __launch_bounds__(256) void quant_rows_block(const uint16_t* __restri
     for (int64_t c = threadIdx.x; c < ld_q; c += 256) {
         uint8_t o = 0;
         if (c < k) {
-            float f = bf16_bits_to_f32(xr[c]);
+            float f = x_bits_to_f32<XT>(xr[c]);
             if (FMT != 0) {
-                o = (uint8_t)(cvt_pk_f8<FMT>(q_f8_pre<FMT, SCALE_IN>(f, s, inv), 0.0f, 0, false) & 0xff);
+                // the reciprocal sequence is verified exhaustively for bf16 elements only; other types divide
+                o = (uint8_t)(cvt_pk_f8<FMT>(q_f8_pre<FMT, SCALE_IN || XT != DAXQ_BF16>(f, s, inv), 0.0f, 0, false) & 0xff);
             } else {
                 o = (uint8_t)(q_i8_bits(f, inv) & 0xffu);
             }
@@ -117,52 +131,79 @@ __global__ __launch_bounds__(256) void quant_rows_block(const uint16_t* __restri
     }
 }
 
-template <int FMT, bool ROUND_BF16, bool SCALE_IN>
-static int launch_quant_rows(const void* x, int64_t m, int64_t k, int64_t ld_x, void* q, int64_t ld_q, float* scale,
-                             float qmax, hipStream_t st) {
+template <int FMT, bool ROUND_BF16, bool SCALE_IN, int XT>
+static int launch_quant_rows_t(const void* x, int64_t m, int64_t k, int64_t ld_x, void* q, int64_t ld_q, float* scale,
+                               float qmax, hipStream_t st) {
+    constexpr int XB = XT == DAXQ_F32 ? 4 : 2;
     if (m < 0 || k <= 0 || ld_x < k || ld_q < k) return fail(DAXQ_ERR_ARG, "quant_rows: bad shape m=%lld k=%lld ld_x=%lld ld_q=%lld",
                                                                (long long)m, (long long)k, (long long)ld_x, (long long)ld_q);
     if (m == 0) return DAXQ_OK;
     if (!x || !q || !scale) return fail(DAXQ_ERR_ARG, "quant_rows: null pointer");
-    if (((uintptr_t)x & 1) != 0 || ((uintptr_t)scale & 3) != 0) return fail(DAXQ_ERR_ALIGN, "quant_rows: x must be 2-byte and scale 4-byte aligned");
-    const uint16_t* xp = static_cast<const uint16_t*>(x);
+    if (((uintptr_t)x & (XB - 1)) != 0 || ((uintptr_t)scale & 3) != 0) return fail(DAXQ_ERR_ALIGN, "quant_rows: x must be element aligned and scale 4-byte aligned");
     uint8_t* qp = static_cast<uint8_t*>(q);
-    const bool vec_ok = (k % 8 == 0) && (ld_x % 8 == 0) && (ld_q % 8 == 0) && (((uintptr_t)x & 15) == 0) &&
-                        (((uintptr_t)q & 7) == 0) && (ld_q / 8 <= 36 * 64) && (m <= (int64_t)4 * 0x7fffffff);
-    if (vec_ok) {
-        const int nchunks = (int)((ld_q / 8 + 63) / 64);
-        const dim3 grid((unsigned)((m + 3) / 4)), block(256);
+    if constexpr (XT != DAXQ_F32) {
+        const uint16_t* xp = static_cast<const uint16_t*>(x);
+        const bool vec_ok = (k % 8 == 0) && (ld_x % 8 == 0) && (ld_q % 8 == 0) && (((uintptr_t)x & 15) == 0) &&
+                            (((uintptr_t)q & 7) == 0) && (ld_q / 8 <= 36 * 64) && (m <= (int64_t)4 * 0x7fffffff);
+        if (vec_ok) {
+            const int nchunks = (int)((ld_q / 8 + 63) / 64);
+            const dim3 grid((unsigned)((m + 3) / 4)), block(256);
 #define DAXQ_Q_CASE(N)                                                                                      \
     if (nchunks <= N) {                                                                                     \
-        hipLaunchKernelGGL((quant_rows_wave<N, FMT, ROUND_BF16, SCALE_IN>), grid, block, 0, st, xp, m, (int)k, ld_x, qp, \
+        hipLaunchKernelGGL((quant_rows_wave<N, FMT, ROUND_BF16, SCALE_IN, XT>), grid, block, 0, st, xp, m, (int)k, ld_x, qp, \
                            ld_q, scale, qmax);                                                              \
         return check_launch("quant_rows_wave");                                                             \
     }
-        DAXQ_Q_CASE(2)
-        DAXQ_Q_CASE(4)
-        DAXQ_Q_CASE(8)
-        DAXQ_Q_CASE(12)
-        DAXQ_Q_CASE(20)
-        DAXQ_Q_CASE(28)
-        DAXQ_Q_CASE(36)
+            DAXQ_Q_CASE(2)
+            DAXQ_Q_CASE(4)
+            DAXQ_Q_CASE(8)
+            DAXQ_Q_CASE(12)
+            DAXQ_Q_CASE(20)
+            DAXQ_Q_CASE(28)
+            DAXQ_Q_CASE(36)
 #undef DAXQ_Q_CASE
+        }
     }
     if (m > 0x7fffffff) return fail(DAXQ_ERR_ARG, "quant_rows: too many rows for the general kernel");
-    hipLaunchKernelGGL((quant_rows_block<FMT, ROUND_BF16, SCALE_IN>), dim3((unsigned)m), dim3(256), 0, st, xp, m, k, ld_x, qp,
+    hipLaunchKernelGGL((quant_rows_block<FMT, ROUND_BF16, SCALE_IN, XT>), dim3((unsigned)m), dim3(256), 0, st, x, m, k, ld_x, qp,
                        ld_q, scale, qmax);
     return check_launch("quant_rows_block");
 }
 
+template <int FMT, bool ROUND_BF16, bool SCALE_IN>
+static int launch_quant_rows(const void* x, int64_t m, int64_t k, int64_t ld_x, void* q, int64_t ld_q, float* scale,
+                             float qmax, hipStream_t st, int x_dtype = DAXQ_BF16) {
+    switch (x_dtype) {
+        case DAXQ_BF16: return launch_quant_rows_t<FMT, ROUND_BF16, SCALE_IN, DAXQ_BF16>(x, m, k, ld_x, q, ld_q, scale, qmax, st);
+        case DAXQ_F16: return launch_quant_rows_t<FMT, ROUND_BF16, SCALE_IN, DAXQ_F16>(x, m, k, ld_x, q, ld_q, scale, qmax, st);
+        case DAXQ_F32: return launch_quant_rows_t<FMT, ROUND_BF16, SCALE_IN, DAXQ_F32>(x, m, k, ld_x, q, ld_q, scale, qmax, st);
+        default: return fail(DAXQ_ERR_ARG, "quant_rows: unknown element type %d", x_dtype);
+    }
+}
 
-// Per-row min and max of a bf16 matrix in fp32 (weight observer statistics).
-__global__ __launch_bounds__(256) void row_minmax_kernel(const uint16_t* __restrict__ x, int64_t k, int64_t ld_x,
+template <bool ROUND_BF16, bool SCALE_IN>
+static int launch_quant_rows_fmt(int q_fmt, const void* x, int x_dtype, int64_t m, int64_t k, int64_t ld_x, void* q,
+                                 int64_t ld_q, float* scale, hipStream_t st) {
+    switch (q_fmt) {
+        case DAXQ_FMT_I8: return launch_quant_rows<0, ROUND_BF16, SCALE_IN>(x, m, k, ld_x, q, ld_q, scale, 127.0f, st, x_dtype);
+        case DAXQ_FMT_E4M3: return launch_quant_rows<1, ROUND_BF16, SCALE_IN>(x, m, k, ld_x, q, ld_q, scale, 448.0f, st, x_dtype);
+        case DAXQ_FMT_E5M2: return launch_quant_rows<2, ROUND_BF16, SCALE_IN>(x, m, k, ld_x, q, ld_q, scale, 57344.0f, st, x_dtype);
+        default: return fail(DAXQ_ERR_ARG, "quant_rows: unknown quantised format %d", q_fmt);
+    }
+}
+
+
+// Per-row min and max of a bf16 / fp16 / fp32 matrix in fp32 (weight observer statistics).
+template <int XT>
+__global__ __launch_bounds__(256) void row_minmax_kernel(const void* __restrict__ xv, int64_t k, int64_t ld_x,
                                                          float* __restrict__ mn, float* __restrict__ mx) {
+    typedef typename XWord<XT>::type word_t;
     __shared__ float rlo[4], rhi[4];
     const int64_t row = blockIdx.x;
-    const uint16_t* xr = x + row * ld_x;
+    const word_t* xr = static_cast<const word_t*>(xv) + row * ld_x;
     float lo = __builtin_inff(), hi = -__builtin_inff();
     for (int64_t c = threadIdx.x; c < k; c += 256) {
-        float f = bf16_bits_to_f32(xr[c]);
+        float f = x_bits_to_f32<XT>(xr[c]);
         lo = min_nan(lo, f);
         hi = max_nan(hi, f);
     }
@@ -229,15 +270,36 @@ int daxq_quantize_rows_e5m2(const void* x, int64_t m, int64_t k, int64_t ld_x, c
                                                       (hipStream_t)stream);
 }
 
-int daxq_row_minmax(const void* x, int64_t m, int64_t k, int64_t ld_x, float* min_out, float* max_out,
-                    daxq_stream_t stream) {
+int daxq_row_minmax_t(const void* x, int x_dtype, int64_t m, int64_t k, int64_t ld_x, float* min_out, float* max_out,
+                      daxq_stream_t stream) {
     using namespace daxq;
     if (m < 0 || k <= 0 || ld_x < k || m > 0x7fffffff) return fail(DAXQ_ERR_ARG, "row_minmax: bad shape m=%lld k=%lld", (long long)m, (long long)k);
     if (m == 0) return DAXQ_OK;
     if (!x || !min_out || !max_out) return fail(DAXQ_ERR_ARG, "row_minmax: null pointer");
-    hipLaunchKernelGGL(row_minmax_kernel, dim3((unsigned)m), dim3(256), 0, (hipStream_t)stream,
-                       static_cast<const uint16_t*>(x), k, ld_x, min_out, max_out);
+    const dim3 grid((unsigned)m), block(256);
+    switch (x_dtype) {
+        case DAXQ_BF16: hipLaunchKernelGGL(row_minmax_kernel<DAXQ_BF16>, grid, block, 0, (hipStream_t)stream, x, k, ld_x, min_out, max_out); break;
+        case DAXQ_F16: hipLaunchKernelGGL(row_minmax_kernel<DAXQ_F16>, grid, block, 0, (hipStream_t)stream, x, k, ld_x, min_out, max_out); break;
+        case DAXQ_F32: hipLaunchKernelGGL(row_minmax_kernel<DAXQ_F32>, grid, block, 0, (hipStream_t)stream, x, k, ld_x, min_out, max_out); break;
+        default: return fail(DAXQ_ERR_ARG, "row_minmax: unknown element type %d", x_dtype);
+    }
     return check_launch("row_minmax");
+}
+
+int daxq_row_minmax(const void* x, int64_t m, int64_t k, int64_t ld_x, float* min_out, float* max_out,
+                    daxq_stream_t stream) {
+    return daxq_row_minmax_t(x, DAXQ_BF16, m, k, ld_x, min_out, max_out, stream);
+}
+
+int daxq_act_quant_rows(const void* x, int x_dtype, int q_fmt, int64_t m, int64_t k, int64_t ld_x, void* q, int64_t ld_q,
+                        float* scale, daxq_stream_t stream) {
+    return daxq::launch_quant_rows_fmt<true, false>(q_fmt, x, x_dtype, m, k, ld_x, q, ld_q, scale, (hipStream_t)stream);
+}
+
+int daxq_quantize_rows(const void* x, int x_dtype, int q_fmt, int64_t m, int64_t k, int64_t ld_x, const float* scale,
+                       void* q, int64_t ld_q, daxq_stream_t stream) {
+    return daxq::launch_quant_rows_fmt<false, true>(q_fmt, x, x_dtype, m, k, ld_x, q, ld_q, const_cast<float*>(scale),
+                                                    (hipStream_t)stream);
 }
 
 int daxq_scale_from_minmax(const float* min_in, const float* max_in, int64_t n, float qmax, float* scale,

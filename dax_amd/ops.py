@@ -6,7 +6,7 @@ surrounding ``torch.compile`` graph can trace through it.  No op has a CPU kerne
 """
 from __future__ import annotations
 
-from typing import Optional, Tuple
+from typing import List, Optional, Tuple
 
 import torch
 
@@ -71,6 +71,24 @@ def _same_device(what: str, ref: torch.Tensor, **others) -> None:
                              f"and the first operand on {ref.device}")
 
 
+FLOAT_KIND = {torch.bfloat16: 0, torch.float16: 1, torch.float32: 2}  # DAXQ_BF16 / DAXQ_F16 / DAXQ_F32
+FMT = {"i8": 0, "e4m3": 1, "e5m2": 2}  # DAXQ_FMT_*
+FMT_OF_DTYPE = {torch.int8: "i8", torch.float8_e4m3fn: "e4m3", torch.float8_e5m2: "e5m2"}
+QMAX = {"i8": 127.0, "e4m3": 448.0, "e5m2": 57344.0}
+
+
+def _rows_float(x: torch.Tensor, what: str) -> int:
+    """Checks a [rows, K] matrix of one of the element types the reference's quantisers accept
+    (dax/quant/nn/dynamic/functional.py:99-103) and returns its DAXQ_* type code."""
+    _need_gpu(x, what)
+    if x.dtype not in FLOAT_KIND:
+        raise AssertionError(f"Unsupported input dtype: {x.dtype}")
+    if x.dim() != 2 or x.stride(1) != 1:
+        raise ValueError(f"daxq::{what}: expected a 2-d tensor with contiguous rows, got shape {tuple(x.shape)} "
+                         f"strides {x.stride()}")
+    return FLOAT_KIND[x.dtype]
+
+
 def _rows_bf16(x: torch.Tensor, what: str) -> None:
     _need_gpu(x, what)
     if x.dtype != torch.bfloat16:
@@ -82,23 +100,24 @@ def _rows_bf16(x: torch.Tensor, what: str) -> None:
 
 # ----------------------------------------------------------------------------- act quant
 def _act_quant(x: torch.Tensor, fp8, e5m2: bool = False) -> Tuple[torch.Tensor, torch.Tensor]:
-    name = "act_quant_e5m2" if e5m2 else "act_quant_e4m3" if fp8 else "act_quant_i8"
-    _rows_bf16(x, name)
+    fmt = "e5m2" if e5m2 else "e4m3" if fp8 else "i8"
+    name = "act_quant_" + fmt
+    kind = _rows_float(x, name)
     m, k = x.shape
     kp = pad_k(k)
     with _on_device(x):
         q = torch.empty((m, kp), dtype=torch.uint8 if fp8 else torch.int8, device=x.device)
         s = torch.empty((m,), dtype=torch.float32, device=x.device)
         if m:
-            fn = getattr(_capi.lib(), "daxq_" + name)
             ld_x = x.stride(0) if m > 1 else k
-            _capi.check(fn(x.data_ptr(), m, k, ld_x, q.data_ptr(), kp, s.data_ptr(), _stream(x)), name)
+            _capi.check(_capi.lib().daxq_act_quant_rows(x.data_ptr(), kind, FMT[fmt], m, k, ld_x, q.data_ptr(), kp,
+                                                        s.data_ptr(), _stream(x)), name)
     return q, s
 
 
 @torch.library.custom_op("daxq::act_quant_i8", mutates_args=(), device_types="cuda")
 def act_quant_i8(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
-    """bf16 [M,K] -> (int8 [M, pad128(K)] zero padded, fp32 [M] per-token scale)."""
+    """bf16 / fp16 / fp32 [M,K] -> (int8 [M, pad128(K)] zero padded, fp32 [M] per-token scale)."""
     return _act_quant(x, False)
 
 
@@ -231,7 +250,7 @@ gelu_tanh_act_quant_e5m2.register_fake(lambda x, want_y=False: _fused_fake(x, "e
 # ----------------------------------------------------------------------------- leaf quantisers
 def _quantize_rows(x: torch.Tensor, scale: torch.Tensor, fmt: str, padded: bool) -> torch.Tensor:
     name = "quantize_rows_" + fmt
-    _rows_bf16(x, name)
+    kind = _rows_float(x, name)
     m, k = x.shape
     if scale.dtype != torch.float32 or scale.numel() != m or scale.device != x.device:
         raise ValueError(f"daxq::{name}: scale must be fp32 with one value per row on {x.device}")
@@ -240,9 +259,9 @@ def _quantize_rows(x: torch.Tensor, scale: torch.Tensor, fmt: str, padded: bool)
     with _on_device(x):
         q = torch.empty((m, ld_q), dtype=torch.int8 if fmt == "i8" else torch.uint8, device=x.device)
         if m:
-            fn = getattr(_capi.lib(), "daxq_" + name)
             ld_x = x.stride(0) if m > 1 else k
-            _capi.check(fn(x.data_ptr(), m, k, ld_x, scale.data_ptr(), q.data_ptr(), ld_q, _stream(x)), name)
+            _capi.check(_capi.lib().daxq_quantize_rows(x.data_ptr(), kind, FMT[fmt], m, k, ld_x, scale.data_ptr(),
+                                                       q.data_ptr(), ld_q, _stream(x)), name)
     return q
 
 
@@ -272,16 +291,16 @@ quantize_rows_e4m3.register_fake(
 # ----------------------------------------------------------------------------- weight observer statistics
 @torch.library.custom_op("daxq::row_minmax", mutates_args=(), device_types="cuda")
 def row_minmax(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
-    """Per-row (min, max) of a bf16 matrix in fp32."""
-    _rows_bf16(x, "row_minmax")
+    """Per-row (min, max) of a bf16 / fp16 / fp32 matrix in fp32."""
+    kind = _rows_float(x, "row_minmax")
     m, k = x.shape
     with _on_device(x):
         lo = torch.empty((m,), dtype=torch.float32, device=x.device)
         hi = torch.empty((m,), dtype=torch.float32, device=x.device)
         if m:
             ld_x = x.stride(0) if m > 1 else k
-            _capi.check(_capi.lib().daxq_row_minmax(x.data_ptr(), m, k, ld_x, lo.data_ptr(), hi.data_ptr(), _stream(x)),
-                        "row_minmax")
+            _capi.check(_capi.lib().daxq_row_minmax_t(x.data_ptr(), kind, m, k, ld_x, lo.data_ptr(), hi.data_ptr(),
+                                                      _stream(x)), "row_minmax")
     return lo, hi
 
 
@@ -308,8 +327,37 @@ scale_from_minmax.register_fake(lambda min_val, max_val, qmax: torch.empty_like(
 
 
 # ----------------------------------------------------------------------------- GEMM + epilogue
-def _linear(xq, sx, wq, sw, bias, fp8: bool, want_acc: bool, x_e5m2: bool = False):
-    name = "linear_e5m2_e4m3" if x_e5m2 else "linear_e4m3" if fp8 else "linear_i8"
+# Workspaces of the split-K launches: one per (device, stream), zero-filled when it is made (the kernels leave the
+# counters at its head zero), grown when a larger problem comes along.  Launches on one stream are ordered, so they can
+# share it; another stream gets its own.
+_splitk_ws = {}
+SPLITK_AUTO = True  # few-tile launches (a few hundred rows) cut K into ranges when it pays
+
+
+def _splitk_workspace(device, stream: int, need: int):
+    key = (device.index, stream)
+    ws = _splitk_ws.get(key)
+    if ws is None or ws.numel() < need:
+        if torch.cuda.is_current_stream_capturing():
+            return None  # an allocation recorded into a graph belongs to that graph: take the plain launch instead
+        ws = torch.zeros(max(need, 1 << 20), dtype=torch.uint8, device=device)
+        _splitk_ws[key] = ws
+    return ws
+
+
+def _auto_splits(m: int, n: int, k: int, out_dtype, want_acc: bool, fp8: bool) -> int:
+    # INT8 only: its partial sums are integers, so the result does not depend on how K is cut and a row's output stays
+    # the same whatever the batch it arrives in; FP8 sums would change in the last bits with the number of rows
+    if not SPLITK_AUTO or fp8 or want_acc or out_dtype != torch.bfloat16 or _capi.kernel_arg() != 0:
+        return 1
+    return _capi.lib().daxq_linear_splitk_choice(m, n, k)
+
+
+def _linear(xq, sx, wq, sw, bias, fp8: bool, want_acc: bool, x_e5m2: bool = False, w_e5m2: bool = False,
+            out_dtype: torch.dtype = torch.bfloat16, splits: Optional[int] = None):
+    x_fmt = "e5m2" if x_e5m2 else "e4m3" if fp8 else "i8"
+    w_fmt = "e5m2" if w_e5m2 else "e4m3" if fp8 else "i8"
+    name = f"linear_{x_fmt}_{w_fmt}"
     _need_gpu(xq, name)
     _same_device(name, xq, sx=sx, wq=wq, sw=sw, bias=bias)
     qdt = torch.uint8 if fp8 else torch.int8
@@ -322,22 +370,75 @@ def _linear(xq, sx, wq, sw, bias, fp8: bool, want_acc: bool, x_e5m2: bool = Fals
     n = wq.shape[0]
     if sx.dtype != torch.float32 or sw.dtype != torch.float32 or sx.numel() != m or sw.numel() != n:
         raise ValueError(f"daxq::{name}: sx must be fp32 [M] and sw fp32 [N]")
-    if bias is not None and (bias.dtype != torch.bfloat16 or bias.numel() != n):
-        raise ValueError(f"daxq::{name}: bias must be bf16 [N]")
+    if out_dtype not in FLOAT_KIND:
+        raise ValueError(f"daxq::{name}: out_dtype must be bfloat16, float16 or float32, got {out_dtype}")
+    if bias is not None and (bias.dtype != out_dtype or bias.numel() != n):
+        raise ValueError(f"daxq::{name}: bias must be {out_dtype} [N]")
     sx = sx.reshape(-1).contiguous()
     sw = sw.reshape(-1).contiguous()
     bias_c = bias.contiguous() if bias is not None else None
     with _on_device(xq):
-        out = torch.empty((m, n), dtype=torch.bfloat16, device=xq.device)
+        out = torch.empty((m, n), dtype=out_dtype, device=xq.device)
         acc = torch.empty((m, n), dtype=torch.float32 if fp8 else torch.int32, device=xq.device) if want_acc else None
         if m and n:
-            fn = getattr(_capi.lib(), "daxq_" + name)
             ld_x = xq.stride(0) if m > 1 else k
             ld_w = wq.stride(0) if n > 1 else k
-            _capi.check(fn(xq.data_ptr(), ld_x, sx.data_ptr(), wq.data_ptr(), ld_w, sw.data_ptr(),
-                           bias_c.data_ptr() if bias_c is not None else None, out.data_ptr(), n,
-                           acc.data_ptr() if acc is not None else None, n, m, n, k, _stream(xq)), name)
+            splits = splits if splits is not None else _auto_splits(m, n, k, out_dtype, want_acc, fp8)
+            if splits > 1:
+                stream = _stream(xq)
+                need = _capi.lib().daxq_linear_splitk_workspace_bytes(m, n, splits)
+                ws = _splitk_workspace(xq.device, stream, need)
+                if ws is not None:
+                    _capi.check(_capi.lib().daxq_linear_w8a8_splitk(
+                        FMT[x_fmt], FMT[w_fmt], xq.data_ptr(), ld_x, sx.data_ptr(), wq.data_ptr(), ld_w, sw.data_ptr(),
+                        bias_c.data_ptr() if bias_c is not None else None, out.data_ptr(), n, m, n, k, splits,
+                        ws.data_ptr(), ws.numel(), stream), name + "_splitk")
+                    return out, acc
+            _capi.check(_capi.lib().daxq_linear_w8a8(
+                FMT[x_fmt], FMT[w_fmt], FLOAT_KIND[out_dtype], xq.data_ptr(), ld_x, sx.data_ptr(), wq.data_ptr(), ld_w,
+                sw.data_ptr(), bias_c.data_ptr() if bias_c is not None else None, out.data_ptr(), n,
+                acc.data_ptr() if acc is not None else None, n, m, n, k, _capi.kernel_arg(), _stream(xq)), name)
     return out, acc
+
+
+@torch.library.custom_op("daxq::linear_w8a8", mutates_args=(), device_types="cuda")
+def linear_w8a8(xq: torch.Tensor, sx: torch.Tensor, wq: torch.Tensor, sw: torch.Tensor, bias: Optional[torch.Tensor],
+                x_fmt: str, w_fmt: str, out_dtype: torch.dtype) -> torch.Tensor:
+    """The GEMM + epilogue for any operand pairing ("i8" x "i8", or "e4m3" / "e5m2" activations against "e4m3" /
+    "e5m2" weights, bytes as uint8) and any module dtype: out and bias are bf16, fp16 or fp32."""
+    if (x_fmt == "i8") != (w_fmt == "i8") or x_fmt not in FMT or w_fmt not in FMT:
+        raise ValueError(f"daxq::linear_w8a8: unsupported operand formats {x_fmt} x {w_fmt}")
+    return _linear(xq, sx, wq, sw, bias, x_fmt != "i8", False, x_fmt == "e5m2", w_fmt == "e5m2", out_dtype)[0]
+
+
+@torch.library.custom_op("daxq::linear_w8a8_acc", mutates_args=(), device_types="cuda")
+def linear_w8a8_acc(xq: torch.Tensor, sx: torch.Tensor, wq: torch.Tensor, sw: torch.Tensor, bias: Optional[torch.Tensor],
+                    x_fmt: str, w_fmt: str, out_dtype: torch.dtype) -> Tuple[torch.Tensor, torch.Tensor]:
+    """As linear_w8a8, also returning the raw accumulators (int32 / fp32 [M,N])."""
+    if (x_fmt == "i8") != (w_fmt == "i8") or x_fmt not in FMT or w_fmt not in FMT:
+        raise ValueError(f"daxq::linear_w8a8: unsupported operand formats {x_fmt} x {w_fmt}")
+    return _linear(xq, sx, wq, sw, bias, x_fmt != "i8", True, x_fmt == "e5m2", w_fmt == "e5m2", out_dtype)
+
+
+@torch.library.custom_op("daxq::linear_w8a8_splitk", mutates_args=(), device_types="cuda")
+def linear_w8a8_splitk(xq: torch.Tensor, sx: torch.Tensor, wq: torch.Tensor, sw: torch.Tensor, bias: Optional[torch.Tensor],
+                       x_fmt: str, w_fmt: str, splits: int) -> torch.Tensor:
+    """linear_w8a8 (bf16) with K cut into `splits` ranges that run as separate workgroups (0 = the library's choice):
+    for launches with too few output tiles to fill the device."""
+    if (x_fmt == "i8") != (w_fmt == "i8") or x_fmt not in FMT or w_fmt not in FMT:
+        raise ValueError(f"daxq::linear_w8a8_splitk: unsupported operand formats {x_fmt} x {w_fmt}")
+    if splits == 0:
+        splits = _capi.lib().daxq_linear_splitk_choice(xq.shape[0], wq.shape[0], xq.shape[1])
+    return _linear(xq, sx, wq, sw, bias, x_fmt != "i8", False, x_fmt == "e5m2", w_fmt == "e5m2", torch.bfloat16, splits)[0]
+
+
+linear_w8a8_splitk.register_fake(lambda xq, sx, wq, sw, bias, x_fmt, w_fmt, splits:
+                                 xq.new_empty((xq.shape[0], wq.shape[0]), dtype=torch.bfloat16))
+linear_w8a8.register_fake(lambda xq, sx, wq, sw, bias, x_fmt, w_fmt, out_dtype:
+                          xq.new_empty((xq.shape[0], wq.shape[0]), dtype=out_dtype))
+linear_w8a8_acc.register_fake(lambda xq, sx, wq, sw, bias, x_fmt, w_fmt, out_dtype: (
+    xq.new_empty((xq.shape[0], wq.shape[0]), dtype=out_dtype),
+    xq.new_empty((xq.shape[0], wq.shape[0]), dtype=torch.int32 if x_fmt == "i8" else torch.float32)))
 
 
 @torch.library.custom_op("daxq::linear_i8", mutates_args=(), device_types="cuda")
@@ -434,9 +535,11 @@ dynamic_linear_e5m2_e4m3.register_fake(_dyn_fake)
 
 # ----------------------------------------------------------------------------- per-tensor scales
 @torch.library.custom_op("daxq::tensor_scale", mutates_args=(), device_types="cuda")
-def tensor_scale(row_min: torch.Tensor, row_max: torch.Tensor, qmax: float, round_bf16: bool,
+def tensor_scale(row_min: torch.Tensor, row_max: torch.Tensor, qmax: float, round_bf16: int,
                  n_expand: int) -> Tuple[torch.Tensor, torch.Tensor]:
-    """Per-tensor scale from per-row (min, max): (scale fp32 [1], the same value n_expand times)."""
+    """Per-tensor scale from per-row (min, max): (scale fp32 [1], the same value n_expand times).  round_bf16: the
+    quotient is rounded to bf16 (1) or fp16 (2), the element type of the tensor the statistics come from, or not
+    at all (0: fp32 tensors and the observer rule)."""
     _need_gpu(row_min, "tensor_scale")
     _same_device("tensor_scale", row_min, row_max=row_max)
     if row_min.dtype != torch.float32 or row_max.dtype != torch.float32 or row_min.shape != row_max.shape or row_min.numel() == 0:
@@ -488,3 +591,74 @@ def broadcast_f32(src: torch.Tensor, n: int) -> torch.Tensor:
 
 broadcast_f32.register_fake(lambda src, n: src.new_empty((n,), dtype=torch.float32))
 
+
+
+
+# ----------------------------------------------------------------------------- any block shape
+def _view_args(view_shape, reduced):
+    import ctypes as C
+
+    nd = len(view_shape)
+    if nd != len(reduced) or not 1 <= nd <= 8:
+        raise NotImplementedError(f"daxq block kernels take views of 1 to 8 dimensions, got {nd}")
+    return nd, (C.c_int64 * nd)(*[int(v) for v in view_shape]), (C.c_int32 * nd)(*[int(bool(r)) for r in reduced])
+
+
+@torch.library.custom_op("daxq::block_scale", mutates_args=(), device_types="cuda")
+def block_scale(x: torch.Tensor, view_shape: List[int], reduced: List[int], qmax: float, round_to_x: bool) -> torch.Tensor:
+    """Scale of every block of the contiguous tensor x seen through `view_shape`, a block spanning the dimensions
+    flagged in `reduced`: fp32, one element per kept index (row-major over the kept dimensions)."""
+    _need_gpu(x, "block_scale")
+    if x.dtype not in FLOAT_KIND:
+        raise AssertionError(f"Unsupported input dtype: {x.dtype}")
+    if not x.is_contiguous():
+        raise ValueError("daxq::block_scale: x must be contiguous")
+    nd, vs, rd = _view_args(view_shape, reduced)
+    kept = 1
+    total = 1
+    for v, r in zip(view_shape, reduced):
+        total *= v
+        kept *= 1 if r else v
+    if total != x.numel():
+        raise ValueError(f"daxq::block_scale: view {list(view_shape)} does not hold {x.numel()} elements")
+    with _on_device(x):
+        s = torch.empty((kept,), dtype=torch.float32, device=x.device)
+        if total:
+            _capi.check(_capi.lib().daxq_block_scale(x.data_ptr(), FLOAT_KIND[x.dtype], nd, vs, rd, float(qmax),
+                                                     int(round_to_x), s.data_ptr(), _stream(x)), "block_scale")
+    return s
+
+
+@torch.library.custom_op("daxq::block_quantize", mutates_args=(), device_types="cuda")
+def block_quantize(x: torch.Tensor, view_shape: List[int], reduced: List[int], scale: torch.Tensor, fmt: str) -> torch.Tensor:
+    """Leaf quantiser of every element of x with its block's scale (the output of block_scale): int8, or fp8 bytes as
+    uint8, in x's shape."""
+    _need_gpu(x, "block_quantize")
+    _same_device("block_quantize", x, scale=scale)
+    if x.dtype not in FLOAT_KIND or fmt not in FMT:
+        raise AssertionError(f"Unsupported input dtype / format: {x.dtype} / {fmt}")
+    if not x.is_contiguous() or scale.dtype != torch.float32 or not scale.is_contiguous():
+        raise ValueError("daxq::block_quantize: x and scale must be contiguous, scale fp32")
+    nd, vs, rd = _view_args(view_shape, reduced)
+    kept = 1
+    for v, r in zip(view_shape, reduced):
+        kept *= 1 if r else v
+    if kept != scale.numel():
+        raise ValueError(f"daxq::block_quantize: {scale.numel()} scales for {kept} blocks")
+    with _on_device(x):
+        q = torch.empty(x.shape, dtype=torch.int8 if fmt == "i8" else torch.uint8, device=x.device)
+        if x.numel():
+            _capi.check(_capi.lib().daxq_block_quantize(x.data_ptr(), FLOAT_KIND[x.dtype], FMT[fmt], nd, vs, rd,
+                                                        scale.data_ptr(), q.data_ptr(), _stream(x)), "block_quantize")
+    return q
+
+
+def _block_scale_fake(x, view_shape, reduced, qmax, round_to_x):
+    kept = 1
+    for v, r in zip(view_shape, reduced):
+        kept *= 1 if r else v
+    return x.new_empty((kept,), dtype=torch.float32)
+
+
+block_scale.register_fake(_block_scale_fake)
+block_quantize.register_fake(lambda x, view_shape, reduced, scale, fmt: x.new_empty(x.shape, dtype=torch.int8 if fmt == "i8" else torch.uint8))

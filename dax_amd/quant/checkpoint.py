@@ -37,9 +37,9 @@ def _empty_quantised(mod: nn.Linear, device) -> nn.Module:
         from .qscheme import per_channel_symmetric
 
         return StaticLinear(mod.in_features, mod.out_features, mod.bias is not None, device, wt.dtype, act.dtype,
-                            torch.bfloat16, wt.qscheme == per_channel_symmetric)
+                            mod.weight.dtype, wt.qscheme == per_channel_symmetric)
     return nndq.Linear(mod.in_features, mod.out_features, mod.bias is not None, device, wt.dtype, act.dtype,
-                       torch.bfloat16, wt.qscheme, act.qscheme)
+                       mod.weight.dtype, wt.qscheme, act.qscheme)
 
 
 def _swap_empty(module: nn.Module, device) -> None:

@@ -43,6 +43,9 @@ def _is_per_token(block_size, shape) -> bool:
     return tuple(block_size) == (1,) * (len(shape) - 1) + (shape[-1],)
 
 
+_ROUND_KIND = {torch.bfloat16: 1, torch.float16: 2, torch.float32: 0}  # how daxq_tensor_scale rounds the quotient
+
+
 def _dynamic_quantize_func(
     input: Optional[torch.Tensor],
     block_size: List[int],
@@ -51,51 +54,57 @@ def _dynamic_quantize_func(
     eps: Optional[float] = None,
     scale_dtype: Optional[torch.dtype] = None,
 ) -> Tuple[torch.Tensor, torch.Tensor]:
-    """Quantises `input` block by block; returns (values in the input's shape, scales with
-    every reduced dim kept as 1).  dax/quant/nn/dynamic/functional.py:54-148."""
+    """Quantises `input` block by block; returns (values in the input's shape, scales in the view shape of the
+    reduction with every reduced dim kept as 1).  dax/quant/nn/dynamic/functional.py:54-148.
+
+    Which kernels run: blocks that lie along the last dimension only (per-token, last-dimension groups) are rows
+    of a matrix and take the one-pass row quantiser; a whole-tensor block takes the row statistics + single
+    reduction; every other block shape takes the general strided kernels.
+    """
     assert input.dtype in [torch.float32, torch.float16, torch.bfloat16], f"Unsupported input dtype: {input.dtype}"
     assert len(block_size) == input.dim(), f"Got input dim:{input.dim()}, block_size: {block_size}"
-    if target_dtype not in FP8_ALLOWED_DTYPES and target_dtype != torch.int8:
+    if target_dtype not in ops.FMT_OF_DTYPE:
         raise NotImplementedError(f"Unsupported dtype {target_dtype}")
-    per_tensor = tuple(block_size) == tuple(input.shape)
-    if not (per_tensor or _is_per_token(block_size, input.shape)):
-        raise NotImplementedError("daxq implements the per-token and per-tensor dynamic schemes; grouped blocks are not built")
+    fmt = ops.FMT_OF_DTYPE[target_dtype]
+    qmax = ops.QMAX[fmt]
+    if quant_max is not None and float(quant_max) != qmax:
+        raise NotImplementedError(f"daxq quantisers use the target dtype's own maximum ({qmax}), got quant_max={quant_max}")
     if scale_dtype not in (None, torch.float32) or (eps is not None and eps != torch.finfo(torch.float32).eps):
         raise NotImplementedError("daxq kernels produce fp32 scales floored at float32 eps")
-    if per_tensor and not _is_per_token(block_size, input.shape):
-        return _per_tensor_quantize(input, target_dtype, float(quant_max))
-    k = input.shape[-1]
-    x2 = input.reshape(-1, k)
-    if target_dtype == torch.int8:
-        q, s = ops.act_quant_i8(x2)
-    elif target_dtype == torch.float8_e5m2:
-        q, s = ops.act_quant_e5m2(x2)
-        q = q.view(torch.float8_e5m2)
-    else:
-        q, s = ops.act_quant_e4m3(x2)
-        q = q.view(torch.float8_e4m3fn)
-    return q[:, :k].view(input.shape), s.view(*input.shape[:-1], 1)
+    view_shape, reduce_dims = _get_reduction_params(tuple(block_size), tuple(input.shape))
+    after = [1 if i in reduce_dims else v for i, v in enumerate(view_shape)]
+    x = input if input.is_contiguous() else input.contiguous()  # the reference's .view needs that layout anyway
+    as_dtype = (lambda q: q) if fmt == "i8" else (lambda q: q.view(target_dtype))
+    if input.numel() == 0:
+        return as_dtype(torch.empty(input.shape, dtype=torch.int8 if fmt == "i8" else torch.uint8, device=input.device)), \
+            torch.empty(after, dtype=torch.float32, device=input.device)
+    if tuple(block_size) == tuple(input.shape) and not _is_per_token(block_size, input.shape):
+        q, s1 = _per_tensor_quantize(x, fmt, qmax)
+        return as_dtype(q).view(input.shape), s1.view(after)
+    g = block_size[-1] if len(block_size) else 1
+    if all(b == 1 for b in block_size[:-1]) and g > 1 and input.dim() >= 1:
+        # rows of the [numel / g, g] view: per-token (g = K) and last-dimension groups
+        x2 = x.view(-1, g)
+        q, s = getattr(ops, "act_quant_" + fmt)(x2)
+        return as_dtype(q[:, :g]).reshape(input.shape), s.view(after)
+    reduced = [1 if i in reduce_dims else 0 for i in range(len(view_shape))]
+    s = ops.block_scale(x, view_shape, reduced, qmax, True)
+    q = ops.block_quantize(x, view_shape, reduced, s, fmt)
+    return as_dtype(q).view(input.shape), s.view(after)
 
 
 def per_tensor_scale(x2: torch.Tensor, quant_max: float):
-    """(scale fp32 [1], the same value once per row of x2) of the whole bf16 matrix x2."""
+    """(scale fp32 [1], the same value once per row of x2) of the whole matrix x2; the quotient is rounded to x2's
+    own element type before the floor, as the eager dtype chain does (:124-129)."""
     lo, hi = ops.row_minmax(x2)
-    return ops.tensor_scale(lo, hi, quant_max, True, x2.shape[0])
+    return ops.tensor_scale(lo, hi, quant_max, _ROUND_KIND[x2.dtype], x2.shape[0])
 
 
-def _per_tensor_quantize(input, target_dtype, quant_max):
-    k = input.shape[-1]
-    x2 = input.reshape(-1, k)
-    if x2.stride(1) != 1:
-        x2 = x2.contiguous()
+def _per_tensor_quantize(x, fmt, quant_max):
+    k = x.shape[-1] if x.dim() else 1
+    x2 = x.reshape(-1, k)
     s1, rows = per_tensor_scale(x2, quant_max)
-    if target_dtype == torch.int8:
-        q = ops.quantize_rows_i8(x2, rows)
-    elif target_dtype == torch.float8_e5m2:
-        q = ops.quantize_rows_e5m2(x2, rows).view(torch.float8_e5m2)
-    else:
-        q = ops.quantize_rows_e4m3(x2, rows).view(torch.float8_e4m3fn)
-    return q.view(input.shape), s1.view((1,) * input.dim())
+    return getattr(ops, "quantize_rows_" + fmt)(x2, rows), s1
 
 
 def dynamic_quantize_to_fp8(

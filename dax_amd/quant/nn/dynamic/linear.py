@@ -97,11 +97,9 @@ class Linear(DerivedOperands, nn.Module):
             raise NotImplementedError(
                 "daxq implements per-token / per-tensor activations with per-channel / per-tensor weights; "
                 f"got input_qscheme={input_qscheme}, weight_qscheme={weight_qscheme}")
-        if compute_dtype == "FP8" and weight_dtype != torch.float8_e4m3fn:
-            raise NotImplementedError(
-                f"daxq implements float8_e4m3fn weights (with e4m3fn or e5m2 activations); got weight {weight_dtype}")
-        if out_dtype not in (None, torch.bfloat16):
-            raise NotImplementedError(f"daxq kernels produce bfloat16 outputs, got out_dtype={out_dtype}")
+        if out_dtype not in (None, torch.bfloat16, torch.float16, torch.float32):
+            raise NotImplementedError(f"daxq kernels produce bfloat16, float16 or float32 outputs, got out_dtype={out_dtype}")
+        out_dtype = out_dtype if out_dtype is not None else torch.bfloat16
 
         super().__init__()
         self.in_features = in_features
@@ -110,8 +108,10 @@ class Linear(DerivedOperands, nn.Module):
         self.register_buffer(
             "qweight", torch.empty((out_features, in_features), device=device, dtype=weight_dtype), persistent=True)
         if bias:
-            # bf16 either way: FP8 row-wise needs it (:111-116), and out_dtype is bf16 here
-            self.bias = nn.Parameter(torch.empty(out_features, device=device, dtype=torch.bfloat16))
+            # the row-wise FP8 matmul writes bf16 and takes a bf16 bias whatever the module's dtype (:106-118)
+            row_wise_fp8 = compute_dtype == "FP8" and weight_qscheme == per_channel_symmetric
+            self.bias = nn.Parameter(torch.empty(out_features, device=device,
+                                                 dtype=torch.bfloat16 if row_wise_fp8 else out_dtype))
         else:
             self.register_parameter("bias", None)
         # [1, N] per channel, [1] per tensor (:122-130)
@@ -121,7 +121,7 @@ class Linear(DerivedOperands, nn.Module):
                        dtype=torch.float32),
             persistent=True)
 
-        self.out_dtype = out_dtype if out_dtype is not None else torch.bfloat16
+        self.out_dtype = out_dtype
         self.weight_dtype = weight_dtype
         self.input_dtype = input_dtype
         self.compute_dtype = compute_dtype
@@ -147,10 +147,8 @@ class Linear(DerivedOperands, nn.Module):
         else:
             from .functional import per_tensor_scale
 
-            qmax = 127.0 if self.input_dtype == torch.int8 else float(torch.finfo(self.input_dtype).max)
-            _, sx = per_tensor_scale(flat, qmax)
-            xq = getattr(ops, "quantize_rows_" + {torch.int8: "i8", torch.float8_e4m3fn: "e4m3",
-                                                 torch.float8_e5m2: "e5m2"}[self.input_dtype])(flat, sx, True)
+            _, sx = per_tensor_scale(flat, ops.QMAX[ops.FMT_OF_DTYPE[self.input_dtype]])
+            xq = getattr(ops, "quantize_rows_" + ops.FMT_OF_DTYPE[self.input_dtype])(flat, sx, True)
         return QuantizedActivation(xq, sx, input.shape[:-1], self.in_features, self.input_dtype)
 
     def _takes_float_fallback(self, input) -> bool:
@@ -168,29 +166,27 @@ class Linear(DerivedOperands, nn.Module):
             logger.warning("int8 matmul not taken for this combination of dimensions, float implementation instead. "
                            "M: %d, K: %d, N: %d", input.numel() // self.in_features, self.in_features, self.out_features)
             return torch.nn.functional.linear(input, self.weight, self.bias)
-        if not isinstance(input, QuantizedActivation) and self.input_qscheme == per_token_symmetric:
-            # the common case: quantiser and GEMM behind one op call
+        # the kernels are inference-only (no autograd formula): the bias enters as a plain tensor
+        bias = None if self.bias is None else self.bias.detach()
+        if (not isinstance(input, QuantizedActivation) and self.input_qscheme == per_token_symmetric
+                and input.dtype == torch.bfloat16 and self.out_dtype == torch.bfloat16
+                and self.weight_dtype != torch.float8_e5m2):
+            # the common case (a bf16 DiT): quantiser and GEMM behind one op call
             flat = input.view(-1, self.in_features)
             if flat.stride(-1) != 1:
                 flat = flat.contiguous()
-            bias = None if self.bias is None else self.bias.detach()
             out = getattr(ops, _DYNAMIC_LINEAR[self.input_dtype])(flat, self._gemm_weight(), self._weight_scale_vector(), bias)
-            out = out.view(*input.shape[:-1], self.out_features)
-            return out if out.dtype == self.out_dtype else out.to(self.out_dtype)
+            return out.view(*input.shape[:-1], self.out_features)
         qa = input if isinstance(input, QuantizedActivation) else self.quantize_activation(input)
         if qa.dtype != self.input_dtype or qa.in_features != self.in_features:
             raise ValueError(f"quantised activation ({qa.dtype}, K={qa.in_features}) does not fit this linear "
                              f"({self.input_dtype}, K={self.in_features})")
-        wq = self._gemm_weight()
-        sw = self._weight_scale_vector()
-        # the kernels are inference-only (no autograd formula): the bias enters as a plain tensor
-        bias = None if self.bias is None else self.bias.detach()
-        if self.compute_dtype == "FP8" and self.input_dtype == torch.float8_e5m2:
-            out = ops.linear_e5m2_e4m3(qa.xq, qa.sx, wq, sw, bias)
-        elif self.compute_dtype == "FP8":
-            out = ops.linear_e4m3(qa.xq, qa.sx, wq, sw, bias)
-        else:
-            out = ops.linear_i8(qa.xq, qa.sx, wq, sw, bias)
+        # What the matmul writes: INT8 scales in fp32 and casts to the module's dtype (:221-228); the row-wise FP8
+        # matmul writes bf16 and the result is cast afterwards (:166-178); per-tensor FP8 writes the module's dtype.
+        row_wise_fp8 = self.compute_dtype == "FP8" and self.input_qscheme == per_token_symmetric
+        mm_dtype = torch.bfloat16 if row_wise_fp8 else self.out_dtype
+        out = ops.linear_w8a8(qa.xq, qa.sx, self._gemm_weight(), self._weight_scale_vector(), bias,
+                              ops.FMT_OF_DTYPE[self.input_dtype], ops.FMT_OF_DTYPE[self.weight_dtype], mm_dtype)
         out = out.view(*qa.prev_dims, self.out_features)
         if out.dtype != self.out_dtype:
             out = out.to(self.out_dtype)

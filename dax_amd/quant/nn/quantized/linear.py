@@ -29,12 +29,13 @@ class Linear(DerivedOperands, nn.Module):
 
     def __init__(self, in_features: int, out_features: int, bias: bool = True, device=None, weight_dtype=None,
                  input_dtype=None, out_dtype=None, row_wise_scale=False) -> None:
-        if weight_dtype is not None and weight_dtype != torch.float8_e4m3fn:
-            raise NotImplementedError(f"daxq implements float8_e4m3fn weights, got {weight_dtype}")
+        if weight_dtype is not None and weight_dtype not in FP8_ALLOWED_DTYPES:
+            raise NotImplementedError(f"the static linear is an FP8 module, got weight dtype {weight_dtype}")
         if input_dtype is not None and input_dtype not in FP8_ALLOWED_DTYPES:
             raise NotImplementedError(f"the static linear is an FP8 module, got input dtype {input_dtype}")
-        if out_dtype not in (None, torch.bfloat16):
-            raise NotImplementedError(f"daxq kernels produce bfloat16 outputs, got out_dtype={out_dtype}")
+        if out_dtype not in (None, torch.bfloat16, torch.float16, torch.float32):
+            raise NotImplementedError(f"daxq kernels produce bfloat16, float16 or float32 outputs, got out_dtype={out_dtype}")
+        out_dtype = out_dtype if out_dtype is not None else torch.bfloat16
         super().__init__()
         self.in_features = in_features
         self.out_features = out_features
@@ -42,14 +43,16 @@ class Linear(DerivedOperands, nn.Module):
             torch.empty((out_features, in_features), device=device, dtype=weight_dtype or torch.float8_e4m3fn),
             requires_grad=False)
         if bias:
-            self.bias = nn.Parameter(torch.empty(out_features, device=device, dtype=torch.bfloat16))
+            # the row-wise matmul writes bf16 and takes a bf16 bias whatever the module's dtype (:57-66)
+            self.bias = nn.Parameter(torch.empty(out_features, device=device,
+                                                 dtype=torch.bfloat16 if row_wise_scale else out_dtype))
         else:
             self.register_parameter("bias", None)
         self.register_buffer(
             "weight_scale", torch.ones((1, out_features) if row_wise_scale else 1, device=device, dtype=torch.float32),
             persistent=True)
         self.register_buffer("input_scale", torch.tensor([1.0], device=device, dtype=torch.float32), persistent=True)
-        self.out_dtype = out_dtype if out_dtype is not None else torch.bfloat16
+        self.out_dtype = out_dtype
         self.weight_dtype = weight_dtype or torch.float8_e4m3fn
         self.input_dtype = input_dtype or torch.float8_e4m3fn
         self.row_wise_scale = row_wise_scale
@@ -64,14 +67,15 @@ class Linear(DerivedOperands, nn.Module):
         self._check_device(input.device)
         prev_dims = input.shape[:-1]
         flat = input.view(-1, self.in_features)
+        if flat.stride(-1) != 1:
+            flat = flat.contiguous()
         sx = ops.broadcast_f32(self.input_scale.reshape(1), flat.shape[0])
         bias = None if self.bias is None else self.bias.detach()  # inference-only kernels
-        if self.input_dtype == torch.float8_e5m2:
-            xq = ops.quantize_rows_e5m2(flat, sx, True)
-            out = ops.linear_e5m2_e4m3(xq, sx, self._gemm_weight(), self._weight_scale_vector(), bias)
-        else:
-            xq = ops.quantize_rows_e4m3(flat, sx, True)
-            out = ops.linear_e4m3(xq, sx, self._gemm_weight(), self._weight_scale_vector(), bias)
+        x_fmt, w_fmt = ops.FMT_OF_DTYPE[self.input_dtype], ops.FMT_OF_DTYPE[self.weight_dtype]
+        xq = getattr(ops, "quantize_rows_" + x_fmt)(flat, sx, True)
+        # row-wise weight scales: the matmul writes bf16 and the result is cast afterwards (:96-104, :116-117)
+        mm_dtype = torch.bfloat16 if self.row_wise_scale else self.out_dtype
+        out = ops.linear_w8a8(xq, sx, self._gemm_weight(), self._weight_scale_vector(), bias, x_fmt, w_fmt, mm_dtype)
         out = out.view(*prev_dims, self.out_features)
         if out.dtype != self.out_dtype:
             out = out.to(self.out_dtype)

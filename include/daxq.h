@@ -10,7 +10,9 @@
  *   - matrices are row-major with an explicit leading dimension in ELEMENTS;
  *   - return value 0 on success, a negative DAXQ_ERR_* otherwise; the text of
  *     the last error on the calling thread is returned by daxq_last_error();
- *   - calls on different streams may run concurrently.
+ *   - calls on different streams, and from different host threads, may run concurrently: the library keeps no
+ *     mutable process state apart from a per-kernel record of the devices whose launch attributes it has set
+ *     (atomic; filled by daxq_init or by a kernel's first launch on a device).
  *
  * Reference paths cited below are relative to the DAX checkout.
  */
@@ -23,7 +25,7 @@
 extern "C" {
 #endif
 
-#define DAXQ_ABI_VERSION 1
+#define DAXQ_ABI_VERSION 2
 
 #define DAXQ_OK 0
 #define DAXQ_ERR_ARG (-1)    /* null pointer, negative size, bad enum */
@@ -35,6 +37,16 @@ extern "C" {
  * multiple of this are zero-padded by the producer (the quantisers below pad
  * columns [k, ld_q) with zeros). */
 #define DAXQ_K_ALIGN 128
+
+/* quantised formats (one byte per element) */
+#define DAXQ_FMT_I8 0   /* two's-complement int8 */
+#define DAXQ_FMT_E4M3 1 /* OCP float8 e4m3fn */
+#define DAXQ_FMT_E5M2 2 /* OCP float8 e5m2 */
+
+/* floating-point element types of activations, outputs and bias */
+#define DAXQ_BF16 0
+#define DAXQ_F16 1
+#define DAXQ_F32 2
 
 typedef void* daxq_stream_t;
 
@@ -136,13 +148,42 @@ int daxq_quantize_rows_e5m2(const void* x, int64_t m, int64_t k, int64_t ld_x, c
                             uint8_t* q, int64_t ld_q, daxq_stream_t stream);
 
 /*
+ * The quantisers above for any element type the reference accepts (fp32, fp16, bf16:
+ *   dax/quant/nn/dynamic/functional.py:99-103) and any quantised format, selected by arguments:
+ * x_dtype DAXQ_BF16 / DAXQ_F16 / DAXQ_F32, q_fmt DAXQ_FMT_I8 / _E4M3 / _E5M2.
+ * daxq_act_quant_rows: per-row dynamic scale, computed and floored in x's own type before it is widened
+ *   (the eager dtype chain of :124-129: fp16 rounds the quotient to fp16, fp32 does not round);
+ * daxq_quantize_rows: leaf quantiser with the caller's per-row scale (dax/quant/nn/quantized/functional.py:11-20).
+ * Last-dimension groups (block (1, ..., 1, G)) are rows of the [numel / G, G] view and use these two.
+ */
+int daxq_act_quant_rows(const void* x, int x_dtype, int q_fmt, int64_t m, int64_t k, int64_t ld_x,
+                        void* q, int64_t ld_q, float* scale, daxq_stream_t stream);
+int daxq_quantize_rows(const void* x, int x_dtype, int q_fmt, int64_t m, int64_t k, int64_t ld_x, const float* scale,
+                       void* q, int64_t ld_q, daxq_stream_t stream);
+
+/*
+ * Any other block shape of _dynamic_quantize_func (dax/quant/nn/dynamic/functional.py:54-148: per-channel
+ * activations, 2-d tiles, blocks over leading dimensions).  The contiguous tensor x is seen through the view of
+ * _get_reduction_params (:13-51): nd <= 8 dimensions view_shape[0..nd), reduced[d] != 0 for the dimensions a block
+ * spans.  view_shape and reduced are HOST arrays, read before the call returns.
+ * daxq_block_scale:    scale[b] = max( round( absmax(block b) / qmax ), 2^-23 ), b row-major over the kept
+ *                      dimensions; round = to x's own type when round_to_x != 0 (dynamic rule), none otherwise.
+ * daxq_block_quantize: q[i] = leaf quantiser of x[i] with its block's scale; q has x's shape, one byte per element.
+ */
+int daxq_block_scale(const void* x, int x_dtype, int nd, const int64_t* view_shape, const int32_t* reduced, float qmax,
+                     int round_to_x, float* scale, daxq_stream_t stream);
+int daxq_block_quantize(const void* x, int x_dtype, int q_fmt, int nd, const int64_t* view_shape, const int32_t* reduced,
+                        const float* scale, void* q, daxq_stream_t stream);
+
+/*
  * Per-tensor schemes (the block of dax/quant/qscheme.py:10-26 is the whole tensor).  The GEMM and the leaf
  * quantisers above take a scale per row / per channel; a per-tensor scale is handed to them written out as a
  * vector, which gives the same arithmetic per element.  These entry points keep that on the device.
  *
  * daxq_tensor_scale: dynamic per-tensor scale from per-row statistics (daxq_row_minmax):
- *   a = max_i max(-row_min[i], row_max[i]);  scale1[0] = max( round(a / qmax), 2^-23 ), round = bf16 RNE when
- *   round_bf16 != 0 (the activation rule, dax/quant/nn/dynamic/functional.py:124-129) or none (observer rule,
+ *   a = max_i max(-row_min[i], row_max[i]);  scale1[0] = max( round(a / qmax), 2^-23 ), round = RNE to bf16 when
+ *   round_bf16 == 1, to fp16 when it is 2 (the activation rule for a tensor of that type,
+ *   dax/quant/nn/dynamic/functional.py:124-129) or none when 0 (fp32 tensors, and the observer rule,
  *   dax/quant/quantization/observer.py:97-134); expand[0..n_expand) receives the same value.
  * daxq_tensor_minmax_update: running min / max of a calibration observer,
  *   dax/quant/quantization/observer.py:200-214:  min_inout[0] = min(min_inout[0], min_i row_min[i]), same for max.
@@ -160,6 +201,9 @@ int daxq_broadcast_f32(const float* src, float* dst, int64_t n, daxq_stream_t st
  */
 int daxq_row_minmax(const void* x, int64_t m, int64_t k, int64_t ld_x,
                     float* min_out, float* max_out, daxq_stream_t stream);
+/* the same for x of element type x_dtype (DAXQ_BF16 / DAXQ_F16 / DAXQ_F32): weights of fp16 / fp32 modules */
+int daxq_row_minmax_t(const void* x, int x_dtype, int64_t m, int64_t k, int64_t ld_x,
+                      float* min_out, float* max_out, daxq_stream_t stream);
 
 /*
  * scale[i] = max( max(-min[i], max[i]) / qmax, 2^-23 ) in fp32 (no bf16 rounding).
@@ -205,12 +249,50 @@ int daxq_linear_e5m2_e4m3(const uint8_t* xq, int64_t ld_xq, const float* sx,
                           float* acc, int64_t ld_acc,
                           int64_t m, int64_t n, int64_t k, daxq_stream_t stream);
 
-/* Selects a GEMM kernel for tests and comparisons; every choice computes the same results.
- * 0 = library default (by shape), 2 / 5 = generic 256x256 / 128x128 tiles, 6 = two-stage 256x256 kernel,
- * 8 = five-stage 256x256 kernel, 9 = the same with 32x32x32 INT8 MFMAs, 11 = the same on 128x128 tiles;
- * 1000 + d sets the depth d of the
- * tile-order groups.  Process-wide; not part of the reference interface. */
-int daxq_set_gemm_variant(int variant);
+/*
+ * The general form of the three entry points above: any operand pairing the reference's constructor accepts
+ *   dax/quant/nn/dynamic/linear.py:42-89   (int8 x int8; any of FP8_ALLOWED_DTYPES for activations and weights,
+ *                                           dax/quant/nn/quantized/functional.py:4-7)
+ * and any module dtype (out_dtype = the float weight's dtype, :263): out and bias are out_dtype elements
+ * (DAXQ_BF16 / DAXQ_F16 / DAXQ_F32).
+ *   int8: out = T( f32( T( f32_rne(acc) * sx[i] * sw[j] ) ) + f32(bias[j]) )   T = round to out_dtype   (:221-228)
+ *   fp8:  out = T( acc * sx[i] * sw[j] + f32(bias[j]) )                        (torch._scaled_mm, :155-173)
+ * acc: optional int32 (int8) / fp32 (fp8) dump of the raw accumulators.
+ * kernel: 0 = the library's choice by shape.  Other values pick one implementation, for tests and comparisons
+ * (every choice computes the same results): 2 / 5 = generic kernel on 256x256 / 128x128 tiles, 6 = two-stage 256x256
+ * kernel, 8 = five-stage 256x256 kernel, 9 = the same with 32x32x32 INT8 MFMAs, 11 = the same on 128x128 tiles;
+ * bits 16-23, when not zero, set the depth of the tile-order groups.  fp16 / fp32 outputs exist in the generic
+ * kernel only.  The choice is an argument of the call: the library keeps no process-wide selection.
+ */
+int daxq_linear_w8a8(int x_fmt, int w_fmt, int out_dtype,
+                     const void* xq, int64_t ld_xq, const float* sx,
+                     const void* wq, int64_t ld_wq, const float* sw,
+                     const void* bias, void* out, int64_t ld_out,
+                     void* acc, int64_t ld_acc,
+                     int64_t m, int64_t n, int64_t k, int kernel, daxq_stream_t stream);
+
+/*
+ * Split-K form of daxq_linear_w8a8 for launches with too few output tiles to fill the CUs (a few hundred rows: the
+ * text-token k / v projections of cross-attention, a single prompt): K is cut into `splits` equal ranges that run as
+ * separate workgroups on 128x128 tiles, partial accumulators (int32 / fp32) go through `workspace`, and the workgroup
+ * that finishes a tile last adds them in range order and applies the epilogue.  Results equal daxq_linear_w8a8's:
+ * bit for bit for int8 (integer partial sums), to fp32 summation order for fp8.  bf16 outputs.  No counterpart in
+ * the reference, whose matmul comes from a vendor library.
+ *   splits     0 = daxq_linear_splitk_choice(m, n, k); 1 = the plain launch (workspace unused); else K / 128 must
+ *              divide by it; needs m, n >= 128.
+ *   workspace  device memory, 256-byte aligned, at least daxq_linear_splitk_workspace_bytes(m, n, splits) bytes.
+ *              Its first 16 KiB are tile counters (at most 4096 output tiles of 128x128): they must be ZERO when
+ *              the call is made and every call leaves them zero, so a workspace is cleared once (hipMemsetAsync of
+ *              those 16 KiB) and then reused for any shapes.  Calls that share a workspace must not overlap in time.
+ */
+int daxq_linear_splitk_choice(int64_t m, int64_t n, int64_t k);
+int64_t daxq_linear_splitk_workspace_bytes(int64_t m, int64_t n, int splits);
+int daxq_linear_w8a8_splitk(int x_fmt, int w_fmt,
+                            const void* xq, int64_t ld_xq, const float* sx,
+                            const void* wq, int64_t ld_wq, const float* sw,
+                            const void* bias, void* out, int64_t ld_out,
+                            int64_t m, int64_t n, int64_t k,
+                            int splits, void* workspace, int64_t workspace_bytes, daxq_stream_t stream);
 
 #ifdef __cplusplus
 }

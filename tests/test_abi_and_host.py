@@ -27,7 +27,7 @@ def test_library_exports_every_declared_symbol():
     for name in declared:
         assert hasattr(lib, name), f"{name} declared in include/daxq.h but not exported"
     assert set(declared) == set(_capi.SIGNATURES), "binding table and header disagree"
-    assert _capi.lib().daxq_abi_version() == 1
+    assert _capi.lib().daxq_abi_version() == _capi.ABI_VERSION == 2
     assert "undefined symbol" not in _capi.last_error()
 
 
@@ -207,8 +207,9 @@ def test_static_linear_state_and_validation():
     assert sd["weight_scale"].shape == (1,) and sd["input_scale"].shape == (1,) and sd["qweight"].dtype == torch.float8_e4m3fn
     assert Linear(64, 32, False, None, torch.float8_e4m3fn, torch.float8_e4m3fn, torch.bfloat16, True).weight_scale.shape == (1, 32)
     assert "input_scale" in lin.extra_repr()
-    with pytest.raises(NotImplementedError):
-        Linear(8, 8, True, None, torch.float8_e5m2, torch.float8_e5m2, torch.bfloat16)     # e5m2 weights
+    e5 = Linear(8, 8, True, None, torch.float8_e5m2, torch.float8_e5m2, torch.float16)     # e5m2 weights, fp16 module
+    assert e5.qweight.dtype == torch.float8_e5m2 and e5.bias.dtype == torch.float16 and e5.out_dtype == torch.float16
+    assert Linear(8, 8, True, None, torch.float8_e4m3fn, torch.float8_e4m3fn, torch.float32, True).bias.dtype == torch.bfloat16
     with pytest.raises(NotImplementedError):
         Linear(8, 8, True, None, torch.float8_e4m3fn, torch.int8, torch.bfloat16)
     with pytest.raises(ValueError, match="Input must be quantized"):
@@ -243,8 +244,16 @@ def test_linear_constructor_validation_and_state_layout():
     assert Linear(8, 8, True, None, torch.float8_e4m3fn, torch.float8_e5m2, torch.bfloat16, te, te).compute_dtype == "FP8"
     mixed = Linear(8, 8, True, None, torch.float8_e4m3fn, torch.float8_e5m2, torch.bfloat16, ch, tok)
     assert mixed.compute_dtype == "FP8" and mixed.input_dtype == torch.float8_e5m2   # the reference's FP8 default
-    with pytest.raises(NotImplementedError):   # e5m2 weights: valid in the reference, not built here
-        Linear(8, 8, True, None, torch.float8_e5m2, torch.float8_e5m2, torch.bfloat16, ch, tok)
+    e5 = Linear(8, 8, True, None, torch.float8_e5m2, torch.float8_e5m2, torch.bfloat16, ch, tok)   # e5m2 weights
+    assert e5.qweight.dtype == torch.float8_e5m2 and e5.compute_dtype == "FP8"
+    # module dtypes other than bf16 (out_dtype = the float weight's dtype, dax/quant/nn/dynamic/linear.py:263): the bias is
+    # kept in that dtype, except for the row-wise FP8 matmul, which takes a bf16 bias (:106-118)
+    assert Linear(8, 8, True, None, torch.int8, torch.int8, torch.float16, ch, tok).bias.dtype == torch.float16
+    assert Linear(8, 8, True, None, torch.int8, torch.int8, torch.float32, ch, tok).bias.dtype == torch.float32
+    assert Linear(8, 8, True, None, torch.float8_e4m3fn, torch.float8_e4m3fn, torch.float16, ch, tok).bias.dtype == torch.bfloat16
+    assert Linear(8, 8, True, None, torch.float8_e4m3fn, torch.float8_e4m3fn, torch.float16, te, te).bias.dtype == torch.float16
+    with pytest.raises(NotImplementedError):
+        Linear(8, 8, True, None, torch.int8, torch.int8, torch.float64, ch, tok)
     # dequantised weight property is plain tensor algebra on the stored state
     with torch.no_grad():
         lin.qweight.copy_(torch.randint(-127, 128, (128, 256), dtype=torch.int8))
@@ -442,3 +451,14 @@ def test_product_never_touches_the_oracle_or_a_cpu_path():
     ops_src = open(os.path.join(pkg, "ops.py")).read()
     decls = [line for line in ops_src.splitlines() if line.startswith("@torch.library.custom_op(")]
     assert decls and all('device_types="cuda"' in d for d in decls)
+
+
+def test_bench_inputs_follow_the_seeded_recipe():
+    """bench.py generates its operands with the oracle's seeded CPU recipe (the column scaling is written as one
+    multiplication by a vector there): same bits."""
+    import bench
+    from oracle import daxq_oracle as O
+
+    for seed, (m, k, n) in enumerate([(64, 1536, 24), (33, 200, 8)]):
+        a, b = bench.synth_inputs(m, k, n, seed), O.make_inputs(m, k, n, seed)
+        assert all(torch.equal(u, v) and u.dtype == torch.bfloat16 for u, v in zip(a, b))

@@ -38,7 +38,7 @@ def _default_variant():
     yield
     from dax_amd import _capi
 
-    _capi.set_gemm_variant(0)
+    _capi.debug_select_gemm(0)
 
 
 def dev(t):
@@ -55,7 +55,7 @@ def test_linear_i8_bit_exact(ops, variant, m, n, k):
     from dax_amd import _capi
 
     _skip_if_too_small(variant, m, n)
-    _capi.set_gemm_variant(variant)
+    _capi.debug_select_gemm(variant)
     x, w, b = O.make_inputs(m, k, n, seed=m + n + k)
     qw, sw = O.weight_quant_int8(w)
     ref = O.linear_int8(x, qw, sw, b)
@@ -88,7 +88,7 @@ def test_linear_i8_random_shapes_and_strides_bit_exact(ops, variant, m, n, k, pa
     dimensions, raw int8 operands straight through the C ABI: accumulators and outputs against the integer oracle."""
     from dax_amd import _capi
 
-    _capi.set_gemm_variant(variant)
+    _capi.debug_select_gemm(variant)
     g = torch.Generator("cpu").manual_seed(m * 7 + n * 3 + k)
     xq = torch.randint(-127, 128, (m, k), generator=g, dtype=torch.int32).to(torch.int8)
     wq = torch.randint(-127, 128, (n, k), generator=g, dtype=torch.int32).to(torch.int8)
@@ -104,9 +104,10 @@ def test_linear_i8_random_shapes_and_strides_bit_exact(ops, variant, m, n, k, pa
     out_wide = torch.full((m, n + pad_n), 3.0, dtype=torch.bfloat16, device="cuda")
     acc_wide = torch.full((m, n + pad_n), -1, dtype=torch.int32, device="cuda")
     sxd, swd, bd = dev(sx), dev(sw), dev(b)
-    rc = _capi.lib().daxq_linear_i8(xq_wide.data_ptr(), k + pad_k, sxd.data_ptr(), wq_wide.data_ptr(), k + pad_k,
-                                    swd.data_ptr(), bd.data_ptr(), out_wide.data_ptr(), n + pad_n, acc_wide.data_ptr(),
-                                    n + pad_n, m, n, k, torch.cuda.current_stream().cuda_stream)
+    # the general entry point names its kernel per call (the library keeps no selection of its own)
+    rc = _capi.lib().daxq_linear_w8a8(0, 0, 0, xq_wide.data_ptr(), k + pad_k, sxd.data_ptr(), wq_wide.data_ptr(), k + pad_k,
+                                      swd.data_ptr(), bd.data_ptr(), out_wide.data_ptr(), n + pad_n, acc_wide.data_ptr(),
+                                      n + pad_n, m, n, k, variant, torch.cuda.current_stream().cuda_stream)
     _capi.check(rc, "linear_i8")
     torch.cuda.synchronize()
     assert torch.equal(acc_wide[:, :n].cpu(), want_acc)
@@ -118,7 +119,7 @@ def test_linear_i8_random_shapes_and_strides_bit_exact(ops, variant, m, n, k, pa
 def test_linear_i8_adversarial_extremes(ops, variant):
     from dax_amd import _capi
 
-    _capi.set_gemm_variant(variant)
+    _capi.debug_select_gemm(variant)
     m, n, k = 300, 264, 13824
     xq = torch.full((m, k), -128, dtype=torch.int8)
     xq[1::2] = 127
@@ -140,7 +141,7 @@ def test_linear_i8_one_hot_layout(ops, variant):
     # row/column or operand transposition inside the MFMA tiling
     from dax_amd import _capi
 
-    _capi.set_gemm_variant(variant)
+    _capi.debug_select_gemm(variant)
     m, n, k = 300, 300, 256
     rng = np.random.default_rng(0)
     for _ in range(6):
@@ -160,7 +161,7 @@ def test_linear_e4m3_within_tolerance(ops, variant, m, n, k):
     from dax_amd import _capi
 
     _skip_if_too_small(variant, m, n)
-    _capi.set_gemm_variant(variant)
+    _capi.debug_select_gemm(variant)
     x, w, b = O.make_inputs(m, k, n, seed=m + n + k + 1)
     qw, sw = O.weight_quant_e4m3(w)
     ref = O.linear_e4m3(x, qw, sw, b)
@@ -184,7 +185,7 @@ def test_linear_fp8_random_shapes_accumulators(ops, variant, e5m2, m, n, k, pad_
     against the exact sum of the decoded products (float64), element by element."""
     from dax_amd import _capi
 
-    _capi.set_gemm_variant(variant)
+    _capi.debug_select_gemm(variant)
     g = torch.Generator("cpu").manual_seed(m + 5 * n + 11 * k)
     act_dtype = torch.float8_e5m2 if e5m2 else torch.float8_e4m3fn
     xf = (torch.randn(m, k, generator=g) * 3).to(act_dtype)
@@ -198,10 +199,16 @@ def test_linear_fp8_random_shapes_accumulators(ops, variant, e5m2, m, n, k, pad_
     out_wide = torch.zeros((m, n + pad_n), dtype=torch.bfloat16, device="cuda")
     acc_wide = torch.full((m, n + pad_n), -1.0, dtype=torch.float32, device="cuda")
     ones_m, ones_n = torch.ones(m, device="cuda"), torch.ones(n, device="cuda")
-    fn = _capi.lib().daxq_linear_e5m2_e4m3 if e5m2 else _capi.lib().daxq_linear_e4m3
-    rc = fn(xq_wide.data_ptr(), k + pad_k, ones_m.data_ptr(), wq_wide.data_ptr(), k + pad_k, ones_n.data_ptr(), None,
-            out_wide.data_ptr(), n + pad_n, acc_wide.data_ptr(), n + pad_n, m, n, k,
-            torch.cuda.current_stream().cuda_stream)
+    if variant == 0:   # the named entry points (library's own choice of kernel)
+        fn = _capi.lib().daxq_linear_e5m2_e4m3 if e5m2 else _capi.lib().daxq_linear_e4m3
+        rc = fn(xq_wide.data_ptr(), k + pad_k, ones_m.data_ptr(), wq_wide.data_ptr(), k + pad_k, ones_n.data_ptr(), None,
+                out_wide.data_ptr(), n + pad_n, acc_wide.data_ptr(), n + pad_n, m, n, k,
+                torch.cuda.current_stream().cuda_stream)
+    else:
+        rc = _capi.lib().daxq_linear_w8a8(2 if e5m2 else 1, 1, 0, xq_wide.data_ptr(), k + pad_k, ones_m.data_ptr(),
+                                          wq_wide.data_ptr(), k + pad_k, ones_n.data_ptr(), None, out_wide.data_ptr(),
+                                          n + pad_n, acc_wide.data_ptr(), n + pad_n, m, n, k, variant,
+                                          torch.cuda.current_stream().cuda_stream)
     _capi.check(rc, "linear fp8")
     torch.cuda.synchronize()
     got = acc_wide[:, :n].cpu().double()
@@ -217,7 +224,7 @@ def test_linear_e5m2_activations_within_tolerance(ops, variant, m, n, k):
     from dax_amd import _capi
 
     _skip_if_too_small(variant, m, n)
-    _capi.set_gemm_variant(variant)
+    _capi.debug_select_gemm(variant)
     x, w, b = O.make_inputs(m, k, n, seed=m + n + k + 2)
     qw, sw = O.weight_quant_e4m3(w)
     ref = O.linear_e4m3(x, qw, sw, b, act_dtype=torch.float8_e5m2)
@@ -244,7 +251,7 @@ def test_linear_leading_dimensions_through_the_c_abi(ops, variant):
     what a caller does that writes q | k | v into one [M, 3N] tensor with three launches."""
     from dax_amd import _capi
 
-    _capi.set_gemm_variant(variant)
+    _capi.debug_select_gemm(variant)
     m, n, k = 600, 520, 384
     x, w, b = O.make_inputs(m, k, n, seed=77)
     qw, sw = O.weight_quant_int8(w)
@@ -257,16 +264,21 @@ def test_linear_leading_dimensions_through_the_c_abi(ops, variant):
     acc_wide = torch.zeros((m, n + 4), dtype=torch.int32, device="cuda")
     sx, swd, bd = dev(ref["sx"].reshape(-1).contiguous()), dev(sw.reshape(-1).contiguous()), dev(b)
     col0 = n + 8                                                    # 16-byte aligned column offset
-    rc = _capi.lib().daxq_linear_i8(xq_wide.data_ptr(), k + 128, sx.data_ptr(), wq_wide.data_ptr(), k + 256, swd.data_ptr(),
-                                    bd.data_ptr(), out_wide.data_ptr() + 2 * col0, 3 * n + 8, acc_wide.data_ptr(), n + 4,
-                                    m, n, k, torch.cuda.current_stream().cuda_stream)
+    if variant == 0:
+        rc = _capi.lib().daxq_linear_i8(xq_wide.data_ptr(), k + 128, sx.data_ptr(), wq_wide.data_ptr(), k + 256, swd.data_ptr(),
+                                        bd.data_ptr(), out_wide.data_ptr() + 2 * col0, 3 * n + 8, acc_wide.data_ptr(), n + 4,
+                                        m, n, k, torch.cuda.current_stream().cuda_stream)
+    else:
+        rc = _capi.lib().daxq_linear_w8a8(0, 0, 0, xq_wide.data_ptr(), k + 128, sx.data_ptr(), wq_wide.data_ptr(), k + 256,
+                                          swd.data_ptr(), bd.data_ptr(), out_wide.data_ptr() + 2 * col0, 3 * n + 8,
+                                          acc_wide.data_ptr(), n + 4, m, n, k, variant, torch.cuda.current_stream().cuda_stream)
     _capi.check(rc, "linear_i8")
     torch.cuda.synchronize()
     assert torch.equal(out_wide[:, col0:col0 + n].cpu().view(torch.int16), ref["out"].view(torch.int16))
     assert torch.equal(acc_wide[:, :n].cpu(), ref["acc"])
     assert bool((out_wide[:, :col0] == 1).all()) and bool((out_wide[:, col0 + n:] == 1).all())   # nothing outside the slice
     assert bool((acc_wide[:, n:] == 0).all())
-    _capi.set_gemm_variant(0)
+    _capi.debug_select_gemm(0)
 
 
 # --------------------------------------------------------------------------- the swapped module
@@ -391,10 +403,18 @@ def test_fp8_default_qconfig_e5m2_activations_e4m3_weights():
     y = model.to_q(x.to("cuda"))
     ref = O.linear_e4m3(x, qw, sw, b, act_dtype=torch.float8_e5m2)["out"]
     assert rel_l2(y, ref) < FP8_TOL
-    # e5m2 weights are not built: the layer stays a float module, as the reference does on NotImplementedError
+    # e5m2 weights (any of FP8_ALLOWED_DTYPES is a valid weight dtype, dax/quant/nn/dynamic/linear.py:42-43)
     model2 = _toy(3).to("cuda")
+    w2 = model2.to_q.weight.detach().cpu().clone()
+    b2 = model2.to_q.bias.detach().cpu().clone()
     quantize_dynamic(model2, {"": cfg(weight_dtype=torch.float8_e5m2)})
-    assert type(model2.to_q) is nn.Linear
+    assert isinstance(model2.to_q, QLinear) and model2.to_q.qweight.dtype == torch.float8_e5m2
+    qw2, sw2 = O.weight_quant_fp8(w2, torch.float8_e5m2)
+    assert torch.equal(model2.to_q.qweight.cpu().view(torch.uint8), qw2.view(torch.uint8))
+    assert torch.equal(model2.to_q.weight_scale.cpu(), sw2)
+    y2 = model2.to_q(x.to("cuda"))
+    ref2 = O.linear_fp8(x, qw2, sw2, b2, act_dtype=torch.float8_e5m2)["out"]
+    assert rel_l2(y2, ref2) < FP8_TOL
 
 
 def test_state_dict_round_trip_and_hooks():
@@ -460,3 +480,76 @@ def test_full_size_14b_out_proj_rows_and_checksum(ops, fp8):
         # idempotence: a second launch over the same operands gives the same bits
         out2 = ops.linear_i8(xq, sx, dev(qw), dev(sw.view(-1)), dev(b))
         assert torch.equal(out2, out)
+
+
+# ------------------------------------------------------------------ split-K (few output tiles)
+@pytest.mark.parametrize("m,n,k,splits", [(512, 5120, 5120, 2), (512, 5120, 5120, 4), (300, 520, 1024, 2), (128, 128, 1024, 8),
+                                          (1000, 392, 1536, 3), (512, 5120, 5120, 0)])
+def test_linear_i8_splitk_bit_exact(ops, m, n, k, splits):
+    """K cut into ranges that run as separate workgroups: integer partial sums, so outputs equal the oracle's bit for bit;
+    two calls in a row on the same workspace (the counters are left at zero), the second on another problem."""
+    x, w, b = O.make_inputs(m, k, n, seed=m + n + k + splits)
+    qw, sw = O.weight_quant_int8(w)
+    ref = O.linear_int8(x, qw, sw, b)
+    xq, sx = ops.act_quant_i8(dev(x))
+    out = ops.linear_w8a8_splitk(xq, sx, dev(qw), dev(sw.view(-1)), dev(b), "i8", "i8", splits)
+    np.testing.assert_array_equal(bf16_bits(out), bf16_bits(ref["out"]))
+    out_nb = ops.linear_w8a8_splitk(xq[: m - 100 if m > 300 else m], sx[: m - 100 if m > 300 else m], dev(qw), dev(sw.view(-1)), None,
+                                    "i8", "i8", splits)
+    rows = m - 100 if m > 300 else m
+    ref_nb = O.epilogue_int8(ref["acc"][:rows], ref["sx"][:rows], sw, None)
+    np.testing.assert_array_equal(bf16_bits(out_nb), bf16_bits(ref_nb))
+    out2 = ops.linear_w8a8_splitk(xq, sx, dev(qw), dev(sw.view(-1)), dev(b), "i8", "i8", splits)
+    np.testing.assert_array_equal(bf16_bits(out2), bf16_bits(ref["out"]))
+
+
+def test_splitk_workspace_shared_by_launches_of_different_shapes(ops):
+    """One workspace, a launch with few tiles and many ranges, then one with more tiles: the second launch's counters
+    must not sit where the first one kept partial results."""
+    cases = [(172, 5120, 13824, 6), (512, 5120, 5120, 2), (300, 640, 1024, 4), (512, 5120, 5120, 2)]
+    for m, n, k, splits in cases:
+        x, w, b = O.make_inputs(m, k, n, seed=k + splits)
+        qw, sw = O.weight_quant_int8(w)
+        ref = O.linear_int8(x, qw, sw, b, keep_acc=False)["out"]
+        xq, sx = ops.act_quant_i8(dev(x))
+        out = ops.linear_w8a8_splitk(xq, sx, dev(qw), dev(sw.view(-1)), dev(b), "i8", "i8", splits)
+        np.testing.assert_array_equal(bf16_bits(out), bf16_bits(ref), err_msg=str((m, n, k, splits)))
+
+
+@pytest.mark.parametrize("e5m2", [False, True])
+def test_linear_fp8_splitk_within_tolerance_and_deterministic(ops, e5m2):
+    m, n, k = 512, 1536, 2048
+    x, w, b = O.make_inputs(m, k, n, seed=91)
+    qw, sw = O.weight_quant_e4m3(w)
+    act = torch.float8_e5m2 if e5m2 else torch.float8_e4m3fn
+    ref = O.linear_fp8(x, qw, sw, b, act_dtype=act)
+    xq, sx = (ops.act_quant_e5m2 if e5m2 else ops.act_quant_e4m3)(dev(x))
+    fmt = "e5m2" if e5m2 else "e4m3"
+    outs = [ops.linear_w8a8_splitk(xq, sx, dev(qw.view(torch.uint8)), dev(sw.view(-1)), dev(b), fmt, "e4m3", 4) for _ in range(3)]
+    assert rel_l2(outs[0], ref["out"]) < 3e-3
+    assert all(torch.equal(o, outs[0]) for o in outs[1:])       # partial sums are added in range order: no run-to-run noise
+    plain = ops.linear_w8a8(xq, sx, dev(qw.view(torch.uint8)), dev(sw.view(-1)), dev(b), fmt, "e4m3", torch.bfloat16)
+    assert rel_l2(outs[0], plain) < 3e-3
+
+
+def test_splitk_argument_checks(ops):
+    from dax_amd import _capi
+
+    L = _capi.lib()
+    assert L.daxq_linear_splitk_choice(75600, 5120, 5120) == 1 and L.daxq_linear_splitk_choice(512, 5120, 5120) > 1
+    assert L.daxq_linear_splitk_choice(64, 5120, 5120) == 1
+    need = L.daxq_linear_splitk_workspace_bytes(512, 5120, 2)
+    assert need == 16384 + 160 * 2 * 65536      # the counter head (fixed) + two partial results for each of 160 tiles
+    xq = torch.zeros(512, 1024, dtype=torch.int8, device="cuda")
+    wq = torch.zeros(256, 1024, dtype=torch.int8, device="cuda")
+    ones_m, ones_n = torch.ones(512, device="cuda"), torch.ones(256, device="cuda")
+    out = torch.empty(512, 256, dtype=torch.bfloat16, device="cuda")
+    ws = torch.zeros(2 << 20, dtype=torch.uint8, device="cuda")
+    st = torch.cuda.current_stream().cuda_stream
+    args = (0, 0, xq.data_ptr(), 1024, ones_m.data_ptr(), wq.data_ptr(), 1024, ones_n.data_ptr(), None, out.data_ptr(), 256, 512, 256, 1024)
+    assert L.daxq_linear_w8a8_splitk(*args, 2, ws.data_ptr(), 1000, st) == -1 and "workspace" in _capi.last_error()
+    assert L.daxq_linear_w8a8_splitk(*args, 3, ws.data_ptr(), ws.numel(), st) == -2        # 8 units of K do not divide by 3
+    assert L.daxq_linear_w8a8_splitk(*args, 2, ws.data_ptr() + 16, ws.numel() - 16, st) == -2
+    assert L.daxq_linear_w8a8_splitk(*args, 2, ws.data_ptr(), ws.numel(), st) == 0
+    torch.cuda.synchronize()
+    assert bool((out == 0).all()) and bool((ws[:16384] == 0).all())
