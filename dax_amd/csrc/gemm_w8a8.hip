@@ -447,9 +447,78 @@ static int splitk_formats(int x_fmt, int w_fmt, bool& fp8, int& f8) {
     return fail(DAXQ_ERR_ARG, "linear: unsupported operand formats x=%d w=%d (int8 x int8, or fp8 x fp8)", x_fmt, w_fmt);
 }
 
+// ---- split-K on the library's own scratch memory (for callers that cannot allocate) ------------------------------
+// The workspace of daxq_linear_w8a8_splitk as a file-scope device array: tile counters at its head, then room for 512
+// partial results of 64 KiB (tiles x ranges <= 512, which is also the most that splitk_choice ever asks for).  Every
+// device the library runs on holds its own copy at its own address until the process ends.  `scratch` is only the
+// host-side handle of the array: host code uses the per-device address that hipGetSymbolAddress returned, never the name.
+constexpr int64_t kStaticSlots = 512;
+constexpr int64_t kStaticScratchBytes = kCounterBytes + kStaticSlots * kPartialBytes;
+static __device__ __align__(256) __attribute__((used)) unsigned char scratch[kStaticScratchBytes];
+
+constexpr int kMaxDevices = 64;
+static std::atomic<void*> g_scratch_ptr[kMaxDevices];      // device address of `scratch`, per device
+static std::atomic<int> g_scratch_cleared[kMaxDevices];    // counters cleared once on that device
+
+__global__ void clear_counters_kernel(int32_t* counters, int n) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) counters[i] = 0;
+}
+
+// Address of the current device's copy of `scratch`, looked up once per device.
+static int scratch_of_current_device(void** ptr, int* dev_out) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return fail(DAXQ_ERR_LAUNCH, "hipGetDevice failed");
+    if (dev < 0 || dev >= kMaxDevices) return fail(DAXQ_ERR_DEVICE, "linear_splitk_static: device index %d, at most %d devices", dev, kMaxDevices);
+    void* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (!p) {
+        hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p) return fail(DAXQ_ERR_LAUNCH, "hipGetSymbolAddress(scratch) on device %d: %s", dev, hipGetErrorString(e));
+        if ((uintptr_t)p & 255) return fail(DAXQ_ERR_ALIGN, "the library's scratch array is not 256-byte aligned on device %d", dev);
+        g_scratch_ptr[dev].store(p, std::memory_order_release);
+    }
+    *ptr = p;
+    *dev_out = dev;
+    return DAXQ_OK;
+}
+
 }  // namespace daxq
 
 extern "C" {
+
+int daxq_linear_w8a8_splitk_static(int x_fmt, int w_fmt, const void* xq, int64_t ld_xq, const float* sx, const void* wq,
+                                   int64_t ld_wq, const float* sw, const void* bias, void* out, int64_t ld_out,
+                                   int64_t m, int64_t n, int64_t k, int splits, daxq_stream_t stream) {
+    using namespace daxq;
+    bool fp8;
+    int f8;
+    if (int rc = splitk_formats(x_fmt, w_fmt, fp8, f8)) return rc;
+    if (splits < 0 || splits > 64) return fail(DAXQ_ERR_ARG, "linear_splitk_static: splits must be 0 (library's choice) to 64");
+    if (m < 0 || n < 0 || k <= 0) return fail(DAXQ_ERR_ARG, "linear_splitk_static: bad shape m=%lld n=%lld k=%lld", (long long)m, (long long)n, (long long)k);
+    if (splits == 0) splits = splitk_choice(m, n, k);
+    hipStream_t st = (hipStream_t)stream;
+    void* ws = nullptr;
+    if (splits > 1) {
+        const int64_t slots = splitk_tiles(m, n) * splits;
+        if (slots > kStaticSlots)
+            return fail(DAXQ_ERR_ARG, "linear_splitk_static: %lld output tiles of 128x128 in %d ranges need %lld partial results, the library's "
+                        "scratch array holds %lld (%lld bytes); use daxq_linear_w8a8_splitk with a workspace", (long long)splitk_tiles(m, n),
+                        splits, (long long)slots, (long long)kStaticSlots, (long long)kStaticScratchBytes);
+        int dev = 0;
+        if (int rc = scratch_of_current_device(&ws, &dev)) return rc;
+        if (!g_scratch_cleared[dev].load(std::memory_order_acquire)) {
+            // first use on this device: the counters start at zero (a kernel on the caller's stream, in front of the GEMM)
+            hipLaunchKernelGGL(clear_counters_kernel, dim3((unsigned)(kMaxSplitTiles / 256)), dim3(256), 0, st,
+                               static_cast<int32_t*>(ws), (int)kMaxSplitTiles);
+            if (int rc = check_launch("clear_counters")) return rc;
+            g_scratch_cleared[dev].store(1, std::memory_order_release);
+        }
+    }
+    return fp8 ? launch_gemm_splitk<true>(xq, ld_xq, sx, wq, ld_wq, sw, bias, out, ld_out, m, n, k, splits, ws,
+                                          kStaticScratchBytes, st, f8)
+               : launch_gemm_splitk<false>(xq, ld_xq, sx, wq, ld_wq, sw, bias, out, ld_out, m, n, k, splits, ws,
+                                           kStaticScratchBytes, st, 0);
+}
 
 int daxq_linear_splitk_choice(int64_t m, int64_t n, int64_t k) { return daxq::splitk_choice(m, n, k); }
 
@@ -491,6 +560,11 @@ int daxq_init(void) {
     DAXQ_PREP_F8(2)
     DAXQ_PREP_F8(3)
 #undef DAXQ_PREP_F8
+    if (!rc) {  // this device's address of the scratch array behind daxq_linear_w8a8_splitk_static
+        void* p = nullptr;
+        int dev = 0;
+        rc = scratch_of_current_device(&p, &dev);
+    }
     return rc;
 }
 

@@ -25,7 +25,7 @@
 extern "C" {
 #endif
 
-#define DAXQ_ABI_VERSION 2
+#define DAXQ_ABI_VERSION 3
 
 #define DAXQ_OK 0
 #define DAXQ_ERR_ARG (-1)    /* null pointer, negative size, bad enum */
@@ -293,6 +293,24 @@ int daxq_linear_w8a8_splitk(int x_fmt, int w_fmt,
                             const void* bias, void* out, int64_t ld_out,
                             int64_t m, int64_t n, int64_t k,
                             int splits, void* workspace, int64_t workspace_bytes, daxq_stream_t stream);
+
+/*
+ * daxq_linear_w8a8_splitk without a workspace argument, for callers that cannot allocate device memory (code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.
+ * Counters and partial results live in a device array inside the library (16 KiB + 512 x 64 KiB = 33 570 816 bytes on
+ * every GPU the library runs on, held until the process ends); the call allocates and frees nothing.
+ *   limit   ceil(m / 128) * ceil(n / 128) * splits <= 512 (what daxq_linear_splitk_choice picks always fits);
+ *           larger requests return DAXQ_ERR_ARG and launch nothing.
+ *   sharing every call on a GPU uses that GPU's one array: calls that overlap in time on one GPU (two streams, two
+ *           threads, two graphs replayed side by side) race.  Calls on one stream are ordered and safe.
+ * Results equal daxq_linear_w8a8_splitk's for the same arguments, bit for bit (same kernels, same summation order).
+ */
+int daxq_linear_w8a8_splitk_static(int x_fmt, int w_fmt,
+                                   const void* xq, int64_t ld_xq, const float* sx,
+                                   const void* wq, int64_t ld_wq, const float* sw,
+                                   const void* bias, void* out, int64_t ld_out,
+                                   int64_t m, int64_t n, int64_t k,
+                                   int splits, daxq_stream_t stream);
 
 #ifdef __cplusplus
 }
