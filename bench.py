@@ -209,6 +209,7 @@ def main():
                          "config0 (one linear, M = 4096, K = N = 1536); the sub-records exist for 14b only")
     ap.add_argument("--variant", type=int, default=0, help="GEMM kernel selection for comparisons (0 = library default)")
     ap.add_argument("--tile-group", type=int, default=0, help="tile-order group depth (0 = library default)")
+    ap.add_argument("--tile-order", type=int, default=0, help="tile order of the five-stage kernel: 0 = library default, 1 = row groups, 2 = whole patches per XCD")
     ap.add_argument("--m", type=int, default=0, help="tokens (0 = the model's own count)")
     ap.add_argument("--cpu-rows", type=int, default=0, help="tokens in the CPU-baseline sample (0 = pick for 10-30 s)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -228,10 +229,12 @@ def main():
 
     assert torch.cuda.is_available(), "bench.py needs an MI355X"
     _capi.require_gfx950(0)
-    if args.variant or args.tile_group:
+    if args.variant or args.tile_group or args.tile_order:
         _capi.debug_select_gemm(args.variant)
         if args.tile_group:
             _capi.debug_select_gemm(1000 + args.tile_group)
+        if args.tile_order:
+            _capi.debug_select_gemm(2000 + args.tile_order)
     dev = torch.device("cuda:0")
     model_name, model_tag, m_model, shapes = MODELS[args.model]
     m = args.m or m_model

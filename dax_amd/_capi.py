@@ -125,15 +125,18 @@ FLOAT_KIND = {"bf16": 0, "f16": 1, "f32": 2}  # DAXQ_BF16 / DAXQ_F16 / DAXQ_F32
 # Host-side only: the library itself keeps no selection, every call names its kernel.
 _kernel_choice = 0
 _tile_group = 0
+_tile_order = 0
 
 
 def debug_select_gemm(v: int) -> None:
     """0 = the library's choice by shape; 2 / 5 / 6 / 8 / 9 / 11 = one implementation (include/daxq.h);
     1000 + d = depth d of the tile-order groups (1000 = default)."""
-    global _kernel_choice, _tile_group
+    global _kernel_choice, _tile_group, _tile_order
     v = int(v)
     if 1000 <= v < 1064:
         _tile_group = v - 1000
+    elif 2000 <= v < 2004:
+        _tile_order = v - 2000
     elif v in (0, 2, 5, 6, 8, 9, 11):
         _kernel_choice = v
     else:
@@ -141,4 +144,4 @@ def debug_select_gemm(v: int) -> None:
 
 
 def kernel_arg() -> int:
-    return _kernel_choice | (_tile_group << 16)
+    return _kernel_choice | (_tile_group << 16) | (_tile_order << 24)

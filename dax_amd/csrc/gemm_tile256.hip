@@ -624,7 +624,11 @@ __global__ __launch_bounds__(256) void gemm_tile256s5_kernel(const GemmArgs p) {
         split = blockIdx.x - tile_id * p.splits;
         klen = p.k / p.splits;
     }
-    tile_of_block(p.gm, tile_id, p.tiles_m, p.tiles_n, tm, tn);
+    if (!SPLITK && p.order == 1) {
+        if (!tile_of_block_patched(tile_id, p.tiles_m, p.tiles_n, tm, tn)) return;  // padding slot (before any barrier)
+    } else {
+        tile_of_block(p.gm, tile_id, p.tiles_m, p.tiles_n, tm, tn);
+    }
     int m0 = tm * BT, n0 = tn * BT;
     m0 = m0 + BT <= p.m ? m0 : p.m - BT;
     n0 = n0 + BT <= p.n ? n0 : p.n - BT;
@@ -869,57 +873,79 @@ __global__ __launch_bounds__(256) void gemm_tile256s5_kernel(const GemmArgs p) {
         }
     }
     if constexpr (SPLITK) {
-        // ---- partial accumulators -> workspace; the last workgroup of the tile sums all of them
+        // ---- partial accumulators -> workspace; the last workgroup of the tile sums all of them.
+        // Partial results cross from one XCD's L2 to another's.  A device-wide fence would do that by writing back
+        // and invalidating the whole L2 of the XCD, once per wavefront (measured: 0.3 us per workgroup, serialised,
+        // 4x the time of the plain launch).  Instead every access to the workspace is itself an agent-scope relaxed
+        // atomic (a store / load with the device-coherent cache policy), the stores are waited for (vmcnt) before the
+        // workgroup's barrier, and only then does one thread count the workgroup in; the last arriver reads behind
+        // a barrier that follows its own count.
         __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));  // the scale / bias loads have landed: the waits above count them
         constexpr int VPB = N16 ? 1 : 4;           // 16-byte vectors per lane and MFMA block
         constexpr int NV = NB * NB * VPB;          // per lane: 16 of them = 64 registers either way
-        typedef int v4raw __attribute__((ext_vector_type(4)));
-        v4raw* mine = static_cast<v4raw*>(p.partials) + (int64_t)blockIdx.x * NV * 256 + t;
+        typedef uint64_t u64x2 __attribute__((ext_vector_type(2)));
+        uint64_t* mine = static_cast<uint64_t*>(p.partials) + ((int64_t)blockIdx.x * NV * 256 + t) * 2;
 #pragma unroll
         for (int j = 0; j < NB; ++j)
 #pragma unroll
             for (int i = 0; i < NB; ++i)
 #pragma unroll
                 for (int v = 0; v < VPB; ++v) {
-                    v4raw w;
+                    v4i w;
                     if constexpr (N16) {
                         w = acc[j][i];
                     } else {
 #pragma unroll
                         for (int e = 0; e < 4; ++e) w[e] = __float_as_int(acc[j][i][4 * v + e]);  // (a by-value call: __builtin_bit_cast of a vector element reads element 0)
                     }
-                    mine[((j * NB + i) * VPB + v) * 256] = w;
+                    const u64x2 w2 = __builtin_bit_cast(u64x2, w);
+                    uint64_t* dst = mine + (int64_t)((j * NB + i) * VPB + v) * 512;
+                    __hip_atomic_store(dst, w2[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    __hip_atomic_store(dst + 1, w2[1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 }
-        __threadfence();  // the partial result is visible device-wide before the counter moves
-        __syncthreads();
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));  // this lane's partial results have reached device-coherent memory
+        __syncthreads();                           // ... and every lane's
         int* flag = reinterpret_cast<int*>(smem + 2048);  // LDS is free: nobody reads a stage after the last barrier
-        if (t == 0) *flag = atomicAdd(p.counters + tile_id, 1) == p.splits - 1;
+        if (t == 0) *flag = __hip_atomic_fetch_add(p.counters + tile_id, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == p.splits - 1;
         __syncthreads();
         if (!*flag) return;
-        __threadfence();  // acquire: the other workgroups' partial results
-        const v4raw* all = static_cast<const v4raw*>(p.partials) + (int64_t)tile_id * p.splits * NV * 256 + t;
+        const uint64_t* all = static_cast<const uint64_t*>(p.partials) + ((int64_t)tile_id * p.splits * NV * 256 + t) * 2;
+        // one range at a time, in range order (FP8 sums then do not depend on who came last); all loads of a range
+        // are in flight together, so a range costs one trip to memory, not one per vector
+        v4i sum[NV];
+        for (int sp = 0; sp < p.splits; ++sp) {
+            const uint64_t* src = all + (int64_t)sp * NV * 512;
+            u64x2 w2[NV];
+#pragma unroll
+            for (int x = 0; x < NV; ++x) {
+                w2[x][0] = __hip_atomic_load(src + x * 512, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                w2[x][1] = __hip_atomic_load(src + x * 512 + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+#pragma unroll
+            for (int x = 0; x < NV; ++x) {
+                const v4i w = __builtin_bit_cast(v4i, w2[x]);
+                if (sp == 0) {
+                    sum[x] = w;  // (0.0f + x would turn a -0.0 partial sum into +0.0)
+                } else if constexpr (FP8) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) sum[x][e] = __float_as_int(__int_as_float(sum[x][e]) + __int_as_float(w[e]));
+                } else {
+                    sum[x] += w;
+                }
+            }
+        }
 #pragma unroll
         for (int j = 0; j < NB; ++j)
 #pragma unroll
             for (int i = 0; i < NB; ++i)
 #pragma unroll
                 for (int v = 0; v < VPB; ++v) {
-                    v4raw sum = all[((j * NB + i) * VPB + v) * 256];
-                    for (int sp = 1; sp < p.splits; ++sp) {
-                        const v4raw w = all[((int64_t)sp * NV + (j * NB + i) * VPB + v) * 256];
-                        if constexpr (FP8) {
-#pragma unroll
-                            for (int e = 0; e < 4; ++e)
-                                sum[e] = __float_as_int(__int_as_float(sum[e]) + __int_as_float(w[e]));
-                        } else {
-                            sum += w;
-                        }
-                    }
+                    const v4i sv = sum[(j * NB + i) * VPB + v];
                     if constexpr (N16) {
-                        acc[j][i] = sum;
+                        acc[j][i] = sv;
                     } else {
 #pragma unroll
-                        for (int e = 0; e < 4; ++e) acc[j][i][4 * v + e] = __int_as_float(sum[e]);
+                        for (int e = 0; e < 4; ++e) acc[j][i][4 * v + e] = __int_as_float(sv[e]);
                     }
                 }
         if (t == 0) p.counters[tile_id] = 0;  // ready for the next launch on this workspace
@@ -979,7 +1005,7 @@ static int launch_tile256s5_impl(const GemmArgs& a, hipStream_t st) {
     constexpr int SMEM = NST * 2 * BT * BKS;  // 160 KB (256 tile), 80 KB (128 tile)
     auto kern = gemm_tile256s5_kernel<FP8, DUMP, F8, N16, BT>;
     if (int rc = prepare_tile256s5<FP8, DUMP, F8, N16, BT>()) return rc;
-    const int64_t nt = (int64_t)a.tiles_m * a.tiles_n;
+    const int64_t nt = a.order == 1 ? patched_grid(a.tiles_m, a.tiles_n) : (int64_t)a.tiles_m * a.tiles_n;
     if (nt > 0x7fffffff) return fail(DAXQ_ERR_ARG, "gemm: too many tiles");
     hipLaunchKernelGGL(kern, dim3((unsigned)nt), dim3(T), SMEM, st, a);
     return check_launch("gemm_tile256s5");

@@ -323,6 +323,12 @@ static int launch_gemm(const void* xq, int64_t ld_xq, const float* sx, const voi
     a.k = (int)k;
     a.tiles_m = a.tiles_n = 0;
     a.gm = (kernel >> 16) & 0xff ? (kernel >> 16) & 0xff : 4;
+    // Tile order of the five-stage 256x256 kernel (bits 24-25 of `kernel`: 0 = by shape, 1 = row groups, 2 = whole
+    // patches per XCD).  The patch order brings the L2-miss traffic down to what eight separate L2s must fetch (measured:
+    // 1.00x that floor on the four 14B shapes against 1.15-1.36x for the row groups), but only the long-K launch gets
+    // faster by it (K = 13824: +2 %; K = 5120: -0.5 to -7 %, 32 CUs in lockstep on the same 12 panels), so long K takes it.
+    const int order_bits = (kernel >> 24) & 3;
+    a.order = order_bits == 2 || (order_bits == 0 && k >= 8192 && m >= 8192) ? 1 : 0;
     a.out_kind = out_kind;
     a.splits = 1;
     a.counters = nullptr;
@@ -373,15 +379,17 @@ static int64_t splitk_tiles(int64_t m, int64_t n) { return ((m + 127) / 128) * (
 constexpr int64_t kCounterBytes = 16384;
 constexpr int64_t kMaxSplitTiles = kCounterBytes / 4;
 
-// How many ranges pay: as many as keep every range at least 512 bytes of K deep, divide K / 128 evenly and do not put
-// more than two workgroups on a CU (two is what the LDS holds); 1 = no split.
+// How many ranges pay: as many as give every workgroup a CU of its own (tiles x ranges <= 256), keep a range at
+// least 1024 bytes of K deep and divide K / 128 evenly; 1 = no split.  Measured at N = K = 5120 (INT8, us, plain launch /
+// 2 / 4 ranges): M = 256 (80 tiles) 34 / 28 / 40, M = 512 (160 tiles) 24 / 35 / 52, M = 1024 52 / 71 / -: the partial
+// results make a round trip through device-coherent memory (about 10 us for 20 MB), which only idle CUs pay for.
 static int splitk_choice(int64_t m, int64_t n, int64_t k) {
     if (m < 128 || n < 128 || k % DAXQ_K_ALIGN) return 1;
     const int64_t tiles = splitk_tiles(m, n), units = k / DAXQ_K_ALIGN;
     int best = 1;
     for (int s = 2; s <= 8; ++s)
-        if (units % s == 0 && k / s >= 512 && tiles * s <= 512) best = s;
-    return tiles >= 256 ? 1 : best;
+        if (units % s == 0 && k / s >= 1024 && tiles * s <= 256) best = s;
+    return best;
 }
 
 template <bool FP8>
@@ -425,6 +433,7 @@ static int launch_gemm_splitk(const void* xq, int64_t ld_xq, const float* sx, co
     a.k = (int)k;
     a.tiles_m = a.tiles_n = 0;
     a.gm = 4;
+    a.order = 0;
     a.out_kind = DAXQ_BF16;
     a.splits = splits;
     a.counters = static_cast<int32_t*>(workspace);

@@ -39,6 +39,7 @@ def _default_variant():
     from dax_amd import _capi
 
     _capi.debug_select_gemm(0)
+    _capi.debug_select_gemm(2000)
 
 
 def dev(t):
@@ -68,6 +69,39 @@ def test_linear_i8_bit_exact(ops, variant, m, n, k):
     out2 = ops.linear_i8(xq, sx, dev(qw), dev(sw.view(-1)), None)
     ref2 = O.epilogue_int8(ref["acc"], ref["sx"], sw, None)
     np.testing.assert_array_equal(bf16_bits(out2), bf16_bits(ref2))
+
+
+# tile grids (in 256-tiles) whose remainder band is 0 to 7 columns wide, with and without a partial last patch
+PATCH_SHAPES = [(256, 2048, 128), (1100, 2304, 128), (2600, 1024 + 256 * 2, 256), (700, 2048 + 256 * 3, 128), (2100, 256 * 4, 128),
+                (1300, 2048 + 256 * 5, 128), (1500, 256 * 6, 256), (520, 4096 + 256 * 7, 128), (8500, 304, 128), (300, 5120, 384)]
+
+
+@pytest.mark.parametrize("m,n,k", PATCH_SHAPES)
+def test_patch_tile_order_bit_exact(ops, m, n, k):
+    """The five-stage kernel with whole 32-slot patches per XCD (padding workgroups exit): every output tile is
+    computed exactly once, accumulators and outputs equal the integer oracle's; FP8 equals the row-group order's bits."""
+    from dax_amd import _capi
+
+    _capi.debug_select_gemm(8)
+    _capi.debug_select_gemm(2002)
+    g = torch.Generator().manual_seed(m + n + k)
+    xq = torch.randint(-127, 128, (m, k), dtype=torch.int8, generator=g)
+    wq = torch.randint(-127, 128, (n, k), dtype=torch.int8, generator=g)
+    sx, sw = torch.rand(m, generator=g) + 0.5, torch.rand(n, generator=g) * 0.01
+    b = torch.randn(n, generator=g).bfloat16()
+    ref_acc = O.int_mm(xq, wq)
+    ref_out = O.epilogue_int8(ref_acc, sx.view(-1, 1), sw.view(1, -1), b)
+    out, acc = ops.linear_i8_acc(dev(xq), dev(sx), dev(wq), dev(sw), dev(b))
+    assert torch.equal(acc.cpu(), ref_acc)
+    np.testing.assert_array_equal(bf16_bits(out), bf16_bits(ref_out))
+    out_plain = ops.linear_i8(dev(xq), dev(sx), dev(wq), dev(sw), dev(b))      # the launch without the accumulator dump
+    np.testing.assert_array_equal(bf16_bits(out_plain), bf16_bits(ref_out))
+    xf = torch.where((xq.view(torch.uint8) & 0x7f) == 0x7f, torch.zeros((), dtype=torch.uint8), xq.view(torch.uint8))
+    wf = torch.where((wq.view(torch.uint8) & 0x7f) == 0x7f, torch.zeros((), dtype=torch.uint8), wq.view(torch.uint8))
+    f_patch = ops.linear_e4m3(dev(xf), dev(sx), dev(wf), dev(sw), dev(b))
+    _capi.debug_select_gemm(2001)
+    f_rows = ops.linear_e4m3(dev(xf), dev(sx), dev(wf), dev(sw), dev(b))
+    assert torch.equal(f_patch.view(torch.int16), f_rows.view(torch.int16))
 
 
 def _random_shapes(count, seed):
@@ -484,7 +518,7 @@ def test_full_size_14b_out_proj_rows_and_checksum(ops, fp8):
 
 # ------------------------------------------------------------------ split-K (few output tiles)
 @pytest.mark.parametrize("m,n,k,splits", [(512, 5120, 5120, 2), (512, 5120, 5120, 4), (300, 520, 1024, 2), (128, 128, 1024, 8),
-                                          (1000, 392, 1536, 3), (512, 5120, 5120, 0)])
+                                          (1000, 392, 1536, 3), (512, 5120, 5120, 0), (256, 5120, 5120, 0)])
 def test_linear_i8_splitk_bit_exact(ops, m, n, k, splits):
     """K cut into ranges that run as separate workgroups: integer partial sums, so outputs equal the oracle's bit for bit;
     two calls in a row on the same workspace (the counters are left at zero), the second on another problem."""
@@ -536,7 +570,8 @@ def test_splitk_argument_checks(ops):
     from dax_amd import _capi
 
     L = _capi.lib()
-    assert L.daxq_linear_splitk_choice(75600, 5120, 5120) == 1 and L.daxq_linear_splitk_choice(512, 5120, 5120) > 1
+    assert L.daxq_linear_splitk_choice(75600, 5120, 5120) == 1 and L.daxq_linear_splitk_choice(256, 5120, 5120) == 2
+    assert L.daxq_linear_splitk_choice(512, 5120, 5120) == 1     # 160 tiles: a second range would have to share CUs
     assert L.daxq_linear_splitk_choice(64, 5120, 5120) == 1
     need = L.daxq_linear_splitk_workspace_bytes(512, 5120, 2)
     assert need == 16384 + 160 * 2 * 65536      # the counter head (fixed) + two partial results for each of 160 tiles
