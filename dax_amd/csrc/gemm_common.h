@@ -11,6 +11,7 @@ typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v8i __attribute__((ext_vector_type(8)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 typedef float v16f __attribute__((ext_vector_type(16)));
+typedef float v4f __attribute__((ext_vector_type(4)));
 typedef unsigned v2u __attribute__((ext_vector_type(2)));
 
 #define DAXQ_LDS __attribute__((address_space(3)))
@@ -69,6 +70,8 @@ constexpr int vmcnt_imm(int n) { return (n & 15) | ((n >> 4) << 14) | 0x0070 | 0
 
 // and-mask that turns an s_waitcnt immediate into one that also waits for lgkmcnt == 0
 constexpr int lgkmcnt0_mask() { return ~0x0f00; }
+// ... for lgkmcnt <= n (n < 16)
+constexpr int lgkmcnt_mask(int n) { return ~0x0f00 | (n << 8); }
 
 __device__ __forceinline__ int swz(int row) { return (row & 7) ^ ((row >> 3) & 1); }
 

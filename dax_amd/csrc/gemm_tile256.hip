@@ -243,14 +243,24 @@ __device__ __forceinline__ void tile256_epilogue(const GemmArgs& p, typename Acc
     }
 }
 
-// The same epilogue for INT8 accumulators held as 8 x 8 blocks of 16x16 (v_mfma_i32_16x16x64_i8).
+// accumulators of one 16x16 block: int32 (v_mfma_i32_16x16x64_i8) or fp32 (v_mfma_f32_16x16x128_f8f6f4)
+template <bool FP8>
+struct Acc16 {
+    typedef v4i type;
+};
+template <>
+struct Acc16<true> {
+    typedef v4f type;
+};
+
+// The same epilogue for accumulators held as 8 x 8 blocks of 16x16 (v_mfma_i32_16x16x64_i8, v_mfma_f32_16x16x128_f8f6f4).
 // In a block a lane owns output row m = l%16 and the columns n = 4*(l/16) + {0..3}.  One
 // v_permlane16_swap per word over two neighbouring blocks gives each lane 8 consecutive columns of one
 // of them: lanes 0-15 block 2jp columns 0-7, lanes 16-31 block 2jp+1 columns 0-7, lanes 32-47 block
 // 2jp columns 8-15, lanes 48-63 block 2jp+1 columns 8-15.
 // NB: 16x16 blocks per operand and wavefront (8: 256x256 tile, 4: 128x128 tile); the tile edge is 32 * NB.
-template <bool DUMP, int NB = 8>
-__device__ __forceinline__ void tile256_epilogue16(const GemmArgs& p, v4i (&acc)[NB][NB], uint8_t* smem, int m0, int n0, int t,
+template <bool DUMP, int NB = 8, bool FP8 = false>
+__device__ __forceinline__ void tile256_epilogue16(const GemmArgs& p, typename Acc16<FP8>::type (&acc)[NB][NB], uint8_t* smem, int m0, int n0, int t,
                                                    int wm, int wn, int l15, int g4, float pre_sx, float pre_sw,
                                                    float pre_bias) {
     constexpr int BT = 32 * NB, WT = 16 * NB;
@@ -271,8 +281,10 @@ __device__ __forceinline__ void tile256_epilogue16(const GemmArgs& p, v4i (&acc)
             for (int i = 0; i < NB; ++i) {
                 const int64_t m = m0 + wm * WT + i * 16 + l15;
 #pragma unroll
-                for (int v = 0; v < 4; ++v)
-                    static_cast<int32_t*>(p.acc)[m * p.ldacc + n0 + wn * WT + j * 16 + 4 * g4 + v] = acc[j][i][v];
+                for (int v = 0; v < 4; ++v) {
+                    if constexpr (FP8) static_cast<float*>(p.acc)[m * p.ldacc + n0 + wn * WT + j * 16 + 4 * g4 + v] = acc[j][i][v];
+                    else static_cast<int32_t*>(p.acc)[m * p.ldacc + n0 + wn * WT + j * 16 + 4 * g4 + v] = acc[j][i][v];
+                }
             }
     }
 
@@ -304,15 +316,19 @@ __device__ __forceinline__ void tile256_epilogue16(const GemmArgs& p, v4i (&acc)
 #pragma unroll
                 for (int h = 0; h < 2; ++h) {
                     const int r = 2 * h;
-                    float y0 = (float)acc[j][i][r];  // v_cvt_f32_i32, round to nearest even
-                    float y1 = (float)acc[j][i][r + 1];
-                    y0 = y0 * sxv;
-                    y1 = y1 * sxv;
-                    y0 = y0 * sws[r];
-                    y1 = y1 * sws[r + 1];
-                    const uint32_t o1 = pack_bf16_rne(y0, y1);
-                    // second rounding: the bias is added to the bf16 value
-                    pk[jj][h] = pack_bf16_rne(__uint_as_float(o1 << 16) + bs[r], __uint_as_float(o1 & 0xffff0000u) + bs[r + 1]);
+                    if constexpr (FP8) {
+                        pk[jj][h] = pack_bf16_rne(acc[j][i][r] * sxv * sws[r] + bs[r], acc[j][i][r + 1] * sxv * sws[r + 1] + bs[r + 1]);
+                    } else {
+                        float y0 = (float)acc[j][i][r];  // v_cvt_f32_i32, round to nearest even
+                        float y1 = (float)acc[j][i][r + 1];
+                        y0 = y0 * sxv;
+                        y1 = y1 * sxv;
+                        y0 = y0 * sws[r];
+                        y1 = y1 * sws[r + 1];
+                        const uint32_t o1 = pack_bf16_rne(y0, y1);
+                        // second rounding: the bias is added to the bf16 value
+                        pk[jj][h] = pack_bf16_rne(__uint_as_float(o1 << 16) + bs[r], __uint_as_float(o1 & 0xffff0000u) + bs[r + 1]);
+                    }
                 }
             }
             v2u s0 = __builtin_amdgcn_permlane16_swap(pk[0][0], pk[1][0], false, false);
@@ -959,6 +975,302 @@ __global__ __launch_bounds__(256) void gemm_tile256s5_kernel(const GemmArgs p) {
                                         p.bias ? bf16_bits_to_f32(pre_b) : -0.0f);
 }
 
+// ---------------------------------------------------------------------------------------------
+// FP8 on v_mfma_f32_16x16x128_f8f6f4: the 256x256 tile with 8 x 8 blocks of 16x16 per wavefront.
+//
+// The narrow FP8 MFMA draws less power per operation than the 32x32x64 form (register-only loops on this
+// workload's values: 4.41 against 4.02 P-op/s), as the 16x16x64 form does for INT8.  Its K is 128 bytes, a PAIR of
+// 64-byte slices, and the operand fragments of a pair fill 128 registers, so they cannot all be held twice beside
+// 256 accumulators.  Register plan (8 registers per fragment: 16 bytes of either slice of the pair):
+//   A (activation rows, MFMA "B" operand)  two sets of 8 fragments, the next pair's set read during the odd half
+//   B (weight rows, MFMA "A" operand)      ONE set: the MFMAs run B block by B block (j outer, A block i inner), block
+//                                          j is dead after its 8 MFMAs and is refilled in place for the next pair
+//                                          right behind them; block 7, which is in use until the pair ends, has a
+//                                          second register set
+// LDS: five 32 KB parts, each ONE operand of ONE pair, [slice of the pair][256 rows][64 B] with the 16-byte chunk
+// swizzle of the 16x16 INT8 form (chunk ^ ((row >> 1) & 3): a fragment read takes 16 rows x 4 chunks).  They form a
+// ring in the order the loads are issued, ... B(q+1), A(q+1), B(q+2), A(q+2), B(q+3) ...:
+//   pair q, even half   MFMAs of B blocks 0-3; DMA loads of A(q+2) into the part B(q) has left; reads B block 7 and
+//                       blocks 0-2 of pair q+1
+//   pair q, odd half    MFMAs of B blocks 4-7; DMA loads of B(q+3) into the part A(q) has left; reads B blocks 3-6
+//                       and all of A of pair q+1
+// One barrier per half: at the first B(q+1) has landed, at the second A(q+1); every load has two to three slice
+// times to land, as in the 64-byte-slice kernels above, and the half-line pairing of the loads is the same.
+// A and B of a lane hold the same K bytes (chunk l/16 of the pair's first slice, then of its second), which is all
+// the MFMA needs: the order of K inside an instruction is free as long as both operands agree.
+namespace f16 {
+constexpr int BT = 256, BKS = 64, T = 256, NPART = 5;
+constexpr int HALF = BT * BKS;   // one slice of one operand: 16 KB
+constexpr int PART = 2 * HALF;   // one operand of one pair: 32 KB
+constexpr int SMEM = NPART * PART;
+constexpr int RD_LAG = 0;  // regions between the last MFMA that reads a B fragment and the LDS read that refills it
+constexpr int TRAIL_READS = 0;  // ds_read_b128 issued behind the last B read of a pair (block 6 at region 56)
+}  // namespace f16
+
+template <bool DUMP, int F8>
+__global__ __launch_bounds__(256) void gemm_tile256f16_kernel(const GemmArgs p) {
+    using namespace f16;
+    constexpr int NB = 8;
+    extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    int tm, tn;
+    if (p.order == 1) {
+        if (!tile_of_block_patched(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn)) return;  // padding slot (before any barrier)
+    } else {
+        tile_of_block(p.gm, blockIdx.x, p.tiles_m, p.tiles_n, tm, tn);
+    }
+    int m0 = tm * BT, n0 = tn * BT;
+    m0 = m0 + BT <= p.m ? m0 : p.m - BT;
+    n0 = n0 + BT <= p.n ? n0 : p.n - BT;
+
+    // ---- HBM side: one wave instruction fills 1 KB of LDS = 16 rows x 64 B; lane l -> row l/4, stored chunk l%4,
+    //      i.e. global chunk (l%4) ^ ((row >> 1) & 3).  Load g of an operand and pair: row block g/2 (64 rows, of which
+    //      this wave fills 16), slice g%2 of the pair (the two halves of a 128-byte line, adjacent instructions).
+    const uint32_t gsw = (uint32_t)(((t & 3) ^ ((t >> 3) & 3)) << 4);
+    uint32_t voff_a = (uint32_t)(t >> 2) * (uint32_t)p.lda + gsw;
+    uint32_t voff_b = (uint32_t)(t >> 2) * (uint32_t)p.ldb + gsw;
+    uint32_t voff_a1 = voff_a + BKS, voff_b1 = voff_b + BKS;
+    const uint8_t* abase = p.a + (int64_t)m0 * p.lda;
+    const uint8_t* bbase = p.b + (int64_t)n0 * p.ldb;
+    const int64_t a_step = 64 * p.lda, b_step = 64 * p.ldb;
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(DAXQ_LDS uint8_t*)smem;
+    const uint32_t wave_lds = lds0 + (uint32_t)__builtin_amdgcn_readfirstlane(wave * 1024);
+    auto issue_a = [&](uint32_t part, int g) {
+        const int j = g >> 1, half = g & 1;
+        const uint32_t dst = wave_lds + part + half * HALF + j * 4096;
+        __builtin_amdgcn_global_load_lds((const DAXQ_GLOBAL void*)(abase + j * a_step + (half ? voff_a1 : voff_a)),
+                                         (DAXQ_LDS void*)(uintptr_t)dst, 16, 0, 0);
+    };
+    auto issue_b = [&](uint32_t part, int g) {
+        const int j = g >> 1, half = g & 1;
+        const uint32_t dst = wave_lds + part + half * HALF + j * 4096;
+        __builtin_amdgcn_global_load_lds((const DAXQ_GLOBAL void*)(bbase + j * b_step + (half ? voff_b1 : voff_b)),
+                                         (DAXQ_LDS void*)(uintptr_t)dst, 16, 0, 0);
+    };
+    auto advance_a = [&]() {
+        voff_a += 2 * BKS;
+        voff_a1 += 2 * BKS;
+    };
+    auto advance_b = [&]() {
+        voff_b += 2 * BKS;
+        voff_b1 += 2 * BKS;
+    };
+
+    // ---- LDS side: row (w*128 + i*16 + l%16), K chunk l/16 of either slice, stored at chunk (l/16) ^ ((l%16 >> 1) & 3)
+    const int lr = lane & 15, kg = lane >> 4;
+    const int xo = (kg ^ ((lr >> 1) & 3)) << 4;
+    const uint8_t* a_rd = smem + (wm * 128 + lr) * BKS + xo;
+    const uint8_t* b_rd = smem + (wn * 128 + lr) * BKS + xo;
+    // A fragment is refilled as two updates of half of its registers: the register allocator then keeps the
+    // fragment where it is (a fresh 8-register value per refill made it rotate the fragment sets through one
+    // another with copies and spills).
+    auto read_into = [&](v8i& dst, const uint8_t* base, uint32_t part, int blk) __attribute__((always_inline)) {
+        const uint8_t* pr = base + part + blk * 16 * BKS;
+        const v4i lo = *reinterpret_cast<const v4i*>(pr);
+        const v4i up = *reinterpret_cast<const v4i*>(pr + HALF);
+        const v8i lo8 = __builtin_shufflevector(lo, lo, 0, 1, 2, 3, -1, -1, -1, -1);  // (widened; the upper lanes are never taken)
+        const v8i up8 = __builtin_shufflevector(up, up, 0, 1, 2, 3, -1, -1, -1, -1);
+        dst = __builtin_shufflevector(lo8, dst, 0, 1, 2, 3, 12, 13, 14, 15);
+        dst = __builtin_shufflevector(dst, up8, 0, 1, 2, 3, 8, 9, 10, 11);
+    };
+
+    v4f acc[NB][NB];
+    // (left uninitialised on purpose: every register of a fragment is written by its first refill, and an
+    // initial value would have to be kept alive, and spilled, through the prologue)
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Wuninitialized"
+#pragma clang diagnostic ignored "-Wsometimes-uninitialized"
+    v8i fa0[NB], fa1[NB];  // A fragments of even / odd pairs
+    v8i fb[NB - 1];        // B fragments 0-6, refilled in place
+    v8i fb7_0, fb7_1;      // B fragment 7 of even / odd pairs
+#pragma clang diagnostic pop
+
+    const int Q = p.k / (2 * BKS);  // pairs; K is a multiple of 128
+    // the ring, oldest part first: at the start of pair q it holds B(q), A(q) (both read already), B(q+1), A(q+1), B(q+2)
+    uint32_t r0 = 0, r1 = PART, r2 = 2 * PART, r3 = 3 * PART, r4 = 4 * PART;
+
+    // One pair of slices.  PAR: parity of the pair (which A set and which B-7 set it consumes).
+    //   ISSUE_A  pair q+2 exists: its A loads go out during the even half
+    //   ISSUE_B  pair q+3 exists: its B loads go out during the odd half
+    //   NEXT     pair q+1 exists: read its fragments
+    //   EXTRA    younger loads that are not tile loads (the epilogue's scales) and may stay in flight
+    //   FIRST    pair 0 of the tile: every block's MFMA starts from zero
+    auto pair = [&](auto PAR, auto ISSUE_A, auto ISSUE_B, auto NEXT, auto EXTRA, auto FIRST) __attribute__((always_inline)) {
+        constexpr bool par = PAR.value, nxt = NEXT.value;
+        auto mfma = [&](int g) __attribute__((always_inline)) {
+            const int j = g >> 3, i = g & 7;
+            const v8i bfr = j == 7 ? (par ? fb7_1 : fb7_0) : fb[j < 7 ? j : 0];
+            const v8i afr = par ? fa1[i] : fa0[i];
+            // weights are the MFMA "A" operand (format select cbsz), activations the "B" operand (blgp); accumulators
+            // tied in place in AGPRs
+            if constexpr (FIRST.value) {
+                if constexpr (F8 == 0) asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, 0" : "=a"(acc[j][i]) : "v"(bfr), "v"(afr));
+                else if constexpr (F8 == kF8XE5) asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, 0 blgp:1" : "=a"(acc[j][i]) : "v"(bfr), "v"(afr));
+                else if constexpr (F8 == kF8WE5) asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, 0 cbsz:1" : "=a"(acc[j][i]) : "v"(bfr), "v"(afr));
+                else asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, 0 cbsz:1 blgp:1" : "=a"(acc[j][i]) : "v"(bfr), "v"(afr));
+            } else {
+                if constexpr (F8 == 0) asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0" : "+a"(acc[j][i]) : "v"(bfr), "v"(afr));
+                else if constexpr (F8 == kF8XE5) asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0 blgp:1" : "+a"(acc[j][i]) : "v"(bfr), "v"(afr));
+                else if constexpr (F8 == kF8WE5) asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0 cbsz:1" : "+a"(acc[j][i]) : "v"(bfr), "v"(afr));
+                else asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0 cbsz:1 blgp:1" : "+a"(acc[j][i]) : "v"(bfr), "v"(afr));
+            }
+        };
+        // ---- even half: B(q+1) has landed; loads younger than it: A(q+1), B(q+2).  The loads of this half overwrite
+        // the part that the B fragments of this pair were read from, so every wavefront's reads of it must be over:
+        // LDS reads complete in order, and behind the last B read of a pair only TRAIL_READS reads of A follow.
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm((nxt ? 8 : 0) + (ISSUE_A.value ? 8 : 0) + EXTRA.value) & lgkmcnt_mask(TRAIL_READS));
+        __builtin_amdgcn_s_barrier();
+#pragma unroll
+        for (int g = 0; g < 32; ++g) {
+            if constexpr (ISSUE_A.value) {
+                if ((g & 3) == 0) issue_a(r0, g >> 2);
+            }
+            if constexpr (nxt) {
+                if (g == 2) {
+                    if constexpr (par) read_into(fb7_0, b_rd, r2, 7);
+                    else read_into(fb7_1, b_rd, r2, 7);
+                }
+                if (g == 8 + RD_LAG) read_into(fb[0], b_rd, r2, 0);   // behind the MFMAs of block 0
+                if (g == 16 + RD_LAG) read_into(fb[1], b_rd, r2, 1);
+                if (g == 24 + RD_LAG) read_into(fb[2], b_rd, r2, 2);
+            }
+            mfma(g);
+            if constexpr (ISSUE_A.value) {
+                if (g == 30) advance_a();
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        // ---- odd half: A(q+1) has landed; loads younger than it: B(q+2), A(q+2).  (Its loads overwrite the part
+        // that this pair's A fragments were read from, a whole half ago: no LDS wait.)
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm((ISSUE_A.value ? 16 : 0) + EXTRA.value));
+        __builtin_amdgcn_s_barrier();
+#pragma unroll
+        for (int g = 32; g < 64; ++g) {
+            if constexpr (ISSUE_B.value) {
+                if ((g & 3) == 0) issue_b(r1, (g - 32) >> 2);
+            }
+            if constexpr (nxt) {
+                if (g == 32 + RD_LAG) read_into(fb[3], b_rd, r2, 3);
+                if (g == 40 + RD_LAG) read_into(fb[4], b_rd, r2, 4);
+                if (g == 48 + RD_LAG) read_into(fb[5], b_rd, r2, 5);
+                if (g == 56 + RD_LAG) read_into(fb[6], b_rd, r2, 6);
+                // A blocks at regions 33, 36, 39, 42, 45, 47, 50, 53: between the B reads, all before the last of them
+                constexpr int a_at[8] = {33, 36, 39, 42, 45, 47, 50, 53};
+#pragma unroll
+                for (int i = 0; i < 8; ++i)
+                    if (g == a_at[i]) {
+                        if constexpr (par) read_into(fa0[i], a_rd, r3, i);
+                        else read_into(fa1[i], a_rd, r3, i);
+                    }
+            }
+            mfma(g);
+            if constexpr (ISSUE_B.value) {
+                if (g == 62) advance_b();
+            }
+            if (g == 63) {
+                const uint32_t o0 = r0, o1 = r1;
+                r0 = r2;
+                r1 = r3;
+                r2 = r4;
+                r3 = o0;
+                r4 = o1;
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+
+    // ---- prologue: A(0) and B(0) first, then B(1), A(1), B(2) in ring order; fragments of pair 0 into registers.
+    //      (The launcher sends K < 512 to the 32x32x64 kernel: here Q >= 4, every pair of the prologue exists and
+    //      pair 0 can be peeled.)
+#pragma unroll
+    for (int g = 0; g < 8; ++g) issue_a(r1, g);
+    advance_a();
+#pragma unroll
+    for (int g = 0; g < 8; ++g) issue_b(r0, g);
+    advance_b();
+#pragma unroll
+    for (int g = 0; g < 8; ++g) issue_b(r2, g);
+    advance_b();
+#pragma unroll
+    for (int g = 0; g < 8; ++g) issue_a(r3, g);
+    advance_a();
+#pragma unroll
+    for (int g = 0; g < 8; ++g) issue_b(r4, g);
+    advance_b();
+    __builtin_amdgcn_s_waitcnt(vmcnt_imm(24));
+    __builtin_amdgcn_s_barrier();
+#pragma unroll
+    for (int j = 0; j < NB - 1; ++j) read_into(fb[j], b_rd, r0, j);
+#pragma unroll
+    for (int i = 0; i < NB; ++i) read_into(fa0[i], a_rd, r1, i);
+    read_into(fb7_0, b_rd, r0, 7);
+
+    // Pair q consumes register set q % 2 and fills the other one.  Pair 0, then the steady pairs 1 .. Q-4 two at a time
+    // (odd, even), then one more if their number is odd.  The three pairs of the tail are code paths of their own with
+    // fixed sets (even, odd, even): when the steady pairs end on an even one, the fragments it has read for the next
+    // pair are moved over to the even set (72 register moves, once per tile).
+    pair(No{}, Yes{}, Yes{}, Yes{}, Int<0>{}, Yes{});
+    int q = 1;
+    for (; q + 4 < Q; q += 2) {
+        pair(Yes{}, Yes{}, Yes{}, Yes{}, Int<0>{}, No{});
+        pair(No{}, Yes{}, Yes{}, Yes{}, Int<0>{}, No{});
+    }
+    if (q + 3 < Q) {
+        pair(Yes{}, Yes{}, Yes{}, Yes{}, Int<0>{}, No{});
+    } else {
+#pragma unroll
+        for (int i = 0; i < NB; ++i) fa0[i] = fa1[i];
+        fb7_0 = fb7_1;
+    }
+    pair(No{}, Yes{}, No{}, Yes{}, Int<0>{}, No{});  // pair Q-3 (even): the last A loads
+
+    // the epilogue's scales and bias, requested behind the last tile loads (always three loads; a missing bias reads
+    // a scale instead and is replaced by -0.0: x + (-0.0) == x bit for bit)
+    const float pre_sx = p.sx[m0 + t], pre_sw = p.sw[n0 + t];
+    const uint16_t pre_b = (p.bias ? p.bias : reinterpret_cast<const uint16_t*>(p.sw))[n0 + t];
+    __builtin_amdgcn_sched_barrier(0);
+
+    pair(Yes{}, No{}, No{}, Yes{}, Int<3>{}, No{});  // pair Q-2 (odd)
+    pair(No{}, No{}, No{}, No{}, Int<3>{}, No{});                // pair Q-1 (even)
+
+    // The MFMAs are inline asm, so the compiler cannot count the wait states between one of them and a VALU read of
+    // its result: idle cycles first, then every accumulator is passed through an empty statement, which no read of
+    // it can move above.
+    asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 7");
+#pragma unroll
+    for (int j = 0; j < NB; j += 2) {
+        asm volatile(""
+                     : "+a"(acc[j][0]), "+a"(acc[j][1]), "+a"(acc[j][2]), "+a"(acc[j][3]), "+a"(acc[j][4]), "+a"(acc[j][5]),
+                       "+a"(acc[j][6]), "+a"(acc[j][7]), "+a"(acc[j + 1][0]), "+a"(acc[j + 1][1]), "+a"(acc[j + 1][2]),
+                       "+a"(acc[j + 1][3]), "+a"(acc[j + 1][4]), "+a"(acc[j + 1][5]), "+a"(acc[j + 1][6]), "+a"(acc[j + 1][7]));
+    }
+    tile256_epilogue16<DUMP, NB, true>(p, acc, smem, m0, n0, t, wm, wn, lr, kg, pre_sx, pre_sw,
+                                       p.bias ? bf16_bits_to_f32(pre_b) : -0.0f);
+}
+
+template <bool DUMP, int F8>
+static int prepare_tile256f16() {
+    static std::atomic<uint64_t> lds_set{0};  // per instantiation
+    return ensure_dynamic_lds(reinterpret_cast<const void*>(gemm_tile256f16_kernel<DUMP, F8>), f16::SMEM, lds_set);
+}
+
+template <bool DUMP, int F8>
+static int launch_tile256f16_impl(const GemmArgs& a, hipStream_t st) {
+    auto kern = gemm_tile256f16_kernel<DUMP, F8>;
+    if (int rc = prepare_tile256f16<DUMP, F8>()) return rc;
+    const int64_t nt = a.order == 1 ? patched_grid(a.tiles_m, a.tiles_n) : (int64_t)a.tiles_m * a.tiles_n;
+    if (nt > 0x7fffffff) return fail(DAXQ_ERR_ARG, "gemm: too many tiles");
+    hipLaunchKernelGGL(kern, dim3((unsigned)nt), dim3(f16::T), f16::SMEM, st, a);
+    return check_launch("gemm_tile256f16");
+}
+
+template <int F8>
+static int launch_tile256f16(const GemmArgs& a, hipStream_t st) {
+    return a.acc ? launch_tile256f16_impl<true, F8>(a, st) : launch_tile256f16_impl<false, F8>(a, st);
+}
+
 template <bool FP8, bool DUMP, int F8, bool N16 = false, int BT = 256, bool SPLITK = false>
 static int prepare_tile256s5() {
     static std::atomic<uint64_t> lds_set{0};  // per instantiation
@@ -1011,11 +1323,12 @@ static int launch_tile256s5_impl(const GemmArgs& a, hipStream_t st) {
     return check_launch("gemm_tile256s5");
 }
 
-// wide:  INT8 with 32x32x32 MFMAs instead of the 16x16x64 form (256 tile only; kept for the tests and for comparisons)
+// wide:  32x32 MFMAs (INT8 32x32x32, FP8 32x32x64) instead of the 16x16 forms (256 tile only; kept for the tests and for comparisons)
 // small: 128x128 tiles (needs m, n >= 128)
 // f8:    FP8 operand formats (kF8XE5 | kF8WE5)
 template <bool FP8, int F8>
-static int launch_tile256s5_f8(const GemmArgs& a, bool small, hipStream_t st) {
+static int launch_tile256s5_f8(const GemmArgs& a, bool wide, bool small, hipStream_t st) {
+    if (!small && !wide && a.k >= 512) return launch_tile256f16<F8>(a, st);  // 16x16x128 MFMAs (at least four pairs of slices); wide: the 32x32x64 form
     if (small) return a.acc ? launch_tile256s5_impl<true, true, F8, false, 128>(a, st) : launch_tile256s5_impl<true, false, F8, false, 128>(a, st);
     return a.acc ? launch_tile256s5_impl<true, true, F8>(a, st) : launch_tile256s5_impl<true, false, F8>(a, st);
 }
@@ -1028,10 +1341,10 @@ int launch_tile256s5(const GemmArgs& a0, int f8, bool wide, bool small, hipStrea
     a.tiles_n = (a.n + bt - 1) / bt;
     if constexpr (FP8) {
         switch (f8) {
-            case 1: return launch_tile256s5_f8<true, 1>(a, small, st);
-            case 2: return launch_tile256s5_f8<true, 2>(a, small, st);
-            case 3: return launch_tile256s5_f8<true, 3>(a, small, st);
-            default: return launch_tile256s5_f8<true, 0>(a, small, st);
+            case 1: return launch_tile256s5_f8<true, 1>(a, wide, small, st);
+            case 2: return launch_tile256s5_f8<true, 2>(a, wide, small, st);
+            case 3: return launch_tile256s5_f8<true, 3>(a, wide, small, st);
+            default: return launch_tile256s5_f8<true, 0>(a, wide, small, st);
         }
     } else {
         if (small) return a.acc ? launch_tile256s5_impl<false, true, 0, true, 128>(a, st) : launch_tile256s5_impl<false, false, 0, true, 128>(a, st);
@@ -1067,6 +1380,14 @@ int prepare_tile256_kernels() {
     DAXQ_PREP(prepare_tile256s5<true, true, F8, false, 256>);    \
     DAXQ_PREP(prepare_tile256s5<true, false, F8, false, 128>);   \
     DAXQ_PREP(prepare_tile256s5<true, true, F8, false, 128>)
+#define DAXQ_PREP_F16(F8)                      \
+    DAXQ_PREP(prepare_tile256f16<false, F8>); \
+    DAXQ_PREP(prepare_tile256f16<true, F8>)
+    DAXQ_PREP_F16(0);
+    DAXQ_PREP_F16(1);
+    DAXQ_PREP_F16(2);
+    DAXQ_PREP_F16(3);
+#undef DAXQ_PREP_F16
     DAXQ_PREP_F8(0);
     DAXQ_PREP_F8(1);
     DAXQ_PREP_F8(2);
