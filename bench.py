@@ -270,8 +270,9 @@ def main():
             "config": {"workload": f"{model_name} linear set, {kind.upper()} W8A8, M={m} tokens: {shape_txt}; {per_lin_txt}",
                        "gemm_variant": args.variant},
             "pct_of_mfma_peak": round(100.0 * res["value"] / PEAK_TOPS, 2),
-            "roofline": roofline(res, kind, f"gemm_tile256s5_kernel, average launch over the {len(shapes)} shape(s); "
-                                 "8-bit ops counted as 2*M*N*K", gemm_traffic(kind) if full else None),
+            "roofline": roofline(res, kind, ("gemm_tile256s5_kernel" if kind == "int8" else "gemm_tile256f16_kernel") +
+                                 f", average launch over the {len(shapes)} shape(s); 8-bit ops counted as 2*M*N*K",
+                                 gemm_traffic(kind) if full else None),
             "per_linear": res["per_linear"],
         }
         if not args.no_cpu_baseline:

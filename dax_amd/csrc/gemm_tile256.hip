@@ -1003,7 +1003,10 @@ constexpr int BT = 256, BKS = 64, T = 256, NPART = 5;
 constexpr int HALF = BT * BKS;   // one slice of one operand: 16 KB
 constexpr int PART = 2 * HALF;   // one operand of one pair: 32 KB
 constexpr int SMEM = NPART * PART;
-constexpr int RD_LAG = 0;  // regions between the last MFMA that reads a B fragment and the LDS read that refills it
+#ifndef DAXQ_F16_RD_LAG
+#define DAXQ_F16_RD_LAG 0
+#endif
+constexpr int RD_LAG = DAXQ_F16_RD_LAG;  // regions between the last MFMA that reads a B fragment and the LDS read that refills it
 constexpr int TRAIL_READS = 0;  // ds_read_b128 issued behind the last B read of a pair (block 6 at region 56)
 }  // namespace f16
 
@@ -1157,7 +1160,13 @@ __global__ __launch_bounds__(256) void gemm_tile256f16_kernel(const GemmArgs p) 
                 if (g == 48 + RD_LAG) read_into(fb[5], b_rd, r2, 5);
                 if (g == 56 + RD_LAG) read_into(fb[6], b_rd, r2, 6);
                 // A blocks at regions 33, 36, 39, 42, 45, 47, 50, 53: between the B reads, all before the last of them
+#if defined(DAXQ_F16_SCHED) && DAXQ_F16_SCHED == 1
+                constexpr int a_at[8] = {33, 34, 35, 37, 38, 39, 41, 42};
+#elif defined(DAXQ_F16_SCHED) && DAXQ_F16_SCHED == 2
+                constexpr int a_at[8] = {34, 37, 41, 44, 47, 50, 53, 55};
+#else
                 constexpr int a_at[8] = {33, 36, 39, 42, 45, 47, 50, 53};
+#endif
 #pragma unroll
                 for (int i = 0; i < 8; ++i)
                     if (g == a_at[i]) {

@@ -252,6 +252,37 @@ def test_linear_fp8_random_shapes_accumulators(ops, variant, e5m2, m, n, k, pad_
     assert torch.equal(out_wide[:, :n].cpu(), acc_wide[:, :n].cpu().bfloat16())   # unit scales, no bias: out = bf16(acc)
 
 
+@pytest.mark.parametrize("e5m2", [False, True])
+@pytest.mark.parametrize("m,n,k", [(8192, 5120, 5120), (4096, 5120, 13824), (2304, 2560, 640)])
+def test_fp8_16x16x128_form_against_the_32x32x64_form_every_element(ops, m, n, k, e5m2):
+    """The FP8 kernel on 16x16x128 MFMAs (fragments refilled in place behind the MFMAs that read them) against the
+    32x32x64 kernel at full depth of K and with every CU busy: raw fp32 accumulators of the whole output, element by
+    element, within the rounding of an fp32 sum (a wrong or torn operand would be off by orders of magnitude);
+    three launches, identical bits each time; a row sample against the exact float64 sum."""
+    from dax_amd import _capi
+
+    g = torch.Generator("cpu").manual_seed(m + n + k)
+    act_dtype = torch.float8_e5m2 if e5m2 else torch.float8_e4m3fn
+    xf = (torch.randn(m, k, generator=g) * 3).to(act_dtype)
+    wf = (torch.randn(n, k, generator=g) * 0.5).to(torch.float8_e4m3fn)
+    xd, wd = dev(xf.view(torch.uint8)), dev(wf.view(torch.uint8))
+    one_m, one_n = torch.ones(m, device="cuda"), torch.ones(n, device="cuda")
+    fn = ops.linear_e5m2_e4m3_acc if e5m2 else ops.linear_e4m3_acc
+    _capi.debug_select_gemm(9)
+    _, acc_wide = fn(xd, one_m, wd, one_n, None)
+    _capi.debug_select_gemm(8)
+    runs = [fn(xd, one_m, wd, one_n, None)[1] for _ in range(3)]
+    assert torch.equal(runs[0], runs[1]) and torch.equal(runs[0], runs[2])
+    bound = dev(xf.float().abs()) @ dev(wf.float().abs()).t()      # sum of |products| (fp32 on the device is enough for a bound)
+    err = ((runs[0] - acc_wide).abs() / bound.clamp_min(1e-30)).max().item()
+    assert err < 4e-5, err
+    rows = torch.randint(0, m, (48,), generator=g)
+    want = xf[rows].double() @ wf.double().t()
+    b64 = xf[rows].double().abs() @ wf.double().abs().t()
+    err = ((runs[0][dev(rows)].cpu().double() - want).abs() / b64.clamp_min(1e-30)).max().item()
+    assert err < 2e-5, err
+
+
 @pytest.mark.parametrize("variant", [0, 5, 6])
 @pytest.mark.parametrize("m,n,k", [(300, 520, 256), (17, 24, 384), (512, 1536, 1536), (4096, 1536, 1536)])
 def test_linear_e5m2_activations_within_tolerance(ops, variant, m, n, k):
