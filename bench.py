@@ -405,6 +405,9 @@ def main():
             want = "int8" if head["dtype"] == "int8" else "fp8_e4m3fn"
             if want in sus and "workload" in sus[want]:
                 res["roofline"]["gemm_frac_of_workload_ceiling"] = round(head["roofline"]["achieved"] / sus[want]["workload"], 4)
+            if "fp8" in res and "fp8_e4m3fn" in sus and "workload" in sus["fp8_e4m3fn"]:
+                res["fp8"]["roofline"]["gemm_frac_of_workload_ceiling"] = round(
+                    res["fp8"]["roofline"]["achieved"] / sus["fp8_e4m3fn"]["workload"], 4)
     print(json.dumps(res), flush=True)
 
 

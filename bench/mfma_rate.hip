@@ -21,7 +21,7 @@
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v8i __attribute__((ext_vector_type(8)));
 typedef int v16i __attribute__((ext_vector_type(16)));
-typedef float v16f __attribute__((ext_vector_type(16)));
+typedef float v4f __attribute__((ext_vector_type(4)));
 
 #define CHECK(x)                                                               \
     do {                                                                       \
@@ -34,7 +34,7 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 
 // a, b: 8 operand sets per lane (256 lanes per block share the pattern across blocks).  The loop is the GEMM's
 // own MFMA sequence for one 64-byte K slice of a wavefront's 128 x 128 outputs, with every memory instruction
-// removed: INT8 8 x 8 blocks of v_mfma_i32_16x16x64_i8, FP8 4 x 4 blocks of v_mfma_f32_32x32x64_f8f6f4, 256
+// removed: INT8 8 x 8 blocks of v_mfma_i32_16x16x64_i8, FP8 8 x 8 blocks of v_mfma_f32_16x16x128_f8f6f4 (a pair of slices), 256
 // accumulator registers, one operand held over a row of blocks, one wavefront per SIMD.
 template <bool FP8>
 __global__ __launch_bounds__(256) void spin(const int* __restrict__ a_src, const int* __restrict__ b_src, int iters, int* out) {
@@ -68,28 +68,26 @@ __global__ __launch_bounds__(256) void spin(const int* __restrict__ a_src, const
             for (int i = 0; i < 8; ++i) r += c[j][i][0];
         out[blockIdx.x * 256 + threadIdx.x] = r;
     } else {
-        v16f c[4][4];
-        for (int j = 0; j < 4; ++j)
-            for (int i = 0; i < 4; ++i)
-                for (int v = 0; v < 16; ++v) c[j][i][v] = 0;
+        v4f c[8][8];
+        for (int j = 0; j < 8; ++j)
+            for (int i = 0; i < 8; ++i)
+                for (int v = 0; v < 4; ++v) c[j][i][v] = 0;
         v8i av[8], bv[8];
 #pragma unroll
         for (int s = 0; s < 8; ++s) {
             av[s] = v8i{a[s][0], a[s][1], a[s][2], a[s][3], a[s][4], a[s][5], a[s][6], a[s][7]};
             bv[s] = v8i{b[s][0], b[s][1], b[s][2], b[s][3], b[s][4], b[s][5], b[s][6], b[s][7]};
         }
-        for (int it = 0; it < iters; it += 2) {
+        for (int it = 0; it < iters; it += 2) {  // a pair of slices per trip: K = 128 per MFMA
 #pragma unroll
-            for (int h = 0; h < 2; ++h)  // two slices: operand sets 0-3 and 4-7
+            for (int j = 0; j < 8; ++j)
 #pragma unroll
-                for (int j = 0; j < 4; ++j)
-#pragma unroll
-                    for (int i = 0; i < 4; ++i)
-                        c[j][i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bv[4 * h + j], av[4 * h + i], c[j][i], 0, 0, 0, 0, 0, 0);
+                for (int i = 0; i < 8; ++i)
+                    asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0" : "+a"(c[j][i]) : "v"(bv[j]), "v"(av[i]));
         }
         float r = 0;
-        for (int j = 0; j < 4; ++j)
-            for (int i = 0; i < 4; ++i) r += c[j][i][0];
+        for (int j = 0; j < 8; ++j)
+            for (int i = 0; i < 8; ++i) r += c[j][i][0];
         out[blockIdx.x * 256 + threadIdx.x] = (int)r;
     }
 }

@@ -211,7 +211,7 @@ def test_linear_e4m3_within_tolerance(ops, variant, m, n, k):
     assert r < 3e-3, r                          # what fp32 accumulation actually delivers
 
 
-@pytest.mark.parametrize("variant", [8, 6, 11])
+@pytest.mark.parametrize("variant", [8, 9, 6, 11])
 @pytest.mark.parametrize("e5m2", [False, True])
 @pytest.mark.parametrize("m,n,k,pad_k,pad_n", _random_shapes(8, seed=77))
 def test_linear_fp8_random_shapes_accumulators(ops, variant, e5m2, m, n, k, pad_k, pad_n):
@@ -250,6 +250,29 @@ def test_linear_fp8_random_shapes_accumulators(ops, variant, e5m2, m, n, k, pad_
     assert err < 2e-5, err        # fp32 accumulation of K products: a few 2^-24 of the sum of magnitudes
     assert bool((acc_wide[:, n:] == -1.0).all())
     assert torch.equal(out_wide[:, :n].cpu(), acc_wide[:, :n].cpu().bfloat16())   # unit scales, no bias: out = bf16(acc)
+
+
+@pytest.mark.parametrize("k", [384, 512, 640, 768, 896, 1024, 1152, 1280, 1408, 1536])
+def test_fp8_16x16x128_form_every_count_of_slice_pairs(ops, k):
+    """Every number of 128-byte pairs of K slices from 3 (below four pairs the launch takes the 32x32x64 kernel) to
+    12: first pair, steady pairs in twos, the odd one and the register moves in front of the three tail pairs all
+    occur.  Accumulators against exact float64 sums, element by element, on a 2 x 3 grid of tiles with ragged edges."""
+    from dax_amd import _capi
+
+    m, n = 300, 700
+    g = torch.Generator("cpu").manual_seed(k)
+    xf = (torch.randn(m, k, generator=g) * 3).to(torch.float8_e4m3fn)
+    wf = (torch.randn(n, k, generator=g) * 0.5).to(torch.float8_e4m3fn)
+    want = xf.double() @ wf.double().t()
+    bound = xf.double().abs() @ wf.double().abs().t()
+    _capi.debug_select_gemm(8)
+    sx, sw = torch.rand(m, generator=g) + 0.5, torch.rand(n, generator=g) + 0.5
+    b = torch.randn(n, generator=g).bfloat16()
+    out, acc = ops.linear_e4m3_acc(dev(xf.view(torch.uint8)), dev(sx), dev(wf.view(torch.uint8)), dev(sw), dev(b))
+    err = ((acc.cpu().double() - want).abs() / bound.clamp_min(1e-30)).max().item()
+    assert err < 2e-5, err
+    ref = (acc.cpu() * sx.view(-1, 1) * sw.view(1, -1) + b.float()).bfloat16()     # the epilogue on the kernel's own sums
+    np.testing.assert_array_equal(bf16_bits(out), bf16_bits(ref))
 
 
 @pytest.mark.parametrize("e5m2", [False, True])
