@@ -1,14 +1,15 @@
 // 256x256-tile W8A8 GEMMs for gfx950: the kernels the large DiT shapes run on.
 //
-// Two forms of the same tile live here.  gemm_tile256s5_kernel (second half of the file, K in
-// 64-byte slices through five 32 KB LDS stages) is the one the library launches;
-// gemm_tile256_kernel (K in 128-byte slices, two 64 KB stages) came first and stays as a second
-// implementation for the tests.  They share everything but the main loop.
+// Three kernels on the same tile live here.  The library launches gemm_tile256s5_kernel for INT8 (K in 64-byte slices
+// through five 32 KB LDS stages, v_mfma_i32_16x16x64_i8) and gemm_tile256f16_kernel for FP8 (K in pairs of such slices,
+// v_mfma_f32_16x16x128_f8f6f4, B fragments refilled in place; at the end of the file).  gemm_tile256s5_kernel with
+// 32x32 MFMAs (INT8 32x32x32, FP8 32x32x64) and gemm_tile256_kernel (K in 128-byte slices, two 64 KB stages; it came
+// first) stay as further implementations for the tests and for K < 512 in FP8.
 //
 // Work decomposition
 //   workgroup  256 x 256 outputs, 4 wavefronts (one per SIMD) in a 2 x 2 grid
 //   wavefront  128 x 128 outputs in 256 accumulator registers (AGPRs): 4 x 4 MFMA blocks of 32x32
-//              (FP8, and INT8 in the older forms) or 8 x 8 blocks of 16x16 (INT8 in the five-stage kernel)
+//              (the older forms) or 8 x 8 blocks of 16x16 (the kernels the library launches)
 // A 2 x 2 wave grid is what minimises LDS reads per MFMA for a square tile: 128 bytes of K are
 // read (2 + 2) * 256 * 128 B = 128 KB per workgroup against 4096 MFMA cycles per wave.
 //

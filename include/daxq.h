@@ -259,10 +259,13 @@ int daxq_linear_e5m2_e4m3(const uint8_t* xq, int64_t ld_xq, const float* sx,
  *   fp8:  out = T( acc * sx[i] * sw[j] + f32(bias[j]) )                        (torch._scaled_mm, :155-173)
  * acc: optional int32 (int8) / fp32 (fp8) dump of the raw accumulators.
  * kernel: 0 = the library's choice by shape.  Other values pick one implementation, for tests and comparisons
- * (every choice computes the same results): 2 / 5 = generic kernel on 256x256 / 128x128 tiles, 6 = two-stage 256x256
- * kernel, 8 = five-stage 256x256 kernel, 9 = the same with 32x32x32 INT8 MFMAs, 11 = the same on 128x128 tiles;
- * bits 16-23, when not zero, set the depth of the tile-order groups.  fp16 / fp32 outputs exist in the generic
- * kernel only.  The choice is an argument of the call: the library keeps no process-wide selection.
+ * (int8 results are the same bits for every choice, fp8 results differ by fp32 summation order): low 16 bits 2 / 5 =
+ * generic kernel on 256x256 / 128x128 tiles, 6 = two-stage 256x256 kernel, 8 = the 256x256 kernel on 16x16 MFMAs
+ * (int8 16x16x64; fp8 16x16x128 from k = 512 on), 9 = the 256x256 kernel on 32x32 MFMAs, 11 = the five-stage kernel on
+ * 128x128 tiles; bits 16-23, when not zero, set the depth of the tile-order groups; bits 24-25 the tile order of the
+ * 256x256 kernels (0 = by shape, 1 = groups of tile rows, 2 = whole 32-tile patches per XCD).  fp16 / fp32 outputs
+ * exist in the generic kernel only.  The choice is an argument of the call: the library keeps no process-wide
+ * selection.
  */
 int daxq_linear_w8a8(int x_fmt, int w_fmt, int out_dtype,
                      const void* xq, int64_t ld_xq, const float* sx,
