@@ -1,0 +1,48 @@
+// Host-side check of the patch-aligned tile order (dax_amd/csrc/tile_order.h): for every tile grid up to 320 x 72 the
+// launch of patched_grid() workgroups computes every tile exactly once, padding slots map to no tile, and the 32 slots
+// that one XCD runs side by side lie in one patch of at most 4 x 8 (or (32 / w) x w) tiles.  Built by
+// __graft_entry__.build() with the host compiler; run by tests/test_abi_and_host.py.
+#include <cstdio>
+#include <cstdlib>
+#include <vector>
+
+#include "../../dax_amd/csrc/tile_order.h"
+
+int main() {
+    long bad = 0, grids = 0;
+    for (int tiles_m = 1; tiles_m <= 320; tiles_m += (tiles_m < 48 ? 1 : 17))
+        for (int tiles_n = 1; tiles_n <= 72; ++tiles_n) {
+            ++grids;
+            std::vector<int> seen((size_t)tiles_m * tiles_n, 0);
+            const int64_t grid = daxq::patched_grid(tiles_m, tiles_n);
+            if (grid % 256 != 0 || grid < (int64_t)tiles_m * tiles_n) ++bad;
+            for (int64_t base = 0; base < grid; base += 256)
+                for (int xcd = 0; xcd < 8; ++xcd) {
+                    int lo_m = 1 << 30, hi_m = -1, lo_n = 1 << 30, hi_n = -1;
+                    for (int slot = 0; slot < 32; ++slot) {
+                        const int pid = (int)base + slot * 8 + xcd;  // the 32 consecutive local ids of this XCD
+                        int tm = -1, tn = -1;
+                        if (!daxq::tile_of_block_patched(pid, tiles_m, tiles_n, tm, tn)) continue;
+                        if (tm < 0 || tm >= tiles_m || tn < 0 || tn >= tiles_n) {
+                            ++bad;
+                            continue;
+                        }
+                        ++seen[(size_t)tm * tiles_n + tn];
+                        lo_m = tm < lo_m ? tm : lo_m;
+                        hi_m = tm > hi_m ? tm : hi_m;
+                        lo_n = tn < lo_n ? tn : lo_n;
+                        hi_n = tn > hi_n ? tn : hi_n;
+                    }
+                    if (hi_m >= 0) {
+                        const int rows = hi_m - lo_m + 1, cols = hi_n - lo_n + 1;
+                        if (cols > 8 || rows * cols > 32) ++bad;  // panels shared inside an XCD: rows + cols of one patch
+                    }
+                }
+            for (int v : seen) bad += v != 1;
+        }
+    // the four benchmark launches: grid sizes and padding
+    const long want[3][3] = {{296, 20, 6144}, {296, 60, 17920}, {296, 54, 16128}};
+    for (auto& w : want) bad += daxq::patched_grid((int)w[0], (int)w[1]) != w[2];
+    std::printf("%ld tile grids checked, %ld errors\n", grids, bad);
+    return bad ? 1 : 0;
+}

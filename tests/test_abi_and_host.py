@@ -31,6 +31,20 @@ def test_library_exports_every_declared_symbol():
     assert "undefined symbol" not in _capi.last_error()
 
 
+def test_patch_tile_order_covers_every_tile_once():
+    """tests/host/tile_order_check (built by __graft_entry__.build() from the header the kernels include): every tile
+    grid up to 320 x 72, every tile exactly once, an XCD's 32 slots inside one patch."""
+    import subprocess
+
+    exe = os.path.join(ROOT, "tests", "host", "tile_order_check")
+    if not os.path.exists(exe):     # a tree that was never built: one second of g++
+        import __graft_entry__
+
+        __graft_entry__._build_host_checks()
+    r = subprocess.run([exe], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0 and " 0 errors" in r.stdout, r.stdout + r.stderr
+
+
 def test_no_cpu_kernels_and_clear_errors():
     import dax_amd.ops as ops
 

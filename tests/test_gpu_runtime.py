@@ -146,6 +146,52 @@ def test_captured_graph_replays_match_eager(fp8):
         assert _same(static_out, eager), f"replay with seed {seed} differs from eager"
 
 
+@pytest.mark.parametrize("fp8", [False, True])
+def test_captured_graph_of_the_256_tile_kernels_replays_match_eager(fp8):
+    """The kernels the large shapes run on (INT8 16x16x64, FP8 16x16x128; chosen by argument here because the shape
+    is small) and the patch tile order with its padding workgroups, captured and replayed with new operand contents."""
+    import dax_amd.ops as ops
+    from dax_amd import _capi
+
+    m, n, k = 700, 2304, 1024
+    g = torch.Generator().manual_seed(3)
+    sx, sw = (torch.rand(m, generator=g) + 0.5).cuda(), (torch.rand(n, generator=g) * 0.01).cuda()
+    b = torch.randn(n, generator=g).bfloat16().cuda()
+
+    def operands(seed):
+        gg = torch.Generator().manual_seed(seed)
+        x = torch.randint(-100, 101, (m, k), dtype=torch.int8, generator=gg)
+        w = torch.randint(-100, 101, (n, k), dtype=torch.int8, generator=gg)
+        if fp8:   # any byte but the two NaN codes is a finite e4m3fn value
+            x, w = x.view(torch.uint8), w.view(torch.uint8)
+            x = torch.where((x & 0x7f) == 0x7f, torch.zeros((), dtype=torch.uint8), x)
+            w = torch.where((w & 0x7f) == 0x7f, torch.zeros((), dtype=torch.uint8), w)
+        return x.cuda(), w.cuda()
+
+    fn = ops.linear_e4m3 if fp8 else ops.linear_i8
+    try:
+        _capi.debug_select_gemm(8)
+        _capi.debug_select_gemm(2002)
+        static_x, static_w = operands(0)
+        fn(static_x, sx, static_w, sw, b)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            static_out = fn(static_x, sx, static_w, sw, b)
+        for seed in (1, 2, 3):
+            x, w = operands(seed)
+            eager = fn(x, sx, w, sw, b)
+            torch.cuda.synchronize()
+            static_x.copy_(x)
+            static_w.copy_(w)
+            graph.replay()
+            torch.cuda.synchronize()
+            assert _same(static_out, eager), f"replay with seed {seed} differs from eager"
+    finally:
+        _capi.debug_select_gemm(0)
+        _capi.debug_select_gemm(2000)
+
+
 _FIRST_LAUNCH_IN_CAPTURE = r"""
 import sys
 import torch
