@@ -40,8 +40,13 @@ def _same_scale(got, want):
     np.testing.assert_array_equal(got.cpu()[ok].numpy(), want[ok].numpy())   # inf and finite values bit for bit
 
 
+@pytest.mark.parametrize("variant", [0, 8])   # 8: the kernels of the large shapes (16x16 MFMA forms)
 @pytest.mark.parametrize("fmt", ["i8", "e4m3", "e5m2"])
-def test_poisoned_tokens_get_the_oracles_scale_and_a_nonfinite_row(ops, fmt):
+def test_poisoned_tokens_get_the_oracles_scale_and_a_nonfinite_row(ops, fmt, variant, request):
+    from dax_amd import _capi
+
+    _capi.debug_select_gemm(variant)
+    request.addfinalizer(lambda: _capi.debug_select_gemm(0))
     m, k, n = 300, 512, 384
     x, bad = _poisoned(m, k, seed=1)
     g = torch.Generator("cpu").manual_seed(2)
