@@ -60,14 +60,14 @@ __device__ __forceinline__ float gelu_tanh_f32(float x) {
 // PRE_LN: y = bf16( ((x - mean) * rstd) * mul[g][c] + add[g][c] ), g = row / rows_per_group; the two
 //         vectors of the workgroup's current group are staged in LDS (mul / add may be null: 1 / 0).
 // PRE_GELU: y = bf16( gelu_tanh(x) ).
-// Requires k % 8 == 0, 16-byte aligned rows of x (and y), 8-byte aligned rows of q, ld_q/8 <= NCH*64.
+// Requires k % 8 == 0, 16-byte aligned rows of x (and y), 8-byte aligned rows of q, kfill/8 <= NCH*64.
 // The quantise-only LayerNorm form for rows of up to 12 x 64 chunks holds two rows (the current and the requested
 // next one) and is kept at three wavefronts per SIMD (170 registers).
 template <int NCH, int FMT, int PRE, bool WRITE_Y>
 __global__ __launch_bounds__(256, (PRE == PRE_LN && NCH <= 12 && !WRITE_Y) ? 3 : 1) void fused_rows_wave(
     const uint16_t* __restrict__ x, int64_t m, int k, int64_t ld_x, const float* __restrict__ mul,
     const float* __restrict__ add, int64_t rows_per_group, float eps, uint16_t* __restrict__ y, int64_t ld_y,
-    uint8_t* __restrict__ q, int64_t ld_q, float* __restrict__ scale, float qmax) {
+    uint8_t* __restrict__ q, int64_t ld_q, int kfill, float* __restrict__ scale, float qmax) {
     // PRE_LN: mul then add, each in the order the lanes read them: per 64 chunks of 8 elements, the first halves of
     // the 64 chunks, then the second halves, so that one 16-byte read per lane covers 1 KB without a gap (the plain
     // order makes the lanes read 16 bytes every 32 and half of the banks collide)
@@ -75,7 +75,7 @@ __global__ __launch_bounds__(256, (PRE == PRE_LN && NCH <= 12 && !WRITE_Y) ? 3 :
     const int kpad = ((k + 511) >> 9) << 9;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int nch = k >> 3;
-    const int npad = (int)(ld_q >> 3);
+    const int npad = kfill >> 3;  // columns [k, kfill) are written as zeros
     int64_t staged = -1;
     // The resident LayerNorm form requests the wavefront's next row before it works on the current one.
     constexpr bool AHEAD = PRE == PRE_LN && NCH <= 12;
@@ -236,17 +236,18 @@ static int launch_fused_rows(const char* what, const void* x, int64_t m, int64_t
     if (PRE == PRE_LN && (rows_per_group <= 0 || !(eps >= 0.0f))) return fail(DAXQ_ERR_ARG, "%s: rows_per_group and eps must be positive", what);
     if (m == 0) return DAXQ_OK;
     if (!x || !q || !scale) return fail(DAXQ_ERR_ARG, "%s: null pointer", what);
+    const int64_t kfill = fill_width(k, ld_q);
     // the row has to fit the registers of one wavefront and move in 16-byte pieces
     const bool ok = (k % 8 == 0) && (ld_x % 8 == 0) && (ld_q % 8 == 0) && (!y || ld_y % 8 == 0) && (((uintptr_t)x & 15) == 0) &&
                     (((uintptr_t)y & 15) == 0) && (((uintptr_t)q & 7) == 0) && (((uintptr_t)scale & 3) == 0) &&
-                    (((uintptr_t)mul & 3) == 0) && (((uintptr_t)add & 3) == 0) && (ld_q / 8 <= 28 * 64) &&
+                    (((uintptr_t)mul & 3) == 0) && (((uintptr_t)add & 3) == 0) && (kfill / 8 <= 28 * 64) &&
                     (PRE != PRE_LN || k <= 8192);
     if (!ok)
         return fail(DAXQ_ERR_ALIGN, "%s: needs k %% 8 == 0, k <= 14336 (8192 with LayerNorm), 16-byte aligned rows of x / y and 8-byte aligned rows of q", what);
     const uint16_t* xp = static_cast<const uint16_t*>(x);
     uint16_t* yp = static_cast<uint16_t*>(y);
     uint8_t* qp = static_cast<uint8_t*>(q);
-    const int nchunks = (int)((ld_q / 8 + 63) / 64);
+    const int nchunks = (int)((kfill / 8 + 63) / 64);
     int dev = 0, cus = 0;
     if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
         return fail(DAXQ_ERR_LAUNCH, "%s: cannot read the CU count", what);
@@ -277,10 +278,10 @@ static int launch_fused_rows(const char* what, const void* x, int64_t m, int64_t
         const dim3 grid((unsigned)(quads < want ? quads : want));                                                        \
         if (yp)                                                                                                          \
             hipLaunchKernelGGL((fused_rows_wave<N, FMT, PRE, true>), grid, block, lds, st, xp, m, (int)k, ld_x, mul, add, \
-                               rows_per_group, eps, yp, ld_y, qp, ld_q, scale, qmax);                                    \
+                               rows_per_group, eps, yp, ld_y, qp, ld_q, (int)kfill, scale, qmax);                                    \
         else                                                                                                             \
             hipLaunchKernelGGL((fused_rows_wave<N, FMT, PRE, false>), grid, block, lds, st, xp, m, (int)k, ld_x, mul, add, \
-                               rows_per_group, eps, yp, ld_y, qp, ld_q, scale, qmax);                                    \
+                               rows_per_group, eps, yp, ld_y, qp, ld_q, (int)kfill, scale, qmax);                                    \
         return check_launch(what);                                                                                       \
     }
     DAXQ_F_CASE(4)

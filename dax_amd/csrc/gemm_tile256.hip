@@ -643,6 +643,8 @@ __global__ __launch_bounds__(256) void gemm_tile256s5_kernel(const GemmArgs p) {
     }
     if (!SPLITK && p.order == 1) {
         if (!tile_of_block_patched(tile_id, p.tiles_m, p.tiles_n, tm, tn)) return;  // padding slot (before any barrier)
+    } else if (!SPLITK && p.order == 2) {
+        if (!tile_of_block_supergroups(tile_id, p.tiles_m, p.tiles_n, tm, tn)) return;
     } else {
         tile_of_block(p.gm, tile_id, p.tiles_m, p.tiles_n, tm, tn);
     }
@@ -1022,6 +1024,8 @@ __global__ __launch_bounds__(256) void gemm_tile256f16_kernel(const GemmArgs p) 
     int tm, tn;
     if (p.order == 1) {
         if (!tile_of_block_patched(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn)) return;  // padding slot (before any barrier)
+    } else if (p.order == 2) {
+        if (!tile_of_block_supergroups(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn)) return;
     } else {
         tile_of_block(p.gm, blockIdx.x, p.tiles_m, p.tiles_n, tm, tn);
     }
@@ -1270,7 +1274,7 @@ template <bool DUMP, int F8>
 static int launch_tile256f16_impl(const GemmArgs& a, hipStream_t st) {
     auto kern = gemm_tile256f16_kernel<DUMP, F8>;
     if (int rc = prepare_tile256f16<DUMP, F8>()) return rc;
-    const int64_t nt = a.order == 1 ? patched_grid(a.tiles_m, a.tiles_n) : (int64_t)a.tiles_m * a.tiles_n;
+    const int64_t nt = a.order == 1 ? patched_grid(a.tiles_m, a.tiles_n) : a.order == 2 ? supergroups_grid(a.tiles_m, a.tiles_n) : (int64_t)a.tiles_m * a.tiles_n;
     if (nt > 0x7fffffff) return fail(DAXQ_ERR_ARG, "gemm: too many tiles");
     hipLaunchKernelGGL(kern, dim3((unsigned)nt), dim3(f16::T), f16::SMEM, st, a);
     return check_launch("gemm_tile256f16");
@@ -1327,7 +1331,7 @@ static int launch_tile256s5_impl(const GemmArgs& a, hipStream_t st) {
     constexpr int SMEM = NST * 2 * BT * BKS;  // 160 KB (256 tile), 80 KB (128 tile)
     auto kern = gemm_tile256s5_kernel<FP8, DUMP, F8, N16, BT>;
     if (int rc = prepare_tile256s5<FP8, DUMP, F8, N16, BT>()) return rc;
-    const int64_t nt = a.order == 1 ? patched_grid(a.tiles_m, a.tiles_n) : (int64_t)a.tiles_m * a.tiles_n;
+    const int64_t nt = a.order == 1 ? patched_grid(a.tiles_m, a.tiles_n) : a.order == 2 ? supergroups_grid(a.tiles_m, a.tiles_n) : (int64_t)a.tiles_m * a.tiles_n;
     if (nt > 0x7fffffff) return fail(DAXQ_ERR_ARG, "gemm: too many tiles");
     hipLaunchKernelGGL(kern, dim3((unsigned)nt), dim3(T), SMEM, st, a);
     return check_launch("gemm_tile256s5");

@@ -328,7 +328,7 @@ static int launch_gemm(const void* xq, int64_t ld_xq, const float* sx, const voi
     // 1.00x that floor on the four 14B shapes against 1.15-1.36x for the row groups), but only the long-K launch gets
     // faster by it (K = 13824: +2 %; K = 5120: -0.5 to -7 %, 32 CUs in lockstep on the same 12 panels), so long K takes it.
     const int order_bits = (kernel >> 24) & 3;
-    a.order = order_bits == 2 || (order_bits == 0 && k >= 8192 && m >= 8192) ? 1 : 0;
+    a.order = order_bits == 3 ? 2 : order_bits == 2 || (order_bits == 0 && k >= 8192 && m >= 8192) ? 1 : 0;
     a.out_kind = out_kind;
     a.splits = 1;
     a.counters = nullptr;

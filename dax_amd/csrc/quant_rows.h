@@ -38,6 +38,14 @@ __device__ __forceinline__ float round_to_x(float s) {
     }
 }
 
+// Columns [k, fill_width) of a quantised row are written as zeros: up to the next multiple of the GEMM's K granularity,
+// as far as the row reaches.  A row stride beyond that (rows kept apart on purpose, or a column slice of a wider
+// buffer) is left alone.
+inline int64_t fill_width(int64_t k, int64_t ld_q) {
+    const int64_t kp = (k + DAXQ_K_ALIGN - 1) / DAXQ_K_ALIGN * DAXQ_K_ALIGN;
+    return kp < ld_q ? kp : ld_q;
+}
+
 // abs-max bits (sign cleared) of a block -> fp32 scale, exactly as the reference rounds it: the quotient is
 // computed and floored in the tensor's own dtype when ROUND (dynamic activations,
 // dax/quant/nn/dynamic/functional.py:124-129), in fp32 otherwise (weight observer).

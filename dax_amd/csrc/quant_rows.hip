@@ -20,19 +20,19 @@ namespace daxq {
 
 // Fast path: one wavefront per row, the row lives in registers.
 // Requires k % 8 == 0, ld_x % 8 == 0, ld_q % 8 == 0, 16-byte aligned x, 8-byte aligned q,
-// and ld_q / 8 <= NCH * 64.
+// and kfill / 8 <= NCH * 64.
 // SCALE_IN: the per-row scale is an input (leaf quantiser) instead of being derived from the row.
 // XT: element type of x, DAXQ_BF16 or DAXQ_F16 (8 elements per 16-byte chunk either way).
 template <int NCH, int FMT, bool ROUND_BF16, bool SCALE_IN, int XT = DAXQ_BF16>
 __global__ __launch_bounds__(256) void quant_rows_wave(const uint16_t* __restrict__ x, int64_t m, int k,
-                                                       int64_t ld_x, uint8_t* __restrict__ q, int64_t ld_q,
+                                                       int64_t ld_x, uint8_t* __restrict__ q, int64_t ld_q, int kfill,
                                                        float* __restrict__ scale, float qmax) {
     const int lane = threadIdx.x & 63;
     const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (row >= m) return;
     const uint4* xr = reinterpret_cast<const uint4*>(x + row * ld_x);
     const int nch = k >> 3;
-    const int npad = (int)(ld_q >> 3);
+    const int npad = kfill >> 3;  // columns [k, kfill) are written as zeros
 
     uint4 v[NCH];
     uint32_t mx = 0;
@@ -88,7 +88,7 @@ struct XWord<DAXQ_F32> {
 
 template <int FMT, bool ROUND_BF16, bool SCALE_IN, int XT = DAXQ_BF16>
 __global__ __launch_bounds__(256) void quant_rows_block(const void* __restrict__ xv, int64_t m, int64_t k,
-                                                        int64_t ld_x, uint8_t* __restrict__ q, int64_t ld_q,
+                                                        int64_t ld_x, uint8_t* __restrict__ q, int64_t ld_q, int64_t kfill,
                                                         float* __restrict__ scale, float qmax) {
     typedef typename XWord<XT>::type word_t;
     constexpr uint32_t kAbs = XT == DAXQ_F32 ? 0x7fffffffu : 0x7fffu;
@@ -116,7 +116,7 @@ __global__ __launch_bounds__(256) void quant_rows_block(const void* __restrict__
     }
     const float inv = 1.0f / s;
     uint8_t* qr = q + row * ld_q;
-    for (int64_t c = threadIdx.x; c < ld_q; c += 256) {
+    for (int64_t c = threadIdx.x; c < kfill; c += 256) {
         uint8_t o = 0;
         if (c < k) {
             float f = x_bits_to_f32<XT>(xr[c]);
@@ -139,19 +139,20 @@ static int launch_quant_rows_t(const void* x, int64_t m, int64_t k, int64_t ld_x
                                                                (long long)m, (long long)k, (long long)ld_x, (long long)ld_q);
     if (m == 0) return DAXQ_OK;
     if (!x || !q || !scale) return fail(DAXQ_ERR_ARG, "quant_rows: null pointer");
+    const int64_t kfill = fill_width(k, ld_q);
     if (((uintptr_t)x & (XB - 1)) != 0 || ((uintptr_t)scale & 3) != 0) return fail(DAXQ_ERR_ALIGN, "quant_rows: x must be element aligned and scale 4-byte aligned");
     uint8_t* qp = static_cast<uint8_t*>(q);
     if constexpr (XT != DAXQ_F32) {
         const uint16_t* xp = static_cast<const uint16_t*>(x);
         const bool vec_ok = (k % 8 == 0) && (ld_x % 8 == 0) && (ld_q % 8 == 0) && (((uintptr_t)x & 15) == 0) &&
-                            (((uintptr_t)q & 7) == 0) && (ld_q / 8 <= 36 * 64) && (m <= (int64_t)4 * 0x7fffffff);
+                            (((uintptr_t)q & 7) == 0) && (kfill / 8 <= 36 * 64) && (m <= (int64_t)4 * 0x7fffffff);
         if (vec_ok) {
-            const int nchunks = (int)((ld_q / 8 + 63) / 64);
+            const int nchunks = (int)((kfill / 8 + 63) / 64);
             const dim3 grid((unsigned)((m + 3) / 4)), block(256);
 #define DAXQ_Q_CASE(N)                                                                                      \
     if (nchunks <= N) {                                                                                     \
         hipLaunchKernelGGL((quant_rows_wave<N, FMT, ROUND_BF16, SCALE_IN, XT>), grid, block, 0, st, xp, m, (int)k, ld_x, qp, \
-                           ld_q, scale, qmax);                                                              \
+                           ld_q, (int)kfill, scale, qmax);                                                            \
         return check_launch("quant_rows_wave");                                                             \
     }
             DAXQ_Q_CASE(2)
@@ -166,7 +167,7 @@ static int launch_quant_rows_t(const void* x, int64_t m, int64_t k, int64_t ld_x
     }
     if (m > 0x7fffffff) return fail(DAXQ_ERR_ARG, "quant_rows: too many rows for the general kernel");
     hipLaunchKernelGGL((quant_rows_block<FMT, ROUND_BF16, SCALE_IN, XT>), dim3((unsigned)m), dim3(256), 0, st, x, m, k, ld_x, qp,
-                       ld_q, scale, qmax);
+                       ld_q, kfill, scale, qmax);
     return check_launch("quant_rows_block");
 }
 

@@ -34,8 +34,10 @@ extern "C" {
 #define DAXQ_ERR_LAUNCH (-4) /* the HIP runtime refused the launch */
 
 /* K granularity of the GEMM entry points: operands whose logical K is not a
- * multiple of this are zero-padded by the producer (the quantisers below pad
- * columns [k, ld_q) with zeros). */
+ * multiple of this are zero-padded by the producer: the quantisers below write
+ * zeros into columns [k, roundup(k, DAXQ_K_ALIGN)) as far as the row reaches
+ * (ld_q may be smaller); a row stride ld_q beyond that keeps rows apart, or makes
+ * q a column slice of a wider buffer, and those bytes are not touched. */
 #define DAXQ_K_ALIGN 128
 
 /* quantised formats (one byte per element) */
@@ -70,7 +72,7 @@ int daxq_init(void);
  *   dax/quant/nn/dynamic/functional.py:181-206, :54-148
  *   dax/quant/nn/quantized/functional.py:17-20
  * x      bf16 [m, k], leading dimension ld_x
- * q      int8 [m, ld_q]; columns [k, ld_q) are written as zeros
+ * q      int8 [m, ld_q]; columns [k, min(ld_q, roundup(k, DAXQ_K_ALIGN))) are written as zeros
  * scale  fp32 [m]   = f32( max( bf16_rne( f32(rowamax) / 127 ), 2^-23 ) )
  * q[r,c] = clamp( rint( f32(x[r,c]) * (1.0f / scale[r]) ), -128, 127 )
  */
@@ -138,7 +140,7 @@ int daxq_gelu_tanh_act_quant_e5m2(const void* x, int64_t m, int64_t k, int64_t l
  * Leaf quantisers with a caller-supplied per-row scale (used once per weight at conversion).
  * Replace quantize_to_int8 / quantize_to_fp8 with a [rows,1] scale
  *   dax/quant/nn/quantized/functional.py:11-20, called from dax/quant/nn/dynamic/linear.py:292-296
- * x bf16 [m, k]; scale fp32 [m]; q [m, ld_q] with columns [k, ld_q) zero.
+ * x bf16 [m, k]; scale fp32 [m]; q [m, ld_q] with columns [k, min(ld_q, roundup(k, DAXQ_K_ALIGN))) zero.
  */
 int daxq_quantize_rows_i8(const void* x, int64_t m, int64_t k, int64_t ld_x, const float* scale,
                           int8_t* q, int64_t ld_q, daxq_stream_t stream);

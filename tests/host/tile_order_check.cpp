@@ -8,13 +8,14 @@
 
 #include "../../dax_amd/csrc/tile_order.h"
 
-int main() {
-    long bad = 0, grids = 0;
+template <class Map, class Grid>
+static long check_order(Map map, Grid grid_of, long& grids) {
+    long bad = 0;
     for (int tiles_m = 1; tiles_m <= 320; tiles_m += (tiles_m < 48 ? 1 : 17))
         for (int tiles_n = 1; tiles_n <= 72; ++tiles_n) {
             ++grids;
             std::vector<int> seen((size_t)tiles_m * tiles_n, 0);
-            const int64_t grid = daxq::patched_grid(tiles_m, tiles_n);
+            const int64_t grid = grid_of(tiles_m, tiles_n);
             if (grid % 256 != 0 || grid < (int64_t)tiles_m * tiles_n) ++bad;
             for (int64_t base = 0; base < grid; base += 256)
                 for (int xcd = 0; xcd < 8; ++xcd) {
@@ -22,7 +23,7 @@ int main() {
                     for (int slot = 0; slot < 32; ++slot) {
                         const int pid = (int)base + slot * 8 + xcd;  // the 32 consecutive local ids of this XCD
                         int tm = -1, tn = -1;
-                        if (!daxq::tile_of_block_patched(pid, tiles_m, tiles_n, tm, tn)) continue;
+                        if (!map(pid, tiles_m, tiles_n, tm, tn)) continue;
                         if (tm < 0 || tm >= tiles_m || tn < 0 || tn >= tiles_n) {
                             ++bad;
                             continue;
@@ -40,9 +41,20 @@ int main() {
                 }
             for (int v : seen) bad += v != 1;
         }
+    return bad;
+}
+
+int main() {
+    long grids = 0;
+    long bad = check_order([](int pid, int a, int b, int& tm, int& tn) { return daxq::tile_of_block_patched(pid, a, b, tm, tn); },
+                           [](int a, int b) { return daxq::patched_grid(a, b); }, grids);
+    bad += check_order([](int pid, int a, int b, int& tm, int& tn) { return daxq::tile_of_block_supergroups(pid, a, b, tm, tn); },
+                       [](int a, int b) { return daxq::supergroups_grid(a, b); }, grids);
     // the four benchmark launches: grid sizes and padding
     const long want[3][3] = {{296, 20, 6144}, {296, 60, 17920}, {296, 54, 16128}};
     for (auto& w : want) bad += daxq::patched_grid((int)w[0], (int)w[1]) != w[2];
+    const long want_sg[3] = {6144, 17920, 16384};  // 296 x 54: super-groups of 20 rows, the last one holds 6 empty patches
+    for (int i = 0; i < 3; ++i) bad += daxq::supergroups_grid((int)want[i][0], (int)want[i][1]) != want_sg[i];
     std::printf("%ld tile grids checked, %ld errors\n", grids, bad);
     return bad ? 1 : 0;
 }

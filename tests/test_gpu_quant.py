@@ -194,6 +194,54 @@ def test_weight_observer_kernels(ops, qmax):
     np.testing.assert_array_equal(s.numpy().view(np.uint32), so.numpy().view(np.uint32))
 
 
+@pytest.mark.parametrize("k,ld_q", [(200, 512), (5120, 5248), (7, 300), (384, 384), (1000, 1008)])
+def test_quantisers_leave_a_wider_row_stride_alone(ops, k, ld_q):
+    """Through the C ABI with a row stride beyond the padded row: values in [0, k), zeros up to the next multiple of
+    128 (as far as the row reaches), and not a byte touched behind that (the output may be a column slice of a wider
+    buffer, or rows kept apart on purpose)."""
+    from dax_amd import _capi
+
+    L = _capi.lib()
+    m = 37
+    x, _, _ = O.make_inputs(m, k, 8, seed=k)
+    xd = dev(x)
+    st = torch.cuda.current_stream().cuda_stream
+    kp = min(ld_q, (k + 127) // 128 * 128)
+    ref_q, ref_s = O.act_quant_int8(x)
+    for fn, extra in ((L.daxq_act_quant_i8, ()), (L.daxq_gelu_tanh_act_quant_i8, None)):
+        q = torch.full((m, ld_q), 0x55, dtype=torch.int8, device="cuda")
+        s = torch.zeros(m, device="cuda")
+        if extra is None:
+            if k % 8:
+                continue           # the fused producers take rows of whole 16-byte pieces only
+            rc = fn(xd.data_ptr(), m, k, k, None, 0, q.data_ptr(), ld_q, s.data_ptr(), st)
+        else:
+            rc = fn(xd.data_ptr(), m, k, k, q.data_ptr(), ld_q, s.data_ptr(), st)
+        assert rc == 0, _capi.last_error()
+        torch.cuda.synchronize()
+        assert bool((q[:, k:kp] == 0).all()) and bool((q[:, kp:] == 0x55).all())
+        if extra is not None:
+            assert torch.equal(q[:, :k].cpu(), ref_q[:, :k]) and torch.equal(s.cpu(), ref_s.view(-1))
+
+
+def test_activation_rows_of_whole_kilobytes_are_kept_apart(ops):
+    """Quantised activations whose rows are a multiple of 1 KB long come back with a row stride 128 bytes larger
+    (memory channels, see ops.Q_ROW_PAD); the GEMM follows the stride, values and results are the oracle's."""
+    m, k, n = 300, 1024, 256
+    x, w, b = O.make_inputs(m, k, n, seed=3)
+    qw, sw = O.weight_quant_int8(w)
+    ref = O.linear_int8(x, qw, sw, b)
+    xq, sx = ops.act_quant_i8(dev(x))
+    assert xq.shape == (m, k) and xq.stride() == (k + 128, 1)
+    assert torch.equal(xq.cpu(), ref["xq"])
+    out = ops.linear_i8(xq, sx, dev(qw), dev(sw.view(-1)), dev(b))
+    assert torch.equal(out.cpu().view(torch.int16), ref["out"].view(torch.int16))
+    xq2, _ = ops.act_quant_i8(dev(x[:, :896].contiguous()))
+    assert xq2.stride() == (896, 1)          # 7 x 128: not a multiple of 1 KB, rows contiguous
+    q3, _, _ = ops.gelu_tanh_act_quant_i8(dev(x))
+    assert q3.shape == (m, k) and q3.stride() == (k + 128, 1)
+
+
 def test_cpu_tensor_is_rejected_loudly(ops):
     with pytest.raises((RuntimeError, NotImplementedError)):
         ops.act_quant_i8(torch.zeros(4, 128, dtype=torch.bfloat16))
