@@ -370,8 +370,9 @@ def main():
 
     # ---- the fused producer + quantiser kernels (outside the timed step): LayerNorm multiply-add in front of
     #      the K=5120 linears, GELU-tanh in front of the 13824 -> 5120 one; algorithmic bytes 3 per element
-    def timed(fn, reps=5):
-        fn()
+    def timed(fn, reps=20):
+        for _ in range(3):  # the first calls pay for fresh allocations and cold clocks
+            fn()
         a, b2 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         a.record()
         for _ in range(reps):
