@@ -323,10 +323,11 @@ static int launch_gemm(const void* xq, int64_t ld_xq, const float* sx, const voi
     a.k = (int)k;
     a.tiles_m = a.tiles_n = 0;
     a.gm = (kernel >> 16) & 0xff ? (kernel >> 16) & 0xff : 4;
-    // Tile order of the five-stage 256x256 kernel (bits 24-25 of `kernel`: 0 = by shape, 1 = row groups, 2 = whole
-    // patches per XCD).  The patch order brings the L2-miss traffic down to what eight separate L2s must fetch (measured:
-    // 1.00x that floor on the four 14B shapes against 1.15-1.36x for the row groups), but only the long-K launch gets
-    // faster by it (K = 13824: +2 %; K = 5120: -0.5 to -7 %, 32 CUs in lockstep on the same 12 panels), so long K takes it.
+    // Tile order of the 256x256 kernels (bits 24-25 of `kernel`: 0 = by shape, 1 = row groups, 2 = whole patches per
+    // XCD, 3 = the same patches in super-groups of rows).  The patch orders bring the L2-miss traffic down to what eight
+    // separate L2s must fetch (measured: 1.00x that floor on the four 14B shapes against 1.15-1.36x for the row groups),
+    // but only the long-K launch gets faster by it (K = 13824: +2 %; K = 5120: -0.5 to -7 %: same occupancy and
+    // s_waitcnt share, higher clock, lower MFMA duty, i.e. longer waits at the slice barriers), so long K takes it.
     const int order_bits = (kernel >> 24) & 3;
     a.order = order_bits == 3 ? 2 : order_bits == 2 || (order_bits == 0 && k >= 8192 && m >= 8192) ? 1 : 0;
     a.out_kind = out_kind;
@@ -458,7 +459,7 @@ static int splitk_formats(int x_fmt, int w_fmt, bool& fp8, int& f8) {
 
 // ---- split-K on the library's own scratch memory (for callers that cannot allocate) ------------------------------
 // The workspace of daxq_linear_w8a8_splitk as a file-scope device array: tile counters at its head, then room for 512
-// partial results of 64 KiB (tiles x ranges <= 512, which is also the most that splitk_choice ever asks for).  Every
+// partial results of 64 KiB (tiles x ranges <= 512; splitk_choice never asks for more than 256).  Every
 // device the library runs on holds its own copy at its own address until the process ends.  `scratch` is only the
 // host-side handle of the array: host code uses the per-device address that hipGetSymbolAddress returned, never the name.
 constexpr int64_t kStaticSlots = 512;
