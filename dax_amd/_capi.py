@@ -131,12 +131,13 @@ _tile_order = 0
 def debug_select_gemm(v: int) -> None:
     """0 = the library's choice by shape; 2 / 5 / 6 / 8 / 9 / 11 = one implementation (include/daxq.h);
     1000 + d = depth d of the tile-order groups (1000 = default); 2000 + o = tile order of the 256x256 kernels
-    (2000 = by shape, 2001 = groups of tile rows, 2002 = whole patches per XCD)."""
+    (2000 = by shape, 2001 = groups of tile rows, 2002 = whole patches per XCD, 2003 = patches in super-groups,
+    2004 / 2005 = banded patches 8 / 4 columns wide, 2006 / 2007 = swept patches 4 / 8 columns wide)."""
     global _kernel_choice, _tile_group, _tile_order
     v = int(v)
     if 1000 <= v < 1064:
         _tile_group = v - 1000
-    elif 2000 <= v < 2004:
+    elif 2000 <= v < 2008:
         _tile_order = v - 2000
     elif v in (0, 2, 5, 6, 8, 9, 11):
         _kernel_choice = v

@@ -589,6 +589,19 @@ int launch_tile256(const GemmArgs& a0, bool x_e5m2, hipStream_t st) {
 //
 // BT: tile edge.  256 is the form described above; 128 (wavefronts of 64 x 64, five 16 KB stages, two workgroups
 // per CU) is the same pipeline for launches with too few 256-tiles to fill the CUs.
+// workgroups of a launch of 256x256 tiles in the tile order a.order
+static inline int64_t grid_of_order(const GemmArgs& a) {
+    switch (a.order) {
+        case 1: return patched_grid(a.tiles_m, a.tiles_n);
+        case 2: return supergroups_grid(a.tiles_m, a.tiles_n);
+        case 3: return banded_grid(a.tiles_m, a.tiles_n, 8);
+        case 4: return banded_grid(a.tiles_m, a.tiles_n, 4);
+        case 5: return swept_grid(a.tiles_m, a.tiles_n, 4);
+        case 6: return swept_grid(a.tiles_m, a.tiles_n, 8);
+        default: return (int64_t)a.tiles_m * a.tiles_n;
+    }
+}
+
 namespace t5 {
 constexpr int BKS = 64, NST = 5, T = 256;
 }  // namespace t5
@@ -645,6 +658,10 @@ __global__ __launch_bounds__(256) void gemm_tile256s5_kernel(const GemmArgs p) {
         if (!tile_of_block_patched(tile_id, p.tiles_m, p.tiles_n, tm, tn)) return;  // padding slot (before any barrier)
     } else if (!SPLITK && p.order == 2) {
         if (!tile_of_block_supergroups(tile_id, p.tiles_m, p.tiles_n, tm, tn)) return;
+    } else if (!SPLITK && p.order >= 5) {
+        if (!tile_of_block_swept(tile_id, p.tiles_m, p.tiles_n, p.order == 5 ? 4 : 8, tm, tn)) return;
+    } else if (!SPLITK && p.order >= 3) {
+        if (!tile_of_block_banded(tile_id, p.tiles_m, p.tiles_n, p.order == 3 ? 8 : 4, tm, tn)) return;
     } else {
         tile_of_block(p.gm, tile_id, p.tiles_m, p.tiles_n, tm, tn);
     }
@@ -1026,6 +1043,10 @@ __global__ __launch_bounds__(256) void gemm_tile256f16_kernel(const GemmArgs p) 
         if (!tile_of_block_patched(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn)) return;  // padding slot (before any barrier)
     } else if (p.order == 2) {
         if (!tile_of_block_supergroups(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn)) return;
+    } else if (p.order >= 5) {
+        if (!tile_of_block_swept(blockIdx.x, p.tiles_m, p.tiles_n, p.order == 5 ? 4 : 8, tm, tn)) return;
+    } else if (p.order >= 3) {
+        if (!tile_of_block_banded(blockIdx.x, p.tiles_m, p.tiles_n, p.order == 3 ? 8 : 4, tm, tn)) return;
     } else {
         tile_of_block(p.gm, blockIdx.x, p.tiles_m, p.tiles_n, tm, tn);
     }
@@ -1274,7 +1295,7 @@ template <bool DUMP, int F8>
 static int launch_tile256f16_impl(const GemmArgs& a, hipStream_t st) {
     auto kern = gemm_tile256f16_kernel<DUMP, F8>;
     if (int rc = prepare_tile256f16<DUMP, F8>()) return rc;
-    const int64_t nt = a.order == 1 ? patched_grid(a.tiles_m, a.tiles_n) : a.order == 2 ? supergroups_grid(a.tiles_m, a.tiles_n) : (int64_t)a.tiles_m * a.tiles_n;
+    const int64_t nt = grid_of_order(a);
     if (nt > 0x7fffffff) return fail(DAXQ_ERR_ARG, "gemm: too many tiles");
     hipLaunchKernelGGL(kern, dim3((unsigned)nt), dim3(f16::T), f16::SMEM, st, a);
     return check_launch("gemm_tile256f16");
@@ -1331,7 +1352,7 @@ static int launch_tile256s5_impl(const GemmArgs& a, hipStream_t st) {
     constexpr int SMEM = NST * 2 * BT * BKS;  // 160 KB (256 tile), 80 KB (128 tile)
     auto kern = gemm_tile256s5_kernel<FP8, DUMP, F8, N16, BT>;
     if (int rc = prepare_tile256s5<FP8, DUMP, F8, N16, BT>()) return rc;
-    const int64_t nt = a.order == 1 ? patched_grid(a.tiles_m, a.tiles_n) : a.order == 2 ? supergroups_grid(a.tiles_m, a.tiles_n) : (int64_t)a.tiles_m * a.tiles_n;
+    const int64_t nt = grid_of_order(a);
     if (nt > 0x7fffffff) return fail(DAXQ_ERR_ARG, "gemm: too many tiles");
     hipLaunchKernelGGL(kern, dim3((unsigned)nt), dim3(T), SMEM, st, a);
     return check_launch("gemm_tile256s5");

@@ -290,6 +290,19 @@ static int launch_generic(const GemmArgs& a, int f8, hipStream_t st) {
 // depth of the tile-order groups (0 = 4 tile rows).
 enum { K_DEFAULT = 0, K_GENERIC256 = 2, K_GENERIC128 = 5, K_TWO_STAGE = 6, K_FIVE_STAGE = 8, K_FIVE_STAGE_WIDE = 9, K_FIVE_STAGE_128 = 11 };
 
+// Tile order a launch of 256x256 tiles takes when the caller names none.  The banded order (tile_order.h: patches of
+// 8 x 4 tiles per XCD, the eight XCDs of a round on the same activation rows and on different weight bands) reads the
+// least from the L2s' far side and was the fastest order on every large shape measured (INT8 and FP8 alike, M = 20000
+// to 75600, K = 2048 to 13824, N = 5120 to 15360: +0.6 to +5.8 % over the row groups, most at long K).  It deals whole
+// patches of 32 tiles to the XCDs, so it is taken only where that costs no extra round of tiles; with fewer than five
+// bands (N < 5120), K below 2048 or few rounds the row groups were as fast or faster (M = 9450, a 1/8 share of the
+// rows: -3 to -16 %; K = 1536: -2 %; N = K = 4096: -2 %).
+static int order_by_shape(int64_t m, int64_t n, int64_t k) {
+    const int64_t tm = (m + 255) / 256, tn = (n + 255) / 256, tiles = tm * tn;
+    if (k < 2048 || tn < 20 || tiles < 2048 || tm > 0x7fffff || tn > 0x7fffff) return 0;
+    return banded_grid((int)tm, (int)tn, 4) == (tiles + 255) / 256 * 256 ? 4 : 0;
+}
+
 template <bool FP8>
 static int launch_gemm(const void* xq, int64_t ld_xq, const float* sx, const void* wq, int64_t ld_wq, const float* sw,
                        const void* bias, void* out, int64_t ld_out, void* acc, int64_t ld_acc, int64_t m, int64_t n,
@@ -323,13 +336,11 @@ static int launch_gemm(const void* xq, int64_t ld_xq, const float* sx, const voi
     a.k = (int)k;
     a.tiles_m = a.tiles_n = 0;
     a.gm = (kernel >> 16) & 0xff ? (kernel >> 16) & 0xff : 4;
-    // Tile order of the 256x256 kernels (bits 24-25 of `kernel`: 0 = by shape, 1 = row groups, 2 = whole patches per
-    // XCD, 3 = the same patches in super-groups of rows).  The patch orders bring the L2-miss traffic down to what eight
-    // separate L2s must fetch (measured: 1.00x that floor on the four 14B shapes against 1.15-1.36x for the row groups),
-    // but only the long-K launch gets faster by it (K = 13824: +2 %; K = 5120: -0.5 to -7 %: same occupancy and
-    // s_waitcnt share, higher clock, lower MFMA duty, i.e. longer waits at the slice barriers), so long K takes it.
-    const int order_bits = (kernel >> 24) & 3;
-    a.order = order_bits == 3 ? 2 : order_bits == 2 || (order_bits == 0 && k >= 8192 && m >= 8192) ? 1 : 0;
+    // Tile order of the 256x256 kernels: bits 24-27 of `kernel`, 0 = by shape (order_by_shape), else 1 + the value of
+    // GemmArgs::order.
+    const int order_bits = (kernel >> 24) & 15;
+    if (order_bits > 7) return fail(DAXQ_ERR_ARG, "linear: unknown tile order %d", order_bits);
+    a.order = order_bits ? order_bits - 1 : ((kernel & 0xffff) == K_FIVE_STAGE_128 ? 0 : order_by_shape(m, n, k));
     a.out_kind = out_kind;
     a.splits = 1;
     a.counters = nullptr;

@@ -101,4 +101,92 @@ inline int64_t supergroups_grid(int tiles_m, int tiles_n) {
     return (int64_t)most * 256;
 }
 
+// Banded order.  Same idea as the patch-aligned order (32 slots of an XCD = one patch of 32 / w rows x w columns), with
+// two changes that keep the XCDs on DIFFERENT weight panels at any one time:
+//   * the columns left over by the main bands (width W = 8 or 4) form one band per set bit of tiles_n % W (widths 4, 2,
+//     1: patches of 8 x 4, 16 x 2, 32 x 1), so no slot is padding in the width;
+//   * those narrow bands are woven into the sequence instead of being appended to it: the tile rows are cut into
+//     super-rows of 32, a super-row into steps of one main-patch height, and a step emits one patch of every main band
+//     followed by the patch of each narrow band that starts at that row.  Patch 8 * round + xcd goes to XCD xcd, so
+//     the eight XCDs of a round sit in eight consecutive entries: different bands when there are at least eight.
+// A full super-row emits tiles_n patches.
+DAXQ_HOST_DEVICE int banded_before(int s, int hmain, int nb_main, int rem) {  // patches of a super-row before step s
+    int c = s * nb_main;
+    for (int wj = 4; wj >= 1; wj >>= 1)
+        if (rem & wj) c += (s * hmain * wj + 31) >> 5;  // ceil(s * hmain / (32 / wj))
+    return c;
+}
+DAXQ_HOST_DEVICE bool tile_of_block_banded(int pid, int tiles_m, int tiles_n, int W, int& tm, int& tn) {
+    const int xcd = pid & 7, local = pid >> 3, slot = local & 31;
+    const int patch = (local >> 5) * 8 + xcd;
+    const int hmain = 32 / W, nb_main = tiles_n / W, rem = tiles_n - nb_main * W;
+    const int sr = patch / tiles_n, u = patch - sr * tiles_n;
+    int s = W - 1;  // steps of a super-row: 32 / hmain = W
+    while (s > 0 && banded_before(s, hmain, nb_main, rem) > u) --s;
+    int v = u - banded_before(s, hmain, nb_main, rem);
+    const int row0 = sr * 32 + s * hmain;
+    int h = hmain, col0 = v * W;
+    if (v >= nb_main) {
+        v -= nb_main;
+        col0 = nb_main * W;
+        h = 0;
+        for (int wj = 4; wj >= 1; wj >>= 1) {
+            if (!(rem & wj)) continue;
+            const int hj = 32 / wj;
+            if ((s * hmain) % hj == 0) {
+                if (v == 0) {
+                    h = hj;
+                    break;
+                }
+                --v;
+            }
+            col0 += wj;
+        }
+        if (h == 0) return false;  // beyond the step's patches (cannot happen for u < patches of the super-row)
+    }
+    tm = row0 + slot % h;
+    tn = col0 + slot / h;
+    return tm < tiles_m;
+}
+inline int64_t banded_grid(int tiles_m, int tiles_n, int W) {
+    const int hmain = 32 / W, nb_main = tiles_n / W, rem = tiles_n - nb_main * W;
+    const int left = tiles_m & 31;
+    const int64_t patches = (int64_t)(tiles_m >> 5) * tiles_n + banded_before((left + hmain - 1) / hmain, hmain, nb_main, rem);
+    return (patches + 7) / 8 * 256;
+}
+
+// Swept order.  Patches of 32 / W rows x W columns again, but every XCD keeps to itself: the patches are listed row
+// block by row block (a row block = one patch height of tile rows, nb = ceil(tiles_n / W) patches), XCD x owns the
+// x-th eighth of that list and walks through it, so that consecutive patches of an XCD share their activation panels
+// and no activation panel is ever wanted by two XCDs at the same time.  Inside a row block the bands are visited in
+// an order rotated per XCD, such that at any one time XCD x is about x * nb / 8 bands ahead of XCD 0: the eight
+// XCDs read different weight panels.  The last band may be narrower than W and the last row block shorter than a
+// patch: those slots are padding.
+DAXQ_HOST_DEVICE int swept_cut(int x, int total) { return (int)(((int64_t)x * total) >> 3); }
+DAXQ_HOST_DEVICE bool tile_of_block_swept(int pid, int tiles_m, int tiles_n, int W, int& tm, int& tn) {
+    const int xcd = pid & 7, local = pid >> 3, round = local >> 5, slot = local & 31;
+    const int H = 32 / W, nb = (tiles_n + W - 1) / W, rbs = (tiles_m + H - 1) / H, total = nb * rbs;
+    const int i = swept_cut(xcd, total) + round;
+    if (i >= swept_cut(xcd + 1, total)) return false;
+    const int rb = i / nb, j = i - rb * nb;
+    int owner = xcd;  // the XCD that owns the first patch of this row block decides the rotation
+    while (owner > 0 && swept_cut(owner, total) > rb * nb) --owner;
+    int rot = (owner * nb) / 8 - swept_cut(owner, total) % nb;
+    rot = rot < 0 ? rot + nb : rot;
+    int band = j + rot;
+    band = band >= nb ? band - nb : band;
+    tm = rb * H + slot % H;
+    tn = band * W + slot / H;
+    return tm < tiles_m && tn < tiles_n;
+}
+inline int64_t swept_grid(int tiles_m, int tiles_n, int W) {
+    const int H = 32 / W, nb = (tiles_n + W - 1) / W, rbs = (tiles_m + H - 1) / H, total = nb * rbs;
+    int most = 0;
+    for (int x = 0; x < 8; ++x) {
+        const int n = swept_cut(x + 1, total) - swept_cut(x, total);
+        most = n > most ? n : most;
+    }
+    return (int64_t)most * 256;
+}
+
 }  // namespace daxq

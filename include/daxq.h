@@ -264,8 +264,10 @@ int daxq_linear_e5m2_e4m3(const uint8_t* xq, int64_t ld_xq, const float* sx,
  * (int8 results are the same bits for every choice, fp8 results differ by fp32 summation order): low 16 bits 2 / 5 =
  * generic kernel on 256x256 / 128x128 tiles, 6 = two-stage 256x256 kernel, 8 = the 256x256 kernel on 16x16 MFMAs
  * (int8 16x16x64; fp8 16x16x128 from k = 512 on), 9 = the 256x256 kernel on 32x32 MFMAs, 11 = the five-stage kernel on
- * 128x128 tiles; bits 16-23, when not zero, set the depth of the tile-order groups; bits 24-25 the tile order of the
- * 256x256 kernels (0 = by shape, 1 = groups of tile rows, 2 = whole 32-tile patches per XCD).  fp16 / fp32 outputs
+ * 128x128 tiles; bits 16-23, when not zero, set the depth of the tile-order groups; bits 24-27 the tile order of the
+ * 256x256 kernels (0 = by shape, 1 = groups of tile rows, 2 = whole 32-tile patches per XCD, 3 = those patches in
+ * super-groups of rows, 4 / 5 = banded patches with main bands 8 / 4 tile columns wide, 6 / 7 = swept patches 4 / 8
+ * columns wide; every order computes every tile once, the results are the same bits).  fp16 / fp32 outputs
  * exist in the generic kernel only.  The choice is an argument of the call: the library keeps no process-wide
  * selection.
  */

@@ -1,6 +1,6 @@
-// Host-side check of the patch-aligned tile order (dax_amd/csrc/tile_order.h): for every tile grid up to 320 x 72 the
-// launch of patched_grid() workgroups computes every tile exactly once, padding slots map to no tile, and the 32 slots
-// that one XCD runs side by side lie in one patch of at most 4 x 8 (or (32 / w) x w) tiles.  Built by
+// Host-side check of the patch tile orders (dax_amd/csrc/tile_order.h: patch-aligned, super-groups, banded, swept): for
+// every tile grid up to 320 x 72 the launch of *_grid() workgroups computes every tile exactly once, padding slots map
+// to no tile, and the 32 slots that one XCD runs side by side lie in one patch of at most 32 tiles, 8 columns wide.  Built by
 // __graft_entry__.build() with the host compiler; run by tests/test_abi_and_host.py.
 #include <cstdio>
 #include <cstdlib>
@@ -50,11 +50,19 @@ int main() {
                            [](int a, int b) { return daxq::patched_grid(a, b); }, grids);
     bad += check_order([](int pid, int a, int b, int& tm, int& tn) { return daxq::tile_of_block_supergroups(pid, a, b, tm, tn); },
                        [](int a, int b) { return daxq::supergroups_grid(a, b); }, grids);
+    for (int W : {8, 4})
+        bad += check_order([W](int pid, int a, int b, int& tm, int& tn) { return daxq::tile_of_block_banded(pid, a, b, W, tm, tn); },
+                           [W](int a, int b) { return daxq::banded_grid(a, b, W); }, grids);
+    for (int W : {8, 4})
+        bad += check_order([W](int pid, int a, int b, int& tm, int& tn) { return daxq::tile_of_block_swept(pid, a, b, W, tm, tn); },
+                           [W](int a, int b) { return daxq::swept_grid(a, b, W); }, grids);
     // the four benchmark launches: grid sizes and padding
     const long want[3][3] = {{296, 20, 6144}, {296, 60, 17920}, {296, 54, 16128}};
     for (auto& w : want) bad += daxq::patched_grid((int)w[0], (int)w[1]) != w[2];
     const long want_sg[3] = {6144, 17920, 16384};  // 296 x 54: super-groups of 20 rows, the last one holds 6 empty patches
     for (int i = 0; i < 3; ++i) bad += daxq::supergroups_grid((int)want[i][0], (int)want[i][1]) != want_sg[i];
+    // banded order, 8 x 4 patches: no more rounds of tiles than the tile count itself needs on the four benchmark launches
+    for (auto& w : want) bad += daxq::banded_grid((int)w[0], (int)w[1], 4) != (w[0] * w[1] + 255) / 256 * 256;
     std::printf("%ld tile grids checked, %ld errors\n", grids, bad);
     return bad ? 1 : 0;
 }

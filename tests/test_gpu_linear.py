@@ -73,17 +73,20 @@ def test_linear_i8_bit_exact(ops, variant, m, n, k):
 
 # tile grids (in 256-tiles) whose remainder band is 0 to 7 columns wide, with and without a partial last patch
 PATCH_SHAPES = [(256, 2048, 128), (1100, 2304, 128), (2600, 1024 + 256 * 2, 256), (700, 2048 + 256 * 3, 128), (2100, 256 * 4, 128),
-                (1300, 2048 + 256 * 5, 128), (1500, 256 * 6, 256), (520, 4096 + 256 * 7, 128), (8500, 304, 128), (300, 5120, 384)]
+                (1300, 2048 + 256 * 5, 128), (1500, 256 * 6, 256), (520, 4096 + 256 * 7, 128), (8500, 304, 128), (300, 5120, 384),
+                (9100, 256 * 7, 128)]
 
 
+@pytest.mark.parametrize("order", [2002, 2003, 2004, 2005, 2006, 2007])
 @pytest.mark.parametrize("m,n,k", PATCH_SHAPES)
-def test_patch_tile_order_bit_exact(ops, m, n, k):
-    """The five-stage kernel with whole 32-slot patches per XCD (padding workgroups exit): every output tile is
-    computed exactly once, accumulators and outputs equal the integer oracle's; FP8 equals the row-group order's bits."""
+def test_patch_tile_order_bit_exact(ops, m, n, k, order):
+    """The 256x256 kernels in every tile order that deals whole 32-slot patches to the XCDs (padding workgroups exit):
+    every output tile is computed exactly once, accumulators and outputs equal the integer oracle's; FP8 equals the
+    row-group order's bits."""
     from dax_amd import _capi
 
     _capi.debug_select_gemm(8)
-    _capi.debug_select_gemm(2002)
+    _capi.debug_select_gemm(order)
     g = torch.Generator().manual_seed(m + n + k)
     xq = torch.randint(-127, 128, (m, k), dtype=torch.int8, generator=g)
     wq = torch.randint(-127, 128, (n, k), dtype=torch.int8, generator=g)

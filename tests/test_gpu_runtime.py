@@ -149,7 +149,7 @@ def test_captured_graph_replays_match_eager(fp8):
 @pytest.mark.parametrize("fp8", [False, True])
 def test_captured_graph_of_the_256_tile_kernels_replays_match_eager(fp8):
     """The kernels the large shapes run on (INT8 16x16x64, FP8 16x16x128; chosen by argument here because the shape
-    is small) and the patch tile order with its padding workgroups, captured and replayed with new operand contents."""
+    is small) and the banded tile order with its padding workgroups, captured and replayed with new operand contents."""
     import dax_amd.ops as ops
     from dax_amd import _capi
 
@@ -171,7 +171,7 @@ def test_captured_graph_of_the_256_tile_kernels_replays_match_eager(fp8):
     fn = ops.linear_e4m3 if fp8 else ops.linear_i8
     try:
         _capi.debug_select_gemm(8)
-        _capi.debug_select_gemm(2002)
+        _capi.debug_select_gemm(2005)
         static_x, static_w = operands(0)
         fn(static_x, sx, static_w, sw, b)
         torch.cuda.synchronize()
