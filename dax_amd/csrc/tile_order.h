@@ -148,6 +148,29 @@ DAXQ_HOST_DEVICE bool tile_of_block_banded(int pid, int tiles_m, int tiles_n, in
     tn = col0 + slot / h;
     return tm < tiles_m;
 }
+// Tile times the slowest XCD needs in the banded order: ceil(its tiles / 32 CUs).  Patches of the full super-rows hold
+// 32 tiles each; only those of the last, partial super-row are counted one by one.
+inline int64_t banded_xcd_rounds(int tiles_m, int tiles_n, int W) {
+    const int hmain = 32 / W, nb_main = tiles_n / W, rem = tiles_n - nb_main * W;
+    const int64_t full = (int64_t)(tiles_m >> 5) * tiles_n;
+    int64_t load[8];
+    for (int x = 0; x < 8; ++x) load[x] = (full / 8 + (x < full % 8 ? 1 : 0)) * 32;
+    const int left = tiles_m & 31;
+    int next = (int)(full % 8);
+    for (int s = 0; s * hmain < left; ++s) {
+        const int row = s * hmain, rows_main = left - row < hmain ? left - row : hmain;
+        for (int b = 0; b < nb_main; ++b, next = (next + 1) & 7) load[next] += rows_main * W;
+        for (int wj = 4; wj >= 1; wj >>= 1) {
+            if (!(rem & wj) || row % (32 / wj)) continue;
+            const int hj = 32 / wj;
+            load[next] += (left - row < hj ? left - row : hj) * wj;
+            next = (next + 1) & 7;
+        }
+    }
+    int64_t most = 0;
+    for (int x = 0; x < 8; ++x) most = load[x] > most ? load[x] : most;
+    return (most + 31) / 32;
+}
 inline int64_t banded_grid(int tiles_m, int tiles_n, int W) {
     const int hmain = 32 / W, nb_main = tiles_n / W, rem = tiles_n - nb_main * W;
     const int left = tiles_m & 31;

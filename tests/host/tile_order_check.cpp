@@ -61,6 +61,21 @@ int main() {
     for (auto& w : want) bad += daxq::patched_grid((int)w[0], (int)w[1]) != w[2];
     const long want_sg[3] = {6144, 17920, 16384};  // 296 x 54: super-groups of 20 rows, the last one holds 6 empty patches
     for (int i = 0; i < 3; ++i) bad += daxq::supergroups_grid((int)want[i][0], (int)want[i][1]) != want_sg[i];
+    // banded_xcd_rounds against a count of the tiles that tile_of_block_banded gives every XCD
+    for (int W : {8, 4})
+        for (int tiles_m = 1; tiles_m <= 300; tiles_m += (tiles_m < 70 ? 1 : 23))
+            for (int tiles_n = 1; tiles_n <= 72; ++tiles_n) {
+                long load[8] = {0};
+                const int64_t grid = daxq::banded_grid(tiles_m, tiles_n, W);
+                for (int64_t pid = 0; pid < grid; ++pid) {
+                    int tm, tn;
+                    if (daxq::tile_of_block_banded((int)pid, tiles_m, tiles_n, W, tm, tn)) ++load[pid & 7];
+                }
+                long most = 0;
+                for (long v : load) most = v > most ? v : most;
+                ++grids;
+                bad += daxq::banded_xcd_rounds(tiles_m, tiles_n, W) != (most + 31) / 32;
+            }
     // banded order, 8 x 4 patches: no more rounds of tiles than the tile count itself needs on the four benchmark launches
     for (auto& w : want) bad += daxq::banded_grid((int)w[0], (int)w[1], 4) != (w[0] * w[1] + 255) / 256 * 256;
     std::printf("%ld tile grids checked, %ld errors\n", grids, bad);
