@@ -23,6 +23,10 @@
 //   MFMA + one DMA load + one fragment read so that the loads of slice kt+2 and the first
 //   fragments of slice kt+1 are spread over its MFMAs.
 //
+// Which tile a workgroup computes is a launch argument (GemmArgs::order): groups of tile rows per XCD (tile_of_block,
+// gemm_common.h) or one of the orders of tile_order.h that give the 32 CUs of an XCD a patch of 32 tiles; the large
+// launches take the banded one (the eight XCDs on the same activation rows and on different weight columns).
+//
 // Tiles at the M / N edge are shifted inwards (origin min(tile*256, dim-256)) instead of being
 // predicated: the overlap rows are computed twice with identical results.  The five-stage kernel
 // also exists on 128x128 tiles (launches with too few 256-tiles to fill the CUs); shapes with
@@ -570,6 +574,19 @@ int launch_tile256(const GemmArgs& a0, bool x_e5m2, hipStream_t st) {
     return a.acc ? launch_tile256_impl<FP8, true>(a, st) : launch_tile256_impl<FP8, false>(a, st);
 }
 
+// workgroups of a launch of 256x256 tiles in the tile order a.order
+static inline int64_t grid_of_order(const GemmArgs& a) {
+    switch (a.order) {
+        case 1: return patched_grid(a.tiles_m, a.tiles_n);
+        case 2: return supergroups_grid(a.tiles_m, a.tiles_n);
+        case 3: return banded_grid(a.tiles_m, a.tiles_n, 8);
+        case 4: return banded_grid(a.tiles_m, a.tiles_n, 4);
+        case 5: return swept_grid(a.tiles_m, a.tiles_n, 4);
+        case 6: return swept_grid(a.tiles_m, a.tiles_n, 8);
+        default: return (int64_t)a.tiles_m * a.tiles_n;
+    }
+}
+
 // ---------------------------------------------------------------------------------------------
 // Five-stage form of the same tile: K in 64-byte slices, five 32 KB LDS stages (all 160 KB).
 //
@@ -589,19 +606,6 @@ int launch_tile256(const GemmArgs& a0, bool x_e5m2, hipStream_t st) {
 //
 // BT: tile edge.  256 is the form described above; 128 (wavefronts of 64 x 64, five 16 KB stages, two workgroups
 // per CU) is the same pipeline for launches with too few 256-tiles to fill the CUs.
-// workgroups of a launch of 256x256 tiles in the tile order a.order
-static inline int64_t grid_of_order(const GemmArgs& a) {
-    switch (a.order) {
-        case 1: return patched_grid(a.tiles_m, a.tiles_n);
-        case 2: return supergroups_grid(a.tiles_m, a.tiles_n);
-        case 3: return banded_grid(a.tiles_m, a.tiles_n, 8);
-        case 4: return banded_grid(a.tiles_m, a.tiles_n, 4);
-        case 5: return swept_grid(a.tiles_m, a.tiles_n, 4);
-        case 6: return swept_grid(a.tiles_m, a.tiles_n, 8);
-        default: return (int64_t)a.tiles_m * a.tiles_n;
-    }
-}
-
 namespace t5 {
 constexpr int BKS = 64, NST = 5, T = 256;
 }  // namespace t5
