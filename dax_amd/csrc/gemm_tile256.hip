@@ -630,11 +630,13 @@ struct TileAcc<false, true> {
 // counts itself in at the tile's counter; the workgroup that arrives last adds the partial results of all ranges
 // in range order (so FP8 sums do not depend on who was last) and runs the epilogue.  No workgroup waits for
 // another.  The last one sets the counter back to zero.
-template <bool FP8, bool DUMP, int F8, bool N16 = false, int BT = 256, bool SPLITK = false>
+template <bool FP8, bool DUMP, int F8, bool N16 = false, int BT = 256, bool SPLITK = false, int D = 2>
 __global__ __launch_bounds__(256) void gemm_tile256s5_kernel(const GemmArgs p) {
     using namespace t5;
     static_assert(!(FP8 && N16), "the 16x16 form exists for INT8 only");
     static_assert(BT == 256 || BT == 128, "tile edge");
+    static_assert(D == 2 || (D == 4 && BT == 128 && !SPLITK), "the deep ring exists on 128 tiles (nine 16 KB stages)");
+    constexpr int NSTG = 2 * D + 1;                   // LDS stages: the slice being read plus D pairs in flight
     typedef typename Frag<FP8>::type frag_t;
     constexpr int WT = BT / 2;                        // edge of a wavefront's outputs
     constexpr int NB = WT / (N16 ? 16 : 32);          // MFMA blocks per operand and wavefront: 8 / 4 (256), 4 / 2 (128)
@@ -743,21 +745,23 @@ __global__ __launch_bounds__(256) void gemm_tile256s5_kernel(const GemmArgs p) {
     frag_t fa00[4] = {}, fb00[4] = {}, fa01[4] = {}, fb01[4] = {}, fa10[4] = {}, fb10[4] = {}, fa11[4] = {}, fb11[4] = {};
 
     const int S = klen / BKS;  // slices; even because K (and each split range) is a multiple of 128
-    // stage offsets of slices s .. s+4 (s = the even slice of the current pair)
-    uint32_t st0 = 0, st1 = STAGE, st2 = 2 * STAGE, st3 = 3 * STAGE, st4 = 4 * STAGE;
+    // stage offsets of slices s .. s+2D-1 and, last, of slice s-1 (s = the even slice of the current pair)
+    uint32_t st[NSTG];
+#pragma unroll
+    for (int i = 0; i < NSTG; ++i) st[i] = i * STAGE;
 
     // One slice.  ODD: slice parity (which register set is consumed).  At its barrier slice s+1 has
     // landed for every wave and every wave has the fragments of slice s in registers.
-    //   ISSUE  start half of pair (s+4, s+5) (s even: the A loads; s odd: the B loads of the same
+    //   ISSUE  start half of pair (s+2D, s+2D+1) (s even: the A loads; s odd: the B loads of the same
     //          pair) into the stages o_ld0 / o_ld1 that slices s-1 and s have left
     //   NEXT   slice s+1 exists: read its fragments into the other set
-    //   YOUNG  loads issued after those of slice s+1 exist and may stay in flight: a whole pair at
-    //          an even slice, the A half of the newest pair at an odd one (vmcnt retires in order)
+    //   YOUNG  number of loads issued after those of slice s+1 that may stay in flight: D-1 whole pairs at
+    //          an even slice, D-2 pairs and the A half of the newest pair at an odd one (vmcnt retires in order)
     //   EXTRA  younger loads that are not tile loads (the epilogue's scales) and may stay in flight
     //   FIRST  slice 0 of the tile: its MFMAs start from zero, the accumulators need no clearing
     auto slice = [&](auto ODD, auto ISSUE, auto NEXT, auto YOUNG, auto EXTRA, auto FIRST, uint32_t o_next, uint32_t o_ld0, uint32_t o_ld1)
                      __attribute__((always_inline)) {
-        __builtin_amdgcn_s_waitcnt(vmcnt_imm((YOUNG.value ? (ODD.value ? PAIR_LOADS / 2 : PAIR_LOADS) : 0) + EXTRA.value) & lgkmcnt0_mask());
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm(YOUNG.value + EXTRA.value) & lgkmcnt0_mask());
         __builtin_amdgcn_s_barrier();
 #pragma unroll
         for (int g = 0; g < NREG; ++g) {
@@ -831,35 +835,51 @@ __global__ __launch_bounds__(256) void gemm_tile256s5_kernel(const GemmArgs p) {
             }
             if constexpr (ODD.value) {
                 if (g == NREG - 1) {
-                    const uint32_t r0 = st0, r1 = st1;
-                    st0 = st2;
-                    st1 = st3;
-                    st2 = st4;
-                    st3 = r0;
-                    st4 = r1;
+                    const uint32_t r0 = st[0], r1 = st[1];
+#pragma unroll
+                    for (int i = 0; i + 2 < NSTG; ++i) st[i] = st[i + 2];
+                    st[NSTG - 2] = r0;
+                    st[NSTG - 1] = r1;
                 }
             }
             __builtin_amdgcn_sched_barrier(0);
         }
     };
-    // a pair of slices (s, s+1), s even; YOUNG of the odd slice equals ISSUE (the pair this one started).
-    // The stage offsets are passed by value: the odd slice rotates them in its last region.
-    auto pair = [&](auto ISSUE, auto YOUNG_E, auto NEXT_O, auto EXTRA, auto FIRST) __attribute__((always_inline)) {
-        slice(No{}, ISSUE, Yes{}, YOUNG_E, EXTRA, FIRST, st1, st4, st0);
-        slice(Yes{}, ISSUE, NEXT_O, ISSUE, EXTRA, No{}, st2, st4, st0);
+    // a pair of slices (s, s+1), s even.  The stage offsets are passed by value: the odd slice rotates them in its
+    // last region.
+    auto pair = [&](auto ISSUE, auto YOUNG_E, auto YOUNG_O, auto NEXT_O, auto EXTRA, auto FIRST) __attribute__((always_inline)) {
+        slice(No{}, ISSUE, Yes{}, YOUNG_E, EXTRA, FIRST, st[1], st[NSTG - 1], st[0]);
+        slice(Yes{}, ISSUE, NEXT_O, YOUNG_O, EXTRA, No{}, st[2], st[NSTG - 1], st[0]);
+    };
+    // a pair of the steady state (it starts pair q+D), and tail pair TL of the D pairs behind the last loads
+    typedef Int<(D - 1) * PAIR_LOADS> SteadyE;
+    typedef Int<(D - 2) * PAIR_LOADS + PAIR_LOADS / 2> SteadyO;
+    auto tail_pair = [&](auto TL) __attribute__((always_inline)) {
+        constexpr int t = decltype(TL)::value;
+        pair(No{}, Int<(D - 1 - t) * PAIR_LOADS>{}, Int<(D - 2 - t > 0 ? D - 2 - t : 0) * PAIR_LOADS>{}, Int<(t < D - 1)>{}, Int<3>{}, No{});
     };
 
-    // ---- prologue: pairs 0 and 1 in flight, pair 0 landed, fragments of slice 0 in set 0
+    // ---- prologue: pairs 0 .. D-1 in flight, pair 0 landed, fragments of slice 0 in set 0
 #pragma unroll
     for (int g = 0; g < PAIR_LOADS; ++g) issue_one(0, STAGE, g);
     advance();
-    if (S >= 4) {
+    if constexpr (D == 2) {
+        if (S >= 4) {
 #pragma unroll
-        for (int g = 0; g < PAIR_LOADS; ++g) issue_one(2 * STAGE, 3 * STAGE, g);
-        advance();
-        __builtin_amdgcn_s_waitcnt(vmcnt_imm(PAIR_LOADS));
-    } else {
-        __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+            for (int g = 0; g < PAIR_LOADS; ++g) issue_one(2 * STAGE, 3 * STAGE, g);
+            advance();
+            __builtin_amdgcn_s_waitcnt(vmcnt_imm(PAIR_LOADS));
+        } else {
+            __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+        }
+    } else {  // the launcher sends only K of at least 2 D pairs here
+#pragma unroll
+        for (int d = 1; d < D; ++d) {
+#pragma unroll
+            for (int g = 0; g < PAIR_LOADS; ++g) issue_one(2 * d * STAGE, (2 * d + 1) * STAGE, g);
+            advance();
+        }
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm((D - 1) * PAIR_LOADS));
     }
     __builtin_amdgcn_s_barrier();
 #pragma unroll
@@ -869,15 +889,15 @@ __global__ __launch_bounds__(256) void gemm_tile256s5_kernel(const GemmArgs p) {
     }
 
     const int Q = S >> 1;  // pairs
-    if (Q >= 3) {
-        pair(Yes{}, Yes{}, Yes{}, Int<0>{}, Yes{});
+    if (D > 2 || Q >= 3) {
+        pair(Yes{}, SteadyE{}, SteadyO{}, Yes{}, Int<0>{}, Yes{});
     } else {  // short K: no pair to peel, clear the accumulators instead
 #pragma unroll
         for (int j = 0; j < NB; ++j)
 #pragma unroll
             for (int i = 0; i < NB; ++i) acc[j][i] = typename TileAcc<FP8, N16>::type{};
     }
-    for (int q = 1; q + 2 < Q; ++q) pair(Yes{}, Yes{}, Yes{}, Int<0>{}, No{});
+    for (int q = 1; q + D < Q; ++q) pair(Yes{}, SteadyE{}, SteadyO{}, Yes{}, Int<0>{}, No{});
 
     // The epilogue's scales and bias are requested here, behind the last tile loads, so that their
     // latency is covered by the remaining two pairs of slices.  Always three loads (a missing bias
@@ -889,8 +909,15 @@ __global__ __launch_bounds__(256) void gemm_tile256s5_kernel(const GemmArgs p) {
     const uint16_t pre_b = (p.bias ? p.bias : reinterpret_cast<const uint16_t*>(p.sw))[n0 + tt];
     __builtin_amdgcn_sched_barrier(0);
 
-    if (Q >= 2) pair(No{}, Yes{}, Yes{}, Int<3>{}, No{});
-    pair(No{}, No{}, No{}, Int<3>{}, No{});
+    if constexpr (D == 2) {
+        if (Q >= 2) tail_pair(Int<0>{});
+        tail_pair(Int<1>{});
+    } else {
+        tail_pair(Int<0>{});
+        tail_pair(Int<1>{});
+        tail_pair(Int<2>{});
+        tail_pair(Int<3>{});
+    }
 
     if constexpr (N16) {
         // The 16x16 MFMAs are inline asm, so the compiler cannot count the wait states between one of them and a
@@ -1310,11 +1337,11 @@ static int launch_tile256f16(const GemmArgs& a, hipStream_t st) {
     return a.acc ? launch_tile256f16_impl<true, F8>(a, st) : launch_tile256f16_impl<false, F8>(a, st);
 }
 
-template <bool FP8, bool DUMP, int F8, bool N16 = false, int BT = 256, bool SPLITK = false>
+template <bool FP8, bool DUMP, int F8, bool N16 = false, int BT = 256, bool SPLITK = false, int D = 2>
 static int prepare_tile256s5() {
     static std::atomic<uint64_t> lds_set{0};  // per instantiation
-    return ensure_dynamic_lds(reinterpret_cast<const void*>(gemm_tile256s5_kernel<FP8, DUMP, F8, N16, BT, SPLITK>),
-                              t5::NST * 2 * BT * t5::BKS, lds_set);
+    return ensure_dynamic_lds(reinterpret_cast<const void*>(gemm_tile256s5_kernel<FP8, DUMP, F8, N16, BT, SPLITK, D>),
+                              (2 * D + 1) * 2 * BT * t5::BKS, lds_set);
 }
 
 // split-K launch on 128 tiles: a.splits ranges of K, a.counters zero, a.partials large enough (checked by the caller)
@@ -1350,16 +1377,31 @@ int launch_tile128_splitk(const GemmArgs& a0, int f8, hipStream_t st) {
 template int launch_tile128_splitk<false>(const GemmArgs&, int, hipStream_t);
 template int launch_tile128_splitk<true>(const GemmArgs&, int, hipStream_t);
 
-template <bool FP8, bool DUMP, int F8, bool N16 = false, int BT = 256>
+template <bool FP8, bool DUMP, int F8, bool N16 = false, int BT = 256, int D = 2>
 static int launch_tile256s5_impl(const GemmArgs& a, hipStream_t st) {
     using namespace t5;
-    constexpr int SMEM = NST * 2 * BT * BKS;  // 160 KB (256 tile), 80 KB (128 tile)
-    auto kern = gemm_tile256s5_kernel<FP8, DUMP, F8, N16, BT>;
-    if (int rc = prepare_tile256s5<FP8, DUMP, F8, N16, BT>()) return rc;
+    constexpr int SMEM = (2 * D + 1) * 2 * BT * BKS;  // 160 KB (256 tile), 80 KB (128 tile), 144 KB (128 tile, nine stages)
+    auto kern = gemm_tile256s5_kernel<FP8, DUMP, F8, N16, BT, false, D>;
+    if (int rc = prepare_tile256s5<FP8, DUMP, F8, N16, BT, false, D>()) return rc;
     const int64_t nt = grid_of_order(a);
     if (nt > 0x7fffffff) return fail(DAXQ_ERR_ARG, "gemm: too many tiles");
     hipLaunchKernelGGL(kern, dim3((unsigned)nt), dim3(T), SMEM, st, a);
     return check_launch("gemm_tile256s5");
+}
+
+// 128x128 tiles.  A launch that gives no CU a second workgroup (at most 256 tiles) has the whole LDS of a CU to itself
+// and takes the form with nine 16 KB stages (four pairs of slices in flight instead of two) when K is long: measured
+// against the five-stage form, M = 512 x N = 5120: K = 5120 22.5 against 23.2 us with the weights near, 31.8 against
+// 33.9 us with weights no launch has touched before; K = 13824 71 against 79 us; K = 20480 66 against 76 us; at
+// K = 1536 the longer fill and tail cost 4 %, so K < 4096 keeps five stages.  With more tiles two workgroups share a
+// CU and its LDS.  What bounds these launches is the CU's path into LDS: a 128x128 tile moves 16 KB per 64-byte slice
+// for 256 MFMA cycles, which is the 64 bytes per cycle that path has (a 256x256 tile needs half of that), and a slice
+// takes about 480 cycles here, FP8 (4 MFMAs a slice) and INT8 (16) alike.
+template <bool FP8, int F8, bool N16>
+static int launch_tile128(const GemmArgs& a, hipStream_t st) {
+    if ((int64_t)a.tiles_m * a.tiles_n <= 256 && a.k >= 4096)
+        return a.acc ? launch_tile256s5_impl<FP8, true, F8, N16, 128, 4>(a, st) : launch_tile256s5_impl<FP8, false, F8, N16, 128, 4>(a, st);
+    return a.acc ? launch_tile256s5_impl<FP8, true, F8, N16, 128>(a, st) : launch_tile256s5_impl<FP8, false, F8, N16, 128>(a, st);
 }
 
 // wide:  32x32 MFMAs (INT8 32x32x32, FP8 32x32x64) instead of the 16x16 forms (256 tile only; kept for the tests and for comparisons)
@@ -1368,7 +1410,7 @@ static int launch_tile256s5_impl(const GemmArgs& a, hipStream_t st) {
 template <bool FP8, int F8>
 static int launch_tile256s5_f8(const GemmArgs& a, bool wide, bool small, hipStream_t st) {
     if (!small && !wide && a.k >= 512) return launch_tile256f16<F8>(a, st);  // 16x16x128 MFMAs (at least four pairs of slices); wide: the 32x32x64 form
-    if (small) return a.acc ? launch_tile256s5_impl<true, true, F8, false, 128>(a, st) : launch_tile256s5_impl<true, false, F8, false, 128>(a, st);
+    if (small) return launch_tile128<true, F8, false>(a, st);
     return a.acc ? launch_tile256s5_impl<true, true, F8>(a, st) : launch_tile256s5_impl<true, false, F8>(a, st);
 }
 
@@ -1386,7 +1428,7 @@ int launch_tile256s5(const GemmArgs& a0, int f8, bool wide, bool small, hipStrea
             default: return launch_tile256s5_f8<true, 0>(a, wide, small, st);
         }
     } else {
-        if (small) return a.acc ? launch_tile256s5_impl<false, true, 0, true, 128>(a, st) : launch_tile256s5_impl<false, false, 0, true, 128>(a, st);
+        if (small) return launch_tile128<false, 0, true>(a, st);
         if (wide) return a.acc ? launch_tile256s5_impl<false, true, 0>(a, st) : launch_tile256s5_impl<false, false, 0>(a, st);
         return a.acc ? launch_tile256s5_impl<false, true, 0, true>(a, st) : launch_tile256s5_impl<false, false, 0, true>(a, st);
     }
@@ -1412,13 +1454,17 @@ int prepare_tile256_kernels() {
     DAXQ_PREP(prepare_tile256s5<false, true, 0, false, 256>);
     DAXQ_PREP(prepare_tile256s5<false, false, 0, true, 128>);
     DAXQ_PREP(prepare_tile256s5<false, true, 0, true, 128>);
+    DAXQ_PREP(prepare_tile256s5<false, false, 0, true, 128, false, 4>);
+    DAXQ_PREP(prepare_tile256s5<false, true, 0, true, 128, false, 4>);
     DAXQ_PREP(prepare_tile256s5<false, false, 0, true, 128, true>);
 #define DAXQ_PREP_F8(F8)                                         \
     DAXQ_PREP(prepare_tile256s5<true, false, F8, false, 128, true>); \
     DAXQ_PREP(prepare_tile256s5<true, false, F8, false, 256>);   \
     DAXQ_PREP(prepare_tile256s5<true, true, F8, false, 256>);    \
     DAXQ_PREP(prepare_tile256s5<true, false, F8, false, 128>);   \
-    DAXQ_PREP(prepare_tile256s5<true, true, F8, false, 128>)
+    DAXQ_PREP(prepare_tile256s5<true, true, F8, false, 128>);    \
+    DAXQ_PREP(prepare_tile256s5<true, false, F8, false, 128, false, 4>); \
+    DAXQ_PREP(prepare_tile256s5<true, true, F8, false, 128, false, 4>)
 #define DAXQ_PREP_F16(F8)                      \
     DAXQ_PREP(prepare_tile256f16<false, F8>); \
     DAXQ_PREP(prepare_tile256f16<true, F8>)

@@ -278,6 +278,39 @@ def test_fp8_16x16x128_form_every_count_of_slice_pairs(ops, k):
     np.testing.assert_array_equal(bf16_bits(out), bf16_bits(ref))
 
 
+@pytest.mark.parametrize("k", [3968, 4096, 4224, 4352, 4480, 5120, 13824])
+def test_nine_stage_128_tile_form_every_count_of_slice_pairs(ops, k):
+    """Launches of at most 256 tiles of 128x128 with K >= 4096 run the five-stage pipeline with nine stages (four pairs
+    of slices in flight): the shortest K it takes, odd and even pair counts, one K below it (the five-stage form), and
+    the depths of the cross-attention and FFN-down projections.  INT8 accumulators and outputs against the integer oracle, FP8 accumulators
+    against exact float64 sums, on a 3 x 6 grid of tiles with ragged edges, chosen by shape and by argument."""
+    from dax_amd import _capi
+
+    m, n = 300, 700
+    g = torch.Generator("cpu").manual_seed(k)
+    xq = torch.randint(-127, 128, (m, k), generator=g, dtype=torch.int32).to(torch.int8)
+    wq = torch.randint(-127, 128, (n, k), generator=g, dtype=torch.int32).to(torch.int8)
+    sx, sw = torch.rand(m, generator=g) * 0.02 + 1e-3, torch.rand(n, generator=g) * 0.002 + 1e-4
+    b = torch.randn(n, generator=g).bfloat16()
+    want_acc = O.int_mm(xq, wq)
+    want_out = O.epilogue_int8(want_acc, sx.view(-1, 1), sw.view(1, -1), b)
+    xf = (torch.randn(m, k, generator=g) * 3).to(torch.float8_e4m3fn)
+    wf = (torch.randn(n, k, generator=g) * 0.5).to(torch.float8_e4m3fn)
+    want_f = xf.double() @ wf.double().t()
+    bound = xf.double().abs() @ wf.double().abs().t()
+    for variant in (11, 0):     # 300 x 700 has 6 tiles of 256x256: the library's own choice is the 128-tile form too
+        _capi.debug_select_gemm(variant)
+        out, acc = ops.linear_i8_acc(dev(xq), dev(sx), dev(wq), dev(sw), dev(b))
+        assert torch.equal(acc.cpu(), want_acc)
+        np.testing.assert_array_equal(bf16_bits(out), bf16_bits(want_out))
+        np.testing.assert_array_equal(bf16_bits(ops.linear_i8(dev(xq), dev(sx), dev(wq), dev(sw), dev(b))), bf16_bits(want_out))
+        outf, accf = ops.linear_e4m3_acc(dev(xf.view(torch.uint8)), dev(sx), dev(wf.view(torch.uint8)), dev(sw), dev(b))
+        err = ((accf.cpu().double() - want_f).abs() / bound.clamp_min(1e-30)).max().item()
+        assert err < 2e-5, err
+        ref = (accf.cpu() * sx.view(-1, 1) * sw.view(1, -1) + b.float()).bfloat16()
+        np.testing.assert_array_equal(bf16_bits(outf), bf16_bits(ref))
+
+
 @pytest.mark.parametrize("e5m2", [False, True])
 @pytest.mark.parametrize("m,n,k", [(8192, 5120, 5120), (4096, 5120, 13824), (2304, 2560, 640)])
 def test_fp8_16x16x128_form_against_the_32x32x64_form_every_element(ops, m, n, k, e5m2):
