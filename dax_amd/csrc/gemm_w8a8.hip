@@ -301,7 +301,8 @@ enum { K_DEFAULT = 0, K_GENERIC256 = 2, K_GENERIC128 = 5, K_TWO_STAGE = 6, K_FIV
 // the rows: -3 to -16 %; K = 1536: -2 %; N = K = 4096: -2 %).
 static int order_by_shape(int64_t m, int64_t n, int64_t k) {
     const int64_t tm = (m + 255) / 256, tn = (n + 255) / 256, tiles = tm * tn;
-    if (k < 2048 || tn < 20 || tiles < 2048 || tm > 0x7fffff || tn > 4096) return 0;  // (the balance count below walks over one row of patches)
+    // (tm >= 32: at least one super-row of whole 8 x 4 patches; tn <= 4096: the balance count walks over one row of patches)
+    if (k < 2048 || tn < 20 || tm < 32 || tiles < 2048 || tm > 0x7fffff || tn > 4096) return 0;
     return banded_xcd_rounds((int)tm, (int)tn, 4) * 100 <= (tiles + 255) / 256 * 105 ? 4 : 0;
 }
 
