@@ -546,6 +546,8 @@ int daxq_linear_w8a8_splitk_static(int x_fmt, int w_fmt, const void* xq, int64_t
 
 int daxq_linear_splitk_choice(int64_t m, int64_t n, int64_t k) { return daxq::splitk_choice(m, n, k); }
 
+int daxq_linear_tile_order_choice(int64_t m, int64_t n, int64_t k) { return 1 + daxq::order_by_shape(m, n, k); }
+
 int64_t daxq_linear_splitk_workspace_bytes(int64_t m, int64_t n, int splits) {
     using namespace daxq;
     if (m <= 0 || n <= 0 || splits <= 1) return 0;

@@ -25,7 +25,7 @@
 extern "C" {
 #endif
 
-#define DAXQ_ABI_VERSION 3
+#define DAXQ_ABI_VERSION 4
 
 #define DAXQ_OK 0
 #define DAXQ_ERR_ARG (-1)    /* null pointer, negative size, bad enum */
@@ -277,6 +277,12 @@ int daxq_linear_w8a8(int x_fmt, int w_fmt, int out_dtype,
                      const void* bias, void* out, int64_t ld_out,
                      void* acc, int64_t ld_acc,
                      int64_t m, int64_t n, int64_t k, int kernel, daxq_stream_t stream);
+
+/* The tile order daxq_linear_w8a8 takes for a launch of 256x256 tiles when bits 24-27 of `kernel` are 0, as the value
+ * of those bits: 1 = groups of tile rows, 5 = banded patches 4 tile columns wide (large launches: K >= 2048,
+ * N >= 5120, M >= 7937 and no XCD more than 5 % over its share of the tiles).  For tests and diagnostics; no
+ * counterpart in the reference, whose matmul comes from a vendor library. */
+int daxq_linear_tile_order_choice(int64_t m, int64_t n, int64_t k);
 
 /*
  * Split-K form of daxq_linear_w8a8 for launches with too few output tiles to fill the CUs (a few hundred rows: the

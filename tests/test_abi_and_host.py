@@ -27,7 +27,7 @@ def test_library_exports_every_declared_symbol():
     for name in declared:
         assert hasattr(lib, name), f"{name} declared in include/daxq.h but not exported"
     assert set(declared) == set(_capi.SIGNATURES), "binding table and header disagree"
-    assert _capi.lib().daxq_abi_version() == _capi.ABI_VERSION == 3
+    assert _capi.lib().daxq_abi_version() == _capi.ABI_VERSION == 4
     assert "undefined symbol" not in _capi.last_error()
 
 
@@ -43,6 +43,24 @@ def test_patch_tile_order_covers_every_tile_once():
         __graft_entry__._build_host_checks()
     r = subprocess.run([exe], capture_output=True, text=True, timeout=120)
     assert r.returncode == 0 and " 0 errors" in r.stdout, r.stdout + r.stderr
+
+
+def test_tile_order_by_shape():
+    """daxq_linear_tile_order_choice (host arithmetic only): the four Wan2.1-14B launches at 75600 tokens and their
+    neighbours take the banded order; a 1/8 share of the rows, short K, narrow N and small launches keep the row
+    groups."""
+    from dax_amd import _capi
+
+    f = _capi.lib().daxq_linear_tile_order_choice
+    for n, k in ((15360, 5120), (5120, 5120), (13824, 5120), (5120, 13824)):
+        assert f(75600, n, k) == 5
+        assert all(f(m, n, k) == 5 for m in range(63488, 75777, 512))
+        assert f(9450, n, k) == 1            # one XCD would end a whole patch ahead of its share
+    assert f(32760, 15360, 5120) == 5 and f(20000, 15360, 5120) == 5
+    assert f(75600, 5120, 1536) == 1         # K below 2048
+    assert f(65536, 4096, 4096) == 1         # fewer than five bands
+    assert f(4096, 15360, 5120) == 1         # less than one super-row of patches
+    assert f(512, 5120, 5120) == 1 and f(1, 8, 128) == 1 and f(0, 0, 0) == 1
 
 
 def test_no_cpu_kernels_and_clear_errors():
