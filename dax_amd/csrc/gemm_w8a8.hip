@@ -292,8 +292,8 @@ enum { K_DEFAULT = 0, K_GENERIC256 = 2, K_GENERIC128 = 5, K_TWO_STAGE = 6, K_FIV
 
 // Tile order a launch of 256x256 tiles takes when the caller names none.  The banded order (tile_order.h: patches of
 // 8 x 4 tiles per XCD, the eight XCDs of a round on the same activation rows and on different weight bands) reads the
-// least from the L2s' far side and was the fastest order on every large shape measured (INT8 and FP8 alike, M = 20000
-// to 75600 in steps of two tile rows around 65536 to 75600, K = 2048 to 13824, N = 5120 to 15360: +0.6 to +5.8 % over
+// least from the L2s' far side and was the fastest order on every large shape measured (INT8 and FP8 alike; M = 20000
+// to 75600, among them every second tile row from 63488 up; K = 2048 to 13824; N = 5120 to 15360: +0.6 to +5.8 % over
 // the row groups, most at long K, and none of the row groups' 3-4 % dips where the XCD ranges start on the same
 // columns).  It deals whole patches of 32 tiles to the XCDs, so one XCD can end up with more tiles than an eighth of
 // them: it is taken when the slowest XCD needs at most 5 % more tile times than the row groups do; with fewer than
