@@ -120,30 +120,48 @@ __global__ __launch_bounds__(256, (PRE == PRE_LN && NCH <= 12 && !WRITE_Y) ? 3 :
         }
 
         if constexpr (PRE == PRE_LN) {
-            // mean and biased variance in fp32, two passes over the registers
-            float sum = 0.0f;
+            // Mean and biased variance in fp32.  Both row sums come straight from the packed bf16 pairs: v_dot2_f32_bf16
+            // multiplies two pairs exactly and adds the products to an fp32 accumulator, so sum(x) = dot(x, 1) and
+            // sum(x^2) = dot(x, x) cost one instruction per pair each, where unpacking, subtracting the mean and
+            // squaring cost five per element.  var = E[x^2] - mean^2 loses bits when the mean is large against the
+            // spread (the two terms cancel), so that form is kept only while mean^2 <= 7 var (the error of the sums,
+            // at most 40 roundings per lane, is then amplified eightfold at worst: 2e-5 of var, 1e-5 of rstd, a 400th
+            // of a bf16 step); any other row -- large offset, constant, non-finite -- takes the second pass over the
+            // registers with the mean subtracted first.  The choice is uniform over the wavefront.
+            float sum = 0.0f, sq = 0.0f;
 #pragma unroll
-            for (int i = 0; i < NCH; ++i) {
-                float f[8];
-                unpack8(v[i], f);  // padding chunks are zero and add nothing
-                sum += ((f[0] + f[1]) + (f[2] + f[3])) + ((f[4] + f[5]) + (f[6] + f[7]));
-            }
-            const float mean = wave_sum_f32(sum) / (float)k;
-            forget_values(v);
-            float ssq = 0.0f;
+            for (int i = 0; i < NCH; ++i) {  // padding chunks are zero and add nothing
+                const uint32_t w[4] = {v[i].x, v[i].y, v[i].z, v[i].w};
 #pragma unroll
-            for (int i = 0; i < NCH; ++i) {
-                if (i * 64 + lane < nch) {
-                    float f[8];
-                    unpack8(v[i], f);
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) {
-                        const float d = f[e] - mean;
-                        ssq += d * d;
-                    }
+                for (int h = 0; h < 4; ++h) {
+                    asm("v_dot2_f32_bf16 %0, %1, %2, %0" : "+v"(sum) : "v"(w[h]), "v"(0x3f803f80u));
+                    asm("v_dot2_f32_bf16 %0, %1, %1, %0" : "+v"(sq) : "v"(w[h]));
                 }
             }
-            const float var = wave_sum_f32(ssq) / (float)k;
+            float mean = wave_sum_f32(sum) / (float)k;
+            float var = wave_sum_f32(sq) / (float)k - mean * mean;
+            if (!(mean * mean <= 7.0f * var)) {
+                // The deviations from the first mean also give what that mean is off by: a plain fp32 sum of K values
+                // near 1000 is uncertain by a few units, i.e. the mean by 1e-3, which is a large part of an output
+                // that lies close to zero.  mean += sum(d) / K, var = sum(d^2) / K - (sum(d) / K)^2.
+                float sd = 0.0f, ssq = 0.0f;
+#pragma unroll
+                for (int i = 0; i < NCH; ++i) {
+                    if (i * 64 + lane < nch) {
+                        float f[8];
+                        unpack8(v[i], f);
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) {
+                            const float d = f[e] - mean;
+                            sd += d;
+                            ssq += d * d;
+                        }
+                    }
+                }
+                const float dm = wave_sum_f32(sd) / (float)k;
+                var = wave_sum_f32(ssq) / (float)k - dm * dm;
+                mean += dm;
+            }
             forget_values(v);
             const float rstd = 1.0f / sqrtf(var + eps);  // IEEE sqrt and division
             const int64_t g = row / rows_per_group;

@@ -350,6 +350,10 @@ def layernorm_affine_bf16(x: torch.Tensor, mul: Optional[torch.Tensor], add: Opt
 
     Operation order of dax/adapters/wan/transformer_adapter.py:151-153 (mul = 1 + scale, add = shift);
     with mul = weight, add = bias and one group it is an affine fp32 LayerNorm cast back to bf16.
+
+    torch's CPU kernel evaluates ``x * rstd - mean * rstd``; for a row whose offset is fifty or more times its spread
+    that difference cancels and outputs next to zero lose digits, where ``(x - mean) * rstd`` (torch's GPU kernel)
+    does not: tests of such rows compare with a float64 evaluation instead (tests/test_gpu_fused.py).
     """
     m, k = x.shape
     y = torch.nn.functional.layer_norm(x.float(), (k,), None, None, eps)

@@ -83,6 +83,47 @@ def test_layernorm_multiply_add(ops, fmt, m, k, rpg, vecs):
     assert torch.equal(q2, q) and torch.equal(s2, s)
 
 
+@pytest.mark.parametrize("fmt", ["i8", "e4m3"])
+def test_layernorm_rows_with_an_offset(ops, fmt):
+    """The variance comes from sum(x^2) / K - mean^2 while the mean is small against the spread and from the second
+    pass over the row otherwise: rows whose offset runs from none to a thousand times the spread (both sides of the
+    switch at mean^2 = 7 var), a row that is constant but for one element, tiny and huge magnitudes."""
+    g = torch.Generator().manual_seed(11)
+    k = 5120
+    offsets = [0.0, 0.5, 1.0, 2.0, 2.5, 2.6, 2.7, 3.0, 4.0, 10.0, 100.0, 1000.0, -2.6, -50.0]
+    rows = [torch.randn(k, generator=g) + o for o in offsets]
+    rows += [torch.randn(k, generator=g) * 1e-3 + 1.0, torch.randn(k, generator=g) * 300 + 5e4, torch.randn(k, generator=g) * 1e-20]
+    spike = torch.full((k,), 7.0)
+    spike[123] = 9.0
+    rows.append(spike)
+    x = torch.stack(rows).bfloat16()
+    mul = 1 + 0.2 * torch.randn(1, k, generator=g)
+    add = 0.1 * torch.randn(1, k, generator=g)
+    fn = getattr(ops, "layernorm_act_quant_" + fmt)
+    q, s, y = fn(dev(x), dev(mul), dev(add), x.shape[0], 1e-6, True)
+    # Against the exact result (float64): torch's CPU kernel, which the oracle calls, evaluates x * rstd - mean * rstd
+    # and loses digits to that cancellation once the offset is 50 times the spread; (x - mean) * rstd, which the
+    # kernel and torch's GPU kernel evaluate, does not.
+    xd = x.double()
+    mean = xd.mean(1, keepdim=True)
+    exact = ((xd - mean) / (xd.var(1, unbiased=False, keepdim=True) + 1e-6).sqrt() * mul.double() + add.double()).float().bfloat16()
+    ref = O.layernorm_affine_bf16(x, mul, add, x.shape[0], 1e-6)
+    rstd = (xd.var(1, unbiased=False, keepdim=True) + 1e-6).rsqrt()
+    for r in range(x.shape[0]):          # row by row: the bound on the share of one-step differences holds for every row
+        # an fp32 mean resolves 6e-8 of itself, so x - mean carries that much absolute error, times rstd and mul: it
+        # shows only where the output lies next to zero (the multiply-add cancels), where bf16 steps are tiny
+        tol = max(1e-6, 2.4e-7 * abs(float(mean[r])) * float(rstd[r]))
+        diff = (y[r].cpu().double() - exact[r].double()).abs()
+        ulps = bf16_ulps(y[r:r + 1], exact[r:r + 1]).view(-1)
+        assert bool(((ulps <= 1) | (diff < tol)).all()), (r, int(ulps.max()), float(diff.max()), tol)
+        # (rows 11, 14 and 17 hold two to five distinct bf16 values, so their outputs sit in as many narrow clusters and a
+        # cluster next to a rounding boundary is several per cent of the row at once)
+        assert float(((ulps > 0) & (diff >= tol)).float().mean()) < (5e-2 if r in (11, 14, 17) else 1e-2), r
+        if r < 10:                       # offsets up to ten times the spread: the oracle agrees as well
+            _check_y(y[r:r + 1], ref[r:r + 1], 1e-2)
+    _check_quant_of_own_y(fmt, y, q, s, k)
+
+
 def test_layernorm_constant_rows_and_strided_input(ops):
     x = torch.full((8, 512), -3.0).bfloat16()
     add = torch.linspace(-2, 2, 512).reshape(1, 512)
