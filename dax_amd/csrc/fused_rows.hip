@@ -171,7 +171,18 @@ __global__ __launch_bounds__(256, (PRE == PRE_LN && NCH <= 12 && !WRITE_Y) ? 3 :
                 const int c = i * 64 + lane;
                 if (c < nch) {
                     float f[8], a[8], b[8];
-                    unpack8(v[i], f);
+                    {
+                        // x - mean in one instruction per element: the pair times (1, 0) or (0, 1) plus -mean.  (A
+                        // non-finite neighbour turns the element into NaN through its zero product; such a row is
+                        // NaN throughout anyway, its mean being non-finite.)
+                        const uint32_t w[4] = {v[i].x, v[i].y, v[i].z, v[i].w};
+                        const float nm = -mean;
+#pragma unroll
+                        for (int h = 0; h < 4; ++h) {
+                            asm("v_dot2_f32_bf16 %0, %1, %2, %3" : "=v"(f[2 * h]) : "v"(w[h]), "v"(0x00003f80u), "v"(nm));
+                            asm("v_dot2_f32_bf16 %0, %1, %2, %3" : "=v"(f[2 * h + 1]) : "v"(w[h]), "v"(0x3f800000u), "v"(nm));
+                        }
+                    }
                     if (in_lds) {
                         const float* sv = s_vec + (i * 128 + lane) * 4;
                         const float4 a0 = *reinterpret_cast<const float4*>(sv);
@@ -190,7 +201,7 @@ __global__ __launch_bounds__(256, (PRE == PRE_LN && NCH <= 12 && !WRITE_Y) ? 3 :
 #pragma unroll
                     for (int e = 0; e < 8; ++e) {
                         // three separately rounded fp32 operations, like the unfused graph
-                        const float xh = __fmul_rn(f[e] - mean, rstd);
+                        const float xh = __fmul_rn(f[e], rstd);
                         f[e] = __fadd_rn(__fmul_rn(xh, a[e]), b[e]);
                     }
                     v[i] = pack8(f);
