@@ -118,14 +118,15 @@ def _random_shapes(count, seed):
     return shapes
 
 
-@pytest.mark.parametrize("variant", [8, 9, 6, 11])
+@pytest.mark.parametrize("variant", [8, 9, 6, 11, 8 | (5 << 24), 8 | (2 << 24)])
 @pytest.mark.parametrize("m,n,k,pad_k,pad_n", _random_shapes(14, seed=2024))
 def test_linear_i8_random_shapes_and_strides_bit_exact(ops, variant, m, n, k, pad_k, pad_n):
     """Seeded random M, N, K (edge tiles shifted inwards in both directions, short and long K) with padded leading
-    dimensions, raw int8 operands straight through the C ABI: accumulators and outputs against the integer oracle."""
+    dimensions, raw int8 operands straight through the C ABI: accumulators and outputs against the integer oracle.
+    (Bits 24-27 of the kernel argument: the banded and the patch tile order on the same operands.)"""
     from dax_amd import _capi
 
-    _capi.debug_select_gemm(variant)
+    _capi.debug_select_gemm(variant & 0xffff)
     g = torch.Generator("cpu").manual_seed(m * 7 + n * 3 + k)
     xq = torch.randint(-127, 128, (m, k), generator=g, dtype=torch.int32).to(torch.int8)
     wq = torch.randint(-127, 128, (n, k), generator=g, dtype=torch.int32).to(torch.int8)
