@@ -106,6 +106,7 @@ def _rows_bf16(x: torch.Tensor, what: str) -> None:
 # average +0.55 %), nothing or a small loss at K = 13824, which keeps its rows contiguous.  The pad is never read or
 # written.
 Q_ROW_PAD = 128
+MIN_TILE_ROWS = 128  # rows of the smallest tile of the tiled GEMM kernels
 
 
 def _row_pad(kp: int) -> int:
@@ -122,15 +123,16 @@ def _fake_q(x, m: int, kp: int, dtype) -> torch.Tensor:
     return x.new_empty_strided((m, kp), (kp + _row_pad(kp), 1), dtype=dtype)
 
 
-def _act_quant(x: torch.Tensor, fp8, e5m2: bool = False) -> Tuple[torch.Tensor, torch.Tensor]:
+def _act_quant(x: torch.Tensor, fp8, e5m2: bool = False, rows: int = 0) -> Tuple[torch.Tensor, torch.Tensor]:
+    """rows > M: the buffers get that many rows and only the first M are written."""
     fmt = "e5m2" if e5m2 else "e4m3" if fp8 else "i8"
     name = "act_quant_" + fmt
     kind = _rows_float(x, name)
     m, k = x.shape
     kp = pad_k(k)
     with _on_device(x):
-        q = _alloc_q(m, kp, torch.uint8 if fp8 else torch.int8, x.device)
-        s = torch.empty((m,), dtype=torch.float32, device=x.device)
+        q = _alloc_q(max(m, rows), kp, torch.uint8 if fp8 else torch.int8, x.device)
+        s = torch.empty((max(m, rows),), dtype=torch.float32, device=x.device)
         if m:
             ld_x = x.stride(0) if m > 1 else k
             _capi.check(_capi.lib().daxq_act_quant_rows(x.data_ptr(), kind, FMT[fmt], m, k, ld_x, q.data_ptr(), kp + _row_pad(kp),
@@ -525,10 +527,16 @@ def _dynamic_linear(x, wq, sw, bias, fmt: str):
     instead of two halves the host time per forward, which is what a small linear costs."""
     fp8 = fmt != "i8"
     _same_device("dynamic_linear_" + fmt, x, wq=wq, sw=sw, bias=bias)  # before the quantiser is launched
-    xq, sx = _act_quant(x, fp8, fmt == "e5m2")
+    # Fewer rows than one 128-row tile: the quantiser fills the first M rows of a 128-row buffer and the tiled kernel
+    # runs on all of it (twice as fast as the generic kernel that takes M < 128 otherwise); what the rows beyond M
+    # hold is never looked at, and their outputs are cut off.
+    m = x.shape[0] if x.dim() == 2 else 0
+    rows = MIN_TILE_ROWS if 0 < m < MIN_TILE_ROWS and wq.dim() == 2 and wq.shape[0] >= MIN_TILE_ROWS else 0
+    xq, sx = _act_quant(x, fp8, fmt == "e5m2", rows)
     if xq.shape[1] != wq.shape[1]:
         raise ValueError(f"daxq::dynamic_linear_{fmt}: x has K={x.shape[1]} (padded {xq.shape[1]}), the weight {wq.shape[1]}")
-    return _linear(xq, sx, wq, sw, bias, fp8, False, fmt == "e5m2")[0]
+    out = _linear(xq, sx, wq, sw, bias, fp8, False, fmt == "e5m2")[0]
+    return out[:m] if rows else out
 
 
 @torch.library.custom_op("daxq::dynamic_linear_i8", mutates_args=(), device_types="cuda")

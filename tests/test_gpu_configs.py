@@ -103,6 +103,31 @@ def test_config4_cross_attention_small_m():
         np.testing.assert_array_equal(bf16_bits(y), bf16_bits(ref))
 
 
+@pytest.mark.parametrize("fp8", [False, True])
+def test_fewer_rows_than_a_tile(fp8):
+    """M below 128: the module quantises into a 128-row buffer and runs the tiled kernel on it (the rows beyond M hold
+    whatever the allocation held); the result has M rows, is contiguous, views like any other, and equals the oracle
+    (INT8 bit for bit).  Shapes that the generic kernel still takes (N < 128) beside them."""
+    for m, k, n in ((1, 1536, 1536), (16, 1536, 1536), (17, 5120, 640), (100, 640, 5120), (127, 1536, 256), (60, 1536, 120), (3, 200, 128)):
+        x, w, b = O.make_inputs(m, k, n, seed=m + n)
+        q = _quantised(k, n, w, b, fp8)
+        y = q(x.to("cuda").view(1, m, k))
+        assert y.shape == (1, m, n) and y.is_contiguous()
+        y = y.view(m, n)
+        if fp8:
+            qw, sw = O.weight_quant_e4m3(w)
+            ref = O.linear_e4m3(x, qw, sw, b)["out"]
+            assert rel_l2(y, ref) < 2e-2
+        else:
+            qw, sw = O.weight_quant_int8(w)
+            ref = O.linear_int8(x, qw, sw, b, keep_acc=False)["out"]
+            np.testing.assert_array_equal(bf16_bits(y), bf16_bits(ref))
+        poisoned = x.clone()                      # a NaN row stays a NaN row and stays alone, also in the padded buffer
+        poisoned[m // 2, 5] = float("nan")
+        yp = q(poisoned.to("cuda"))
+        assert bool(torch.isnan(yp[m // 2]).all()) and bool(torch.equal(torch.isnan(yp).any(1).cpu(), torch.arange(m) == m // 2))
+
+
 def test_q_k_v_separate_equals_n_concatenated():
     # the reference keeps to_q / to_k / to_v as three modules; one GEMM against the N-concatenated
     # weight is the benchmark's "fused QKV" shape.  Per-token / per-channel scales make them identical.
