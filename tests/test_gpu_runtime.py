@@ -65,6 +65,31 @@ def test_traced_graph_matches_eager(fp8, k, backend):
 
 
 @pytest.mark.parametrize("fp8", [False, True])
+def test_few_rows_traced_and_in_a_captured_graph(fp8):
+    """Ten rows: the op quantises into a 128-row buffer and returns the first ten rows of the tiled kernel's output.
+    Traced (the fake kernel promises a [10, N] tensor) and captured into a HIP graph, every call equals eager."""
+    model = _mlp(384, 520, fp8, seed=21)
+    x = _input(5, 384, seed=22)
+    ref = model(x)
+    traced = torch.compile(model, backend="aot_eager", fullgraph=True)
+    assert _same(traced(x), ref)
+    static_x = x.clone()
+    model(static_x)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        static_out = model(static_x)
+    for seed in (23, 24, 25):
+        x2 = _input(5, 384, seed=seed)
+        want = model(x2)
+        torch.cuda.synchronize()
+        static_x.copy_(x2)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert _same(static_out, want), f"replay with seed {seed} differs from eager"
+
+
+@pytest.mark.parametrize("fp8", [False, True])
 def test_compiled_with_graph_replay_matches_eager(fp8):
     """torch.compile(mode="reduce-overhead"): the generated code and the daxq ops are captured into a HIP graph by
     the compiler's runtime and replayed from the third call on; every call equals eager."""
