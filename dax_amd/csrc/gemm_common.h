@@ -48,6 +48,12 @@ struct GemmArgs {
     int splits;
     int32_t* counters;
     void* partials;
+    // A launch of 256x256 tiles with few rounds of workgroups leaves most CUs idle during its last, partial round.
+    // Such a launch is cut in two: `grid` > 0 launches only the first `grid` workgroups of the tile order (the whole
+    // rounds), and a second launch on 128x128 tiles with quad_base > 0 computes the four quadrants of each 256x256
+    // tile from id quad_base - 1 on, one workgroup per quadrant (tiles_m / tiles_n count 256x256 tiles in both).
+    // 0 = off.
+    int grid, quad_base;
 };
 
 // FP8 operand formats of a launch as one template parameter: bit 0 = activations are e5m2, bit 1 = weights are e5m2

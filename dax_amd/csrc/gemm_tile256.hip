@@ -668,12 +668,19 @@ __global__ __launch_bounds__(256) void gemm_tile256s5_kernel(const GemmArgs p) {
         if (!tile_of_block_swept(tile_id, p.tiles_m, p.tiles_n, p.order == 5 ? 4 : 8, tm, tn)) return;
     } else if (!SPLITK && p.order >= 3) {
         if (!tile_of_block_banded(tile_id, p.tiles_m, p.tiles_n, p.order == 3 ? 8 : 4, tm, tn)) return;
+    } else if (BT == 128 && !SPLITK && p.quad_base) {
+        tile_of_block(p.gm, p.quad_base - 1 + (tile_id >> 2), p.tiles_m, p.tiles_n, tm, tn);  // the 256x256 tile
     } else {
         tile_of_block(p.gm, tile_id, p.tiles_m, p.tiles_n, tm, tn);
     }
     int m0 = tm * BT, n0 = tn * BT;
     m0 = m0 + BT <= p.m ? m0 : p.m - BT;
     n0 = n0 + BT <= p.n ? n0 : p.n - BT;
+    if (BT == 128 && !SPLITK && p.quad_base) {  // quadrant tile_id % 4 of the 256x256 tile, whose origin is shifted inwards at the edges
+        m0 = tm * 256, n0 = tn * 256;
+        m0 = (m0 + 256 <= p.m ? m0 : p.m - 256) + ((tile_id >> 1) & 1) * 128;
+        n0 = (n0 + 256 <= p.n ? n0 : p.n - 256) + (tile_id & 1) * 128;
+    }
 
     // ---- HBM side.  One wave instruction fills 1 KB of LDS = 16 rows x 64 B: lane l -> row l/4,
     //      stored chunk l%4, i.e. global chunk (l%4) ^ ((row>>2)&3).  Instruction j of a thread
@@ -1326,7 +1333,7 @@ template <bool DUMP, int F8>
 static int launch_tile256f16_impl(const GemmArgs& a, hipStream_t st) {
     auto kern = gemm_tile256f16_kernel<DUMP, F8>;
     if (int rc = prepare_tile256f16<DUMP, F8>()) return rc;
-    const int64_t nt = grid_of_order(a);
+    const int64_t nt = a.grid > 0 ? a.grid : grid_of_order(a);
     if (nt > 0x7fffffff) return fail(DAXQ_ERR_ARG, "gemm: too many tiles");
     hipLaunchKernelGGL(kern, dim3((unsigned)nt), dim3(f16::T), f16::SMEM, st, a);
     return check_launch("gemm_tile256f16");
@@ -1383,7 +1390,7 @@ static int launch_tile256s5_impl(const GemmArgs& a, hipStream_t st) {
     constexpr int SMEM = (2 * D + 1) * 2 * BT * BKS;  // 160 KB (256 tile), 80 KB (128 tile), 144 KB (128 tile, nine stages)
     auto kern = gemm_tile256s5_kernel<FP8, DUMP, F8, N16, BT, false, D>;
     if (int rc = prepare_tile256s5<FP8, DUMP, F8, N16, BT, false, D>()) return rc;
-    const int64_t nt = grid_of_order(a);
+    const int64_t nt = a.grid > 0 ? a.grid : grid_of_order(a);
     if (nt > 0x7fffffff) return fail(DAXQ_ERR_ARG, "gemm: too many tiles");
     hipLaunchKernelGGL(kern, dim3((unsigned)nt), dim3(T), SMEM, st, a);
     return check_launch("gemm_tile256s5");
@@ -1399,7 +1406,7 @@ static int launch_tile256s5_impl(const GemmArgs& a, hipStream_t st) {
 // takes about 480 cycles here, FP8 (4 MFMAs a slice) and INT8 (16) alike.
 template <bool FP8, int F8, bool N16>
 static int launch_tile128(const GemmArgs& a, hipStream_t st) {
-    if ((int64_t)a.tiles_m * a.tiles_n <= 256 && a.k >= 4096)
+    if ((a.grid > 0 ? (int64_t)a.grid : (int64_t)a.tiles_m * a.tiles_n) <= 256 && a.k >= 4096)
         return a.acc ? launch_tile256s5_impl<FP8, true, F8, N16, 128, 4>(a, st) : launch_tile256s5_impl<FP8, false, F8, N16, 128, 4>(a, st);
     return a.acc ? launch_tile256s5_impl<FP8, true, F8, N16, 128>(a, st) : launch_tile256s5_impl<FP8, false, F8, N16, 128>(a, st);
 }
@@ -1415,11 +1422,7 @@ static int launch_tile256s5_f8(const GemmArgs& a, bool wide, bool small, hipStre
 }
 
 template <bool FP8>
-int launch_tile256s5(const GemmArgs& a0, int f8, bool wide, bool small, hipStream_t st) {
-    GemmArgs a = a0;
-    const int bt = small ? 128 : 256;
-    a.tiles_m = (a.m + bt - 1) / bt;
-    a.tiles_n = (a.n + bt - 1) / bt;
+static int launch_tile256s5_one(const GemmArgs& a, int f8, bool wide, bool small, hipStream_t st) {
     if constexpr (FP8) {
         switch (f8) {
             case 1: return launch_tile256s5_f8<true, 1>(a, wide, small, st);
@@ -1434,8 +1437,59 @@ int launch_tile256s5(const GemmArgs& a0, int f8, bool wide, bool small, hipStrea
     }
 }
 
-template int launch_tile256s5<false>(const GemmArgs&, int, bool, bool, hipStream_t);
-template int launch_tile256s5<true>(const GemmArgs&, int, bool, bool, hipStream_t);
+// CUs of the current device (0 if the query fails), asked once per device
+static int cu_count() {
+    static std::atomic<int> cached[64];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return 0;
+    if (dev >= 0 && dev < 64) {
+        if (int c = cached[dev].load(std::memory_order_relaxed)) return c;
+    }
+    int cus = 0;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) return 0;
+    if (dev >= 0 && dev < 64) cached[dev].store(cus, std::memory_order_relaxed);
+    return cus;
+}
+
+// Tiles of the last, partial round of a 256x256 launch that go to a second launch on 128x128 tiles; 0 = none.
+// One workgroup of 256x256 tiles fills a CU, so a launch of R whole rounds and L more tiles takes R + 1 tile times
+// however small L is.  As 4 L quadrants with a CU each (L <= a quarter of the CUs) the L tiles take half a tile time
+// or less.  Measured against the single launch (INT8 / e4m3, K = 5120 unless noted):
+//   4725 x 13824 (4 rounds + 2 tiles) +5.6 / +6.1 %; 8500 x 4096, K = 2048 (2 + 32) +9.9 / +9.9 %;
+//   20000 x 5120 (6 + 44) +3.3 / +2.4 %; 75600 x 5120 in row groups (23 + 32) -0.6 / -0.8 %: over many rounds the CUs
+//   drift apart and the early ones pick the last tiles up, so the cut is taken up to kTailMaxRounds whole rounds;
+//   with two quadrants per CU (L up to half the CUs: 4725 x 5120, 1 + 124) -5.3 / -5.9 %: a round of 128x128 tiles
+//   at two per CU takes as long as a round of 256x256 tiles, so those launches stay whole.
+constexpr int kTailMaxRounds = 8;
+static int tail_tiles(const GemmArgs& a, int tail) {
+    if (tail == 1 || a.order != 0) return 0;  // the patch orders deal whole patches: their ids are not tile counts
+    const int cus = cu_count();
+    if (cus < 8) return 0;
+    const int64_t tiles = (int64_t)a.tiles_m * a.tiles_n, rounds = tiles / cus, left = tiles - rounds * cus;
+    if (rounds < 1 || left == 0 || 4 * left > cus) return 0;
+    return (tail == 2 || rounds <= kTailMaxRounds) ? (int)left : 0;
+}
+
+// tail: 0 = cut the last partial round off by shape (tail_tiles), 1 = never, 2 = whenever every quadrant gets a CU
+template <bool FP8>
+int launch_tile256s5(const GemmArgs& a0, int f8, bool wide, bool small, int tail, hipStream_t st) {
+    GemmArgs a = a0;
+    const int bt = small ? 128 : 256;
+    a.tiles_m = (a.m + bt - 1) / bt;
+    a.tiles_n = (a.n + bt - 1) / bt;
+    a.grid = a.quad_base = 0;
+    const int left = small || wide ? 0 : tail_tiles(a, tail);
+    if (left == 0) return launch_tile256s5_one<FP8>(a, f8, wide, small, st);
+    const int whole = a.tiles_m * a.tiles_n - left;
+    a.grid = whole;
+    if (int rc = launch_tile256s5_one<FP8>(a, f8, false, false, st)) return rc;
+    a.grid = 4 * left;
+    a.quad_base = whole + 1;
+    return launch_tile256s5_one<FP8>(a, f8, false, true, st);
+}
+
+template int launch_tile256s5<false>(const GemmArgs&, int, bool, bool, int, hipStream_t);
+template int launch_tile256s5<true>(const GemmArgs&, int, bool, bool, int, hipStream_t);
 
 // Every instantiation the launchers above can pick, prepared on the current device: afterwards no launch changes a
 // kernel attribute any more, so the first launch may already sit inside a stream capture.

@@ -244,7 +244,7 @@ template <bool FP8>
 int launch_tile256(const GemmArgs& a, bool x_e5m2, hipStream_t st);
 bool tile256_applies(const GemmArgs& a);
 template <bool FP8>
-int launch_tile256s5(const GemmArgs& a, int f8, bool wide, bool small, hipStream_t st);
+int launch_tile256s5(const GemmArgs& a, int f8, bool wide, bool small, int tail, hipStream_t st);
 template <bool FP8>
 int launch_tile128_splitk(const GemmArgs& a, int f8, hipStream_t st);
 
@@ -348,6 +348,11 @@ static int launch_gemm(const void* xq, int64_t ld_xq, const float* sx, const voi
     a.splits = 1;
     a.counters = nullptr;
     a.partials = nullptr;
+    a.grid = a.quad_base = 0;
+    // bits 28-29 of `kernel`: the last partial round of a launch of 256x256 tiles as a second launch on 128x128 tiles:
+    // 0 = by shape, 1 = never, 2 = whenever every 128x128 tile of it gets a CU of its own
+    const int tail = (kernel >> 28) & 3;
+    if (tail > 2) return fail(DAXQ_ERR_ARG, "linear: unknown tail choice %d", tail);
     const int which = kernel & 0xffff;
     const bool fits32 = a.lda < (1 << 26) && a.ldb < (1 << 26);  // 32-bit row offsets of the tiled kernels
     if (out_kind != DAXQ_BF16 && which != K_DEFAULT && which != K_GENERIC256 && which != K_GENERIC128)
@@ -363,8 +368,8 @@ static int launch_gemm(const void* xq, int64_t ld_xq, const float* sx, const voi
             // M = 512 -> 1127 / 551, M = 1024 (80 large tiles) -> 1275 / 1055, M = 2048 (160) -> 1542 / 1817;
             // 4096 x 1536 x 1536 (96) -> 1182 / 895, 8192 x 1536 x 1536 (192) -> 1517 / 1587.
             const int64_t tiles256 = ((m + 255) / 256) * ((n + 255) / 256);
-            if (tile256_applies(a) && tiles256 >= 128) return launch_tile256s5<FP8>(a, f8, false, false, st);
-            if (m >= 128 && n >= 128 && fits32) return launch_tile256s5<FP8>(a, f8, false, true, st);
+            if (tile256_applies(a) && tiles256 >= 128) return launch_tile256s5<FP8>(a, f8, false, false, tail, st);
+            if (m >= 128 && n >= 128 && fits32) return launch_tile256s5<FP8>(a, f8, false, true, 1, st);
             return launch_generic<FP8, 128>(a, f8, st);
         }
         case K_GENERIC256: return launch_generic<FP8, 256>(a, f8, st);
@@ -376,10 +381,10 @@ static int launch_gemm(const void* xq, int64_t ld_xq, const float* sx, const voi
         case K_FIVE_STAGE:
         case K_FIVE_STAGE_WIDE:  // INT8 with 32x32x32 MFMAs
             if (!tile256_applies(a)) return fail(DAXQ_ERR_ARG, "linear: the 256x256 kernel needs m, n >= 256");
-            return launch_tile256s5<FP8>(a, f8, which == K_FIVE_STAGE_WIDE, false, st);
+            return launch_tile256s5<FP8>(a, f8, which == K_FIVE_STAGE_WIDE, false, tail, st);
         case K_FIVE_STAGE_128:
             if (m < 128 || n < 128 || !fits32) return fail(DAXQ_ERR_ARG, "linear: the 128x128 kernel needs m, n >= 128");
-            return launch_tile256s5<FP8>(a, f8, false, true, st);
+            return launch_tile256s5<FP8>(a, f8, false, true, 1, st);
         default: return fail(DAXQ_ERR_ARG, "linear: unknown kernel choice %d", which);
     }
 }
@@ -451,6 +456,7 @@ static int launch_gemm_splitk(const void* xq, int64_t ld_xq, const float* sx, co
     a.order = 0;
     a.out_kind = DAXQ_BF16;
     a.splits = splits;
+    a.grid = a.quad_base = 0;
     a.counters = static_cast<int32_t*>(workspace);
     a.partials = static_cast<uint8_t*>(workspace) + cbytes;
     return launch_tile128_splitk<FP8>(a, f8, st);

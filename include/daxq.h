@@ -267,7 +267,11 @@ int daxq_linear_e5m2_e4m3(const uint8_t* xq, int64_t ld_xq, const float* sx,
  * 128x128 tiles; bits 16-23, when not zero, set the depth of the tile-order groups; bits 24-27 the tile order of the
  * 256x256 kernels (0 = by shape, 1 = groups of tile rows, 2 = whole 32-tile patches per XCD, 3 = those patches in
  * super-groups of rows, 4 / 5 = banded patches with main bands 8 / 4 tile columns wide, 6 / 7 = swept patches 4 / 8
- * columns wide; every order computes every tile once, the results are the same bits).  fp16 / fp32 outputs
+ * columns wide; every order computes every tile once, the results are the same bits); bits 28-29 the treatment of
+ * the last, partial round of workgroups of a launch of 256x256 tiles in row groups (0 = by shape: when the launch
+ * has one to eight whole rounds and the tiles left over number at most a quarter of the CUs, they run as a second
+ * launch of 128x128 tiles with a CU each; 1 = never; 2 = whenever they number at most a quarter of the CUs; int8
+ * results are the same bits either way).  fp16 / fp32 outputs
  * exist in the generic kernel only.  The choice is an argument of the call: the library keeps no process-wide
  * selection.
  */

@@ -40,6 +40,7 @@ def _default_variant():
 
     _capi.debug_select_gemm(0)
     _capi.debug_select_gemm(2000)
+    _capi.debug_select_gemm(3000)
 
 
 def dev(t):
@@ -105,6 +106,57 @@ def test_patch_tile_order_bit_exact(ops, m, n, k, order):
     _capi.debug_select_gemm(2001)
     f_rows = ops.linear_e4m3(dev(xf), dev(sx), dev(wf), dev(sw), dev(b))
     assert torch.equal(f_patch.view(torch.int16), f_rows.view(torch.int16))
+
+
+# (m, n, k): grids of 256-tiles with one to four whole rounds of 256 workgroups and 1 to 64 tiles left over, edge tiles
+# (shifted inwards) among the tiles left over
+TAIL_SHAPES = [(4100, 4352, 128), (8500, 4096, 256), (4725, 13824, 128), (16300, 1024 + 40, 128), (8200, 8192 - 8, 128)]
+
+
+@pytest.mark.parametrize("m,n,k", TAIL_SHAPES)
+def test_last_round_as_a_second_launch_bit_exact(ops, m, n, k):
+    """A launch of 256x256 tiles whose last round of workgroups is a few tiles: the whole rounds run as 256x256 tiles,
+    the tiles left over as a second launch of their 128x128 quadrants.  Accumulators and outputs equal the integer
+    oracle's with the cut forced and by shape; FP8 outputs stay within tolerance of the single launch's (the second
+    launch adds in another order)."""
+    from dax_amd import _capi
+
+    tiles = -(-m // 256) * -(-n // 256)
+    assert tiles // 256 >= 1 and 0 < tiles % 256 <= 64, "the shape must leave at most a quarter of 256 CUs' worth of tiles"
+    g = torch.Generator().manual_seed(m + n + k)
+    xq = torch.randint(-127, 128, (m, k), dtype=torch.int8, generator=g)
+    wq = torch.randint(-127, 128, (n, k), dtype=torch.int8, generator=g)
+    sx, sw = torch.rand(m, generator=g) + 0.5, torch.rand(n, generator=g) * 0.01
+    b = torch.randn(n, generator=g).bfloat16()
+    ref_acc = O.int_mm(xq, wq)
+    ref_out = O.epilogue_int8(ref_acc, sx.view(-1, 1), sw.view(1, -1), b)
+    xf = torch.where((xq.view(torch.uint8) & 0x7f) == 0x7f, torch.zeros((), dtype=torch.uint8), xq.view(torch.uint8))
+    wf = torch.where((wq.view(torch.uint8) & 0x7f) == 0x7f, torch.zeros((), dtype=torch.uint8), wq.view(torch.uint8))
+    _capi.debug_select_gemm(8)
+    _capi.debug_select_gemm(2001)     # row groups: the order the cut exists for
+    f8 = {}
+    for tail in (3002, 3000, 3001):
+        _capi.debug_select_gemm(tail)
+        out, acc = ops.linear_i8_acc(dev(xq), dev(sx), dev(wq), dev(sw), dev(b))
+        assert torch.equal(acc.cpu(), ref_acc), f"accumulators, tail choice {tail}"
+        np.testing.assert_array_equal(bf16_bits(out), bf16_bits(ref_out))
+        out_plain = ops.linear_i8(dev(xq), dev(sx), dev(wq), dev(sw), None)
+        np.testing.assert_array_equal(bf16_bits(out_plain), bf16_bits(O.epilogue_int8(ref_acc, sx.view(-1, 1), sw.view(1, -1), None)))
+        f8[tail] = ops.linear_e4m3(dev(xf), dev(sx), dev(wf), dev(sw), dev(b)).float().cpu()
+    assert not torch.isnan(f8[3002]).any()
+    assert float((f8[3002] - f8[3001]).norm() / f8[3001].norm()) < 1e-3
+    assert torch.equal(f8[3002], f8[3000]), "one to four whole rounds: the cut is taken by shape"
+
+
+def test_tail_choice_bits_are_validated(ops):
+    from dax_amd import _capi
+
+    x = torch.zeros(256, 128, dtype=torch.int8, device="cuda")
+    s = torch.ones(256, device="cuda")
+    out = torch.empty(256, 256, dtype=torch.bfloat16, device="cuda")
+    rc = _capi.lib().daxq_linear_w8a8(0, 0, 0, x.data_ptr(), 128, s.data_ptr(), x.data_ptr(), 128, s.data_ptr(), None, out.data_ptr(), 256,
+                                      None, 0, 256, 256, 128, 3 << 28, torch.cuda.current_stream().cuda_stream)
+    assert rc < 0 and "tail" in _capi.last_error()
 
 
 def _random_shapes(count, seed):

@@ -171,14 +171,15 @@ def test_captured_graph_replays_match_eager(fp8):
         assert _same(static_out, eager), f"replay with seed {seed} differs from eager"
 
 
+@pytest.mark.parametrize("m,n,k,order,tail", [(700, 2304, 1024, 2005, 3000), (4100, 4352, 256, 2001, 3002)])
 @pytest.mark.parametrize("fp8", [False, True])
-def test_captured_graph_of_the_256_tile_kernels_replays_match_eager(fp8):
+def test_captured_graph_of_the_256_tile_kernels_replays_match_eager(fp8, m, n, k, order, tail):
     """The kernels the large shapes run on (INT8 16x16x64, FP8 16x16x128; chosen by argument here because the shape
-    is small) and the banded tile order with its padding workgroups, captured and replayed with new operand contents."""
+    is small), captured and replayed with new operand contents: in the banded tile order with its padding workgroups,
+    and as the two launches of a grid whose last round of workgroups is cut off (289 tiles: 256 + 33 as quadrants)."""
     import dax_amd.ops as ops
     from dax_amd import _capi
 
-    m, n, k = 700, 2304, 1024
     g = torch.Generator().manual_seed(3)
     sx, sw = (torch.rand(m, generator=g) + 0.5).cuda(), (torch.rand(n, generator=g) * 0.01).cuda()
     b = torch.randn(n, generator=g).bfloat16().cuda()
@@ -196,7 +197,8 @@ def test_captured_graph_of_the_256_tile_kernels_replays_match_eager(fp8):
     fn = ops.linear_e4m3 if fp8 else ops.linear_i8
     try:
         _capi.debug_select_gemm(8)
-        _capi.debug_select_gemm(2005)
+        _capi.debug_select_gemm(order)
+        _capi.debug_select_gemm(tail)
         static_x, static_w = operands(0)
         fn(static_x, sx, static_w, sw, b)
         torch.cuda.synchronize()
@@ -215,6 +217,7 @@ def test_captured_graph_of_the_256_tile_kernels_replays_match_eager(fp8):
     finally:
         _capi.debug_select_gemm(0)
         _capi.debug_select_gemm(2000)
+        _capi.debug_select_gemm(3000)
 
 
 _FIRST_LAUNCH_IN_CAPTURE = r"""
