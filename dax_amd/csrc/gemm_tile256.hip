@@ -1456,6 +1456,7 @@ static int cu_count() {
 // however small L is.  As 4 L quadrants with a CU each (L <= a quarter of the CUs) the L tiles take half a tile time
 // or less.  Measured against the single launch (INT8 / e4m3, K = 5120 unless noted):
 //   4725 x 13824 (4 rounds + 2 tiles) +5.6 / +6.1 %; 8500 x 4096, K = 2048 (2 + 32) +9.9 / +9.9 %;
+//   4095 x 4608, K = 1536 (1 + 32) +10.7 / +9.8 %, K = 8960 +24 / +26 %;
 //   20000 x 5120 (6 + 44) +3.3 / +2.4 %; 75600 x 5120 in row groups (23 + 32) -0.6 / -0.8 %: over many rounds the CUs
 //   drift apart and the early ones pick the last tiles up, so the cut is taken up to kTailMaxRounds whole rounds;
 //   with two quadrants per CU (L up to half the CUs: 4725 x 5120, 1 + 124) -5.3 / -5.9 %: a round of 128x128 tiles
