@@ -63,6 +63,25 @@ def test_tile_order_by_shape():
     assert f(512, 5120, 5120) == 1 and f(1, 8, 128) == 1 and f(0, 0, 0) == 1
 
 
+def test_kernel_argument_fields():
+    """The host-side selection (tests, comparisons) packs the fields of the `kernel` argument as include/daxq.h lays
+    them out: implementation in the low 16 bits, group depth in bits 16-23, tile order in 24-27, treatment of the last
+    partial round of workgroups in 28-29."""
+    from dax_amd import _capi
+
+    try:
+        for v in (8, 1005, 2004, 3002):
+            _capi.debug_select_gemm(v)
+        assert _capi.kernel_arg() == 8 | (5 << 16) | (4 << 24) | (2 << 28)
+        for bad in (3, 1064, 2008, 3003, -1):
+            with pytest.raises(_capi.DaxqError):
+                _capi.debug_select_gemm(bad)
+    finally:
+        for v in (0, 1000, 2000, 3000):
+            _capi.debug_select_gemm(v)
+    assert _capi.kernel_arg() == 0
+
+
 def test_no_cpu_kernels_and_clear_errors():
     import dax_amd.ops as ops
 
