@@ -18,6 +18,11 @@ int check_launch(const char* what);
 constexpr float kEps = 1.1920928955078125e-07f;  // 2^-23 = torch.finfo(float32).eps
 
 __device__ __forceinline__ float bf16_bits_to_f32(uint32_t b) { return __uint_as_float(b << 16); }
+__device__ __forceinline__ float f16_bits_to_f32(uint16_t b) { return (float)__builtin_bit_cast(_Float16, b); }
+// two floats rounded to fp16 (nearest even; overflow gives infinity, as a cast does), lo in the low half
+__device__ __forceinline__ uint32_t pack_f16_rne(float lo, float hi) {
+    return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)lo) | ((uint32_t)__builtin_bit_cast(uint16_t, (_Float16)hi) << 16);
+}
 
 // max / min that give NaN when either operand is NaN, like torch.max / torch.min / torch.clamp on tensors
 // (fmaxf and fminf drop a NaN operand, which would turn a poisoned row into finite garbage)
