@@ -1419,8 +1419,9 @@ static int launch_tile256s5_impl(const GemmArgs& a, hipStream_t st) {
 // 33.9 us with weights no launch has touched before; K = 13824 71 against 79 us; K = 20480 66 against 76 us; at
 // K = 1536 the longer fill and tail cost 4 %, so K < 4096 keeps five stages.  With more tiles two workgroups share a
 // CU and its LDS.  A slice takes about 480 cycles here, FP8 (4 MFMAs a slice) and INT8 (16, 256 cycles) alike, and
-// what it spends the rest on is the issue of its four loads per wavefront: variants that load into registers instead
-// of LDS, read no fragments, wait for no load or drop the barriers take as long, one without loads 17 against 22 us.
+// what it spends the rest on is its four loads per wavefront, whichever way they go: variants that load into registers
+// instead of LDS, read no fragments, wait for no load, drop the barriers or leave the loads to four more wavefronts
+// take as long or longer, one without loads 17 against 22 us.
 template <bool FP8, int F8, bool N16>
 static int launch_tile128(const GemmArgs& a, hipStream_t st) {
     if ((a.grid > 0 ? (int64_t)a.grid : (int64_t)a.tiles_m * a.tiles_n) <= 256 && a.k >= 4096)
