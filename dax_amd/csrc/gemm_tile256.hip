@@ -264,7 +264,11 @@ struct Acc16<true> {
 // of them: lanes 0-15 block 2jp columns 0-7, lanes 16-31 block 2jp+1 columns 0-7, lanes 32-47 block
 // 2jp columns 8-15, lanes 48-63 block 2jp+1 columns 8-15.
 // NB: 16x16 blocks per operand and wavefront (8: 256x256 tile, 4: 128x128 tile); the tile edge is 32 * NB.
-template <bool DUMP, int NB = 8, bool FP8 = false>
+// OUTK (int8 form): element type of out and bias, DAXQ_BF16 / DAXQ_F16 / DAXQ_F32.  A template argument, i.e. a kernel
+// of its own per type: with all three forms inside one kernel behind uniform branches its code grew from 27 to 44 KB
+// and the bf16 launches at K = 1536, which change between main loop and epilogue every 24 slices, lost 2.7 %; with
+// the choice inside the loops they lost 2 to 11 % everywhere.
+template <bool DUMP, int NB = 8, bool FP8 = false, int OUTK = DAXQ_BF16>
 __device__ __forceinline__ void tile256_epilogue16(const GemmArgs& p, typename Acc16<FP8>::type (&acc)[NB][NB], uint8_t* smem, int m0, int n0, int t,
                                                    int wm, int wn, int l15, int g4, float pre_sx, float pre_sw,
                                                    float pre_bias) {
@@ -305,10 +309,34 @@ __device__ __forceinline__ void tile256_epilogue16(const GemmArgs& p, typename A
     }
     __builtin_amdgcn_sched_barrier(0);
 
-    // F16 (int8 form only): out and bias are fp16 instead of bf16.  The two forms are two copies of the whole loop nest
-    // behind one uniform branch: with the choice inside the loops the bf16 form ran 2 to 11 % slower.
-    auto write_out = [&](auto F16) __attribute__((always_inline)) {
-    constexpr bool f16 = decltype(F16)::value;
+    // fp32 module (int8 form): one rounding less and four-byte outputs, a lane's four columns of a block as one store
+    if constexpr (!FP8 && OUTK == DAXQ_F32) {
+        {
+#pragma unroll
+            for (int i = 0; i < NB; ++i) {
+                const float sxv = sxr[i];
+                float* orow = reinterpret_cast<float*>(p.out) + (int64_t)(m0 + wm * WT + i * 16 + l15) * p.ldo + n0 + wn * WT + 4 * g4;
+#pragma unroll
+                for (int j = 0; j < NB; ++j) {
+                    const float sws[4] = {swr[j].x, swr[j].y, swr[j].z, swr[j].w};
+                    const float bs[4] = {br[j].x, br[j].y, br[j].z, br[j].w};
+                    float o[4];
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        float y = (float)acc[j][i][r];
+                        y = y * sxv;
+                        y = y * sws[r];
+                        o[r] = y + bs[r];
+                    }
+                    *reinterpret_cast<float4*>(orow + j * 16) = make_float4(o[0], o[1], o[2], o[3]);
+                }
+            }
+        }
+        return;
+    }
+    // (int8 form only) out and bias are fp16 instead of bf16
+    constexpr bool f16 = !FP8 && OUTK == DAXQ_F16;
+    {
 #pragma unroll
     for (int i = 0; i < NB; ++i) {
         const int ml = wm * WT + i * 16 + l15;
@@ -355,9 +383,7 @@ __device__ __forceinline__ void tile256_epilogue16(const GemmArgs& p, typename A
             *reinterpret_cast<uint4*>(orow + jp * 32) = make_uint4(s0.x, s1.x, s0.y, s1.y);
         }
     }
-    };
-    if (!FP8 && p.out_kind == DAXQ_F16) write_out(Yes{});
-    else write_out(No{});
+    }
 }
 
 // DUMP: also write the raw accumulators to p.acc (tests); a separate instantiation so that the
@@ -647,8 +673,9 @@ struct TileAcc<false, true> {
 // counts itself in at the tile's counter; the workgroup that arrives last adds the partial results of all ranges
 // in range order (so FP8 sums do not depend on who was last) and runs the epilogue.  No workgroup waits for
 // another.  The last one sets the counter back to zero.
-template <bool FP8, bool DUMP, int F8, bool N16 = false, int BT = 256, bool SPLITK = false, int D = 2>
+template <bool FP8, bool DUMP, int F8, bool N16 = false, int BT = 256, bool SPLITK = false, int D = 2, int OUTK = DAXQ_BF16>
 __global__ __launch_bounds__(256) void gemm_tile256s5_kernel(const GemmArgs p) {
+    static_assert(OUTK == DAXQ_BF16 || (N16 && !SPLITK && !DUMP), "fp16 / fp32 outputs exist in the 16x16 int8 form");
     using namespace t5;
     static_assert(!(FP8 && N16), "the 16x16 form exists for INT8 only");
     static_assert(BT == 256 || BT == 128, "tile edge");
@@ -930,7 +957,9 @@ __global__ __launch_bounds__(256) void gemm_tile256s5_kernel(const GemmArgs p) {
     // two wavefronts repeat the loads of the lower two and drop the values)
     const int tt = t & (BT - 1);
     const float pre_sx = p.sx[m0 + tt], pre_sw = p.sw[n0 + tt];
-    const uint16_t pre_b = (p.bias ? p.bias : reinterpret_cast<const uint16_t*>(p.sw))[n0 + tt];
+    uint32_t pre_b;  // the bias element's bits: bf16 / fp16, or fp32
+    if constexpr (OUTK == DAXQ_F32) pre_b = __float_as_uint((p.bias ? reinterpret_cast<const float*>(p.bias) : p.sw)[n0 + tt]);
+    else pre_b = (p.bias ? p.bias : reinterpret_cast<const uint16_t*>(p.sw))[n0 + tt];
     __builtin_amdgcn_sched_barrier(0);
 
     if constexpr (D == 2) {
@@ -1043,8 +1072,8 @@ __global__ __launch_bounds__(256) void gemm_tile256s5_kernel(const GemmArgs p) {
         __syncthreads();                      // every thread has read the flag before the epilogue reuses the LDS
     }
     if constexpr (N16)
-        tile256_epilogue16<DUMP, NB>(p, acc, smem, m0, n0, t, wm, wn, lr, lane >> 4, pre_sx, pre_sw,
-                                     p.bias ? (p.out_kind == DAXQ_F16 ? f16_bits_to_f32(pre_b) : bf16_bits_to_f32(pre_b)) : -0.0f);
+        tile256_epilogue16<DUMP, NB, false, OUTK>(p, acc, smem, m0, n0, t, wm, wn, lr, lane >> 4, pre_sx, pre_sw,
+                                                  !p.bias ? -0.0f : OUTK == DAXQ_F32 ? __uint_as_float(pre_b) : OUTK == DAXQ_F16 ? f16_bits_to_f32((uint16_t)pre_b) : bf16_bits_to_f32(pre_b));
     else
         tile256_epilogue<FP8, DUMP, NB>(p, acc, smem, m0, n0, t, wm, wn, l31, hi, pre_sx, pre_sw,
                                         p.bias ? bf16_bits_to_f32(pre_b) : -0.0f);
@@ -1361,10 +1390,10 @@ static int launch_tile256f16(const GemmArgs& a, hipStream_t st) {
     return a.acc ? launch_tile256f16_impl<true, F8>(a, st) : launch_tile256f16_impl<false, F8>(a, st);
 }
 
-template <bool FP8, bool DUMP, int F8, bool N16 = false, int BT = 256, bool SPLITK = false, int D = 2>
+template <bool FP8, bool DUMP, int F8, bool N16 = false, int BT = 256, bool SPLITK = false, int D = 2, int OUTK = DAXQ_BF16>
 static int prepare_tile256s5() {
     static std::atomic<uint64_t> lds_set{0};  // per instantiation
-    return ensure_dynamic_lds(reinterpret_cast<const void*>(gemm_tile256s5_kernel<FP8, DUMP, F8, N16, BT, SPLITK, D>),
+    return ensure_dynamic_lds(reinterpret_cast<const void*>(gemm_tile256s5_kernel<FP8, DUMP, F8, N16, BT, SPLITK, D, OUTK>),
                               (2 * D + 1) * 2 * BT * t5::BKS, lds_set);
 }
 
@@ -1401,12 +1430,13 @@ int launch_tile128_splitk(const GemmArgs& a0, int f8, hipStream_t st) {
 template int launch_tile128_splitk<false>(const GemmArgs&, int, hipStream_t);
 template int launch_tile128_splitk<true>(const GemmArgs&, int, hipStream_t);
 
-template <bool FP8, bool DUMP, int F8, bool N16 = false, int BT = 256, int D = 2>
+template <bool FP8, bool DUMP, int F8, bool N16 = false, int BT = 256, int D = 2, int OUTK = DAXQ_BF16>
 static int launch_tile256s5_impl(const GemmArgs& a, hipStream_t st) {
     using namespace t5;
     constexpr int SMEM = (2 * D + 1) * 2 * BT * BKS;  // 160 KB (256 tile), 80 KB (128 tile), 144 KB (128 tile, nine stages)
-    auto kern = gemm_tile256s5_kernel<FP8, DUMP, F8, N16, BT, false, D>;
-    if (int rc = prepare_tile256s5<FP8, DUMP, F8, N16, BT, false, D>()) return rc;
+    if (a.out_kind != OUTK) return fail(DAXQ_ERR_ARG, "gemm: this kernel writes output type %d, not %d", OUTK, a.out_kind);
+    auto kern = gemm_tile256s5_kernel<FP8, DUMP, F8, N16, BT, false, D, OUTK>;
+    if (int rc = prepare_tile256s5<FP8, DUMP, F8, N16, BT, false, D, OUTK>()) return rc;
     const int64_t nt = a.grid > 0 ? a.grid : grid_of_order(a);
     if (nt > 0x7fffffff) return fail(DAXQ_ERR_ARG, "gemm: too many tiles");
     hipLaunchKernelGGL(kern, dim3((unsigned)nt), dim3(T), SMEM, st, a);
@@ -1424,6 +1454,13 @@ static int launch_tile256s5_impl(const GemmArgs& a, hipStream_t st) {
 // take as long or longer, one without loads 17 against 22 us.
 template <bool FP8, int F8, bool N16>
 static int launch_tile128(const GemmArgs& a, hipStream_t st) {
+    if constexpr (N16) {  // fp16 / fp32 modules (these forms have no accumulator dump: the dispatcher sends that to the generic kernel)
+        const bool deep = (a.grid > 0 ? (int64_t)a.grid : (int64_t)a.tiles_m * a.tiles_n) <= 256 && a.k >= 4096;
+        if (a.out_kind == DAXQ_F16)
+            return deep ? launch_tile256s5_impl<false, false, 0, true, 128, 4, DAXQ_F16>(a, st) : launch_tile256s5_impl<false, false, 0, true, 128, 2, DAXQ_F16>(a, st);
+        if (a.out_kind == DAXQ_F32)
+            return deep ? launch_tile256s5_impl<false, false, 0, true, 128, 4, DAXQ_F32>(a, st) : launch_tile256s5_impl<false, false, 0, true, 128, 2, DAXQ_F32>(a, st);
+    }
     if ((a.grid > 0 ? (int64_t)a.grid : (int64_t)a.tiles_m * a.tiles_n) <= 256 && a.k >= 4096)
         return a.acc ? launch_tile256s5_impl<FP8, true, F8, N16, 128, 4>(a, st) : launch_tile256s5_impl<FP8, false, F8, N16, 128, 4>(a, st);
     return a.acc ? launch_tile256s5_impl<FP8, true, F8, N16, 128>(a, st) : launch_tile256s5_impl<FP8, false, F8, N16, 128>(a, st);
@@ -1451,6 +1488,8 @@ static int launch_tile256s5_one(const GemmArgs& a, int f8, bool wide, bool small
     } else {
         if (small) return launch_tile128<false, 0, true>(a, st);
         if (wide) return a.acc ? launch_tile256s5_impl<false, true, 0>(a, st) : launch_tile256s5_impl<false, false, 0>(a, st);
+        if (a.out_kind == DAXQ_F16) return launch_tile256s5_impl<false, false, 0, true, 256, 2, DAXQ_F16>(a, st);
+        if (a.out_kind == DAXQ_F32) return launch_tile256s5_impl<false, false, 0, true, 256, 2, DAXQ_F32>(a, st);
         return a.acc ? launch_tile256s5_impl<false, true, 0, true>(a, st) : launch_tile256s5_impl<false, false, 0, true>(a, st);
     }
 }
@@ -1529,6 +1568,12 @@ int prepare_tile256_kernels() {
     DAXQ_PREP(prepare_tile256s5<false, true, 0, true, 128>);
     DAXQ_PREP(prepare_tile256s5<false, false, 0, true, 128, false, 4>);
     DAXQ_PREP(prepare_tile256s5<false, true, 0, true, 128, false, 4>);
+    DAXQ_PREP(prepare_tile256s5<false, false, 0, true, 256, false, 2, DAXQ_F16>);
+    DAXQ_PREP(prepare_tile256s5<false, false, 0, true, 128, false, 2, DAXQ_F16>);
+    DAXQ_PREP(prepare_tile256s5<false, false, 0, true, 128, false, 4, DAXQ_F16>);
+    DAXQ_PREP(prepare_tile256s5<false, false, 0, true, 256, false, 2, DAXQ_F32>);
+    DAXQ_PREP(prepare_tile256s5<false, false, 0, true, 128, false, 2, DAXQ_F32>);
+    DAXQ_PREP(prepare_tile256s5<false, false, 0, true, 128, false, 4, DAXQ_F32>);
     DAXQ_PREP(prepare_tile256s5<false, false, 0, true, 128, true>);
 #define DAXQ_PREP_F8(F8)                                         \
     DAXQ_PREP(prepare_tile256s5<true, false, F8, false, 128, true>); \

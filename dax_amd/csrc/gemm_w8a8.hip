@@ -355,15 +355,15 @@ static int launch_gemm(const void* xq, int64_t ld_xq, const float* sx, const voi
     if (tail > 2) return fail(DAXQ_ERR_ARG, "linear: unknown tail choice %d", tail);
     const int which = kernel & 0xffff;
     const bool fits32 = a.lda < (1 << 26) && a.ldb < (1 << 26);  // 32-bit row offsets of the tiled kernels
-    // the int8 kernels on 16x16 MFMAs (the library's choice, 8, 11) also write fp16; every other tiled kernel bf16 only
-    const bool tiled_out = out_kind == DAXQ_BF16 || (!FP8 && out_kind == DAXQ_F16);
+    // the int8 kernels on 16x16 MFMAs (the library's choice, 8, 11) also write fp16 and fp32; every other tiled kernel bf16 only
+    const bool tiled_out = out_kind == DAXQ_BF16 || (!FP8 && !acc);  // (the accumulator dump of the tiled kernels exists with bf16 outputs)
     if (which != K_DEFAULT && which != K_GENERIC256 && which != K_GENERIC128 &&
         (out_kind != DAXQ_BF16 && !(tiled_out && (which == K_FIVE_STAGE || which == K_FIVE_STAGE_128))))
         return fail(DAXQ_ERR_ARG, "linear: kernel %d does not write this output type", which);
     switch (which) {
         case K_DEFAULT: {
-            // fp32 outputs, and fp16 outputs of the fp8 forms (modules that are not bf16): the generic kernel, which
-            // rounds to any of the three
+            // fp16 / fp32 outputs of the fp8 forms (per-tensor fp8 modules that are not bf16): the generic kernel,
+            // which rounds to any of the three
             if (!tiled_out)
                 return (m >= 256 && n >= 256) ? launch_generic<FP8, 256>(a, f8, st) : launch_generic<FP8, 128>(a, f8, st);
             // library default: the five-stage kernel on 256x256 tiles once there is one for every second CU, on

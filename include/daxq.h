@@ -271,8 +271,8 @@ int daxq_linear_e5m2_e4m3(const uint8_t* xq, int64_t ld_xq, const float* sx,
  * the last, partial round of workgroups of a launch of 256x256 tiles in row groups (0 = by shape: when the launch
  * has one to eight whole rounds and the tiles left over number at most a quarter of the CUs, they run as a second
  * launch of 128x128 tiles with a CU each; 1 = never; 2 = whenever they number at most a quarter of the CUs; int8
- * results are the same bits either way).  fp16 outputs of int8 operands are written by the library's choice and by
- * 8 and 11 (the kernels on 16x16 MFMAs); fp32 outputs, and fp16 outputs of fp8 operands, exist in the generic kernel
+ * results are the same bits either way).  fp16 and fp32 outputs of int8 operands are written by the library's choice
+ * and by 8 and 11 (the kernels on 16x16 MFMAs); fp16 and fp32 outputs of fp8 operands exist in the generic kernel
  * only.  The choice is an argument of the call: the library keeps no process-wide
  * selection.
  */

@@ -107,7 +107,7 @@ def _module(k, n, dtype, seed, bias=True):
 def test_int8_module_fp16_fp32_bit_exact(dtype, m, k, n):
     """out_dtype = the float weight's dtype (dax/quant/nn/dynamic/linear.py:263): scale in the input's dtype, fp32
     scaling of the exact accumulators, cast to fp16 / fp32, bias added in that dtype.  fp16 modules run the tiled
-    kernels (128x128 tiles for the first two shapes, 256x256 with edge tiles for the last), fp32 ones the generic kernel."""
+    and fp32 modules run the tiled kernels (128x128 tiles for the first two shapes, 256x256 with edge tiles for the last)."""
     from dax_amd.quant.quantization import quantize_dynamic
     from dax_amd.quant.quantization.qconfig import get_dynamic_int8_per_token_act_per_channel_weight_qconfig as cfg
 
@@ -131,11 +131,12 @@ def test_int8_module_fp16_fp32_bit_exact(dtype, m, k, n):
     assert yb.dtype == dtype and torch.equal(yb.cpu(), refb)
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
 @pytest.mark.parametrize("variant,m,n,k", [(8, 700, 520, 256), (11, 300, 392, 384), (8, 4100, 4352, 128), (0, 130, 264, 128)])
-def test_int8_fp16_outputs_of_the_tiled_kernels(variant, m, n, k):
-    """fp16 outputs straight from the kernels on 16x16 MFMAs, named by argument, with and without bias, edge tiles
-    included; 289 tiles with the tiles left over after one round forced into a second launch (both write fp16).  Values
-    beyond the fp16 range become infinities, as the reference's cast makes them."""
+def test_int8_fp16_fp32_outputs_of_the_tiled_kernels(variant, m, n, k, dtype):
+    """fp16 / fp32 outputs straight from the kernels on 16x16 MFMAs, named by argument, with and without bias, edge
+    tiles included; 289 tiles with the tiles left over after one round forced into a second launch (both write the
+    type).  Values beyond the fp16 range become infinities, as the reference's cast makes them."""
     import dax_amd.ops as ops
     from dax_amd import _capi
 
@@ -144,17 +145,18 @@ def test_int8_fp16_outputs_of_the_tiled_kernels(variant, m, n, k):
     wq = torch.randint(-127, 128, (n, k), dtype=torch.int8, generator=g)
     sx, sw = torch.rand(m, generator=g) + 0.5, torch.rand(n, generator=g) * 0.01
     sx[0] = 3.0e4                                   # a row that overflows fp16
-    b = torch.randn(n, generator=g).half()
+    b = torch.randn(n, generator=g).to(dtype)
     acc = O.int_mm(xq, wq)
     try:
         _capi.debug_select_gemm(variant)
         _capi.debug_select_gemm(2001)
         _capi.debug_select_gemm(3002)
         for bias in (b, None):
-            out = ops.linear_w8a8(xq.cuda(), sx.cuda(), wq.cuda(), sw.cuda(), bias.cuda() if bias is not None else None, "i8", "i8", torch.float16)
-            ref = O.epilogue_int8(acc, sx.view(-1, 1), sw.view(1, -1), bias, torch.float16)
-            assert out.dtype == torch.float16 and torch.isinf(ref[0]).any()
-            assert torch.equal(out.cpu().view(torch.int16), ref.view(torch.int16)), f"{(out.cpu().view(torch.int16) != ref.view(torch.int16)).sum().item()} outputs differ"
+            out = ops.linear_w8a8(xq.cuda(), sx.cuda(), wq.cuda(), sw.cuda(), bias.cuda() if bias is not None else None, "i8", "i8", dtype)
+            ref = O.epilogue_int8(acc, sx.view(-1, 1), sw.view(1, -1), bias, dtype)
+            assert out.dtype == dtype and (dtype == torch.float32 or torch.isinf(ref[0]).any())
+            bits = torch.int16 if dtype == torch.float16 else torch.int32
+            assert torch.equal(out.cpu().view(bits), ref.view(bits)), f"{(out.cpu().view(bits) != ref.view(bits)).sum().item()} outputs differ"
     finally:
         for v in (0, 2000, 3000):
             _capi.debug_select_gemm(v)
