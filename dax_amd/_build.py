@@ -65,13 +65,6 @@ def build(verbose: bool = False) -> str:
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError(f"hipcc failed on mfma_rate.hip:\n{r.stderr}")
-    # ... and the one behind the epilogue's instruction-rate figure (documentation only; nothing loads it)
-    cmd = [HIPCC, *FLAGS, os.path.join(ROOT, "bench", "valu_rate.hip"), "-o", os.path.join(ROOT, "bench", "valu_rate")]
-    if verbose:
-        print(" ".join(cmd), flush=True)
-    r = subprocess.run(cmd, capture_output=True, text=True)
-    if r.returncode != 0:
-        raise RuntimeError(f"hipcc failed on valu_rate.hip:\n{r.stderr}")
     return LIB
 
 

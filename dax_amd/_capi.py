@@ -11,7 +11,7 @@ import threading
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "libdaxq.so")
-ABI_VERSION = 4
+ABI_VERSION = 5
 
 _lock = threading.Lock()
 _lib = None
@@ -56,6 +56,11 @@ SIGNATURES = {
     "daxq_linear_w8a8_splitk": [_INT, _INT, _P, _I64, _P, _P, _I64, _P, _P, _P, _I64, _I64, _I64, _I64, _INT, _P, _I64, _P],
     "daxq_linear_w8a8_splitk_static": [_INT, _INT, _P, _I64, _P, _P, _I64, _P, _P, _P, _I64, _I64, _I64, _I64, _INT, _P],
     "daxq_linear_w8a8": [_INT, _INT, _INT, _P, _I64, _P, _P, _I64, _P, _P, _P, _I64, _P, _I64, _I64, _I64, _I64, _INT, _P],
+    "daxq_dynamic_linear": [_INT, _INT, _INT, _INT, _P, _I64, _P, _I64, _P, _I64, _P, _I64, _P, _P, _P, _I64, _I64, _I64, _I64,
+                            _P, _I64, _INT, _P],
+    "daxq_dynamic_linear_i8": [_P, _I64, _P, _I64, _P, _P, _I64, _P, _P, _P, _I64, _I64, _I64, _I64, _P],
+    "daxq_dynamic_linear_e4m3": [_P, _I64, _P, _I64, _P, _P, _I64, _P, _P, _P, _I64, _I64, _I64, _I64, _P],
+    "daxq_dynamic_linear_e5m2_e4m3": [_P, _I64, _P, _I64, _P, _P, _I64, _P, _P, _P, _I64, _I64, _I64, _I64, _P],
 }
 
 

@@ -492,12 +492,8 @@ static __device__ __align__(256) __attribute__((used)) unsigned char scratch[kSt
 
 constexpr int kMaxDevices = 64;
 static std::atomic<void*> g_scratch_ptr[kMaxDevices];      // device address of `scratch`, per device
-static std::atomic<int> g_scratch_cleared[kMaxDevices];    // counters cleared once on that device
-
-__global__ void clear_counters_kernel(int32_t* counters, int n) {
-    const int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n) counters[i] = 0;
-}
+// The counters at the head of the array need no clearing: a file-scope device array is zero when the code object is
+// loaded, and every launch leaves the counters it used at zero.
 
 // Address of the current device's copy of `scratch`, looked up once per device.
 static int scratch_of_current_device(void** ptr, int* dev_out) {
@@ -540,13 +536,6 @@ int daxq_linear_w8a8_splitk_static(int x_fmt, int w_fmt, const void* xq, int64_t
                         splits, (long long)slots, (long long)kStaticSlots, (long long)kStaticScratchBytes);
         int dev = 0;
         if (int rc = scratch_of_current_device(&ws, &dev)) return rc;
-        if (!g_scratch_cleared[dev].load(std::memory_order_acquire)) {
-            // first use on this device: the counters start at zero (a kernel on the caller's stream, in front of the GEMM)
-            hipLaunchKernelGGL(clear_counters_kernel, dim3((unsigned)(kMaxSplitTiles / 256)), dim3(256), 0, st,
-                               static_cast<int32_t*>(ws), (int)kMaxSplitTiles);
-            if (int rc = check_launch("clear_counters")) return rc;
-            g_scratch_cleared[dev].store(1, std::memory_order_release);
-        }
     }
     return fp8 ? launch_gemm_splitk<true>(xq, ld_xq, sx, wq, ld_wq, sw, bias, out, ld_out, m, n, k, splits, ws,
                                           kStaticScratchBytes, st, f8)
@@ -616,6 +605,62 @@ int daxq_linear_w8a8(int x_fmt, int w_fmt, int out_dtype, const void* xq, int64_
         return launch_gemm<true>(xq, ld_xq, sx, wq, ld_wq, sw, bias, out, ld_out, acc, ld_acc, m, n, k, (hipStream_t)stream,
                                  (x_fmt == DAXQ_FMT_E5M2 ? kF8XE5 : 0) | (w_fmt == DAXQ_FMT_E5M2 ? kF8WE5 : 0), out_dtype, kernel);
     return fail(DAXQ_ERR_ARG, "linear: unsupported operand formats x=%d w=%d (int8 x int8, or fp8 x fp8)", x_fmt, w_fmt);
+}
+
+// ---- quantiser + GEMM behind one entry point --------------------------------------------------------------------
+int daxq_dynamic_linear(int x_dtype, int x_fmt, int w_fmt, int out_dtype, const void* x, int64_t ld_x, void* xq,
+                        int64_t ld_xq, float* sx, int64_t rows_alloc, const void* wq, int64_t ld_wq, const float* sw,
+                        const void* bias, void* out, int64_t ld_out, int64_t m, int64_t n, int64_t k, void* workspace,
+                        int64_t workspace_bytes, int kernel, daxq_stream_t stream) {
+    using namespace daxq;
+    bool fp8;
+    int f8;
+    if (int rc = splitk_formats(x_fmt, w_fmt, fp8, f8)) return rc;
+    if (m < 0 || n < 0 || k <= 0 || rows_alloc < m)
+        return fail(DAXQ_ERR_ARG, "dynamic_linear: bad shape m=%lld n=%lld k=%lld rows_alloc=%lld", (long long)m, (long long)n,
+                    (long long)k, (long long)rows_alloc);
+    const int64_t kp = (k + DAXQ_K_ALIGN - 1) / DAXQ_K_ALIGN * DAXQ_K_ALIGN;
+    if (ld_xq < kp || ld_wq < kp)
+        return fail(DAXQ_ERR_ARG, "dynamic_linear: ld_xq=%lld and ld_wq=%lld must reach k rounded up to %d (%lld)", (long long)ld_xq,
+                    (long long)ld_wq, DAXQ_K_ALIGN, (long long)kp);
+    if (m == 0 || n == 0) return DAXQ_OK;
+    // the quantiser zero-fills columns [k, kp) of the rows it writes
+    if (int rc = daxq_act_quant_rows(x, x_dtype, x_fmt, m, k, ld_x, xq, ld_xq, sx, stream)) return rc;
+    // Fewer rows than the smallest tile of the tiled kernels: run them on 128 rows of the caller's buffers when those
+    // reach that far (the rows beyond m hold whatever the buffers held; an output row depends on its own operand row only).
+    const int64_t mg = (m < 128 && rows_alloc >= 128 && n >= 128) ? 128 : m;
+    hipStream_t st = (hipStream_t)stream;
+    // INT8 launches with few tiles cut K into ranges when the caller brings a workspace (integer partial sums: the
+    // same bits as the plain launch); FP8 sums would change with the number of rows, so they stay whole.
+    if (!fp8 && workspace && out_dtype == DAXQ_BF16 && kernel == 0) {
+        const int splits = splitk_choice(mg, n, kp);
+        if (splits > 1 && workspace_bytes >= kCounterBytes + splitk_tiles(mg, n) * splits * kPartialBytes)
+            return launch_gemm_splitk<false>(xq, ld_xq, sx, wq, ld_wq, sw, bias, out, ld_out, mg, n, kp, splits, workspace,
+                                             workspace_bytes, st, 0);
+    }
+    return fp8 ? launch_gemm<true>(xq, ld_xq, sx, wq, ld_wq, sw, bias, out, ld_out, nullptr, 0, mg, n, kp, st, f8, out_dtype, kernel)
+               : launch_gemm<false>(xq, ld_xq, sx, wq, ld_wq, sw, bias, out, ld_out, nullptr, 0, mg, n, kp, st, 0, out_dtype, kernel);
+}
+
+int daxq_dynamic_linear_i8(const void* x, int64_t ld_x, int8_t* xq, int64_t ld_xq, float* sx, const int8_t* wq,
+                           int64_t ld_wq, const float* sw, const void* bias, void* out, int64_t ld_out, int64_t m,
+                           int64_t n, int64_t k, daxq_stream_t stream) {
+    return daxq_dynamic_linear(DAXQ_BF16, DAXQ_FMT_I8, DAXQ_FMT_I8, DAXQ_BF16, x, ld_x, xq, ld_xq, sx, m, wq, ld_wq, sw, bias, out,
+                               ld_out, m, n, k, nullptr, 0, 0, stream);
+}
+
+int daxq_dynamic_linear_e4m3(const void* x, int64_t ld_x, uint8_t* xq, int64_t ld_xq, float* sx, const uint8_t* wq,
+                             int64_t ld_wq, const float* sw, const void* bias, void* out, int64_t ld_out, int64_t m,
+                             int64_t n, int64_t k, daxq_stream_t stream) {
+    return daxq_dynamic_linear(DAXQ_BF16, DAXQ_FMT_E4M3, DAXQ_FMT_E4M3, DAXQ_BF16, x, ld_x, xq, ld_xq, sx, m, wq, ld_wq, sw, bias,
+                               out, ld_out, m, n, k, nullptr, 0, 0, stream);
+}
+
+int daxq_dynamic_linear_e5m2_e4m3(const void* x, int64_t ld_x, uint8_t* xq, int64_t ld_xq, float* sx, const uint8_t* wq,
+                                  int64_t ld_wq, const float* sw, const void* bias, void* out, int64_t ld_out, int64_t m,
+                                  int64_t n, int64_t k, daxq_stream_t stream) {
+    return daxq_dynamic_linear(DAXQ_BF16, DAXQ_FMT_E5M2, DAXQ_FMT_E4M3, DAXQ_BF16, x, ld_x, xq, ld_xq, sx, m, wq, ld_wq, sw, bias,
+                               out, ld_out, m, n, k, nullptr, 0, 0, stream);
 }
 
 int daxq_linear_i8(const int8_t* xq, int64_t ld_xq, const float* sx, const int8_t* wq, int64_t ld_wq, const float* sw,

@@ -48,10 +48,16 @@ class _NoGuard:
 _NO_GUARD = _NoGuard()
 
 
+_multi_gpu = None
+
+
 def _on_device(t: torch.Tensor):
     """Context that makes the tensor's device current for the allocations and the launch; with a single GPU it is
     current already and the guard (several microseconds per call) is left out."""
-    return torch.cuda.device(t.device) if torch.cuda.device_count() > 1 else _NO_GUARD
+    global _multi_gpu
+    if _multi_gpu is None:
+        _multi_gpu = torch.cuda.device_count() > 1
+    return torch.cuda.device(t.device) if _multi_gpu else _NO_GUARD
 
 
 def _need_gpu(t: torch.Tensor, what: str) -> None:
@@ -353,19 +359,28 @@ scale_from_minmax.register_fake(lambda min_val, max_val, qmax: torch.empty_like(
 
 # ----------------------------------------------------------------------------- GEMM + epilogue
 # Workspaces of the split-K launches: one per (device, stream), zero-filled when it is made (the kernels leave the
-# counters at its head zero), grown when a larger problem comes along.  Launches on one stream are ordered, so they can
-# share it; another stream gets its own.
+# counters at its head zero).  Launches on one stream are ordered, so they can share it; another stream gets its own.
+# A workspace is never freed once a launch has used it: its address may sit in work that is still queued.  The first
+# one of a stream already holds everything the library's own choice of ranges can ask for (tiles x ranges <= 256); a
+# larger explicit request gets a larger one and the old one stays alive beside it.
 _splitk_ws = {}
+_splitk_retired = []  # outgrown workspaces, kept alive until the process ends
 SPLITK_AUTO = True  # few-tile launches (a few hundred rows) cut K into ranges when it pays
+SPLITK_WS_BYTES = 16384 + 256 * 65536  # counters + 256 partial results of 64 KiB
 
 
 def _splitk_workspace(device, stream: int, need: int):
+    """None while the stream is being captured: a graph replays on whatever stream its owner picks, possibly beside
+    another graph captured on the same stream, and two replays that share one workspace race on its counters.  The
+    caller then takes the plain launch (INT8 results are the same bits either way)."""
+    if torch.cuda.is_current_stream_capturing():
+        return None
     key = (device.index, stream)
     ws = _splitk_ws.get(key)
     if ws is None or ws.numel() < need:
-        if torch.cuda.is_current_stream_capturing():
-            return None  # an allocation recorded into a graph belongs to that graph: take the plain launch instead
-        ws = torch.zeros(max(need, 1 << 20), dtype=torch.uint8, device=device)
+        if ws is not None:
+            _splitk_retired.append(ws)
+        ws = torch.zeros(max(need, SPLITK_WS_BYTES), dtype=torch.uint8, device=device)
         _splitk_ws[key] = ws
     return ws
 
@@ -522,21 +537,67 @@ linear_e4m3_acc.register_fake(lambda xq, sx, wq, sw, bias: (
 
 
 # ----------------------------------------------------------------------------- quantiser + GEMM behind one dispatch
+_Q_DTYPE = {"i8": torch.int8, "e4m3": torch.uint8, "e5m2": torch.uint8}
+_W_FMT = {"i8": 0, "e4m3": 1, "e5m2": 1}  # the weight format each activation format is paired with here
+_splitk_memo = {}  # (rows, n, kp) -> daxq_linear_splitk_choice, host arithmetic asked once per shape
+_dyn_fn = None     # the bound daxq_dynamic_linear
+
+
 def _dynamic_linear(x, wq, sw, bias, fmt: str):
-    """Per-token quantiser and GEMM of one linear, the same two launches as act_quant_* + linear_*; one op call
-    instead of two halves the host time per forward, which is what a small linear costs."""
-    fp8 = fmt != "i8"
-    _same_device("dynamic_linear_" + fmt, x, wq=wq, sw=sw, bias=bias)  # before the quantiser is launched
-    # Fewer rows than one 128-row tile: the quantiser fills the first M rows of a 128-row buffer and the tiled kernel
-    # runs on all of it (twice as fast as the generic kernel that takes M < 128 otherwise); what the rows beyond M
-    # hold is never looked at, and their outputs are cut off.
-    m = x.shape[0] if x.dim() == 2 else 0
-    rows = MIN_TILE_ROWS if 0 < m < MIN_TILE_ROWS and wq.dim() == 2 and wq.shape[0] >= MIN_TILE_ROWS else 0
-    xq, sx = _act_quant(x, fp8, fmt == "e5m2", rows)
-    if xq.shape[1] != wq.shape[1]:
-        raise ValueError(f"daxq::dynamic_linear_{fmt}: x has K={x.shape[1]} (padded {xq.shape[1]}), the weight {wq.shape[1]}")
-    out = _linear(xq, sx, wq, sw, bias, fp8, False, fmt == "e5m2")[0]
-    return out[:m] if rows else out
+    """Per-token quantiser and GEMM of one linear through the library's single entry point for the pair
+    (daxq_dynamic_linear): one ctypes call, and two allocations (the quantised activation with its scales behind it
+    in one buffer, and the output) behind one op dispatch -- the host time per forward is what a small linear costs.
+    The launches are those of act_quant_* followed by linear_*."""
+    global _dyn_fn
+    dev = x.device
+    kind = FLOAT_KIND.get(x.dtype)
+    if dev.type != "cuda" or kind is None or x.dim() != 2 or x.stride(1) != 1:
+        _rows_float(x, "dynamic_linear_" + fmt)  # raises with the reason
+    if dev.index not in _capi._checked_devices:
+        _need_gpu(x, "dynamic_linear_" + fmt)
+    if wq.device != dev or sw.device != dev or (bias is not None and bias.device != dev):
+        _same_device("dynamic_linear_" + fmt, x, wq=wq, sw=sw, bias=bias)  # before anything is launched
+    if wq.dtype != _Q_DTYPE[fmt] or wq.dim() != 2 or wq.stride(1) != 1:
+        raise ValueError(f"daxq::dynamic_linear_{fmt}: the weight must be {_Q_DTYPE[fmt]} [N, pad128(K)] with contiguous rows")
+    m, k = x.shape
+    n, kp = wq.shape
+    if kp != (k + K_ALIGN - 1) // K_ALIGN * K_ALIGN:
+        raise ValueError(f"daxq::dynamic_linear_{fmt}: x has K={k} (padded {pad_k(k)}), the weight {kp}")
+    if sw.dtype != torch.float32 or sw.numel() != n or not sw.is_contiguous():
+        raise ValueError(f"daxq::dynamic_linear_{fmt}: sw must be contiguous fp32 [N]")
+    if bias is not None and (bias.dtype != torch.bfloat16 or bias.numel() != n or not bias.is_contiguous()):
+        raise ValueError(f"daxq::dynamic_linear_{fmt}: bias must be contiguous bfloat16 [N]")
+    # Fewer rows than one 128-row tile: the buffers get 128 rows and the tiled kernel runs on all of them (twice as fast
+    # as the kernel that takes fewer rows); what the rows beyond M hold is never looked at, and their outputs are cut off.
+    rows = MIN_TILE_ROWS if 0 < m < MIN_TILE_ROWS <= n else m
+    ld_q = kp + (Q_ROW_PAD if kp % 1024 == 0 else 0)
+    with _on_device(x):
+        # quantised rows, then the fp32 scales (the row stride is a multiple of 128, so they are aligned)
+        scratch = torch.empty((rows * (ld_q + 4),), dtype=torch.uint8, device=dev)
+        out = torch.empty((rows, n), dtype=torch.bfloat16, device=dev)
+        if m and n:
+            if _dyn_fn is None:
+                _dyn_fn = _capi.lib().daxq_dynamic_linear
+            stream = _stream(x)
+            ws_ptr, ws_bytes = None, 0
+            karg = _capi.kernel_arg()
+            if fmt == "i8" and SPLITK_AUTO and karg == 0:
+                key = (rows, n, kp)
+                splits = _splitk_memo.get(key)
+                if splits is None:
+                    splits = _splitk_memo[key] = _capi.lib().daxq_linear_splitk_choice(rows, n, kp)
+                if splits > 1:
+                    ws = _splitk_workspace(dev, stream, SPLITK_WS_BYTES)
+                    if ws is not None:
+                        ws_ptr, ws_bytes = ws.data_ptr(), ws.numel()
+            base = scratch.data_ptr()
+            rc = _dyn_fn(kind, FMT[fmt], _W_FMT[fmt], 0, x.data_ptr(), x.stride(0) if m > 1 else k, base, ld_q,
+                         base + rows * ld_q, rows, wq.data_ptr(), wq.stride(0) if n > 1 else kp, sw.data_ptr(),
+                         bias.data_ptr() if bias is not None else None, out.data_ptr(), n, m, n, k, ws_ptr, ws_bytes, karg,
+                         stream)
+            if rc:
+                _capi.check(rc, "dynamic_linear_" + fmt)
+    return out[:m] if rows != m else out
 
 
 @torch.library.custom_op("daxq::dynamic_linear_i8", mutates_args=(), device_types="cuda")

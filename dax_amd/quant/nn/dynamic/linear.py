@@ -160,7 +160,60 @@ class Linear(DerivedOperands, nn.Module):
         k, n = self.in_features, self.out_features
         return not (m > 16 and k % 8 == 0 and k > 0 and n % 8 == 0 and n > 0)
 
+    # ------------------------------------------------------------------ the common case, prepared ahead
+    # A bf16 per-token module whose stored state already is what the GEMM reads keeps (op name, weight bytes, weight scale
+    # vector, bias, device) ready: every torch call in a forward costs the host a microsecond or two, and a small
+    # linear's time is the host's.  The tensors alias the module's state, so in-place updates show through; the tuple
+    # also remembers which state tensors it was built from and where they lived, and a forward that finds other ones
+    # (a buffer or parameter replaced by assignment, by a hook of an off-loading framework, or through `.data`)
+    # rebuilds it.  Whatever sets the state afresh (conversion, load_state_dict, .to()) rebuilds it too.
+    _fast = None
+
+    def refresh_derived(self) -> None:
+        super().refresh_derived()
+        self._build_fast()
+
+    def _build_fast(self):
+        object.__setattr__(self, "_fast", None)
+        qw, ws, bp = self._buffers["qweight"], self._buffers["weight_scale"], self._parameters["bias"]
+        if (qw.device.type != "cuda" or self.input_qscheme != per_token_symmetric or self.out_dtype != torch.bfloat16
+                or self.weight_dtype == torch.float8_e5m2 or ws.numel() == 1 or ops.pad_k(qw.shape[1]) != qw.shape[1]
+                or not qw.is_contiguous() or ops.is_tracing(qw) or torch.cuda.is_current_stream_capturing()):
+            return None
+        bias = None if bp is None else bp.detach()
+        if bias is not None and (bias.dtype != torch.bfloat16 or not bias.is_contiguous() or bias.device != qw.device):
+            return None
+        # (plain data only: a module must stay deep-copyable, and a copy finds the addresses changed and rebuilds)
+        fast = (_DYNAMIC_LINEAR[self.input_dtype], self._gemm_weight(), self._weight_scale_vector(), bias,
+                qw.device, qw, ws, bp, qw.data_ptr(), ws.data_ptr(), 0 if bp is None else bp.data_ptr())
+        object.__setattr__(self, "_fast", fast)
+        return fast
+
+    def _fast_is_current(self, f) -> bool:
+        qw, ws, bp = self._buffers["qweight"], self._buffers["weight_scale"], self._parameters["bias"]
+        return (qw is f[5] and ws is f[6] and bp is f[7] and qw.data_ptr() == f[8] and ws.data_ptr() == f[9]
+                and (bp is None or bp.data_ptr() == f[10]))
+
     def forward(self, input) -> Tensor:
+        fast = self._fast
+        if (fast is not None and input.__class__ is Tensor and input.dtype is torch.bfloat16
+                and not self.uncompiled_small_shape_fallback and not torch.compiler.is_compiling()):
+            if not self._fast_is_current(fast):
+                self.refresh_derived()
+                fast = self._fast
+        else:
+            fast = None
+        if fast is not None:
+            op, wq, sw, bias, dev = fast[:5]
+            op = getattr(ops, op)
+            if input.device != dev:
+                self._check_device(input.device)
+            if input.dim() == 2 and input.stride(1) == 1:
+                return op(input, wq, sw, bias)
+            flat = input.view(-1, self.in_features)
+            if flat.stride(-1) != 1:
+                flat = flat.contiguous()
+            return op(flat, wq, sw, bias).view(*input.shape[:-1], self.out_features)
         self._check_device(input.device)
         if self._takes_float_fallback(input):
             logger.warning("int8 matmul not taken for this combination of dimensions, float implementation instead. "

@@ -25,7 +25,7 @@
 extern "C" {
 #endif
 
-#define DAXQ_ABI_VERSION 4
+#define DAXQ_ABI_VERSION 5
 
 #define DAXQ_OK 0
 #define DAXQ_ERR_ARG (-1)    /* null pointer, negative size, bad enum */
@@ -283,6 +283,44 @@ int daxq_linear_w8a8(int x_fmt, int w_fmt, int out_dtype,
                      void* acc, int64_t ld_acc,
                      int64_t m, int64_t n, int64_t k, int kernel, daxq_stream_t stream);
 
+/*
+ * The whole forward of the dynamic W8A8 linear in one call: the per-token quantiser of x followed by the GEMM with the
+ * fused epilogue, i.e. daxq_act_quant_rows + daxq_linear_w8a8 (or its split-K form) on the caller's stream.
+ * Replaces Linear.forward
+ *   dax/quant/nn/dynamic/linear.py:146-228   (FP8 branch :146-178, INT8 branch :181-228)
+ * x     [m, k] of x_dtype elements (DAXQ_BF16 / DAXQ_F16 / DAXQ_F32), leading dimension ld_x
+ * xq    scratch for the quantised activation, one byte per element, [rows_alloc, ld_xq], ld_xq >= roundup(k, DAXQ_K_ALIGN);
+ *       16-byte aligned, ld_xq % 16 == 0; the call writes rows [0, m) (columns [k, roundup(k)) as zeros)
+ * sx    scratch for the per-token scales, fp32 [rows_alloc]
+ * wq    quantised weight [n, roundup(k, DAXQ_K_ALIGN)] (ld_wq), pad columns zero; sw fp32 [n]; bias [n] of out_dtype or NULL
+ * out   [rows_alloc, n] of out_dtype elements (ld_out); rows [0, m) are the result
+ * rows_alloc >= m: rows that xq, sx and out really hold.  With m < 128 <= rows_alloc (and n >= 128) the tiled kernels run
+ *       on 128 rows of those buffers (twice as fast as the kernel that takes fewer rows); rows [m, 128) of out then hold
+ *       unspecified values.  Pass rows_alloc = m to have nothing beyond row m touched.
+ * workspace / workspace_bytes: optional split-K workspace as for daxq_linear_w8a8_splitk (counters zero), or NULL.
+ *       INT8 launches with bf16 outputs and few tiles then cut K into ranges (same bits as the plain launch).
+ * kernel: as for daxq_linear_w8a8 (0 = the library's choice).
+ * Formats and output types as for daxq_linear_w8a8.  The caller owns every buffer; nothing is allocated.
+ */
+int daxq_dynamic_linear(int x_dtype, int x_fmt, int w_fmt, int out_dtype,
+                        const void* x, int64_t ld_x,
+                        void* xq, int64_t ld_xq, float* sx, int64_t rows_alloc,
+                        const void* wq, int64_t ld_wq, const float* sw, const void* bias,
+                        void* out, int64_t ld_out,
+                        int64_t m, int64_t n, int64_t k,
+                        void* workspace, int64_t workspace_bytes, int kernel, daxq_stream_t stream);
+/* The three pairings of the bf16 DiT by name (bf16 x, bias and out; rows_alloc = m; no workspace; the library's kernel):
+ * int8 x int8 (dax/quant/nn/dynamic/linear.py:181-228), e4m3fn x e4m3fn and e5m2 x e4m3fn (:146-178). */
+int daxq_dynamic_linear_i8(const void* x, int64_t ld_x, int8_t* xq, int64_t ld_xq, float* sx,
+                           const int8_t* wq, int64_t ld_wq, const float* sw, const void* bias,
+                           void* out, int64_t ld_out, int64_t m, int64_t n, int64_t k, daxq_stream_t stream);
+int daxq_dynamic_linear_e4m3(const void* x, int64_t ld_x, uint8_t* xq, int64_t ld_xq, float* sx,
+                             const uint8_t* wq, int64_t ld_wq, const float* sw, const void* bias,
+                             void* out, int64_t ld_out, int64_t m, int64_t n, int64_t k, daxq_stream_t stream);
+int daxq_dynamic_linear_e5m2_e4m3(const void* x, int64_t ld_x, uint8_t* xq, int64_t ld_xq, float* sx,
+                                  const uint8_t* wq, int64_t ld_wq, const float* sw, const void* bias,
+                                  void* out, int64_t ld_out, int64_t m, int64_t n, int64_t k, daxq_stream_t stream);
+
 /* The tile order daxq_linear_w8a8 takes for a launch of 256x256 tiles when bits 24-27 of `kernel` are 0, as the value
  * of those bits: 1 = groups of tile rows, 5 = banded patches 4 tile columns wide (large launches: K >= 2048,
  * N >= 5120, M >= 7937 and no XCD more than 5 % over its share of the tiles).  For tests and diagnostics; no
@@ -300,8 +338,9 @@ int daxq_linear_tile_order_choice(int64_t m, int64_t n, int64_t k);
  *              divide by it; needs m, n >= 128.
  *   workspace  device memory, 256-byte aligned, at least daxq_linear_splitk_workspace_bytes(m, n, splits) bytes.
  *              Its first 16 KiB are tile counters (at most 4096 output tiles of 128x128): they must be ZERO when
- *              the call is made and every call leaves them zero, so a workspace is cleared once (hipMemsetAsync of
- *              those 16 KiB) and then reused for any shapes.  Calls that share a workspace must not overlap in time.
+ *              the call is made and every call leaves them zero, so a workspace is cleared once (a hipMemset of those
+ *              16 KiB, or a small clear kernel; not a hipMemsetAsync inside a captured graph) and then reused for any
+ *              shapes.  Calls that share a workspace must not overlap in time.
  */
 int daxq_linear_splitk_choice(int64_t m, int64_t n, int64_t k);
 int64_t daxq_linear_splitk_workspace_bytes(int64_t m, int64_t n, int splits);

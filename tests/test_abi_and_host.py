@@ -27,7 +27,7 @@ def test_library_exports_every_declared_symbol():
     for name in declared:
         assert hasattr(lib, name), f"{name} declared in include/daxq.h but not exported"
     assert set(declared) == set(_capi.SIGNATURES), "binding table and header disagree"
-    assert _capi.lib().daxq_abi_version() == _capi.ABI_VERSION == 4
+    assert _capi.lib().daxq_abi_version() == _capi.ABI_VERSION == 5
     assert "undefined symbol" not in _capi.last_error()
 
 

@@ -171,6 +171,61 @@ def test_captured_graph_replays_match_eager(fp8):
         assert _same(static_out, eager), f"replay with seed {seed} differs from eager"
 
 
+def test_split_k_shape_captured_on_a_stream_that_already_has_a_workspace():
+    """M = 256, N = K = 5120: eagerly this INT8 launch cuts K into ranges and goes through a workspace that belongs
+    to the stream.  A capture on that stream must not record the workspace's address (a graph may replay beside another
+    one, or after a larger eager request has replaced the workspace): under capture the plain launch runs, whose INT8
+    results are the same bits.  The workspace is then outgrown eagerly, and every replay still equals eager."""
+    import dax_amd.ops as ops
+    from oracle import daxq_oracle as O
+
+    m, n, k = 256, 5120, 5120
+    assert ops._capi.lib().daxq_linear_splitk_choice(m, n, k) > 1
+    x, w, b = O.make_inputs(m, k, n, seed=77)
+    dev = torch.device("cuda")
+    wd, bd = w.to(dev), b.to(dev)
+    lo, hi = ops.row_minmax(wd)
+    sw = ops.scale_from_minmax(lo, hi, 127.0)
+    qw = ops.quantize_rows_i8(wd, sw, True)
+
+    def run(xd):
+        return ops.dynamic_linear_i8(xd, qw, sw, bd)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    static_x = x.to(dev)
+    with torch.cuda.stream(side):
+        eager0 = run(static_x)          # split-K: this stream now owns a workspace
+        side.synchronize()
+        key = (dev.index if dev.index is not None else torch.cuda.current_device(), side.cuda_stream)
+        assert key in ops._splitk_ws
+        ws_before = ops._splitk_ws[key]
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            static_out = run(static_x)
+        # an explicit request for more ranges than the first workspace holds replaces it; the old one stays alive
+        big_m = 1024
+        xb, _, _ = O.make_inputs(big_m, k, n, seed=78)
+        xq, sx = ops.act_quant_i8(xb.to(dev))
+        need = ops._capi.lib().daxq_linear_splitk_workspace_bytes(big_m, n, 4)
+        assert need > ws_before.numel()
+        big = ops.linear_w8a8_splitk(xq, sx, qw, sw, bd, "i8", "i8", 4)
+        side.synchronize()
+        assert ops._splitk_ws[key] is not ws_before and any(t is ws_before for t in ops._splitk_retired)
+        assert _same(big, ops.linear_i8(xq, sx, qw, sw, bd))
+    torch.cuda.synchronize()
+    ref = O.linear_int8(x, *O.weight_quant_int8(w), b)["out"]
+    assert _same(eager0, ref)
+    for seed in (79, 80, 81):
+        x2, _, _ = O.make_inputs(m, k, n, seed=seed)
+        want = run(x2.to(dev))
+        torch.cuda.synchronize()
+        static_x.copy_(x2.to(dev))
+        graph.replay()
+        torch.cuda.synchronize()
+        assert _same(static_out, want), f"replay with seed {seed} differs from eager"
+
+
 @pytest.mark.parametrize("m,n,k,order,tail", [(700, 2304, 1024, 2005, 3000), (4100, 4352, 256, 2001, 3002)])
 @pytest.mark.parametrize("fp8", [False, True])
 def test_captured_graph_of_the_256_tile_kernels_replays_match_eager(fp8, m, n, k, order, tail):
