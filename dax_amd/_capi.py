@@ -37,16 +37,18 @@ SIGNATURES = {
     "daxq_quantize_rows_i8": [_P, _I64, _I64, _I64, _P, _P, _I64, _P],
     "daxq_quantize_rows_e4m3": [_P, _I64, _I64, _I64, _P, _P, _I64, _P],
     "daxq_quantize_rows_e5m2": [_P, _I64, _I64, _I64, _P, _P, _I64, _P],
-    "daxq_tensor_scale": [_P, _P, _I64, _F32, _INT, _P, _P, _I64, _P],
+    "daxq_tensor_scale": [_P, _P, _I64, _F32, _F32, _INT, _P, _P, _I64, _P],
     "daxq_tensor_minmax_update": [_P, _P, _I64, _P, _P, _P],
     "daxq_broadcast_f32": [_P, _P, _I64, _P],
     "daxq_row_minmax": [_P, _I64, _I64, _I64, _P, _P, _P],
     "daxq_row_minmax_t": [_P, _INT, _I64, _I64, _I64, _P, _P, _P],
     "daxq_act_quant_rows": [_P, _INT, _INT, _I64, _I64, _I64, _P, _I64, _P, _P],
+    "daxq_act_quant_rows_ex": [_P, _INT, _INT, _I64, _I64, _I64, _P, _I64, _P, _F32, _F32, _INT, _P],
     "daxq_quantize_rows": [_P, _INT, _INT, _I64, _I64, _I64, _P, _P, _I64, _P],
-    "daxq_block_scale": [_P, _INT, _INT, C.POINTER(_I64), C.POINTER(C.c_int32), _F32, _INT, _P, _P],
-    "daxq_block_quantize": [_P, _INT, _INT, _INT, C.POINTER(_I64), C.POINTER(C.c_int32), _P, _P, _P],
+    "daxq_block_scale": [_P, _INT, _INT, C.POINTER(_I64), C.POINTER(C.c_int32), _F32, _F32, _INT, _P, _P],
+    "daxq_block_quantize": [_P, _INT, _INT, _INT, C.POINTER(_I64), C.POINTER(C.c_int32), _P, _INT, _P, _P],
     "daxq_scale_from_minmax": [_P, _P, _I64, _F32, _P, _P],
+    "daxq_scale_from_minmax_eps": [_P, _P, _I64, _F32, _F32, _P, _P],
     "daxq_linear_i8": [_P, _I64, _P, _P, _I64, _P, _P, _P, _I64, _P, _I64, _I64, _I64, _I64, _P],
     "daxq_linear_e4m3": [_P, _I64, _P, _P, _I64, _P, _P, _P, _I64, _P, _I64, _I64, _I64, _I64, _P],
     "daxq_linear_e5m2_e4m3": [_P, _I64, _P, _P, _I64, _P, _P, _P, _I64, _P, _I64, _I64, _I64, _I64, _P],
@@ -56,7 +58,7 @@ SIGNATURES = {
     "daxq_linear_w8a8_splitk": [_INT, _INT, _P, _I64, _P, _P, _I64, _P, _P, _P, _I64, _I64, _I64, _I64, _INT, _P, _I64, _P],
     "daxq_linear_w8a8_splitk_static": [_INT, _INT, _P, _I64, _P, _P, _I64, _P, _P, _P, _I64, _I64, _I64, _I64, _INT, _P],
     "daxq_linear_w8a8": [_INT, _INT, _INT, _P, _I64, _P, _P, _I64, _P, _P, _P, _I64, _P, _I64, _I64, _I64, _I64, _INT, _P],
-    "daxq_dynamic_linear": [_INT, _INT, _INT, _INT, _P, _I64, _P, _I64, _P, _I64, _P, _I64, _P, _P, _P, _I64, _I64, _I64, _I64,
+    "daxq_dynamic_linear": [_INT, _INT, _INT, _INT, _INT, _P, _I64, _P, _I64, _P, _I64, _P, _I64, _P, _P, _P, _I64, _I64, _I64, _I64,
                             _P, _I64, _INT, _P],
     "daxq_dynamic_linear_i8": [_P, _I64, _P, _I64, _P, _P, _I64, _P, _P, _P, _I64, _I64, _I64, _I64, _P],
     "daxq_dynamic_linear_e4m3": [_P, _I64, _P, _I64, _P, _P, _I64, _P, _P, _P, _I64, _I64, _I64, _I64, _P],

@@ -113,7 +113,8 @@ def fuse_linears(linears: Sequence[Linear]) -> Linear:
     first = linears[0]
     for lin in linears:
         if (not isinstance(lin, Linear) or lin.in_features != first.in_features or lin.input_dtype != first.input_dtype
-                or lin.weight_dtype != first.weight_dtype or (lin.bias is None) != (first.bias is None)):
+                or lin.weight_dtype != first.weight_dtype or (lin.bias is None) != (first.bias is None)
+                or lin.act_scale_fp32 != first.act_scale_fp32):
             raise ValueError("fuse_linears needs quantised linears of one kind reading the same input")
     n = sum(lin.out_features for lin in linears)
     fused = Linear(first.in_features, n, first.bias is not None, first.qweight.device, first.weight_dtype,
@@ -122,6 +123,9 @@ def fuse_linears(linears: Sequence[Linear]) -> Linear:
     fused.weight_scale = torch.cat([lin.weight_scale for lin in linears], 1)
     if first.bias is not None:
         fused.bias = nn.Parameter(torch.cat([lin.bias.detach() for lin in linears], 0), requires_grad=False)
+    if first.act_scale_fp32:
+        fused.act_scale_fp32 = True
+    fused.refresh_derived()
     return fused
 
 
@@ -190,6 +194,8 @@ def _block_is_fusable(block) -> bool:
         return False
     lins = [getattr(a1, n, None) for n in ("to_q", "to_k", "to_v")] + [getattr(a2, n, None) for n in ("to_q", "to_k", "to_v")]
     if not all(isinstance(l, Linear) for l in lins):
+        return False
+    if any(l.act_scale_fp32 for l in lins):  # the fused producer kernels round the scale as the eager chain does
         return False
     net = getattr(ffn, "net", None)
     first = getattr(net[0], "proj", None) if net is not None and len(net) else None

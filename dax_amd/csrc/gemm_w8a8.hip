@@ -608,7 +608,7 @@ int daxq_linear_w8a8(int x_fmt, int w_fmt, int out_dtype, const void* xq, int64_
 }
 
 // ---- quantiser + GEMM behind one entry point --------------------------------------------------------------------
-int daxq_dynamic_linear(int x_dtype, int x_fmt, int w_fmt, int out_dtype, const void* x, int64_t ld_x, void* xq,
+int daxq_dynamic_linear(int x_dtype, int x_fmt, int w_fmt, int out_dtype, int act_scale_round, const void* x, int64_t ld_x, void* xq,
                         int64_t ld_xq, float* sx, int64_t rows_alloc, const void* wq, int64_t ld_wq, const float* sw,
                         const void* bias, void* out, int64_t ld_out, int64_t m, int64_t n, int64_t k, void* workspace,
                         int64_t workspace_bytes, int kernel, daxq_stream_t stream) {
@@ -625,7 +625,8 @@ int daxq_dynamic_linear(int x_dtype, int x_fmt, int w_fmt, int out_dtype, const 
                     (long long)ld_wq, DAXQ_K_ALIGN, (long long)kp);
     if (m == 0 || n == 0) return DAXQ_OK;
     // the quantiser zero-fills columns [k, kp) of the rows it writes
-    if (int rc = daxq_act_quant_rows(x, x_dtype, x_fmt, m, k, ld_x, xq, ld_xq, sx, stream)) return rc;
+    const float qmax = x_fmt == DAXQ_FMT_I8 ? 127.0f : x_fmt == DAXQ_FMT_E4M3 ? 448.0f : 57344.0f;
+    if (int rc = daxq_act_quant_rows_ex(x, x_dtype, x_fmt, m, k, ld_x, xq, ld_xq, sx, qmax, kEps, act_scale_round, stream)) return rc;
     // Fewer rows than the smallest tile of the tiled kernels: run them on 128 rows of the caller's buffers when those
     // reach that far (the rows beyond m hold whatever the buffers held; an output row depends on its own operand row only).
     const int64_t mg = (m < 128 && rows_alloc >= 128 && n >= 128) ? 128 : m;
@@ -645,21 +646,21 @@ int daxq_dynamic_linear(int x_dtype, int x_fmt, int w_fmt, int out_dtype, const 
 int daxq_dynamic_linear_i8(const void* x, int64_t ld_x, int8_t* xq, int64_t ld_xq, float* sx, const int8_t* wq,
                            int64_t ld_wq, const float* sw, const void* bias, void* out, int64_t ld_out, int64_t m,
                            int64_t n, int64_t k, daxq_stream_t stream) {
-    return daxq_dynamic_linear(DAXQ_BF16, DAXQ_FMT_I8, DAXQ_FMT_I8, DAXQ_BF16, x, ld_x, xq, ld_xq, sx, m, wq, ld_wq, sw, bias, out,
+    return daxq_dynamic_linear(DAXQ_BF16, DAXQ_FMT_I8, DAXQ_FMT_I8, DAXQ_BF16, DAXQ_SCALE_ROUND_X, x, ld_x, xq, ld_xq, sx, m, wq, ld_wq, sw, bias, out,
                                ld_out, m, n, k, nullptr, 0, 0, stream);
 }
 
 int daxq_dynamic_linear_e4m3(const void* x, int64_t ld_x, uint8_t* xq, int64_t ld_xq, float* sx, const uint8_t* wq,
                              int64_t ld_wq, const float* sw, const void* bias, void* out, int64_t ld_out, int64_t m,
                              int64_t n, int64_t k, daxq_stream_t stream) {
-    return daxq_dynamic_linear(DAXQ_BF16, DAXQ_FMT_E4M3, DAXQ_FMT_E4M3, DAXQ_BF16, x, ld_x, xq, ld_xq, sx, m, wq, ld_wq, sw, bias,
+    return daxq_dynamic_linear(DAXQ_BF16, DAXQ_FMT_E4M3, DAXQ_FMT_E4M3, DAXQ_BF16, DAXQ_SCALE_ROUND_X, x, ld_x, xq, ld_xq, sx, m, wq, ld_wq, sw, bias,
                                out, ld_out, m, n, k, nullptr, 0, 0, stream);
 }
 
 int daxq_dynamic_linear_e5m2_e4m3(const void* x, int64_t ld_x, uint8_t* xq, int64_t ld_xq, float* sx, const uint8_t* wq,
                                   int64_t ld_wq, const float* sw, const void* bias, void* out, int64_t ld_out, int64_t m,
                                   int64_t n, int64_t k, daxq_stream_t stream) {
-    return daxq_dynamic_linear(DAXQ_BF16, DAXQ_FMT_E5M2, DAXQ_FMT_E4M3, DAXQ_BF16, x, ld_x, xq, ld_xq, sx, m, wq, ld_wq, sw, bias,
+    return daxq_dynamic_linear(DAXQ_BF16, DAXQ_FMT_E5M2, DAXQ_FMT_E4M3, DAXQ_BF16, DAXQ_SCALE_ROUND_X, x, ld_x, xq, ld_xq, sx, m, wq, ld_wq, sw, bias,
                                out, ld_out, m, n, k, nullptr, 0, 0, stream);
 }
 

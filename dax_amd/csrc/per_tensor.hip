@@ -38,7 +38,7 @@ __device__ __forceinline__ void block_minmax(float& lo, float& hi, float* s_lo, 
 }
 
 __global__ __launch_bounds__(kRedThreads) void tensor_scale_kernel(const float* __restrict__ mn, const float* __restrict__ mx,
-                                                                   int64_t m, float qmax, int round_bf16,
+                                                                   int64_t m, float qmax, float eps, int round_bf16,
                                                                    float* __restrict__ scale1, float* __restrict__ expand,
                                                                    int64_t n_expand) {
     __shared__ float s_lo[kRedThreads / 64], s_hi[kRedThreads / 64];
@@ -50,9 +50,14 @@ __global__ __launch_bounds__(kRedThreads) void tensor_scale_kernel(const float* 
     block_minmax(lo, hi, s_lo, s_hi);
     const float amax = max_nan(-lo, hi);  // = max |x|: exact, the statistics are the tensor's own values
     float s = amax / qmax;              // IEEE division
-    if (round_bf16 == 1) s = round_to_x<DAXQ_BF16>(s);  // the quotient is rounded to the tensor's own element type
-    else if (round_bf16 == 2) s = round_to_x<DAXQ_F16>(s);
-    s = max_nan(s, kEps);
+    if (round_bf16 == 1) {  // quotient and floor are rounded to the tensor's own element type
+        s = round_to_x<DAXQ_BF16>(s);
+        eps = round_to_x<DAXQ_BF16>(eps);
+    } else if (round_bf16 == 2) {
+        s = round_to_x<DAXQ_F16>(s);
+        eps = round_to_x<DAXQ_F16>(eps);
+    }
+    s = max_nan(s, eps);
     if (threadIdx.x == 0) scale1[0] = s;
     for (int64_t i = threadIdx.x; i < n_expand; i += kRedThreads) expand[i] = s;
 }
@@ -82,13 +87,13 @@ __global__ void broadcast_f32_kernel(const float* __restrict__ src, float* __res
 
 extern "C" {
 
-int daxq_tensor_scale(const float* row_min, const float* row_max, int64_t m, float qmax, int round_bf16, float* scale1,
-                      float* expand, int64_t n_expand, daxq_stream_t stream) {
+int daxq_tensor_scale(const float* row_min, const float* row_max, int64_t m, float qmax, float eps, int round_bf16,
+                      float* scale1, float* expand, int64_t n_expand, daxq_stream_t stream) {
     using namespace daxq;
-    if (m <= 0 || n_expand < 0 || !(qmax > 0.0f)) return fail(DAXQ_ERR_ARG, "tensor_scale: bad argument m=%lld n_expand=%lld", (long long)m, (long long)n_expand);
+    if (m <= 0 || n_expand < 0 || !(qmax > 0.0f) || !(eps >= 0.0f)) return fail(DAXQ_ERR_ARG, "tensor_scale: bad argument m=%lld n_expand=%lld", (long long)m, (long long)n_expand);
     if (!row_min || !row_max || !scale1 || (n_expand > 0 && !expand)) return fail(DAXQ_ERR_ARG, "tensor_scale: null pointer");
     hipLaunchKernelGGL(tensor_scale_kernel, dim3(1), dim3(kRedThreads), 0, (hipStream_t)stream, row_min, row_max, m, qmax,
-                       round_bf16, scale1, expand, n_expand);
+                       eps, round_bf16, scale1, expand, n_expand);
     return check_launch("tensor_scale");
 }
 

@@ -47,7 +47,7 @@ __device__ __forceinline__ int64_t offset_of(const BlockView& v, int64_t idx, in
 
 template <int XT, bool ROUND>
 __global__ __launch_bounds__(256) void block_scale_kernel(const void* __restrict__ xv, const BlockView v, int64_t n_red,
-                                                          float qmax, float* __restrict__ scale) {
+                                                          float qmax, float eps, float* __restrict__ scale) {
     typedef typename XW<XT>::type word_t;
     constexpr uint32_t kAbs = XT == DAXQ_F32 ? 0x7fffffffu : 0x7fffu;
     __shared__ uint32_t red[4];
@@ -65,13 +65,25 @@ __global__ __launch_bounds__(256) void block_scale_kernel(const void* __restrict
         amax = red[1] > amax ? red[1] : amax;
         amax = red[2] > amax ? red[2] : amax;
         amax = red[3] > amax ? red[3] : amax;
-        scale[blockIdx.x] = scale_from_amax_bits<ROUND, XT>(amax, qmax);
+        scale[blockIdx.x] = scale_from_amax_bits_rt<XT>(amax, qmax, eps, ROUND ? 1 : 0);
     }
 }
 
+// f32 rounded to the arithmetic type CT of the leaf quantiser (DAXQ_F32: no rounding)
+__device__ __forceinline__ float round_ct(float v, int ct) {
+    if (ct == DAXQ_BF16) return round_to_x<DAXQ_BF16>(v);
+    if (ct == DAXQ_F16) return round_to_x<DAXQ_F16>(v);
+    return v;
+}
+
+// st / ct: the element type of the scale the caller asked for, and the type torch's type promotion makes of (x, scale).
+// The reference's wrappers always ask for an fp32 scale, and then everything below is fp32.  With a scale of a 16-bit
+// type (dax/quant/nn/dynamic/functional.py:128-129) the leaf quantisers (dax/quant/nn/quantized/functional.py:11-20)
+// round 1.0 / scale to the scale's type, and x * inv and x / scale to the promoted type: bf16 x with a bf16 scale
+// computes in bf16, bf16 x with an fp16 scale in fp32 (but with the reciprocal rounded to fp16).
 template <int XT, int FMT>
 __global__ __launch_bounds__(256) void block_quantize_kernel(const void* __restrict__ xv, const BlockView v, int64_t total,
-                                                             const float* __restrict__ scale, uint8_t* __restrict__ q) {
+                                                             const float* __restrict__ scale, uint8_t* __restrict__ q, int st, int ct) {
     typedef typename XW<XT>::type word_t;
     const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (i >= total) return;
@@ -88,9 +100,24 @@ __global__ __launch_bounds__(256) void block_quantize_kernel(const void* __restr
     const float s = scale[blk];
     const float f = x_bits_to_f32<XT>(static_cast<const word_t*>(xv)[i]);
     if constexpr (FMT == 0) {
-        q[i] = (uint8_t)(q_i8_bits(f, 1.0f / s) & 0xffu);
+        if (ct == DAXQ_F32 && st == DAXQ_F32) {
+            q[i] = (uint8_t)(q_i8_bits(f, 1.0f / s) & 0xffu);
+        } else {
+            const float inv = round_ct(1.0f / s, st);
+            float r = round_ct(f * inv, ct);  // (the product of two 16-bit floats is exact in fp32: one rounding)
+            r = rintf(r);                     // an integer below 2^8 (bf16) or 2^11 (fp16) in magnitude is exact in that type; larger ones clamp
+            r = min_nan(max_nan(r, -128.0f), 127.0f);
+            q[i] = (uint8_t)(int8_t)(r != r ? 0.0f : r);
+        }
     } else {
-        q[i] = (uint8_t)(cvt_pk_f8<FMT>(q_f8_pre<FMT, true>(f, s, 0.0f), 0.0f, 0, false) & 0xff);
+        if (ct == DAXQ_F32) {
+            q[i] = (uint8_t)(cvt_pk_f8<FMT>(q_f8_pre<FMT, true>(f, s, 0.0f), 0.0f, 0, false) & 0xff);
+        } else {
+            constexpr float kMax = FMT == 2 ? 57344.0f : 448.0f;
+            float r = round_ct(f / s, ct);
+            r = min_nan(max_nan(r, -kMax), kMax);
+            q[i] = (uint8_t)(cvt_pk_f8<FMT>(r, 0.0f, 0, false) & 0xff);
+        }
     }
 }
 
@@ -121,20 +148,20 @@ static int64_t make_view(BlockView& v, int nd, const int64_t* view_shape, const 
 extern "C" {
 
 int daxq_block_scale(const void* x, int x_dtype, int nd, const int64_t* view_shape, const int32_t* reduced, float qmax,
-                     int round_to_x, float* scale, daxq_stream_t stream) {
+                     float eps, int round_to_x, float* scale, daxq_stream_t stream) {
     using namespace daxq;
     BlockView v;
     int64_t n_kept, n_red;
     const int64_t total = make_view(v, nd, view_shape, reduced, n_kept, n_red);
-    if (total < 0 || !(qmax > 0.0f)) return fail(DAXQ_ERR_ARG, "block_scale: bad view (1 to %d positive dimensions)", kMaxDims);
+    if (total < 0 || !(qmax > 0.0f) || !(eps >= 0.0f)) return fail(DAXQ_ERR_ARG, "block_scale: bad view (1 to %d positive dimensions), quant_max or eps", kMaxDims);
     if (total == 0) return DAXQ_OK;
     if (!x || !scale) return fail(DAXQ_ERR_ARG, "block_scale: null pointer");
     if (n_kept > 0x7fffffff) return fail(DAXQ_ERR_ARG, "block_scale: too many blocks");
     const dim3 grid((unsigned)n_kept), block(256);
     hipStream_t st = (hipStream_t)stream;
 #define DAXQ_BS(XT)                                                                                             \
-    if (round_to_x) hipLaunchKernelGGL((block_scale_kernel<XT, true>), grid, block, 0, st, x, v, n_red, qmax, scale); \
-    else hipLaunchKernelGGL((block_scale_kernel<XT, false>), grid, block, 0, st, x, v, n_red, qmax, scale)
+    if (round_to_x) hipLaunchKernelGGL((block_scale_kernel<XT, true>), grid, block, 0, st, x, v, n_red, qmax, eps, scale); \
+    else hipLaunchKernelGGL((block_scale_kernel<XT, false>), grid, block, 0, st, x, v, n_red, qmax, eps, scale)
     switch (x_dtype) {
         case DAXQ_BF16: DAXQ_BS(DAXQ_BF16); break;
         case DAXQ_F16: DAXQ_BS(DAXQ_F16); break;
@@ -146,7 +173,7 @@ int daxq_block_scale(const void* x, int x_dtype, int nd, const int64_t* view_sha
 }
 
 int daxq_block_quantize(const void* x, int x_dtype, int q_fmt, int nd, const int64_t* view_shape, const int32_t* reduced,
-                        const float* scale, void* q, daxq_stream_t stream) {
+                        const float* scale, int scale_dtype, void* q, daxq_stream_t stream) {
     using namespace daxq;
     BlockView v;
     int64_t n_kept, n_red;
@@ -154,15 +181,19 @@ int daxq_block_quantize(const void* x, int x_dtype, int q_fmt, int nd, const int
     if (total < 0) return fail(DAXQ_ERR_ARG, "block_quantize: bad view (1 to %d positive dimensions)", kMaxDims);
     if (total == 0) return DAXQ_OK;
     if (!x || !scale || !q) return fail(DAXQ_ERR_ARG, "block_quantize: null pointer");
+    if (scale_dtype != DAXQ_F32 && scale_dtype != DAXQ_BF16 && scale_dtype != DAXQ_F16)
+        return fail(DAXQ_ERR_ARG, "block_quantize: unknown scale type %d", scale_dtype);
+    // type promotion of (x, scale): the same 16-bit type on both sides stays, anything else is fp32
+    const int sk = scale_dtype, ct = (x_dtype == scale_dtype) ? x_dtype : DAXQ_F32;
     if ((total + 255) / 256 > 0x7fffffff) return fail(DAXQ_ERR_ARG, "block_quantize: tensor too large");
     const dim3 grid((unsigned)((total + 255) / 256)), block(256);
     hipStream_t st = (hipStream_t)stream;
     uint8_t* qp = static_cast<uint8_t*>(q);
 #define DAXQ_BQ(XT)                                                                                                   \
     switch (q_fmt) {                                                                                                  \
-        case DAXQ_FMT_I8: hipLaunchKernelGGL((block_quantize_kernel<XT, 0>), grid, block, 0, st, x, v, total, scale, qp); break;   \
-        case DAXQ_FMT_E4M3: hipLaunchKernelGGL((block_quantize_kernel<XT, 1>), grid, block, 0, st, x, v, total, scale, qp); break; \
-        case DAXQ_FMT_E5M2: hipLaunchKernelGGL((block_quantize_kernel<XT, 2>), grid, block, 0, st, x, v, total, scale, qp); break; \
+        case DAXQ_FMT_I8: hipLaunchKernelGGL((block_quantize_kernel<XT, 0>), grid, block, 0, st, x, v, total, scale, qp, sk, ct); break;   \
+        case DAXQ_FMT_E4M3: hipLaunchKernelGGL((block_quantize_kernel<XT, 1>), grid, block, 0, st, x, v, total, scale, qp, sk, ct); break; \
+        case DAXQ_FMT_E5M2: hipLaunchKernelGGL((block_quantize_kernel<XT, 2>), grid, block, 0, st, x, v, total, scale, qp, sk, ct); break; \
         default: return fail(DAXQ_ERR_ARG, "block_quantize: unknown quantised format %d", q_fmt);                    \
     }
     switch (x_dtype) {

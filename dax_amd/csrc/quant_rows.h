@@ -57,6 +57,22 @@ __device__ __forceinline__ float scale_from_amax_bits(uint32_t amax_bits, float 
     return max_nan(s, kEps);  // clamp(min=eps): a NaN abs-max (a NaN anywhere in the row) stays NaN
 }
 
+// The same rule with the caller's floor and the rounding chosen at run time (uniform over the launch):
+// round_x != 0   the eager chain: quotient and floor live in the tensor's own element type, so both are rounded to it
+//                (clamp(min=eps) on a bf16 tensor compares with eps rounded to bf16)
+// round_x == 0   quotient and floor stay in fp32: what a code generator that fuses the chain leaves of it
+//                (the reference's forward carries a torch.compile decorator, dax/quant/nn/dynamic/linear.py:143)
+template <int XT>
+__device__ __forceinline__ float scale_from_amax_bits_rt(uint32_t amax_bits, float qmax, float eps, int round_x) {
+    float a = x_bits_to_f32<XT>(amax_bits);
+    float s = a / qmax;
+    if (round_x) {
+        s = round_to_x<XT>(s);
+        eps = round_to_x<XT>(eps);
+    }
+    return max_nan(s, eps);
+}
+
 // Wavefront-wide reductions with DPP (data-parallel primitives: the partner lane's value is an operand
 // modifier of the VALU instruction, no trip through the LDS crossbar as with ds_bpermute): four steps
 // give every lane the result of its row of 16 lanes, the four row results are then read as scalars.

@@ -26,7 +26,7 @@ namespace daxq {
 template <int NCH, int FMT, bool ROUND_BF16, bool SCALE_IN, int XT = DAXQ_BF16>
 __global__ __launch_bounds__(256) void quant_rows_wave(const uint16_t* __restrict__ x, int64_t m, int k,
                                                        int64_t ld_x, uint8_t* __restrict__ q, int64_t ld_q, int kfill,
-                                                       float* __restrict__ scale, float qmax) {
+                                                       float* __restrict__ scale, float qmax, float eps, int round_x) {
     const int lane = threadIdx.x & 63;
     const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (row >= m) return;
@@ -58,17 +58,28 @@ __global__ __launch_bounds__(256) void quant_rows_wave(const uint16_t* __restric
         }
         uint32_t amax = (mx & 0xffffu) > (mx >> 16) ? (mx & 0xffffu) : (mx >> 16);
         amax = wave_max_u32(amax);
-        s = scale_from_amax_bits<ROUND_BF16, XT>(amax, qmax);
+        s = scale_from_amax_bits_rt<XT>(amax, qmax, eps, round_x);
         if (lane == 0) scale[row] = s;
     }
     const float inv = 1.0f / s;  // IEEE division, not v_rcp_f32
 
     uint2* qr = reinterpret_cast<uint2*>(q + row * ld_q);
+    // The reciprocal sequence of the FP8 forms is verified exhaustively for bf16 elements under bf16-rounded scales:
+    // fp16 rows, and bf16 rows whose scale stays in fp32 (round_x == 0, uniform over the launch), divide.
+    constexpr bool kRecip = FMT != 0 && !SCALE_IN && XT == DAXQ_BF16;
+    if (kRecip && !round_x) {
+#pragma unroll
+        for (int i = 0; i < NCH; ++i) {
+            const int c = i * 64 + lane;
+            if (c < nch) store_stream_8(qr + c, quant_chunk<FMT, true, XT>(v[i], s, inv));
+            else if (c < npad) store_stream_8(qr + c, make_uint2(0, 0));
+        }
+        return;
+    }
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
         const int c = i * 64 + lane;
         if (c < nch) {
-            // the reciprocal sequence of the FP8 forms is verified exhaustively for bf16 elements; fp16 rows divide
             store_stream_8(qr + c, quant_chunk<FMT, SCALE_IN || XT != DAXQ_BF16, XT>(v[i], s, inv));
         } else if (c < npad) {
             store_stream_8(qr + c, make_uint2(0, 0));
@@ -89,7 +100,7 @@ struct XWord<DAXQ_F32> {
 template <int FMT, bool ROUND_BF16, bool SCALE_IN, int XT = DAXQ_BF16>
 __global__ __launch_bounds__(256) void quant_rows_block(const void* __restrict__ xv, int64_t m, int64_t k,
                                                         int64_t ld_x, uint8_t* __restrict__ q, int64_t ld_q, int64_t kfill,
-                                                        float* __restrict__ scale, float qmax) {
+                                                        float* __restrict__ scale, float qmax, float eps, int round_x) {
     typedef typename XWord<XT>::type word_t;
     constexpr uint32_t kAbs = XT == DAXQ_F32 ? 0x7fffffffu : 0x7fffu;
     __shared__ uint32_t red[4];
@@ -111,7 +122,7 @@ __global__ __launch_bounds__(256) void quant_rows_block(const void* __restrict__
         amax = red[1] > amax ? red[1] : amax;
         amax = red[2] > amax ? red[2] : amax;
         amax = red[3] > amax ? red[3] : amax;
-        s = scale_from_amax_bits<ROUND_BF16, XT>(amax, qmax);
+        s = scale_from_amax_bits_rt<XT>(amax, qmax, eps, round_x);
         if (threadIdx.x == 0) scale[row] = s;
     }
     const float inv = 1.0f / s;
@@ -122,7 +133,9 @@ __global__ __launch_bounds__(256) void quant_rows_block(const void* __restrict__
             float f = x_bits_to_f32<XT>(xr[c]);
             if (FMT != 0) {
                 // the reciprocal sequence is verified exhaustively for bf16 elements only; other types divide
-                o = (uint8_t)(cvt_pk_f8<FMT>(q_f8_pre<FMT, SCALE_IN || XT != DAXQ_BF16>(f, s, inv), 0.0f, 0, false) & 0xff);
+                const float pre = (SCALE_IN || XT != DAXQ_BF16 || round_x) ? q_f8_pre<FMT, SCALE_IN || XT != DAXQ_BF16>(f, s, inv)
+                                                                           : q_f8_pre<FMT, true>(f, s, inv);
+                o = (uint8_t)(cvt_pk_f8<FMT>(pre, 0.0f, 0, false) & 0xff);
             } else {
                 o = (uint8_t)(q_i8_bits(f, inv) & 0xffu);
             }
@@ -133,7 +146,7 @@ __global__ __launch_bounds__(256) void quant_rows_block(const void* __restrict__
 
 template <int FMT, bool ROUND_BF16, bool SCALE_IN, int XT>
 static int launch_quant_rows_t(const void* x, int64_t m, int64_t k, int64_t ld_x, void* q, int64_t ld_q, float* scale,
-                               float qmax, hipStream_t st) {
+                               float qmax, hipStream_t st, float eps, int round_x) {
     constexpr int XB = XT == DAXQ_F32 ? 4 : 2;
     if (m < 0 || k <= 0 || ld_x < k || ld_q < k) return fail(DAXQ_ERR_ARG, "quant_rows: bad shape m=%lld k=%lld ld_x=%lld ld_q=%lld",
                                                                (long long)m, (long long)k, (long long)ld_x, (long long)ld_q);
@@ -152,7 +165,7 @@ static int launch_quant_rows_t(const void* x, int64_t m, int64_t k, int64_t ld_x
 #define DAXQ_Q_CASE(N)                                                                                      \
     if (nchunks <= N) {                                                                                     \
         hipLaunchKernelGGL((quant_rows_wave<N, FMT, ROUND_BF16, SCALE_IN, XT>), grid, block, 0, st, xp, m, (int)k, ld_x, qp, \
-                           ld_q, (int)kfill, scale, qmax);                                                            \
+                           ld_q, (int)kfill, scale, qmax, eps, round_x);                                              \
         return check_launch("quant_rows_wave");                                                             \
     }
             DAXQ_Q_CASE(2)
@@ -167,28 +180,31 @@ static int launch_quant_rows_t(const void* x, int64_t m, int64_t k, int64_t ld_x
     }
     if (m > 0x7fffffff) return fail(DAXQ_ERR_ARG, "quant_rows: too many rows for the general kernel");
     hipLaunchKernelGGL((quant_rows_block<FMT, ROUND_BF16, SCALE_IN, XT>), dim3((unsigned)m), dim3(256), 0, st, x, m, k, ld_x, qp,
-                       ld_q, kfill, scale, qmax);
+                       ld_q, kfill, scale, qmax, eps, round_x);
     return check_launch("quant_rows_block");
 }
 
+// eps, round_x: floor and rounding of a dynamic scale (scale_from_amax_bits_rt); unused when the scale is an input
 template <int FMT, bool ROUND_BF16, bool SCALE_IN>
 static int launch_quant_rows(const void* x, int64_t m, int64_t k, int64_t ld_x, void* q, int64_t ld_q, float* scale,
-                             float qmax, hipStream_t st, int x_dtype = DAXQ_BF16) {
+                             float qmax, hipStream_t st, int x_dtype = DAXQ_BF16, float eps = kEps, int round_x = 1) {
+    if (!SCALE_IN && (!(qmax > 0.0f) || !(eps >= 0.0f))) return fail(DAXQ_ERR_ARG, "quant_rows: quant_max must be positive and eps not negative");
     switch (x_dtype) {
-        case DAXQ_BF16: return launch_quant_rows_t<FMT, ROUND_BF16, SCALE_IN, DAXQ_BF16>(x, m, k, ld_x, q, ld_q, scale, qmax, st);
-        case DAXQ_F16: return launch_quant_rows_t<FMT, ROUND_BF16, SCALE_IN, DAXQ_F16>(x, m, k, ld_x, q, ld_q, scale, qmax, st);
-        case DAXQ_F32: return launch_quant_rows_t<FMT, ROUND_BF16, SCALE_IN, DAXQ_F32>(x, m, k, ld_x, q, ld_q, scale, qmax, st);
+        case DAXQ_BF16: return launch_quant_rows_t<FMT, ROUND_BF16, SCALE_IN, DAXQ_BF16>(x, m, k, ld_x, q, ld_q, scale, qmax, st, eps, round_x);
+        case DAXQ_F16: return launch_quant_rows_t<FMT, ROUND_BF16, SCALE_IN, DAXQ_F16>(x, m, k, ld_x, q, ld_q, scale, qmax, st, eps, round_x);
+        case DAXQ_F32: return launch_quant_rows_t<FMT, ROUND_BF16, SCALE_IN, DAXQ_F32>(x, m, k, ld_x, q, ld_q, scale, qmax, st, eps, round_x);
         default: return fail(DAXQ_ERR_ARG, "quant_rows: unknown element type %d", x_dtype);
     }
 }
 
+// qmax <= 0: the format's own maximum
 template <bool ROUND_BF16, bool SCALE_IN>
 static int launch_quant_rows_fmt(int q_fmt, const void* x, int x_dtype, int64_t m, int64_t k, int64_t ld_x, void* q,
-                                 int64_t ld_q, float* scale, hipStream_t st) {
+                                 int64_t ld_q, float* scale, hipStream_t st, float qmax = 0.0f, float eps = kEps, int round_x = 1) {
     switch (q_fmt) {
-        case DAXQ_FMT_I8: return launch_quant_rows<0, ROUND_BF16, SCALE_IN>(x, m, k, ld_x, q, ld_q, scale, 127.0f, st, x_dtype);
-        case DAXQ_FMT_E4M3: return launch_quant_rows<1, ROUND_BF16, SCALE_IN>(x, m, k, ld_x, q, ld_q, scale, 448.0f, st, x_dtype);
-        case DAXQ_FMT_E5M2: return launch_quant_rows<2, ROUND_BF16, SCALE_IN>(x, m, k, ld_x, q, ld_q, scale, 57344.0f, st, x_dtype);
+        case DAXQ_FMT_I8: return launch_quant_rows<0, ROUND_BF16, SCALE_IN>(x, m, k, ld_x, q, ld_q, scale, qmax > 0.0f ? qmax : 127.0f, st, x_dtype, eps, round_x);
+        case DAXQ_FMT_E4M3: return launch_quant_rows<1, ROUND_BF16, SCALE_IN>(x, m, k, ld_x, q, ld_q, scale, qmax > 0.0f ? qmax : 448.0f, st, x_dtype, eps, round_x);
+        case DAXQ_FMT_E5M2: return launch_quant_rows<2, ROUND_BF16, SCALE_IN>(x, m, k, ld_x, q, ld_q, scale, qmax > 0.0f ? qmax : 57344.0f, st, x_dtype, eps, round_x);
         default: return fail(DAXQ_ERR_ARG, "quant_rows: unknown quantised format %d", q_fmt);
     }
 }
@@ -224,13 +240,13 @@ __global__ __launch_bounds__(256) void row_minmax_kernel(const void* __restrict_
     }
 }
 
-// scale[i] = max( max(-min[i], max[i]) / qmax, 2^-23 ), all in fp32
+// scale[i] = max( max(-min[i], max[i]) / qmax, eps ), all in fp32
 __global__ void scale_from_minmax_kernel(const float* __restrict__ mn, const float* __restrict__ mx, int64_t n,
-                                         float qmax, float* __restrict__ scale) {
+                                         float qmax, float eps, float* __restrict__ scale) {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n) {
         const float a = max_nan(-mn[i], mx[i]);
-        scale[i] = max_nan(a / qmax, kEps);
+        scale[i] = max_nan(a / qmax, eps);
     }
 }
 
@@ -297,6 +313,15 @@ int daxq_act_quant_rows(const void* x, int x_dtype, int q_fmt, int64_t m, int64_
     return daxq::launch_quant_rows_fmt<true, false>(q_fmt, x, x_dtype, m, k, ld_x, q, ld_q, scale, (hipStream_t)stream);
 }
 
+int daxq_act_quant_rows_ex(const void* x, int x_dtype, int q_fmt, int64_t m, int64_t k, int64_t ld_x, void* q, int64_t ld_q,
+                           float* scale, float quant_max, float eps, int scale_round, daxq_stream_t stream) {
+    if (scale_round != DAXQ_SCALE_ROUND_X && scale_round != DAXQ_SCALE_ROUND_NONE)
+        return daxq::fail(DAXQ_ERR_ARG, "act_quant_rows_ex: unknown scale rounding %d", scale_round);
+    if (!(quant_max > 0.0f)) return daxq::fail(DAXQ_ERR_ARG, "act_quant_rows_ex: quant_max must be positive");
+    return daxq::launch_quant_rows_fmt<true, false>(q_fmt, x, x_dtype, m, k, ld_x, q, ld_q, scale, (hipStream_t)stream, quant_max,
+                                                    eps, scale_round == DAXQ_SCALE_ROUND_X);
+}
+
 int daxq_quantize_rows(const void* x, int x_dtype, int q_fmt, int64_t m, int64_t k, int64_t ld_x, const float* scale,
                        void* q, int64_t ld_q, daxq_stream_t stream) {
     return daxq::launch_quant_rows_fmt<false, true>(q_fmt, x, x_dtype, m, k, ld_x, q, ld_q, const_cast<float*>(scale),
@@ -305,12 +330,17 @@ int daxq_quantize_rows(const void* x, int x_dtype, int q_fmt, int64_t m, int64_t
 
 int daxq_scale_from_minmax(const float* min_in, const float* max_in, int64_t n, float qmax, float* scale,
                            daxq_stream_t stream) {
+    return daxq_scale_from_minmax_eps(min_in, max_in, n, qmax, daxq::kEps, scale, stream);
+}
+
+int daxq_scale_from_minmax_eps(const float* min_in, const float* max_in, int64_t n, float qmax, float eps, float* scale,
+                               daxq_stream_t stream) {
     using namespace daxq;
-    if (n < 0 || !(qmax > 0.0f)) return fail(DAXQ_ERR_ARG, "scale_from_minmax: bad argument");
+    if (n < 0 || !(qmax > 0.0f) || eps != eps) return fail(DAXQ_ERR_ARG, "scale_from_minmax: bad argument");
     if (n == 0) return DAXQ_OK;
     if (!min_in || !max_in || !scale) return fail(DAXQ_ERR_ARG, "scale_from_minmax: null pointer");
     hipLaunchKernelGGL(scale_from_minmax_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
-                       min_in, max_in, n, qmax, scale);
+                       min_in, max_in, n, qmax, eps, scale);
     return check_launch("scale_from_minmax");
 }
 

@@ -64,6 +64,13 @@ class Linear(DerivedOperands, nn.Module):
     # False: every shape is quantised, as under the reference's own torch.compile decorator (:143); True: the
     # un-compiled reference's float matmul for M <= 16 or K / N not multiples of 8 (:186-202)
     uncompiled_small_shape_fallback = False
+    # False: the activation scale is computed in the input's own element type and only then widened to fp32, the
+    # reference's eager op sequence (dynamic/functional.py:124-129).  True: quotient and floor stay in fp32 -- what is
+    # left of that sequence when the forward runs under the torch.compile decorator it carries (:143; the code generator
+    # does not materialise the bf16 intermediate), which moves the scale of almost every token by up to half a bf16 step
+    # and about 0.4 % of the int8 values by one.  Class or instance attribute; the fused producer kernels and the block
+    # fusion built on them implement the eager form only.
+    act_scale_fp32 = False
 
     def __init__(
         self,
@@ -143,11 +150,11 @@ class Linear(DerivedOperands, nn.Module):
         if flat.stride(-1) != 1:  # a view with strided columns: the reference's torch ops take it, the kernels want rows
             flat = flat.contiguous()
         if self.input_qscheme == per_token_symmetric:
-            xq, sx = getattr(ops, _ACT_QUANT[self.input_dtype])(flat)
+            xq, sx = getattr(ops, _ACT_QUANT[self.input_dtype])(flat, self.act_scale_fp32)
         else:
             from .functional import per_tensor_scale
 
-            _, sx = per_tensor_scale(flat, ops.QMAX[ops.FMT_OF_DTYPE[self.input_dtype]])
+            _, sx = per_tensor_scale(flat, ops.QMAX[ops.FMT_OF_DTYPE[self.input_dtype]], round_x=not self.act_scale_fp32)
             xq = getattr(ops, "quantize_rows_" + ops.FMT_OF_DTYPE[self.input_dtype])(flat, sx, True)
         return QuantizedActivation(xq, sx, input.shape[:-1], self.in_features, self.input_dtype)
 
@@ -209,11 +216,11 @@ class Linear(DerivedOperands, nn.Module):
             if input.device != dev:
                 self._check_device(input.device)
             if input.dim() == 2 and input.stride(1) == 1:
-                return op(input, wq, sw, bias)
+                return op(input, wq, sw, bias, self.act_scale_fp32)
             flat = input.view(-1, self.in_features)
             if flat.stride(-1) != 1:
                 flat = flat.contiguous()
-            return op(flat, wq, sw, bias).view(*input.shape[:-1], self.out_features)
+            return op(flat, wq, sw, bias, self.act_scale_fp32).view(*input.shape[:-1], self.out_features)
         self._check_device(input.device)
         if self._takes_float_fallback(input):
             logger.warning("int8 matmul not taken for this combination of dimensions, float implementation instead. "
@@ -228,7 +235,8 @@ class Linear(DerivedOperands, nn.Module):
             flat = input.view(-1, self.in_features)
             if flat.stride(-1) != 1:
                 flat = flat.contiguous()
-            out = getattr(ops, _DYNAMIC_LINEAR[self.input_dtype])(flat, self._gemm_weight(), self._weight_scale_vector(), bias)
+            out = getattr(ops, _DYNAMIC_LINEAR[self.input_dtype])(flat, self._gemm_weight(), self._weight_scale_vector(), bias,
+                                                                  self.act_scale_fp32)
             return out.view(*input.shape[:-1], self.out_features)
         qa = input if isinstance(input, QuantizedActivation) else self.quantize_activation(input)
         if qa.dtype != self.input_dtype or qa.in_features != self.in_features:

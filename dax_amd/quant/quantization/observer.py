@@ -53,9 +53,7 @@ class UniformQuantizationObserverBase(nn.Module):
     def _calculate_qparams(self, min_val: torch.Tensor, max_val: torch.Tensor):
         if min_val.numel() == 0 or max_val.numel() == 0:
             return None  # nothing observed yet (:116-120)
-        if float(self.eps) != torch.finfo(torch.float32).eps:
-            raise NotImplementedError("daxq_scale_from_minmax floors the scale at float32 eps")
-        return ops.scale_from_minmax(min_val, max_val, float(self.quant_max))
+        return ops.scale_from_minmax(min_val, max_val, float(self.quant_max), float(self.eps))
 
     def reset_min_max_vals(self):
         raise NotImplementedError("Cannot reset min/max values in the given observer.")

@@ -50,6 +50,11 @@ extern "C" {
 #define DAXQ_F16 1
 #define DAXQ_F32 2
 
+/* how a dynamic activation scale, absmax / quant_max, is rounded before the floor (and the floor with it) */
+#define DAXQ_SCALE_ROUND_NONE 0 /* kept in fp32: what is left of the chain when a code generator fuses it, as under the
+                                   torch.compile decorator of the reference's forward (dax/quant/nn/dynamic/linear.py:143) */
+#define DAXQ_SCALE_ROUND_X 1    /* to x's own element type: the eager dtype chain, dax/quant/nn/dynamic/functional.py:124-129 */
+
 typedef void* daxq_stream_t;
 
 int daxq_abi_version(void);
@@ -160,6 +165,16 @@ int daxq_quantize_rows_e5m2(const void* x, int64_t m, int64_t k, int64_t ld_x, c
  */
 int daxq_act_quant_rows(const void* x, int x_dtype, int q_fmt, int64_t m, int64_t k, int64_t ld_x,
                         void* q, int64_t ld_q, float* scale, daxq_stream_t stream);
+/* daxq_act_quant_rows with the arguments _dynamic_quantize_func takes from its caller
+ *   dax/quant/nn/dynamic/functional.py:54-61, :126-127
+ * quant_max (> 0) instead of the format's own maximum, eps (>= 0) instead of 2^-23 as the floor of the scale, and
+ * scale_round = DAXQ_SCALE_ROUND_X (what daxq_act_quant_rows does) or DAXQ_SCALE_ROUND_NONE:
+ *   scale = max( round( f32(rowamax) / quant_max ), round( eps ) ),   round = to x's element type, or none.
+ * The scale is fp32 and the leaf quantiser computes in fp32 (a scale of a 16-bit type changes that arithmetic:
+ * daxq_block_quantize).  e4m3fn / e5m2 rows of bf16 elements divide element by element when the scale is not rounded. */
+int daxq_act_quant_rows_ex(const void* x, int x_dtype, int q_fmt, int64_t m, int64_t k, int64_t ld_x,
+                           void* q, int64_t ld_q, float* scale, float quant_max, float eps, int scale_round,
+                           daxq_stream_t stream);
 int daxq_quantize_rows(const void* x, int x_dtype, int q_fmt, int64_t m, int64_t k, int64_t ld_x, const float* scale,
                        void* q, int64_t ld_q, daxq_stream_t stream);
 
@@ -168,14 +183,19 @@ int daxq_quantize_rows(const void* x, int x_dtype, int q_fmt, int64_t m, int64_t
  * activations, 2-d tiles, blocks over leading dimensions).  The contiguous tensor x is seen through the view of
  * _get_reduction_params (:13-51): nd <= 8 dimensions view_shape[0..nd), reduced[d] != 0 for the dimensions a block
  * spans.  view_shape and reduced are HOST arrays, read before the call returns.
- * daxq_block_scale:    scale[b] = max( round( absmax(block b) / qmax ), 2^-23 ), b row-major over the kept
+ * daxq_block_scale:    scale[b] = max( round( absmax(block b) / qmax ), round( eps ) ), b row-major over the kept
  *                      dimensions; round = to x's own type when round_to_x != 0 (dynamic rule), none otherwise.
  * daxq_block_quantize: q[i] = leaf quantiser of x[i] with its block's scale; q has x's shape, one byte per element.
+ *                      scale_dtype: the element type of the scale the caller asked _dynamic_quantize_func for
+ *                      (:128-129); the values are passed as fp32 either way (exact widening).  DAXQ_F32 (every wrapper
+ *                      of the reference): fp32 arithmetic.  A 16-bit type: 1.0 / scale is rounded to it, and x * inv and
+ *                      x / scale to what type promotion makes of x and the scale -- that 16-bit type when x has it too,
+ *                      fp32 otherwise (dax/quant/nn/quantized/functional.py:11-20).
  */
 int daxq_block_scale(const void* x, int x_dtype, int nd, const int64_t* view_shape, const int32_t* reduced, float qmax,
-                     int round_to_x, float* scale, daxq_stream_t stream);
+                     float eps, int round_to_x, float* scale, daxq_stream_t stream);
 int daxq_block_quantize(const void* x, int x_dtype, int q_fmt, int nd, const int64_t* view_shape, const int32_t* reduced,
-                        const float* scale, void* q, daxq_stream_t stream);
+                        const float* scale, int scale_dtype, void* q, daxq_stream_t stream);
 
 /*
  * Per-tensor schemes (the block of dax/quant/qscheme.py:10-26 is the whole tensor).  The GEMM and the leaf
@@ -183,7 +203,7 @@ int daxq_block_quantize(const void* x, int x_dtype, int q_fmt, int nd, const int
  * vector, which gives the same arithmetic per element.  These entry points keep that on the device.
  *
  * daxq_tensor_scale: dynamic per-tensor scale from per-row statistics (daxq_row_minmax):
- *   a = max_i max(-row_min[i], row_max[i]);  scale1[0] = max( round(a / qmax), 2^-23 ), round = RNE to bf16 when
+ *   a = max_i max(-row_min[i], row_max[i]);  scale1[0] = max( round(a / qmax), round(eps) ), round = RNE to bf16 when
  *   round_bf16 == 1, to fp16 when it is 2 (the activation rule for a tensor of that type,
  *   dax/quant/nn/dynamic/functional.py:124-129) or none when 0 (fp32 tensors, and the observer rule,
  *   dax/quant/quantization/observer.py:97-134); expand[0..n_expand) receives the same value.
@@ -191,7 +211,7 @@ int daxq_block_quantize(const void* x, int x_dtype, int q_fmt, int nd, const int
  *   dax/quant/quantization/observer.py:200-214:  min_inout[0] = min(min_inout[0], min_i row_min[i]), same for max.
  * daxq_broadcast_f32: dst[0..n) = src[0]; how dax/quant/nn/quantized/linear.py:98-100 expands its input scale.
  */
-int daxq_tensor_scale(const float* row_min, const float* row_max, int64_t m, float qmax, int round_bf16,
+int daxq_tensor_scale(const float* row_min, const float* row_max, int64_t m, float qmax, float eps, int round_bf16,
                       float* scale1, float* expand, int64_t n_expand, daxq_stream_t stream);
 int daxq_tensor_minmax_update(const float* row_min, const float* row_max, int64_t m,
                               float* min_inout, float* max_inout, daxq_stream_t stream);
@@ -213,6 +233,9 @@ int daxq_row_minmax_t(const void* x, int x_dtype, int64_t m, int64_t k, int64_t 
  */
 int daxq_scale_from_minmax(const float* min_in, const float* max_in, int64_t n, float qmax,
                            float* scale, daxq_stream_t stream);
+/* the same with the observer's own floor instead of 2^-23 (its `eps` buffer, dax/quant/quantization/observer.py:19-35, :125) */
+int daxq_scale_from_minmax_eps(const float* min_in, const float* max_in, int64_t n, float qmax, float eps,
+                               float* scale, daxq_stream_t stream);
 
 /*
  * INT8 GEMM on MFMA with the fused epilogue.
@@ -300,16 +323,18 @@ int daxq_linear_w8a8(int x_fmt, int w_fmt, int out_dtype,
  * workspace / workspace_bytes: optional split-K workspace as for daxq_linear_w8a8_splitk (counters zero), or NULL.
  *       INT8 launches with bf16 outputs and few tiles then cut K into ranges (same bits as the plain launch).
  * kernel: as for daxq_linear_w8a8 (0 = the library's choice).
+ * act_scale_round: DAXQ_SCALE_ROUND_X, the reference's eager arithmetic, or DAXQ_SCALE_ROUND_NONE, the per-token scale
+ *       kept in fp32 as under the torch.compile decorator of the reference's forward (:143).
  * Formats and output types as for daxq_linear_w8a8.  The caller owns every buffer; nothing is allocated.
  */
-int daxq_dynamic_linear(int x_dtype, int x_fmt, int w_fmt, int out_dtype,
+int daxq_dynamic_linear(int x_dtype, int x_fmt, int w_fmt, int out_dtype, int act_scale_round,
                         const void* x, int64_t ld_x,
                         void* xq, int64_t ld_xq, float* sx, int64_t rows_alloc,
                         const void* wq, int64_t ld_wq, const float* sw, const void* bias,
                         void* out, int64_t ld_out,
                         int64_t m, int64_t n, int64_t k,
                         void* workspace, int64_t workspace_bytes, int kernel, daxq_stream_t stream);
-/* The three pairings of the bf16 DiT by name (bf16 x, bias and out; rows_alloc = m; no workspace; the library's kernel):
+/* The three pairings of the bf16 DiT by name (bf16 x, bias and out; eager scale; rows_alloc = m; no workspace; the library's kernel):
  * int8 x int8 (dax/quant/nn/dynamic/linear.py:181-228), e4m3fn x e4m3fn and e5m2 x e4m3fn (:146-178). */
 int daxq_dynamic_linear_i8(const void* x, int64_t ld_x, int8_t* xq, int64_t ld_xq, float* sx,
                            const int8_t* wq, int64_t ld_wq, const float* sw, const void* bias,

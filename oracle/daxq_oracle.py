@@ -44,6 +44,11 @@ How each function is pinned (see tests/test_oracle_*.py):
                            arithmetic and the C fp8 encoders
 * linear_int8_float_       float64 matmul on the bf16 de-quantised weight (tolerance: the float
   fallback                 matmul's summation order is the library's)
+* act_scale_fp32           closed form max(f32(amax) / qmax, eps) in numpy float32 over every finite bf16 / fp16
+                           abs-max; PARITY UNPINNED against the reference as it runs compiled on an NVIDIA GPU
+                           (which instruction the generated code divides with cannot be observed here)
+* dynamic_quantize with    quant_max / eps / scale_dtype other than the wrappers': numpy restatement of the
+  caller's arguments       dtype chain element by element (scale in x's type, cast, promoted arithmetic)
 """
 
 from __future__ import annotations
@@ -102,10 +107,10 @@ def quantize_to_fp8(x: torch.Tensor, scale: torch.Tensor, dtype: torch.dtype = t
     return (x / scale).clamp(-qmax, qmax).to(dtype)
 
 
-def act_quant_int8(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
-    """dynamic_quantize_to_int8, per-token.  dynamic/functional.py:181-206, :54-148."""
+def act_quant_int8(x: torch.Tensor, scale_fp32: bool = False) -> Tuple[torch.Tensor, torch.Tensor]:
+    """dynamic_quantize_to_int8, per-token.  dynamic/functional.py:181-206, :54-148.  scale_fp32: act_scale_fp32."""
     x2 = x.reshape(-1, x.shape[-1])
-    s = act_scale(x2, INT8_QMAX)
+    s = act_scale_fp32(x2, INT8_QMAX) if scale_fp32 else act_scale(x2, INT8_QMAX)
     return quantize_to_int8(x2, s), s
 
 
@@ -141,18 +146,29 @@ def get_reduction_params(block_size, input_size):
     return view, dims
 
 
-def dynamic_quantize(x: torch.Tensor, block_size, target_dtype: torch.dtype) -> Tuple[torch.Tensor, torch.Tensor]:
-    """``_dynamic_quantize_func`` for any block shape and any of the input dtypes it accepts (fp32 / fp16 / bf16),
-    as its two wrappers call it (quant_max of the target dtype, eps = float32 eps, fp32 scales).
-    dax/quant/nn/dynamic/functional.py:54-148, :152-206.  Returns (values in x's shape, scales with every
-    reduced dim kept as 1, in the view shape of get_reduction_params)."""
-    qmax = INT8_QMAX if target_dtype == torch.int8 else torch.finfo(target_dtype).max
+def dynamic_quantize(x: torch.Tensor, block_size, target_dtype: torch.dtype, quant_max=None, eps=None,
+                     scale_dtype: Optional[torch.dtype] = torch.float32,
+                     fused_chain: bool = False) -> Tuple[torch.Tensor, torch.Tensor]:
+    """``_dynamic_quantize_func`` for any block shape, any of the input dtypes it accepts (fp32 / fp16 / bf16) and
+    any quant_max / eps / scale_dtype.  dax/quant/nn/dynamic/functional.py:54-148.  The defaults are what its two
+    wrappers pass (:152-206): quant_max of the target dtype, eps = eps of the scale dtype, fp32 scales.
+    Returns (values in x's shape, scales with every reduced dim kept as 1, in the view shape of get_reduction_params).
+
+    fused_chain: ``act_scale_fp32`` below applied per block -- abs-max widened to fp32 first, quotient and floor in fp32."""
+    if quant_max is None:
+        quant_max = INT8_QMAX if target_dtype == torch.int8 else torch.finfo(target_dtype).max
+    if scale_dtype is None:  # :104-105
+        scale_dtype = x.dtype
+    if eps is None:
+        eps = torch.finfo(scale_dtype).eps
     view, dims = get_reduction_params(tuple(block_size), tuple(x.shape))
     xv = x.view(view)  # :121
     amax = xv.abs().amax(dim=dims, keepdim=False) if dims else xv.abs()  # :124
-    scale = torch.clamp(amax / float(qmax), min=EPS)  # :126-127, in x's dtype
-    if scale.dtype != torch.float32:  # :128-129
-        scale = scale.to(torch.float32)
+    if fused_chain:
+        amax = amax.to(torch.float32)
+    scale = torch.clamp(amax / float(quant_max), min=eps)  # :126-127, in x's dtype
+    if scale.dtype != scale_dtype:  # :128-129
+        scale = scale.to(scale_dtype)
     after = list(view)
     for i in dims:  # :131-135
         after[i] = 1
@@ -160,6 +176,18 @@ def dynamic_quantize(x: torch.Tensor, block_size, target_dtype: torch.dtype) -> 
     if target_dtype == torch.int8:  # :137-148
         return quantize_to_int8(xv, scale).view(x.shape), scale
     return quantize_to_fp8(xv, scale, target_dtype).view(x.shape), scale
+
+
+def act_scale_fp32(x: torch.Tensor, qmax: float, eps: float = EPS) -> torch.Tensor:
+    """The per-token scale with quotient and floor in fp32: ``max(f32(rowamax) / qmax, eps)``, fp32 [M, 1].
+
+    The reference's forward carries ``@torch.compile`` (dax/quant/nn/dynamic/linear.py:143).  A code generator that
+    fuses dynamic/functional.py:124-129 computes in fp32 and does not materialise the bf16 quotient (torch's inductor
+    leaves such casts out unless told to emulate them), so on an NVIDIA run the scale is this fp32 value.  The
+    division here is IEEE; what instruction the generated code divides with is not something this build can observe.
+    """
+    amax = x.abs().amax(dim=-1, keepdim=False).to(torch.float32)
+    return torch.clamp(amax / float(qmax), min=eps).view(-1, 1)
 
 
 # --------------------------------------------------------------------------- #
@@ -231,7 +259,7 @@ def epilogue_int8(acc: torch.Tensor, sx: torch.Tensor, sw: torch.Tensor,
 
 def linear_int8(x: torch.Tensor, qweight: torch.Tensor, wscale: torch.Tensor,
                 bias: Optional[torch.Tensor], row_chunk: int = 8192,
-                keep_acc: bool = True) -> Dict[str, torch.Tensor]:
+                keep_acc: bool = True, scale_fp32: bool = False) -> Dict[str, torch.Tensor]:
     """Whole INT8 forward.  dax/quant/nn/dynamic/linear.py:180-228.
 
     Processes rows in chunks so that the int32 accumulator of the big shapes is
@@ -239,7 +267,7 @@ def linear_int8(x: torch.Tensor, qweight: torch.Tensor, wscale: torch.Tensor,
     """
     prev = x.shape[:-1]
     x2 = x.reshape(-1, x.shape[-1])
-    xq, sx = act_quant_int8(x2)
+    xq, sx = act_quant_int8(x2, scale_fp32)
     outs, accs = [], []
     for r0 in range(0, x2.shape[0], row_chunk):
         acc = int_mm(xq[r0:r0 + row_chunk], qweight)
@@ -277,7 +305,8 @@ def scaled_mm_fp32(xq: torch.Tensor, qweight: torch.Tensor, scale_a: torch.Tenso
 
 def linear_fp8(x: torch.Tensor, qweight: torch.Tensor, wscale: torch.Tensor, bias: Optional[torch.Tensor],
                act_dtype: torch.dtype = torch.float8_e4m3fn, per_tensor: bool = False,
-               out_dtype: Optional[torch.dtype] = None, row_chunk: int = 8192) -> Dict[str, torch.Tensor]:
+               out_dtype: Optional[torch.dtype] = None, row_chunk: int = 8192,
+               scale_fp32: bool = False) -> Dict[str, torch.Tensor]:
     """Whole FP8 forward of the dynamic module.  dax/quant/nn/dynamic/linear.py:145-178.
 
     ``qweight`` is float8_e4m3fn or float8_e5m2 [N,K]; ``act_dtype`` the activation format (the FP8 qconfig's
@@ -294,7 +323,7 @@ def linear_fp8(x: torch.Tensor, qweight: torch.Tensor, wscale: torch.Tensor, bia
         sx = act_scale_per_tensor(x2, qmax)
         mm_dtype = out_dtype
     else:
-        sx = act_scale(x2, qmax)
+        sx = act_scale_fp32(x2, qmax) if scale_fp32 else act_scale(x2, qmax)
         mm_dtype = torch.bfloat16
     xq = quantize_to_fp8(x2, sx, act_dtype)
     out = scaled_mm_fp32(xq, qweight, sx, wscale, None if bias is None else bias.to(mm_dtype), mm_dtype, row_chunk)

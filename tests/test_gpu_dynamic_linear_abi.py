@@ -59,7 +59,7 @@ def test_dynamic_linear_i8_through_the_c_abi_bit_exact(m, n, k, named):
         rc = L.daxq_dynamic_linear_i8(xd.data_ptr(), k, xq.data_ptr(), kp + pad, sx.data_ptr(), wq.data_ptr(), kp, sw.data_ptr(),
                                       bd.data_ptr(), out.data_ptr(), n + 8, m, n, k, _stream())
     else:
-        rc = L.daxq_dynamic_linear(0, 0, 0, 0, xd.data_ptr(), k, xq.data_ptr(), kp + pad, sx.data_ptr(), rows, wq.data_ptr(), kp,
+        rc = L.daxq_dynamic_linear(0, 0, 0, 0, 1, xd.data_ptr(), k, xq.data_ptr(), kp + pad, sx.data_ptr(), rows, wq.data_ptr(), kp,
                                    sw.data_ptr(), bd.data_ptr(), out.data_ptr(), n + 8, m, n, k, None, 0, 0, _stream())
     _capi.check(rc, "dynamic_linear_i8")
     torch.cuda.synchronize()
@@ -116,7 +116,7 @@ def test_dynamic_linear_with_a_split_k_workspace_bit_exact():
         xq = torch.empty((m, k), dtype=torch.int8, device="cuda")
         sx = torch.empty((m,), dtype=torch.float32, device="cuda")
         out = torch.zeros((m, n), dtype=torch.bfloat16, device="cuda")
-        _capi.check(L.daxq_dynamic_linear(0, 0, 0, 0, xd.data_ptr(), k, xq.data_ptr(), k, sx.data_ptr(), m, wq.data_ptr(), k,
+        _capi.check(L.daxq_dynamic_linear(0, 0, 0, 0, 1, xd.data_ptr(), k, xq.data_ptr(), k, sx.data_ptr(), m, wq.data_ptr(), k,
                                           sw.data_ptr(), bd.data_ptr(), out.data_ptr(), n, m, n, k,
                                           workspace.data_ptr() if workspace is not None else None,
                                           workspace.numel() if workspace is not None else 0, 0, _stream()), "dynamic_linear")
@@ -132,9 +132,9 @@ def test_dynamic_linear_rejects_bad_arguments():
     t = torch.zeros(1 << 16, dtype=torch.uint8, device="cuda")
     p = t.data_ptr()
     # rows_alloc < m, a leading dimension that does not reach the padded K, mixed operand formats
-    assert L.daxq_dynamic_linear(0, 0, 0, 0, p, 128, p, 128, p, 1, p, 128, p, None, p, 8, 2, 8, 128, None, 0, 0, _stream()) == -1
-    assert L.daxq_dynamic_linear(0, 0, 0, 0, p, 100, p, 100, p, 2, p, 128, p, None, p, 8, 2, 8, 100, None, 0, 0, _stream()) == -1
-    assert L.daxq_dynamic_linear(0, 0, 1, 0, p, 128, p, 128, p, 2, p, 128, p, None, p, 8, 2, 8, 128, None, 0, 0, _stream()) == -1
+    assert L.daxq_dynamic_linear(0, 0, 0, 0, 1, p, 128, p, 128, p, 1, p, 128, p, None, p, 8, 2, 8, 128, None, 0, 0, _stream()) == -1
+    assert L.daxq_dynamic_linear(0, 0, 0, 0, 1, p, 100, p, 100, p, 2, p, 128, p, None, p, 8, 2, 8, 100, None, 0, 0, _stream()) == -1
+    assert L.daxq_dynamic_linear(0, 0, 1, 0, 1, p, 128, p, 128, p, 2, p, 128, p, None, p, 8, 2, 8, 128, None, 0, 0, _stream()) == -1
     assert "dynamic_linear" in _capi.last_error() or "unsupported operand formats" in _capi.last_error()
     torch.cuda.synchronize()
 

@@ -652,3 +652,115 @@ def test_linear_int8_other_module_dtypes(closed_form, dtype):
     npdt = np.float16 if dtype == torch.float16 else np.float32
     want = (y.astype(npdt).astype(np.float32) + b.float().numpy()).astype(npdt)
     np.testing.assert_array_equal(r["out"].numpy(), want)
+
+
+# ------------------------------------------------------------------ fp32 scale and caller-supplied quant_max / eps / scale_dtype
+def _np_bf16_rne(v: np.ndarray) -> np.ndarray:
+    """float32 -> nearest bfloat16 (ties to even), returned as float32; finite inputs."""
+    u = np.ascontiguousarray(v, dtype=np.float32).view(np.uint32).astype(np.uint64)
+    u = (u + 0x7FFF + ((u >> 16) & 1)) >> 16 << 16
+    return u.astype(np.uint32).view(np.float32)
+
+
+def test_act_scale_fp32_closed_form_exhaustive():
+    """act_scale_fp32 = max(f32(amax) / qmax, 2^-23) with an IEEE fp32 division and no rounding to the input's type:
+    every non-negative finite bf16 and fp16 abs-max, against numpy float32 arithmetic.  It differs from the eager
+    scale on almost every value whose quotient is not a bf16 number."""
+    bits = ALL_POS_FINITE = np.arange(0, 0x7F80, dtype=np.uint16)
+    a32 = (bits.astype(np.uint32) << 16).view(np.float32)
+    xb = from_bits(bits).view(-1, 1)
+    h = np.arange(0, 0x7C00, dtype=np.uint16).view(np.float16)
+    xh = torch.from_numpy(h.copy()).view(-1, 1)
+    for qmax in (127.0, 448.0, 57344.0):
+        got = O.act_scale_fp32(xb, qmax).view(-1).numpy()
+        want = np.maximum(a32 / np.float32(qmax), np.float32(2.0 ** -23))
+        np.testing.assert_array_equal(got, want)
+        eager = O.act_scale(xb, qmax).view(-1).numpy()
+        np.testing.assert_array_equal(eager, np.maximum(_np_bf16_rne(a32 / np.float32(qmax)), np.float32(2.0 ** -23)))
+        above = want > np.float32(2.0 ** -22)          # (below, both sit on the floor)
+        assert (got[above] != eager[above]).mean() > 0.8          # the two forms are different functions (448 = 7 * 64: one quotient in seven is a bf16 number)
+        assert (np.abs(got - eager)[above] <= eager[above] * 2.0 ** -8).all()   # ... half a bf16 step apart at most
+        goth = O.act_scale_fp32(xh, qmax).view(-1).numpy()
+        np.testing.assert_array_equal(goth, np.maximum(h.astype(np.float32) / np.float32(qmax), np.float32(2.0 ** -23)))
+    # a row's abs-max decides, sign and position do not; another floor is honoured
+    x = torch.tensor([[0.5, -3.0, 2.0], [0.0, 0.0, 0.0]]).bfloat16()
+    np.testing.assert_array_equal(O.act_scale_fp32(x, 127.0).view(-1).numpy(), np.array([np.float32(3.0) / np.float32(127.0), 2.0 ** -23], np.float32))
+    np.testing.assert_array_equal(O.act_scale_fp32(x, 127.0, eps=0.5).view(-1).numpy(), np.array([0.5, 0.5], np.float32))
+
+
+def test_fp32_scale_changes_a_small_share_of_the_int8_values():
+    """On benchmark-shaped data the fp32 scale moves well under 1 % of the int8 values, each by one step."""
+    x, _, _ = O.make_inputs(512, 1536, 8, seed=0)
+    q0, s0 = O.act_quant_int8(x)
+    q1, s1 = O.act_quant_int8(x, scale_fp32=True)
+    assert (s0 != s1).float().mean() > 0.9
+    diff = (q0.int() - q1.int()).abs()
+    assert int(diff.max()) == 1 and 0.0 < float((diff != 0).float().mean()) < 0.01
+
+
+def test_dynamic_quantize_with_the_callers_quant_max_eps_and_scale_dtype(closed_form):
+    """_dynamic_quantize_func honours quant_max, eps and scale_dtype (dax/quant/nn/dynamic/functional.py:54-61,
+    :104-129).  Restated in numpy element by element: abs-max, quotient and floor in x's type; cast to scale_dtype;
+    the leaf quantiser rounds 1.0 / scale to the scale's type and the product / quotient to the promoted type of x and
+    the scale (bf16 x bf16 -> bf16; bf16 x fp16 or anything with an fp32 side -> fp32)."""
+    g = torch.Generator().manual_seed(50)
+    x = (torch.randn(48, 64, generator=g) * torch.logspace(-3, 2, 64)).bfloat16()
+    x[3] = 0
+    xf = x.float().numpy()
+    amax = np.abs(xf).max(axis=1, keepdims=True)
+    for quant_max, eps in ((127.0, 2.0 ** -23), (100.0, 1e-3), (63, 0.0078125), (448.0, 0.3)):
+        s_x = np.maximum(_np_bf16_rne(amax / np.float32(quant_max)), _np_bf16_rne(np.float32([eps])))   # bf16 tensor, bf16 floor
+        # fp32 scale: fp32 arithmetic in the leaf quantiser
+        q, sc = O.dynamic_quantize(x, (1, 64), torch.int8, quant_max=quant_max, eps=eps, scale_dtype=torch.float32)
+        assert sc.dtype == torch.float32
+        np.testing.assert_array_equal(sc.numpy(), s_x)
+        inv = (np.float32(1.0) / s_x).astype(np.float32)
+        np.testing.assert_array_equal(q.numpy(), np.clip(np.rint((xf * inv).astype(np.float32)), -128, 127).astype(np.int8))
+        # bf16 scale (scale_dtype=None means x's own type): bf16 arithmetic
+        for sd in (torch.bfloat16, None):
+            q, sc = O.dynamic_quantize(x, (1, 64), torch.int8, quant_max=quant_max, eps=eps, scale_dtype=sd)
+            assert sc.dtype == torch.bfloat16
+            np.testing.assert_array_equal(sc.float().numpy(), s_x)
+            inv_b = _np_bf16_rne((np.float32(1.0) / s_x).astype(np.float32))
+            prod = _np_bf16_rne((xf * inv_b).astype(np.float32))
+            np.testing.assert_array_equal(q.numpy(), np.clip(np.rint(prod), -128, 127).astype(np.int8))
+        # fp8 with a bf16 scale: the quotient is rounded to bf16 before the clamp and the cast
+        for fdt, enc, fmax in ((torch.float8_e4m3fn, closed_form.f32_to_e4m3fn, 448.0), (torch.float8_e5m2, closed_form.f32_to_e5m2, 57344.0)):
+            q8, sc8 = O.dynamic_quantize(x, (1, 64), fdt, quant_max=quant_max, eps=eps, scale_dtype=torch.bfloat16)
+            np.testing.assert_array_equal(sc8.float().numpy(), s_x)
+            v = np.clip(_np_bf16_rne((xf / s_x).astype(np.float32)), -fmax, fmax).astype(np.float32)
+            np.testing.assert_array_equal(q8.view(torch.uint8).numpy(), enc(v.reshape(-1)).reshape(v.shape))
+        # fp16 scale for a bf16 tensor: the cast can change the value (range); the reciprocal is an fp16 number, the
+        # product is promoted to fp32
+        q, sc = O.dynamic_quantize(x, (1, 64), torch.int8, quant_max=quant_max, eps=eps, scale_dtype=torch.float16)
+        s_h = s_x.astype(np.float16)
+        np.testing.assert_array_equal(sc.numpy(), s_h)
+        inv = (np.float32(1.0) / s_h.astype(np.float32)).astype(np.float16).astype(np.float32)
+        np.testing.assert_array_equal(q.numpy(), np.clip(np.rint((xf * inv).astype(np.float32)), -128, 127).astype(np.int8))
+    # the wrappers' defaults are the special case
+    q_a, s_a = O.dynamic_quantize(x, (1, 64), torch.int8)
+    q_b, s_b = O.dynamic_quantize(x, (1, 64), torch.int8, quant_max=127, eps=torch.finfo(torch.float32).eps, scale_dtype=torch.float32)
+    assert torch.equal(q_a, q_b) and torch.equal(s_a, s_b)
+
+
+def test_scale_by_division_and_by_reciprocal_where_they_differ():
+    """torch on a GPU evaluates ``amax / float(quant_max)`` (a tensor over a Python scalar,
+    dax/quant/nn/dynamic/functional.py:126) as ``amax * (1 / quant_max)``; on the CPU, and in this build's kernels, it
+    is a division.  For bf16 tensors the two give the same scale for every abs-max; for fp16 and fp32 tensors they do
+    not always.  This records the deviation set (parity of fp16 / fp32 scales with an eager GPU run is unpinned)."""
+    b = (np.arange(0, 0x7F80, dtype=np.uint32) << 16).view(np.float32)
+    h = np.arange(0, 0x7C00, dtype=np.uint16).view(np.float16).astype(np.float32)
+    counts = {}
+    for qmax in (127.0, 448.0, 57344.0):
+        r = np.float32(1.0) / np.float32(qmax)
+        assert np.array_equal(_np_bf16_rne(b / np.float32(qmax)), _np_bf16_rne((b * r).astype(np.float32)))   # bf16: never
+        div = (h / np.float32(qmax)).astype(np.float16)
+        mul = (h * r).astype(np.float32).astype(np.float16)
+        counts[qmax] = int((div != mul).sum())
+    assert counts[127.0] == 0 and 0 < counts[448.0] < 100 and 0 < counts[57344.0] < 100   # fp16: a few dozen of 31 744 values
+    f = np.abs(np.random.default_rng(7).standard_normal(200000).astype(np.float32)) * np.float32(3.0)
+    for qmax, lo, hi in ((127.0, 0.01, 0.15), (448.0, 0.3, 0.7)):
+        r = np.float32(1.0) / np.float32(qmax)
+        share = float(((f / np.float32(qmax)) != (f * r).astype(np.float32)).mean())
+        assert lo < share < hi, (qmax, share)       # fp32: a few percent at 127, about half at 448, each one ulp
+        assert np.abs((f / np.float32(qmax)).view(np.int32) - (f * r).astype(np.float32).view(np.int32)).max() <= 1
