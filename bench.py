@@ -209,7 +209,7 @@ def main():
                          "config0 (one linear, M = 4096, K = N = 1536); the sub-records exist for 14b only")
     ap.add_argument("--variant", type=int, default=0, help="GEMM kernel selection for comparisons (0 = library default)")
     ap.add_argument("--tile-group", type=int, default=0, help="tile-order group depth (0 = library default)")
-    ap.add_argument("--tile-order", type=int, default=0, help="tile order of the 256x256 kernels: 0 = library default, 1 = row groups, 2 = whole patches per XCD, 3 = patches in super-groups, 4 / 5 = banded 8 / 4 wide, 6 / 7 = swept 4 / 8 wide")
+    ap.add_argument("--tile-order", type=int, default=0, help="tile order of the 256x256 kernels: 0 = library default, 1 = row groups, 2 = banded patches")
     ap.add_argument("--m", type=int, default=0, help="tokens (0 = the model's own count)")
     ap.add_argument("--cpu-rows", type=int, default=0, help="tokens in the CPU-baseline sample (0 = pick for 10-30 s)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -270,7 +270,7 @@ def main():
             "config": {"workload": f"{model_name} linear set, {kind.upper()} W8A8, M={m} tokens: {shape_txt}; {per_lin_txt}",
                        "gemm_variant": args.variant},
             "pct_of_mfma_peak": round(100.0 * res["value"] / PEAK_TOPS, 2),
-            "roofline": roofline(res, kind, ("gemm_tile256s5_kernel" if kind == "int8" else "gemm_tile256f16_kernel") +
+            "roofline": roofline(res, kind, ("gemm_tile256s5_kernel" if kind == "int8" else "gemm_tile_fp8_kernel") +
                                  f", average launch over the {len(shapes)} shape(s); 8-bit ops counted as 2*M*N*K",
                                  gemm_traffic(kind) if full else None),
             "per_linear": res["per_linear"],

@@ -138,21 +138,20 @@ _tail = 0
 
 
 def debug_select_gemm(v: int) -> None:
-    """0 = the library's choice by shape; 2 / 5 / 6 / 8 / 9 / 11 = one implementation (include/daxq.h);
-    1000 + d = depth d of the tile-order groups (1000 = default); 2000 + o = tile order of the 256x256 kernels
-    (2000 = by shape, 2001 = groups of tile rows, 2002 = whole patches per XCD, 2003 = patches in super-groups,
-    2004 / 2005 = banded patches 8 / 4 columns wide, 2006 / 2007 = swept patches 4 / 8 columns wide); 3000 + t = the
-    last partial round of a 256x256 launch as a second launch on 128x128 tiles (3000 = by shape, 3001 = never,
-    3002 = whenever every such tile gets a CU)."""
+    """0 = the library's choice by shape; 2 / 5 / 8 / 11 = one implementation (include/daxq.h: the generic kernel on
+    256x256 / 128x128 tiles, the tiled kernel on 256x256 / 128x128 tiles); 1000 + d = depth d of the tile-order groups
+    (1000 = default); 2000 + o = tile order of the 256x256 kernels (2000 = by shape, 2001 = groups of tile rows,
+    2002 = banded patches); 3000 + t = the last partial round of a 256x256 launch as a second launch on 128x128 tiles
+    (3000 = by shape, 3001 = never, 3002 = whenever every such tile gets a CU)."""
     global _kernel_choice, _tile_group, _tile_order, _tail
     v = int(v)
     if 1000 <= v < 1064:
         _tile_group = v - 1000
-    elif 2000 <= v < 2008:
+    elif 2000 <= v < 2003:
         _tile_order = v - 2000
     elif 3000 <= v < 3003:
         _tail = v - 3000
-    elif v in (0, 2, 5, 6, 8, 9, 11):
+    elif v in (0, 2, 5, 8, 11):
         _kernel_choice = v
     else:
         raise DaxqError(f"unknown gemm kernel choice {v}")

@@ -39,10 +39,9 @@ struct GemmArgs {
     int m, n, k;
     int tiles_m, tiles_n;
     int gm;  // depth (in tile rows) of the groups the tile order walks through
-    // tile order of the 256x256 kernels (tile_order.h): 0 = groups of gm tile rows, 1 = whole patches per XCD, 2 = the same
-    // patches in super-groups of rows, 3 / 4 = banded with main bands 8 / 4 columns wide, 5 / 6 = swept with bands 4 / 8 wide
+    // tile order of the 256x256 kernels: 0 = groups of gm tile rows, 1 = banded patches of 8 x 4 tiles (tile_order.h)
     int order;
-    int out_kind;  // element type of out and bias: DAXQ_BF16 / DAXQ_F16 / DAXQ_F32 (the tiled kernels write bf16 only)
+    int out_kind;  // element type of out and bias: DAXQ_BF16 / DAXQ_F16 / DAXQ_F32
     // split-K launches only: K is cut into `splits` equal ranges, one workgroup each; partial accumulators go to
     // `partials` ([tile][split][64 KiB]) and the workgroup that arrives last at `counters[tile]` adds them up
     int splits;

@@ -20,7 +20,7 @@
 // congruent mod 8) form a compact patch of the output and share A/B panels in that XCD's L2.
 #include <type_traits>
 
-#include "gemm_common.h"
+#include "gemm_tile.h"
 
 namespace daxq {
 
@@ -240,14 +240,19 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_w8a8_kernel(const GemmArgs p
     else epilogue(std::integral_constant<int, DAXQ_F32>{});
 }
 
-template <bool FP8>
-int launch_tile256(const GemmArgs& a, bool x_e5m2, hipStream_t st);
 bool tile256_applies(const GemmArgs& a);
-template <bool FP8>
-int launch_tile256s5(const GemmArgs& a, int f8, bool wide, bool small, int tail, hipStream_t st);
+int launch_tile_i8(const GemmArgs& a, bool small, int tail, hipStream_t st);           // gemm_tile256.hip
+int launch_tile_fp8(const GemmArgs& a, int f8, bool small, int tail, hipStream_t st);  // gemm_tile_fp8.hip
 template <bool FP8>
 int launch_tile128_splitk(const GemmArgs& a, int f8, hipStream_t st);
 
+template <bool FP8>
+static int launch_tiled(const GemmArgs& a, int f8, bool small, int tail, hipStream_t st) {
+    if constexpr (FP8) return launch_tile_fp8(a, f8, small, tail, st);
+    else return launch_tile_i8(a, small, tail, st);
+}
+
+int prepare_tile_fp8_kernels();
 int prepare_tile256_kernels();
 
 template <bool FP8, int BM, int BN, int BK, int WM, int WN, bool DIRECT, int F8 = 0>
@@ -288,7 +293,7 @@ static int launch_generic(const GemmArgs& a, int f8, hipStream_t st) {
 
 // Kernel choices of the `kernel` argument (daxq_linear_w8a8): low 16 bits pick the implementation, bits 16-23 the
 // depth of the tile-order groups (0 = 4 tile rows).
-enum { K_DEFAULT = 0, K_GENERIC256 = 2, K_GENERIC128 = 5, K_TWO_STAGE = 6, K_FIVE_STAGE = 8, K_FIVE_STAGE_WIDE = 9, K_FIVE_STAGE_128 = 11 };
+enum { K_DEFAULT = 0, K_GENERIC256 = 2, K_GENERIC128 = 5, K_TILED_256 = 8, K_TILED_128 = 11 };
 
 // Tile order a launch of 256x256 tiles takes when the caller names none.  The banded order (tile_order.h: patches of
 // 8 x 4 tiles per XCD, the eight XCDs of a round on the same activation rows and on different weight bands) reads the
@@ -301,9 +306,10 @@ enum { K_DEFAULT = 0, K_GENERIC256 = 2, K_GENERIC128 = 5, K_TWO_STAGE = 6, K_FIV
 // the rows: -3 to -16 %; K = 1536: -2 %; N = K = 4096: -2 %).
 static int order_by_shape(int64_t m, int64_t n, int64_t k) {
     const int64_t tm = (m + 255) / 256, tn = (n + 255) / 256, tiles = tm * tn;
-    // (tm >= 32: at least one super-row of whole 8 x 4 patches; tn <= 4096: the balance count walks over one row of patches)
-    if (k < 2048 || tn < 20 || tm < 32 || tiles < 2048 || tm > 0x7fffff || tn > 4096) return 0;
-    return banded_xcd_rounds((int)tm, (int)tn, 4) * 100 <= (tiles + 255) / 256 * 105 ? 4 : 0;
+    // (tm >= 32: at least one super-row of whole 8 x 4 patches; tm <= 100000 and tn <= 4096: the range the host-side
+    // coverage check of the order reaches, with sampled grids)
+    if (k < 2048 || tn < 20 || tm < 32 || tiles < 2048 || tm > 100000 || tn > 4096) return kOrderRowGroups;
+    return banded_xcd_rounds((int)tm, (int)tn, 4) * 100 <= (tiles + 255) / 256 * 105 ? kOrderBanded : kOrderRowGroups;
 }
 
 template <bool FP8>
@@ -339,11 +345,11 @@ static int launch_gemm(const void* xq, int64_t ld_xq, const float* sx, const voi
     a.k = (int)k;
     a.tiles_m = a.tiles_n = 0;
     a.gm = (kernel >> 16) & 0xff ? (kernel >> 16) & 0xff : 4;
-    // Tile order of the 256x256 kernels: bits 24-27 of `kernel`, 0 = by shape (order_by_shape), else 1 + the value of
-    // GemmArgs::order.
+    // Tile order of the 256x256 kernels: bits 24-27 of `kernel`, 0 = by shape (order_by_shape), 1 = groups of tile rows,
+    // 2 = banded
     const int order_bits = (kernel >> 24) & 15;
-    if (order_bits > 7) return fail(DAXQ_ERR_ARG, "linear: unknown tile order %d", order_bits);
-    a.order = order_bits ? order_bits - 1 : ((kernel & 0xffff) == K_FIVE_STAGE_128 ? 0 : order_by_shape(m, n, k));
+    if (order_bits > 2) return fail(DAXQ_ERR_ARG, "linear: unknown tile order %d", order_bits);
+    a.order = order_bits ? order_bits - 1 : order_by_shape(m, n, k);
     a.out_kind = out_kind;
     a.splits = 1;
     a.counters = nullptr;
@@ -355,40 +361,31 @@ static int launch_gemm(const void* xq, int64_t ld_xq, const float* sx, const voi
     if (tail > 2) return fail(DAXQ_ERR_ARG, "linear: unknown tail choice %d", tail);
     const int which = kernel & 0xffff;
     const bool fits32 = a.lda < (1 << 26) && a.ldb < (1 << 26);  // 32-bit row offsets of the tiled kernels
-    // the int8 kernels on 16x16 MFMAs (the library's choice, 8, 11) also write fp16 and fp32; every other tiled kernel bf16 only
-    const bool tiled_out = out_kind == DAXQ_BF16 || (!FP8 && !acc);  // (the accumulator dump of the tiled kernels exists with bf16 outputs)
-    if (which != K_DEFAULT && which != K_GENERIC256 && which != K_GENERIC128 &&
-        (out_kind != DAXQ_BF16 && !(tiled_out && (which == K_FIVE_STAGE || which == K_FIVE_STAGE_128))))
-        return fail(DAXQ_ERR_ARG, "linear: kernel %d does not write this output type", which);
+    if (acc && out_kind != DAXQ_BF16 && which != K_GENERIC256 && which != K_GENERIC128 && which != K_DEFAULT)
+        return fail(DAXQ_ERR_ARG, "linear: the tiled kernels dump their accumulators with bf16 outputs only");
     switch (which) {
         case K_DEFAULT: {
-            // fp16 / fp32 outputs of the fp8 forms (per-tensor fp8 modules that are not bf16): the generic kernel,
-            // which rounds to any of the three
-            if (!tiled_out)
+            // fp16 / fp32 outputs together with the accumulator dump (tests): the generic kernel
+            if (acc && out_kind != DAXQ_BF16)
                 return (m >= 256 && n >= 256) ? launch_generic<FP8, 256>(a, f8, st) : launch_generic<FP8, 128>(a, f8, st);
-            // library default: the five-stage kernel on 256x256 tiles once there is one for every second CU, on
-            // 128x128 tiles (4x as many workgroups, two per CU) below that, and the generic kernel for operands
-            // smaller than one such tile.  Measured at N = K = 5120 (INT8, T-op/s, 128 / 256 tiles):
+            // library default: the tiled kernel on 256x256 tiles once there is one for every second CU, on 128x128
+            // tiles (4x as many workgroups, two per CU) below that, and the generic kernel for operands smaller than
+            // one such tile.  Measured at N = K = 5120 (INT8, T-op/s, 128 / 256 tiles):
             // M = 512 -> 1127 / 551, M = 1024 (80 large tiles) -> 1275 / 1055, M = 2048 (160) -> 1542 / 1817;
             // 4096 x 1536 x 1536 (96) -> 1182 / 895, 8192 x 1536 x 1536 (192) -> 1517 / 1587.
             const int64_t tiles256 = ((m + 255) / 256) * ((n + 255) / 256);
-            if (tile256_applies(a) && tiles256 >= 128) return launch_tile256s5<FP8>(a, f8, false, false, tail, st);
-            if (m >= 128 && n >= 128 && fits32) return launch_tile256s5<FP8>(a, f8, false, true, 1, st);
+            if (tile256_applies(a) && tiles256 >= 128) return launch_tiled<FP8>(a, f8, false, tail, st);
+            if (m >= 128 && n >= 128 && fits32) return launch_tiled<FP8>(a, f8, true, 1, st);
             return launch_generic<FP8, 128>(a, f8, st);
         }
         case K_GENERIC256: return launch_generic<FP8, 256>(a, f8, st);
         case K_GENERIC128: return launch_generic<FP8, 128>(a, f8, st);
-        case K_TWO_STAGE:
+        case K_TILED_256:
             if (!tile256_applies(a)) return fail(DAXQ_ERR_ARG, "linear: the 256x256 kernel needs m, n >= 256");
-            if (f8 & kF8WE5) return fail(DAXQ_ERR_ARG, "linear: the two-stage kernel has no e5m2-weight form");
-            return launch_tile256<FP8>(a, f8 & kF8XE5, st);
-        case K_FIVE_STAGE:
-        case K_FIVE_STAGE_WIDE:  // INT8 with 32x32x32 MFMAs
-            if (!tile256_applies(a)) return fail(DAXQ_ERR_ARG, "linear: the 256x256 kernel needs m, n >= 256");
-            return launch_tile256s5<FP8>(a, f8, which == K_FIVE_STAGE_WIDE, false, tail, st);
-        case K_FIVE_STAGE_128:
+            return launch_tiled<FP8>(a, f8, false, tail, st);
+        case K_TILED_128:
             if (m < 128 || n < 128 || !fits32) return fail(DAXQ_ERR_ARG, "linear: the 128x128 kernel needs m, n >= 128");
-            return launch_tile256s5<FP8>(a, f8, false, true, 1, st);
+            return launch_tiled<FP8>(a, f8, true, 1, st);
         default: return fail(DAXQ_ERR_ARG, "linear: unknown kernel choice %d", which);
     }
 }
@@ -571,6 +568,7 @@ int daxq_linear_w8a8_splitk(int x_fmt, int w_fmt, const void* xq, int64_t ld_xq,
 int daxq_init(void) {
     using namespace daxq;
     int rc = prepare_tile256_kernels();
+    if (!rc) rc = prepare_tile_fp8_kernels();
 #define DAXQ_PREP_ALL(FP8, BT, WN)                                        \
     if (!rc) rc = prepare_cfg<FP8, BT, BT, 128, 2, WN, true, 0>();
     DAXQ_PREP_ALL(false, 128, 2)

@@ -283,20 +283,20 @@ int daxq_linear_e5m2_e4m3(const uint8_t* xq, int64_t ld_xq, const float* sx,
  *   int8: out = T( f32( T( f32_rne(acc) * sx[i] * sw[j] ) ) + f32(bias[j]) )   T = round to out_dtype   (:221-228)
  *   fp8:  out = T( acc * sx[i] * sw[j] + f32(bias[j]) )                        (torch._scaled_mm, :155-173)
  * acc: optional int32 (int8) / fp32 (fp8) dump of the raw accumulators.
- * kernel: 0 = the library's choice by shape.  Other values pick one implementation, for tests and comparisons
- * (int8 results are the same bits for every choice, fp8 results differ by fp32 summation order): low 16 bits 2 / 5 =
- * generic kernel on 256x256 / 128x128 tiles, 6 = two-stage 256x256 kernel, 8 = the 256x256 kernel on 16x16 MFMAs
- * (int8 16x16x64; fp8 16x16x128 from k = 512 on), 9 = the 256x256 kernel on 32x32 MFMAs, 11 = the five-stage kernel on
- * 128x128 tiles; bits 16-23, when not zero, set the depth of the tile-order groups; bits 24-27 the tile order of the
- * 256x256 kernels (0 = by shape, 1 = groups of tile rows, 2 = whole 32-tile patches per XCD, 3 = those patches in
- * super-groups of rows, 4 / 5 = banded patches with main bands 8 / 4 tile columns wide, 6 / 7 = swept patches 4 / 8
- * columns wide; every order computes every tile once, the results are the same bits); bits 28-29 the treatment of
- * the last, partial round of workgroups of a launch of 256x256 tiles in row groups (0 = by shape: when the launch
- * has one to eight whole rounds and the tiles left over number at most a quarter of the CUs, they run as a second
- * launch of 128x128 tiles with a CU each; 1 = never; 2 = whenever they number at most a quarter of the CUs; int8
- * results are the same bits either way).  fp16 and fp32 outputs of int8 operands are written by the library's choice
- * and by 8 and 11 (the kernels on 16x16 MFMAs); fp16 and fp32 outputs of fp8 operands exist in the generic kernel
- * only.  The choice is an argument of the call: the library keeps no process-wide
+ * kernel: 0 = the library's choice by shape.  Other values pick one implementation, for tests and comparisons: low 16
+ * bits 2 / 5 = the generic kernel on 256x256 / 128x128 tiles (an implementation of its own, any shape), 8 / 11 = the
+ * tiled kernel on 256x256 / 128x128 tiles (int8: 16x16x64 MFMAs; fp8: 16x16x128 MFMAs; needs m, n >= the tile edge);
+ * bits 16-23, when not zero, set the depth of the tile-order groups; bits 24-27 the tile order of the 256x256 kernels
+ * (0 = by shape, 1 = groups of tile rows, 2 = banded patches of 8 x 4 tiles per XCD; every order computes every tile
+ * once, the results are the same bits); bits 28-29 the treatment of the last, partial round of workgroups of a launch
+ * of 256x256 tiles in row groups (0 = by shape: when the launch has one to eight whole rounds and the tiles left over
+ * number at most a quarter of the CUs, they run as a second launch of 128x128 tiles with a CU each; 1 = never;
+ * 2 = whenever they number at most a quarter of the CUs).
+ * int8 results are the same bits for every choice.  fp8 results are the same bits for every choice of tile size, tile
+ * order and cut of the tiled kernel (one sequence of MFMAs per output element), so an output row does not depend on
+ * how many rows the launch has; the generic kernel (any fp8 launch with n < 128, or m < 128 rows) adds in another
+ * order and agrees to fp32 rounding.  Every kernel writes bf16, fp16 and fp32; the accumulator dump of the tiled
+ * kernels exists with bf16 outputs.  The choice is an argument of the call: the library keeps no process-wide
  * selection.
  */
 int daxq_linear_w8a8(int x_fmt, int w_fmt, int out_dtype,
@@ -347,8 +347,8 @@ int daxq_dynamic_linear_e5m2_e4m3(const void* x, int64_t ld_x, uint8_t* xq, int6
                                   void* out, int64_t ld_out, int64_t m, int64_t n, int64_t k, daxq_stream_t stream);
 
 /* The tile order daxq_linear_w8a8 takes for a launch of 256x256 tiles when bits 24-27 of `kernel` are 0, as the value
- * of those bits: 1 = groups of tile rows, 5 = banded patches 4 tile columns wide (large launches: K >= 2048,
- * N >= 5120, M >= 7937 and no XCD more than 5 % over its share of the tiles).  For tests and diagnostics; no
+ * of those bits: 1 = groups of tile rows, 2 = banded patches (large launches: K >= 2048, N >= 5120, M >= 7937 and no
+ * XCD more than 5 % over its share of the tiles).  For tests and diagnostics; no
  * counterpart in the reference, whose matmul comes from a vendor library. */
 int daxq_linear_tile_order_choice(int64_t m, int64_t n, int64_t k);
 

@@ -2,8 +2,8 @@
 through the swapped module.  Rows of a per-token-quantised linear are independent, so at the large M a
 sample of rows (first / last rows of the first / last tiles plus random ones) is compared with the
 oracle bit for bit (INT8) or within 2e-2 relative L2 (FP8), and the whole output is tied to it by
-running the same module on the row sample alone: the two GPU results must be identical (INT8) or equal up to
-rounding flips of the fp32 summation order (FP8)."""
+running the same module on the row sample alone: the two GPU results must be identical, INT8 and FP8 alike (a token's
+output does not depend on the batch it arrives in)."""
 import numpy as np
 import pytest
 import torch
@@ -46,13 +46,8 @@ def _check(m, k, n, seed, fp8, x=None):
     assert y.shape == (m, n) and y.dtype == torch.bfloat16
     rows = _rows(m)
     y_rows = q(xd[rows.to("cuda")].contiguous())
-    if fp8:
-        # the two launches may run different MFMA forms (16x16x128 for many tiles, 32x32x64 for few), whose fp32 sums
-        # differ in the last bits: identical up to bf16 rounding flips
-        same = (y[rows.to("cuda")] == y_rows).float().mean().item()
-        assert same > 0.99 and rel_l2(y[rows.to("cuda")], y_rows) < 5e-4, "full-M launch and row-sample launch disagree"
-    else:
-        assert torch.equal(y[rows.to("cuda")], y_rows), "full-M launch and row-sample launch disagree"
+    # (FP8 too: every tile size, tile order and launch cut runs the same sequence of MFMAs per output element)
+    assert torch.equal(y[rows.to("cuda")], y_rows), "full-M launch and row-sample launch disagree"
     if fp8:
         qw, sw = O.weight_quant_e4m3(w)
         ref = O.linear_e4m3(x[rows], qw, sw, b)["out"]

@@ -163,6 +163,43 @@ def test_int8_fp16_fp32_outputs_of_the_tiled_kernels(variant, m, n, k, dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+@pytest.mark.parametrize("x_fmt,w_fmt", [("e4m3", "e4m3"), ("e5m2", "e4m3"), ("e4m3", "e5m2")])
+@pytest.mark.parametrize("variant,m,n,k", [(8, 700, 520, 640), (11, 300, 392, 384), (8, 4100, 4352, 256), (0, 130, 264, 128)])
+def test_fp8_fp16_fp32_outputs_of_the_tiled_kernels(variant, m, n, k, dtype, x_fmt, w_fmt):
+    """fp16 / fp32 outputs of FP8 operands (what a per-tensor FP8 module that is not bf16 asks for) from the kernel on
+    16x16x128 MFMAs, on both tile sizes, with and without bias, and with the last round cut into a second launch:
+    out = T(acc * sx * sw + bias) with one rounding, against the oracle's scaled matmul at 3e-3 relative L2, and
+    against the same kernel's bf16 launch (its accumulators are the same, so its fp32 result rounded to bf16 must
+    equal the bf16 output bit for bit)."""
+    import dax_amd.ops as ops
+    from dax_amd import _capi
+
+    fdt = {"e4m3": torch.float8_e4m3fn, "e5m2": torch.float8_e5m2}
+    g = torch.Generator().manual_seed(variant + m + len(x_fmt))
+    xf = (torch.randn(m, k, generator=g) * 3).to(fdt[x_fmt])
+    wf = (torch.randn(n, k, generator=g) * 0.5).to(fdt[w_fmt])
+    sx, sw = torch.rand(m, generator=g) * 0.1 + 0.01, torch.rand(n, generator=g) * 0.01 + 1e-3
+    b = torch.randn(n, generator=g).to(dtype)
+    try:
+        _capi.debug_select_gemm(variant)
+        _capi.debug_select_gemm(2001)
+        _capi.debug_select_gemm(3002)
+        for bias in (b, None):
+            bd = bias.cuda() if bias is not None else None
+            out = ops.linear_w8a8(xf.view(torch.uint8).cuda(), sx.cuda(), wf.view(torch.uint8).cuda(), sw.cuda(), bd, x_fmt, w_fmt, dtype)
+            ref = O.scaled_mm_fp32(xf, wf, sx, sw, bias, dtype)
+            assert out.dtype == dtype and rel_l2(out, ref) < 3e-3
+            if dtype == torch.float32:
+                outb = ops.linear_w8a8(xf.view(torch.uint8).cuda(), sx.cuda(), wf.view(torch.uint8).cuda(), sw.cuda(),
+                                       bd.bfloat16() if bd is not None else None, x_fmt, w_fmt, torch.bfloat16)
+                if bias is None:
+                    assert torch.equal(out.bfloat16(), outb)
+    finally:
+        for v in (0, 2000, 3000):
+            _capi.debug_select_gemm(v)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
 @pytest.mark.parametrize("per_tensor", [False, True])
 def test_fp8_module_fp16_fp32(dtype, per_tensor):
     from dax_amd.quant.quantization import quantize_dynamic

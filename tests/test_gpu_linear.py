@@ -14,11 +14,11 @@ from tests.util import bf16_bits, rel_l2
 
 pytestmark = pytest.mark.gpu
 
-VARIANTS = [0, 2, 5, 6, 8, 9, 11]  # 0 = library default, 2 / 5 = generic kernels, 6 = two-stage 256x256, 8 / 9 = five-stage 256x256 (9: INT8 with 32x32 MFMAs), 11 = five-stage 128x128
+VARIANTS = [0, 2, 5, 8, 11]  # 0 = library default, 2 / 5 = generic kernel on 256x256 / 128x128 tiles, 8 / 11 = tiled kernel on 256x256 / 128x128 tiles
 
 
 def _skip_if_too_small(variant, m, n):
-    if variant in (6, 8, 9) and (m < 256 or n < 256):
+    if variant == 8 and (m < 256 or n < 256):
         pytest.skip("the 256x256 kernel needs m, n >= 256")
     if variant == 11 and (m < 128 or n < 128):
         pytest.skip("the 128x128 kernel needs m, n >= 128")
@@ -78,12 +78,12 @@ PATCH_SHAPES = [(256, 2048, 128), (1100, 2304, 128), (2600, 1024 + 256 * 2, 256)
                 (9100, 256 * 7, 128)]
 
 
-@pytest.mark.parametrize("order", [2002, 2003, 2004, 2005, 2006, 2007])
+@pytest.mark.parametrize("order", [2002])
 @pytest.mark.parametrize("m,n,k", PATCH_SHAPES)
 def test_patch_tile_order_bit_exact(ops, m, n, k, order):
-    """The 256x256 kernels in every tile order that deals whole 32-slot patches to the XCDs (padding workgroups exit):
-    every output tile is computed exactly once, accumulators and outputs equal the integer oracle's; FP8 equals the
-    row-group order's bits."""
+    """The 256x256 kernels in the banded tile order, which deals whole 32-slot patches to the XCDs (padding workgroups
+    exit): every output tile is computed exactly once, accumulators and outputs equal the integer oracle's; FP8 equals
+    the row-group order's bits."""
     from dax_amd import _capi
 
     _capi.debug_select_gemm(8)
@@ -117,8 +117,8 @@ TAIL_SHAPES = [(4100, 4352, 128), (8500, 4096, 256), (4725, 13824, 128), (16300,
 def test_last_round_as_a_second_launch_bit_exact(ops, m, n, k):
     """A launch of 256x256 tiles whose last round of workgroups is a few tiles: the whole rounds run as 256x256 tiles,
     the tiles left over as a second launch of their 128x128 quadrants.  Accumulators and outputs equal the integer
-    oracle's with the cut forced and by shape; FP8 outputs stay within tolerance of the single launch's (the second
-    launch adds in another order)."""
+    oracle's with the cut forced and by shape; FP8 outputs are the single launch's bits (both tile sizes run the same
+    sequence of MFMAs per output element)."""
     from dax_amd import _capi
 
     tiles = -(-m // 256) * -(-n // 256)
@@ -144,7 +144,7 @@ def test_last_round_as_a_second_launch_bit_exact(ops, m, n, k):
         np.testing.assert_array_equal(bf16_bits(out_plain), bf16_bits(O.epilogue_int8(ref_acc, sx.view(-1, 1), sw.view(1, -1), None)))
         f8[tail] = ops.linear_e4m3(dev(xf), dev(sx), dev(wf), dev(sw), dev(b)).float().cpu()
     assert not torch.isnan(f8[3002]).any()
-    assert float((f8[3002] - f8[3001]).norm() / f8[3001].norm()) < 1e-3
+    assert torch.equal(f8[3002], f8[3001]), "FP8: the cut launch and the single launch must give the same bits"
     assert torch.equal(f8[3002], f8[3000]), "one to four whole rounds: the cut is taken by shape"
 
 
@@ -170,12 +170,12 @@ def _random_shapes(count, seed):
     return shapes
 
 
-@pytest.mark.parametrize("variant", [8, 9, 6, 11, 8 | (5 << 24), 8 | (2 << 24)])
+@pytest.mark.parametrize("variant", [8, 11, 2, 8 | (2 << 24), 8 | (1 << 24)])
 @pytest.mark.parametrize("m,n,k,pad_k,pad_n", _random_shapes(14, seed=2024))
 def test_linear_i8_random_shapes_and_strides_bit_exact(ops, variant, m, n, k, pad_k, pad_n):
     """Seeded random M, N, K (edge tiles shifted inwards in both directions, short and long K) with padded leading
     dimensions, raw int8 operands straight through the C ABI: accumulators and outputs against the integer oracle.
-    (Bits 24-27 of the kernel argument: the banded and the patch tile order on the same operands.)"""
+    (Bits 24-27 of the kernel argument: the banded order and the row groups on the same operands.)"""
     from dax_amd import _capi
 
     _capi.debug_select_gemm(variant & 0xffff)
@@ -225,7 +225,7 @@ def test_linear_i8_adversarial_extremes(ops, variant):
     np.testing.assert_array_equal(bf16_bits(out), bf16_bits(O.epilogue_int8(want, sx.view(-1, 1), sw.view(1, -1), None)))
 
 
-@pytest.mark.parametrize("variant", [0, 6, 8, 9, 11])
+@pytest.mark.parametrize("variant", [0, 2, 8, 11])
 def test_linear_i8_one_hot_layout(ops, variant):
     # a single non-zero in each operand lands in exactly one accumulator: catches any
     # row/column or operand transposition inside the MFMA tiling
@@ -267,7 +267,7 @@ def test_linear_e4m3_within_tolerance(ops, variant, m, n, k):
     assert r < 3e-3, r                          # what fp32 accumulation actually delivers
 
 
-@pytest.mark.parametrize("variant", [8, 9, 6, 11])
+@pytest.mark.parametrize("variant", [8, 11, 2])
 @pytest.mark.parametrize("e5m2", [False, True])
 @pytest.mark.parametrize("m,n,k,pad_k,pad_n", _random_shapes(8, seed=77))
 def test_linear_fp8_random_shapes_accumulators(ops, variant, e5m2, m, n, k, pad_k, pad_n):
@@ -308,11 +308,13 @@ def test_linear_fp8_random_shapes_accumulators(ops, variant, e5m2, m, n, k, pad_
     assert torch.equal(out_wide[:, :n].cpu(), acc_wide[:, :n].cpu().bfloat16())   # unit scales, no bias: out = bf16(acc)
 
 
-@pytest.mark.parametrize("k", [384, 512, 640, 768, 896, 1024, 1152, 1280, 1408, 1536])
-def test_fp8_16x16x128_form_every_count_of_slice_pairs(ops, k):
-    """Every number of 128-byte pairs of K slices from 3 (below four pairs the launch takes the 32x32x64 kernel) to
-    12: first pair, steady pairs in twos, the odd one and the register moves in front of the three tail pairs all
-    occur.  Accumulators against exact float64 sums, element by element, on a 2 x 3 grid of tiles with ragged edges."""
+@pytest.mark.parametrize("variant", [8, 11])
+@pytest.mark.parametrize("k", [128, 256, 384, 512, 640, 768, 896, 1024, 1152, 1280, 1408, 1536])
+def test_fp8_16x16x128_form_every_count_of_slice_pairs(ops, k, variant):
+    """Every number of 128-byte pairs of K slices from 1 to 12 on both tile sizes: the plain loop below four pairs, then
+    first pair, steady pairs in twos, the odd one and the register moves in front of the three tail pairs all occur.
+    Accumulators against exact float64 sums, element by element, on a grid of tiles with ragged edges; both tile sizes
+    give the same bits."""
     from dax_amd import _capi
 
     m, n = 300, 700
@@ -321,14 +323,19 @@ def test_fp8_16x16x128_form_every_count_of_slice_pairs(ops, k):
     wf = (torch.randn(n, k, generator=g) * 0.5).to(torch.float8_e4m3fn)
     want = xf.double() @ wf.double().t()
     bound = xf.double().abs() @ wf.double().abs().t()
-    _capi.debug_select_gemm(8)
+    _capi.debug_select_gemm(variant)
     sx, sw = torch.rand(m, generator=g) + 0.5, torch.rand(n, generator=g) + 0.5
     b = torch.randn(n, generator=g).bfloat16()
     out, acc = ops.linear_e4m3_acc(dev(xf.view(torch.uint8)), dev(sx), dev(wf.view(torch.uint8)), dev(sw), dev(b))
     err = ((acc.cpu().double() - want).abs() / bound.clamp_min(1e-30)).max().item()
-    assert err < 2e-5, err
+    # (the MFMA adds the 128 products of an instruction in a fixed-point adder of limited width: with one to three
+    # instructions per sum that error, about 3e-5 of the sum of magnitudes, is not averaged down yet)
+    assert err < (4e-5 if k < 512 else 2e-5), err
     ref = (acc.cpu() * sx.view(-1, 1) * sw.view(1, -1) + b.float()).bfloat16()     # the epilogue on the kernel's own sums
     np.testing.assert_array_equal(bf16_bits(out), bf16_bits(ref))
+    _capi.debug_select_gemm(8 if variant == 11 else 11)
+    out2, acc2 = ops.linear_e4m3_acc(dev(xf.view(torch.uint8)), dev(sx), dev(wf.view(torch.uint8)), dev(sw), dev(b))
+    assert torch.equal(acc, acc2) and torch.equal(out, out2), "256x256 and 128x128 tiles must give the same FP8 bits"
 
 
 @pytest.mark.parametrize("k", [3968, 4096, 4224, 4352, 4480, 5120, 13824])
@@ -368,9 +375,10 @@ def test_nine_stage_128_tile_form_every_count_of_slice_pairs(ops, k):
 @pytest.mark.parametrize("m,n,k", [(8192, 5120, 5120), (4096, 5120, 13824), (2304, 2560, 640)])
 def test_fp8_16x16x128_form_against_the_32x32x64_form_every_element(ops, m, n, k, e5m2):
     """The FP8 kernel on 16x16x128 MFMAs (fragments refilled in place behind the MFMAs that read them) against the
-    32x32x64 kernel at full depth of K and with every CU busy: raw fp32 accumulators of the whole output, element by
-    element, within the rounding of an fp32 sum (a wrong or torn operand would be off by orders of magnitude);
-    three launches, identical bits each time; a row sample against the exact float64 sum."""
+    generic kernel (32x32x64 MFMAs) at full depth of K and with every CU busy: raw fp32 accumulators of the whole
+    output, element by element, within the rounding of an fp32 sum (a wrong or torn operand would be off by orders of
+    magnitude); three launches, identical bits each time, and the 128x128-tile launch the same bits again; a row sample
+    against the exact float64 sum."""
     from dax_amd import _capi
 
     g = torch.Generator("cpu").manual_seed(m + n + k)
@@ -380,11 +388,13 @@ def test_fp8_16x16x128_form_against_the_32x32x64_form_every_element(ops, m, n, k
     xd, wd = dev(xf.view(torch.uint8)), dev(wf.view(torch.uint8))
     one_m, one_n = torch.ones(m, device="cuda"), torch.ones(n, device="cuda")
     fn = ops.linear_e5m2_e4m3_acc if e5m2 else ops.linear_e4m3_acc
-    _capi.debug_select_gemm(9)
+    _capi.debug_select_gemm(2)
     _, acc_wide = fn(xd, one_m, wd, one_n, None)
     _capi.debug_select_gemm(8)
     runs = [fn(xd, one_m, wd, one_n, None)[1] for _ in range(3)]
     assert torch.equal(runs[0], runs[1]) and torch.equal(runs[0], runs[2])
+    _capi.debug_select_gemm(11)
+    assert torch.equal(runs[0], fn(xd, one_m, wd, one_n, None)[1]), "128x128 tiles: the same sums"
     bound = dev(xf.float().abs()) @ dev(wf.float().abs()).t()      # sum of |products| (fp32 on the device is enough for a bound)
     err = ((runs[0] - acc_wide).abs() / bound.clamp_min(1e-30)).max().item()
     assert err < 4e-5, err
@@ -395,7 +405,7 @@ def test_fp8_16x16x128_form_against_the_32x32x64_form_every_element(ops, m, n, k
     assert err < 2e-5, err
 
 
-@pytest.mark.parametrize("variant", [0, 5, 6])
+@pytest.mark.parametrize("variant", [0, 5, 8])
 @pytest.mark.parametrize("m,n,k", [(300, 520, 256), (17, 24, 384), (512, 1536, 1536), (4096, 1536, 1536)])
 def test_linear_e5m2_activations_within_tolerance(ops, variant, m, n, k):
     from dax_amd import _capi
@@ -422,7 +432,7 @@ def test_linear_rejects_unaligned_k(ops):
         ops.linear_i8(xq, torch.ones(8, device="cuda"), wq, torch.ones(8, device="cuda"), None)
 
 
-@pytest.mark.parametrize("variant", [0, 5, 6, 8, 9, 11])
+@pytest.mark.parametrize("variant", [0, 5, 2, 8, 11])
 def test_linear_leading_dimensions_through_the_c_abi(ops, variant):
     """Operands and output as column slices of wider buffers (ld > logical width), straight through the C ABI:
     what a caller does that writes q | k | v into one [M, 3N] tensor with three launches."""

@@ -226,7 +226,7 @@ def test_split_k_shape_captured_on_a_stream_that_already_has_a_workspace():
         assert _same(static_out, want), f"replay with seed {seed} differs from eager"
 
 
-@pytest.mark.parametrize("m,n,k,order,tail", [(700, 2304, 1024, 2005, 3000), (4100, 4352, 256, 2001, 3002)])
+@pytest.mark.parametrize("m,n,k,order,tail", [(700, 2304, 1024, 2002, 3000), (4100, 4352, 256, 2001, 3002)])
 @pytest.mark.parametrize("fp8", [False, True])
 def test_captured_graph_of_the_256_tile_kernels_replays_match_eager(fp8, m, n, k, order, tail):
     """The kernels the large shapes run on (INT8 16x16x64, FP8 16x16x128; chosen by argument here because the shape
