@@ -10,6 +10,11 @@ are resident in HBM before the timed region.  Prints ONE JSON line:
   * "model40"      INT8, 40 layers x {QKV, out, cross-q at M tokens; cross-k, cross-v at 512 text tokens; FFN up,
                    FFN down} with distinct weights per layer, timed end to end; "attn2_to_out" (the cross-attention
                    output projection of the real block, not part of that list) is timed and reported beside it
+  * "wan1_3b"      INT8, the four linears of a Wan2.1-1.3B block at 480p (M = 32760, hidden 1536, FFN 8960)
+  * "m9450"        INT8, the 14B step on one GPU's share of the rows under the reference's eight-way sequence
+                   parallelism (M = 9450)
+  * "config0"      INT8, the single linear the reference's CPU path is quoted on (M = 4096, K = N = 1536): one call of the
+                   quantiser + GEMM op per step, eagerly and replayed from a captured HIP graph
 
 each with its own ``roofline`` (GEMM launches, HIP events on the launch stream) and ``cpu_baseline`` (the CPU oracle
 on a bounded sample of the same tensors).
@@ -152,6 +157,85 @@ class Runner:
                 ev[li][2].record()
         return out
 
+    def fused_step(self):
+        """One op call per linear (quantiser + GEMM behind one dispatch): what the swapped module's forward runs."""
+        fused = (self.ops.dynamic_linear_e5m2_e4m3 if self.kind == "fp8_e5m2" else
+                 self.ops.dynamic_linear_e4m3 if self.fp8 else self.ops.dynamic_linear_i8)
+        out = None
+        for (name, k, n, x, qw, sw, b) in self.layers:
+            out = fused(x, qw, sw, b)
+        return out
+
+    def run_host_bound(self, steps, warmup):
+        """For steps of a few tens of microseconds, where event records between the launches would be what is timed: the
+        timed region runs `steps` fused steps with nothing in between (-> ms_per_step, value); the kernel durations behind
+        `roofline` come from a second pass of the same number of steps with events (run()); a third figure replays the
+        step from a captured HIP graph (what a serving loop that cannot afford the host's launch time does)."""
+        import torch
+
+        for _ in range(warmup):
+            self.fused_step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            self.fused_step()
+        torch.cuda.synchronize()
+        ms_eager = (time.perf_counter() - t0) * 1e3 / steps
+        res = self.run(steps, 2)
+        res["ms_per_step_with_events"] = res["ms_per_step"]
+        res["ms_per_step"] = ms_eager
+        res["value"] = res["total_ops"] / (ms_eager * 1e-3) / 1e12
+        res["warmup"] = warmup
+        # graph replay: capture one step on a side stream, replay `steps` times
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            self.fused_step()
+            side.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=side):
+                self.fused_step()
+            for _ in range(3):
+                graph.replay()
+            side.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(steps):
+                graph.replay()
+            side.synchronize()
+            res["ms_per_step_graph_replay"] = (time.perf_counter() - t0) * 1e3 / steps
+            # the GEMM kernel's own duration: 20 launches on pre-quantised rows captured into one graph, so that no host
+            # time sits between them (events around single launches from Python would time the host's launch gaps)
+            per = {}
+            for (name, k, n, x, qw, sw, b) in self.layers:
+                xq, sx = self.act_quant(x)
+                self.linear(xq, sx, qw, sw, b)
+                side.synchronize()
+                g2 = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(g2, stream=side):
+                    for _ in range(20):
+                        self.linear(xq, sx, qw, sw, b)
+                g2.replay()
+                side.synchronize()
+                a, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                a.record(side)
+                for _ in range(5):
+                    g2.replay()
+                e.record(side)
+                side.synchronize()
+                per[name] = a.elapsed_time(e) / 100.0
+            gemm_ms = sum(per.values())
+            res["gemm_ms"] = gemm_ms
+            res["achieved"] = res["total_ops"] / (gemm_ms * 1e-3) / 1e12
+            for name, ms in per.items():
+                e_ = res["per_linear"][name]
+                e_["gemm_ms"] = round(ms, 5)
+                e_["gemm_tops"] = round(2.0 * e_["rows"] * e_["n"] * e_["k"] / (ms * 1e-3) / 1e12, 1)
+                e_["gemm_gbps"] = round((e_["rows"] * e_["k"] + 4.0 * e_["rows"] + e_["n"] * e_["k"] + 6.0 * e_["n"] + 2.0 * e_["rows"] * e_["n"]) / (ms * 1e-3) / 1e9, 1)
+                e_["gemm_hbm_frac"] = round(e_["gemm_gbps"] / 8000.0, 4)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        return res
+
     def run(self, steps, warmup):
         import torch
 
@@ -183,6 +267,7 @@ class Runner:
             e["quant_gbps"] = round(cnt * (3.0 * rows * k + 4.0 * rows) / (e["quant_ms"] * 1e-3) / 1e9, 1)
             # algorithmic bytes of the GEMM launch: both operands, scales, bias, the bf16 output
             e["gemm_gbps"] = round(cnt * (rows * k + 4.0 * rows + n * k + 6.0 * n + 2.0 * rows * n) / (e["gemm_ms"] * 1e-3) / 1e9, 1)
+            e["gemm_hbm_frac"] = round(e["gemm_gbps"] / 8000.0, 4)  # algorithmic bytes of the launch against 8 TB/s
             e["quant_ms"], e["gemm_ms"] = round(e["quant_ms"], 4), round(e["gemm_ms"], 4)
         achieved = total_ops / (gemm_ms * 1e-3) / 1e12
         return {"ms_per_step": ms_per_step, "total_ops": total_ops, "value": total_ops / (ms_per_step * 1e-3) / 1e12,
@@ -215,6 +300,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-mfma-ceiling", action="store_true")
     ap.add_argument("--no-producers", action="store_true")
+    ap.add_argument("--kv-fused", action="store_true", help="40-layer workload: the text tokens' k and v projections as one N-concatenated launch")
+    ap.add_argument("--no-sub-records", action="store_true", help="leave out the wan1_3b / m9450 / config0 sub-records of the default run")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also run one plain 1 GiB device copy (reference point for HBM traffic counters)")
     args = ap.parse_args()
@@ -256,30 +343,42 @@ def main():
     info = _capi.device_info(0)
     shape_txt = ", ".join(f"{nm} {k}->{n}" for nm, k, n in shapes)
     per_lin_txt = "per linear: per-token act quant + MFMA GEMM + fused scale/bias/bf16 epilogue"
-    blocks = {}
-    for kind in [p for p in parts if p != "model40"]:
+    def block_record(kind, name_, tag_, m_, shapes_, dev_layers_, cpu_layers_, steps_, warmup_, traffic, cpu_rows, host_bound=False):
+        """One step over the linears of `shapes_` at m_ tokens: runs it, and returns the record with roofline and cpu_baseline."""
         r = Runner(ops, kind)
-        for name, x, w, b in dev_layers:
+        for name, x, w, b in dev_layers_:
             r.add(name, x, w, b)
-        res = r.run(args.steps, args.warmup)
+        res = r.run_host_bound(steps_, warmup_) if host_bound else r.run(steps_, warmup_)
         del r
+        txt = ", ".join(f"{nm} {k}->{n}" for nm, k, n in shapes_)
         rec = {
-            "metric": f"w8a8_linear_tops_{model_tag}_{kind}",
+            "metric": f"w8a8_linear_tops_{tag_}_{kind}",
             "value": round(res["value"], 2), "unit": "TOPS", "ms_per_step": round(res["ms_per_step"], 4),
             "steps": res["steps"], "warmup": res["warmup"], "dtype": DTYPE_NAME[kind],
-            "config": {"workload": f"{model_name} linear set, {kind.upper()} W8A8, M={m} tokens: {shape_txt}; {per_lin_txt}",
+            "config": {"workload": f"{name_} linear set, {kind.upper()} W8A8, M={m_} tokens: {txt}; {per_lin_txt}",
                        "gemm_variant": args.variant},
             "pct_of_mfma_peak": round(100.0 * res["value"] / PEAK_TOPS, 2),
             "roofline": roofline(res, kind, ("gemm_tile256s5_kernel" if kind == "int8" else "gemm_tile_fp8_kernel") +
-                                 f", average launch over the {len(shapes)} shape(s); 8-bit ops counted as 2*M*N*K",
-                                 gemm_traffic(kind) if full else None),
+                                 f", average launch over the {len(shapes_)} shape(s); 8-bit ops counted as 2*M*N*K", traffic),
             "per_linear": res["per_linear"],
         }
+        if host_bound:
+            rec["ms_per_step_graph_replay"] = round(res["ms_per_step_graph_replay"], 4)
+            rec["value_graph_replay"] = round(res["total_ops"] / (res["ms_per_step_graph_replay"] * 1e-3) / 1e12, 2)
+            rec["config"]["step"] = ("one call of the quantiser + GEMM op per linear with nothing in between (the step is the host's "
+                                     "launch time); roofline = the GEMM kernel's own duration, 20 launches captured into one HIP graph "
+                                     "and replayed between two events; graph replay = the whole step captured once into a HIP graph")
         if not args.no_cpu_baseline:
-            rows = min(args.cpu_rows or (49152 if kind == "int8" else 24576), m)
-            rec["cpu_baseline"] = cpu_baseline(kind, rows, cpu_layers,
-                                               f"first {rows} of {m} tokens of each of the {len(shapes)} linears (same tensors as the GPU step)")
-        blocks[kind] = rec
+            rows = min(cpu_rows, m_)
+            rec["cpu_baseline"] = cpu_baseline(kind, rows, cpu_layers_,
+                                               f"first {rows} of {m_} tokens of each of the {len(shapes_)} linears (same tensors as the GPU step)")
+        return rec
+
+    blocks = {}
+    for kind in [p for p in parts if p != "model40"]:
+        blocks[kind] = block_record(kind, model_name, model_tag, m, shapes, dev_layers, cpu_layers, args.steps, args.warmup,
+                                    gemm_traffic(kind) if full else None, args.cpu_rows or (49152 if kind == "int8" else 24576),
+                                    host_bound=args.model == "config0")
 
     model40 = None
     if "model40" in parts:
@@ -297,6 +396,13 @@ def main():
             base[name] = (w.to(dev), b.to(dev))
         order = [("qkv", x5120), ("out", x5120), ("cross_q", x5120), ("cross_k", text_dev), ("cross_v", text_dev),
                  ("ffn_up", x5120), ("ffn_down", x13824)]
+        if args.kv_fused:
+            # k and v of the text tokens as ONE launch against the N-concatenated weight (per-channel weight scales and
+            # per-token activation scales make it bit-identical to the two launches; the self-attention QKV of this
+            # list is the same construction)
+            base["cross_kv"] = (torch.cat([base["cross_k"][0], base["cross_v"][0]], 0), torch.cat([base["cross_k"][1], base["cross_v"][1]], 0))
+            order = [o for o in order if o[0] not in ("cross_k", "cross_v")]
+            order.insert(3, ("cross_kv", text_dev))
         r = Runner(ops, "int8")
         q0 = {name: r.quantise_weight(base[name][0]) for name, _ in order}
         for layer in range(40):
@@ -339,6 +445,27 @@ def main():
                 "int8", rows, one, f"ONE layer of the 40 (7 linears; first {rows} of {m} tokens, all {TEXT_TOKENS} text tokens); "
                                    "the 40 layers cost the same each, so the rate stands for the whole step")
 
+    # ---- the other configurations the reference is quoted on, as sub-records of the default run (INT8)
+    extra = {}
+    if full and not args.only and not args.no_sub_records:
+        # one GPU's share of the rows under the reference's eight-way sequence parallelism: the first 9450 tokens
+        sl_dev = [(nm, x[:9450], w, b) for nm, x, w, b in dev_layers]
+        sl_cpu = [(nm, x[:9450], w, b) for nm, x, w, b in cpu_layers]
+        extra["m9450"] = block_record("int8", model_name + ", 1/8 of the rows", model_tag + "_m9450", 9450, shapes, sl_dev, sl_cpu,
+                                      args.steps, args.warmup, None, 4096)
+        for key in ("1.3b", "config0"):
+            name_, tag_, m_, shapes_ = MODELS[key]
+            cl, dl = [], []
+            for i, (nm, k, n) in enumerate(shapes_):
+                x, w, b = synth_inputs(m_, k, n, seed=i)
+                cl.append((nm, x, w, b))
+                dl.append((nm, x.to(dev), w.to(dev), b.to(dev)))
+            small = key == "config0"
+            extra["config0" if small else "wan1_3b"] = block_record(
+                "int8", name_, tag_, m_, shapes_, dl, cl, 200 if small else args.steps, 20 if small else args.warmup, None,
+                4096 if small else 16384, host_bound=small)
+            del cl, dl
+
     if args.calib_copy:
         src = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
         dst = torch.empty_like(src)
@@ -358,13 +485,14 @@ def main():
     }
     if "cpu_baseline" in head:
         res["cpu_baseline"] = head["cpu_baseline"]
-    for key in ("per_linear", "attn2_to_out", "total_pops"):
+    for key in ("per_linear", "attn2_to_out", "total_pops", "ms_per_step_graph_replay", "value_graph_replay"):
         if key in head:
             res[key] = head[key]
     for kind, rec in blocks.items():
         res["fp8" if kind == "fp8" else kind] = rec
     if model40 is not None:
         res["model40"] = model40
+    res.update(extra)
     res["device"] = {"arch": info["arch"], "cu_count": info["cu_count"], "max_clock_mhz": info["clock_khz"] / 1000.0}
     res["input_generation_s"] = round(t_gen, 1)
 

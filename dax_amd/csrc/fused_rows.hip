@@ -243,7 +243,7 @@ __global__ __launch_bounds__(256, (PRE == PRE_LN && NCH <= 12 && !WRITE_Y) ? 3 :
         for (int i = 0; i < NCH; ++i) {
             const int c = i * 64 + lane;
             if (c < nch) {
-                store_stream_8(qr + c, quant_chunk<FMT>(v[i], s, inv));
+                store_stream_8(qr + c, quant_chunk<FMT, false, DAXQ_BF16, false>(v[i], s, inv));  // own scale at the format's maximum: no clamp
             } else if (c < npad) {
                 store_stream_8(qr + c, make_uint2(0, 0));
             }

@@ -115,9 +115,15 @@ __device__ __forceinline__ float wave_sum_f32(float x) {
 // clamp(rint(x * inv), -128, 127) as the low byte of a float: the product is clamped first (same result, the
 // bounds are integers) and 1.5 * 2^23 is added, which rounds it to an integer, half to even, in the low mantissa
 // bits; those bits are the two's-complement value.  Two operations fewer than round + convert.
+// CLAMP = false: a row quantised with its own bf16-rounded (or fp32) scale of abs-max / 127 never leaves [-127.4, 127.4]
+// (the rounding of the scale moves x * inv at the row maximum by at most 2^-8 of it: checked for every bf16 abs-max), so
+// the clamp is dead code there and is left out.  (A NaN product -- an infinite element of a row whose scale is infinite
+// -- then gives the byte 0 instead of -128; such a row's output is non-finite through its scale either way.)
+template <bool CLAMP = true>
 __device__ __forceinline__ uint32_t q_i8_bits(float x, float inv) {
     float r = x * inv;
-    r = fminf(fmaxf(r, -128.0f), 127.0f);
+    if constexpr (CLAMP) r = fminf(fmaxf(r, -128.0f), 127.0f);
+    else asm("" : "+v"(r));  // the product is rounded before the addition, as in the reference: no contraction into one fma
     return __float_as_uint(r + 12582912.0f);
 }
 
@@ -127,7 +133,10 @@ __device__ __forceinline__ uint32_t q_i8_bits(float x, float inv) {
 // significand of s is all ones, which a scale whose low 16 bits are zero never has).  The reference's
 // true division costs about ten instructions per element when spelled x / s.
 // TRUE_DIV: spell the division out (leaf quantiser with an arbitrary fp32 scale, used once per weight).
-template <int FMT, bool TRUE_DIV>
+// CLAMP = false: with the row's own scale of abs-max / qmax the quotient at the row maximum stays below qmax * (1 + 2^-8)
+// (449.5 for e4m3fn, 57530 for e5m2: checked for every bf16 abs-max), which the cast's round-to-nearest-even takes to
+// the format's largest finite value by itself (the next step up lies beyond 464 / 61440), so the clamp is left out.
+template <int FMT, bool TRUE_DIV, bool CLAMP = true>
 __device__ __forceinline__ float q_f8_pre(float x, float s, float inv) {
     constexpr float kMax = FMT == 2 ? 57344.0f : 448.0f;
     float v;
@@ -140,6 +149,7 @@ __device__ __forceinline__ float q_f8_pre(float x, float s, float inv) {
     }
     // With a scale from the caller a NaN element must stay NaN through the clamp, as in the reference, and become
     // the format's NaN byte; with the row's own scale a NaN element has already made that scale NaN.
+    if constexpr (!CLAMP) return v;
     if constexpr (TRUE_DIV) return min_nan(max_nan(v, -kMax), kMax);
     return fminf(fmaxf(v, -kMax), kMax);
 }
@@ -153,7 +163,7 @@ __device__ __forceinline__ int cvt_pk_f8(float a, float b, int old, bool hi) {
 }
 
 // 8 bf16 / fp16 values (one 16-byte chunk) -> 8 quantised bytes
-template <int FMT, bool TRUE_DIV = false, int XT = DAXQ_BF16>
+template <int FMT, bool TRUE_DIV = false, int XT = DAXQ_BF16, bool CLAMP = true>
 __device__ __forceinline__ uint2 quant_chunk(const uint4& v, float s, float inv) {
     const uint32_t w[4] = {v.x, v.y, v.z, v.w};
     uint32_t o[2];
@@ -172,13 +182,13 @@ __device__ __forceinline__ uint2 quant_chunk(const uint4& v, float s, float inv)
             f3 = x_bits_to_f32<XT>(w[2 * h + 1] >> 16);
         }
         if (FMT != 0) {
-            int p = cvt_pk_f8<FMT>(q_f8_pre<FMT, TRUE_DIV>(f0, s, inv), q_f8_pre<FMT, TRUE_DIV>(f1, s, inv), 0, false);
-            p = cvt_pk_f8<FMT>(q_f8_pre<FMT, TRUE_DIV>(f2, s, inv), q_f8_pre<FMT, TRUE_DIV>(f3, s, inv), p, true);
+            int p = cvt_pk_f8<FMT>(q_f8_pre<FMT, TRUE_DIV, CLAMP>(f0, s, inv), q_f8_pre<FMT, TRUE_DIV, CLAMP>(f1, s, inv), 0, false);
+            p = cvt_pk_f8<FMT>(q_f8_pre<FMT, TRUE_DIV, CLAMP>(f2, s, inv), q_f8_pre<FMT, TRUE_DIV, CLAMP>(f3, s, inv), p, true);
             o[h] = (uint32_t)p;
         } else {
             // byte 0 of each of the four words: three v_perm_b32
-            const uint32_t p01 = __builtin_amdgcn_perm(q_i8_bits(f1, inv), q_i8_bits(f0, inv), 0x0c0c0400u);
-            const uint32_t p23 = __builtin_amdgcn_perm(q_i8_bits(f3, inv), q_i8_bits(f2, inv), 0x0c0c0400u);
+            const uint32_t p01 = __builtin_amdgcn_perm(q_i8_bits<CLAMP>(f1, inv), q_i8_bits<CLAMP>(f0, inv), 0x0c0c0400u);
+            const uint32_t p23 = __builtin_amdgcn_perm(q_i8_bits<CLAMP>(f3, inv), q_i8_bits<CLAMP>(f2, inv), 0x0c0c0400u);
             o[h] = __builtin_amdgcn_perm(p23, p01, 0x05040100u);
         }
     }

@@ -64,14 +64,18 @@ __global__ __launch_bounds__(256) void quant_rows_wave(const uint16_t* __restric
     const float inv = 1.0f / s;  // IEEE division, not v_rcp_f32
 
     uint2* qr = reinterpret_cast<uint2*>(q + row * ld_q);
-    // The reciprocal sequence of the FP8 forms is verified exhaustively for bf16 elements under bf16-rounded scales:
-    // fp16 rows, and bf16 rows whose scale stays in fp32 (round_x == 0, uniform over the launch), divide.
-    constexpr bool kRecip = FMT != 0 && !SCALE_IN && XT == DAXQ_BF16;
-    if (kRecip && !round_x) {
+    // Two forms of the store loop.  The fast one, for a bf16 row quantised with its own scale at no more than the
+    // format's maximum: no clamp (dead code there, quant_rows.h), and for FP8 the reciprocal sequence, which is verified
+    // exhaustively for bf16 elements under bf16-rounded scales.  The general one -- fp16 rows, a scale from the caller,
+    // a quant_max beyond the format's maximum, an FP8 row whose scale stays in fp32 -- divides and clamps.  The choice
+    // is uniform over the launch.
+    constexpr float kFmtMax = FMT == 0 ? 127.0f : FMT == 1 ? 448.0f : 57344.0f;
+    constexpr bool kFastForm = !SCALE_IN && XT == DAXQ_BF16;
+    if (kFastForm && qmax <= kFmtMax && (FMT == 0 || round_x)) {
 #pragma unroll
         for (int i = 0; i < NCH; ++i) {
             const int c = i * 64 + lane;
-            if (c < nch) store_stream_8(qr + c, quant_chunk<FMT, true, XT>(v[i], s, inv));
+            if (c < nch) store_stream_8(qr + c, quant_chunk<FMT, false, XT, false>(v[i], s, inv));
             else if (c < npad) store_stream_8(qr + c, make_uint2(0, 0));
         }
         return;
@@ -80,7 +84,7 @@ __global__ __launch_bounds__(256) void quant_rows_wave(const uint16_t* __restric
     for (int i = 0; i < NCH; ++i) {
         const int c = i * 64 + lane;
         if (c < nch) {
-            store_stream_8(qr + c, quant_chunk<FMT, SCALE_IN || XT != DAXQ_BF16, XT>(v[i], s, inv));
+            store_stream_8(qr + c, quant_chunk<FMT, (FMT != 0), XT>(v[i], s, inv));
         } else if (c < npad) {
             store_stream_8(qr + c, make_uint2(0, 0));
         }
