@@ -336,7 +336,9 @@ __global__ __launch_bounds__(256) void gemm_tile256s5_kernel(const GemmArgs p) {
                 }
             }
             if constexpr (N16) {
-                const int j = g / NB, i = g % NB;  // B block j, A block i
+                // B block j, A block i: consecutive MFMAs share the weight fragment (holding the activation fragment instead
+                // measured the same: 2985 - 2994 against 2997 - 3000 T-op/s)
+                const int j = g / NB, i = g % NB;
                 const v4i bfr = ODD.value ? (j < 4 ? fb10[j & 3] : fb11[j & 3]) : (j < 4 ? fb00[j & 3] : fb01[j & 3]);
                 const v4i afr = ODD.value ? (i < 4 ? fa10[i & 3] : fa11[i & 3]) : (i < 4 ? fa00[i & 3] : fa01[i & 3]);
                 // accumulator tied in place in AGPRs: left to the register allocator, the 64 four-register
