@@ -302,13 +302,15 @@ enum { K_DEFAULT = 0, K_GENERIC256 = 2, K_GENERIC128 = 5, K_TILED_256 = 8, K_TIL
 // the row groups, most at long K, and none of the row groups' 3-4 % dips where the XCD ranges start on the same
 // columns).  It deals whole patches of 32 tiles to the XCDs, so one XCD can end up with more tiles than an eighth of
 // them: it is taken when the slowest XCD needs at most 5 % more tile times than the row groups do; with fewer than
-// five bands (N < 5120), K below 2048 or few rounds the row groups were as fast or faster (M = 9450, a 1/8 share of
-// the rows: -3 to -16 %; K = 1536: -2 %; N = K = 4096: -2 %).
+// five bands (N < 5120), K below 2048 or few rounds the row groups were as fast or faster (K = 1536: -2 %; N = K = 4096:
+// -2 %; M = 9450, a 1/8 share of the rows, 3 to 9 rounds: -0.8 to +2 % per linear and +0.2 / +1.0 % INT8 / FP8 over the
+// four, now that the rows under the last whole step form dense patches, -3 to -16 % before; M = 4725: -4 to -5 %; M =
+// 20000: +3 % at N >= 13824, -3 % at N = 5120, where the row groups run their last tiles as a second launch).
 static int order_by_shape(int64_t m, int64_t n, int64_t k) {
     const int64_t tm = (m + 255) / 256, tn = (n + 255) / 256, tiles = tm * tn;
-    // (tm >= 32: at least one super-row of whole 8 x 4 patches; tm <= 100000 and tn <= 4096: the range the host-side
+    // (tm >= 64: at least two super-rows of whole 8 x 4 patches; tm <= 100000 and tn <= 4096: the range the host-side
     // coverage check of the order reaches, with sampled grids)
-    if (k < 2048 || tn < 20 || tm < 32 || tiles < 2048 || tm > 100000 || tn > 4096) return kOrderRowGroups;
+    if (k < 2048 || tn < 20 || tm < 64 || tiles < 2048 || tm > 100000 || tn > 4096) return kOrderRowGroups;
     return banded_xcd_rounds((int)tm, (int)tn, 4) * 100 <= (tiles + 255) / 256 * 105 ? kOrderBanded : kOrderRowGroups;
 }
 

@@ -20,34 +20,74 @@ namespace daxq {
 // tile rows are cut into super-rows of 32, a super-row into steps of one main-patch height, and a step emits one patch of
 // every main band followed by the patch of each narrow band that starts at that row.  Patch 8 * round + xcd goes to XCD
 // xcd, so the eight XCDs of a round sit in eight consecutive entries: on the same activation rows and on different weight
-// bands when there are at least eight.  Slots beyond a patch's tiles (below the last tile row) are padding: their
-// workgroups exit at once.  A full super-row emits tiles_n patches.
+// bands when there are at least eight.  A full super-row emits tiles_n patches.
+// The last, partial super-row (tiles_m % 32 rows): whole steps of hmain rows as above; the r < hmain rows left under them
+// form dense patches of r rows x (32 / r) columns over the main bands and over every narrow band that would start a
+// patch at that row (the bands further right are still inside a patch that started higher up).  Slots beyond a patch's
+// tiles are padding: their workgroups exit at once.
+// (Cutting the patches of the last round further so that every XCD works in the launch's last tile time was measured
+// in two forms, tile by tile and in pieces of consecutive rows: both slower than whole patches.)
+struct BandedGrid {
+    int tiles_m, tiles_n, W, hmain, nb_main, rem;
+    int full_sr;               // whole super-rows
+    int full_steps, r, wr;     // partial super-row: whole steps, rows left under them, width of their dense patches
+    int dense_cols, dense_n;   // columns the dense patches cover, and their count
+    int tail_before;           // patches of the partial super-row in front of the dense ones
+    int patches;               // all patches of the grid (the launchers keep grids below 2^31 workgroups)
+};
 DAXQ_HOST_DEVICE int banded_before(int s, int hmain, int nb_main, int rem) {  // patches of a super-row before step s
     int c = s * nb_main;
     for (int wj = 4; wj >= 1; wj >>= 1)
         if (rem & wj) c += (s * hmain * wj + 31) >> 5;  // ceil(s * hmain / (32 / wj))
     return c;
 }
-DAXQ_HOST_DEVICE bool tile_of_block_banded(int pid, int tiles_m, int tiles_n, int W, int& tm, int& tn) {
-    const int xcd = pid & 7, local = pid >> 3, slot = local & 31;
-    const int patch = (local >> 5) * 8 + xcd;
-    const int hmain = 32 / W, nb_main = tiles_n / W, rem = tiles_n - nb_main * W;
-    const int sr = patch / tiles_n, u = patch - sr * tiles_n;
-    int s = W - 1;  // steps of a super-row: 32 / hmain = W
-    while (s > 0 && banded_before(s, hmain, nb_main, rem) > u) --s;
-    int v = u - banded_before(s, hmain, nb_main, rem);
-    const int row0 = sr * 32 + s * hmain;
-    int h = hmain, col0 = v * W;
-    if (v >= nb_main) {
-        v -= nb_main;
-        col0 = nb_main * W;
+DAXQ_HOST_DEVICE BandedGrid banded_make(int tiles_m, int tiles_n, int W) {
+    BandedGrid g;
+    g.tiles_m = tiles_m, g.tiles_n = tiles_n, g.W = W;
+    g.hmain = 32 / W, g.nb_main = tiles_n / W, g.rem = tiles_n - g.nb_main * W;
+    g.full_sr = tiles_m >> 5;
+    const int left = tiles_m & 31;
+    g.full_steps = left / g.hmain;
+    g.r = left - g.full_steps * g.hmain;
+    g.wr = g.r ? 32 / g.r : 0;
+    g.dense_cols = g.nb_main * W;
+    for (int wj = 4; wj >= 1; wj >>= 1)
+        if ((g.rem & wj) && (g.full_steps * g.hmain) % (32 / wj) == 0) g.dense_cols += wj;
+    g.dense_n = g.r ? (g.dense_cols + g.wr - 1) / g.wr : 0;
+    g.tail_before = banded_before(g.full_steps, g.hmain, g.nb_main, g.rem);
+    g.patches = g.full_sr * tiles_n + g.tail_before + g.dense_n;
+    return g;
+}
+// Patch `patch` of the grid: slot s of it is tile (row0 + s % h, col0 + s / h) when s % h < rows and s / h < cols.
+DAXQ_HOST_DEVICE bool banded_patch(const BandedGrid& g, int patch, int& row0, int& col0, int& h, int& rows, int& cols) {
+    if (patch >= g.patches) return false;
+    const int sr = patch / g.tiles_n, u = patch - sr * g.tiles_n;
+    int s = g.W - 1;  // steps of a super-row: 32 / hmain = W
+    if (sr == g.full_sr) {
+        const int v = u - g.tail_before;
+        if (v >= 0) {  // dense patches of the rows under the whole steps
+            row0 = sr * 32 + g.full_steps * g.hmain;
+            col0 = v * g.wr;
+            h = rows = g.r;
+            cols = g.dense_cols - col0 < g.wr ? g.dense_cols - col0 : g.wr;
+            return true;
+        }
+        s = g.full_steps - 1;
+    }
+    while (s > 0 && banded_before(s, g.hmain, g.nb_main, g.rem) > u) --s;
+    int v = u - banded_before(s, g.hmain, g.nb_main, g.rem);
+    row0 = sr * 32 + s * g.hmain;
+    h = g.hmain, col0 = v * g.W, cols = g.W;
+    if (v >= g.nb_main) {
+        v -= g.nb_main;
+        col0 = g.nb_main * g.W;
         h = 0;
         for (int wj = 4; wj >= 1; wj >>= 1) {
-            if (!(rem & wj)) continue;
+            if (!(g.rem & wj)) continue;
             const int hj = 32 / wj;
-            if ((s * hmain) % hj == 0) {
+            if ((s * g.hmain) % hj == 0) {
                 if (v == 0) {
-                    h = hj;
+                    h = hj, cols = wj;
                     break;
                 }
                 --v;
@@ -56,38 +96,34 @@ DAXQ_HOST_DEVICE bool tile_of_block_banded(int pid, int tiles_m, int tiles_n, in
         }
         if (h == 0) return false;  // beyond the step's patches (cannot happen for u < patches of the super-row)
     }
-    tm = row0 + slot % h;
-    tn = col0 + slot / h;
-    return tm < tiles_m;
+    rows = g.tiles_m - row0 < h ? g.tiles_m - row0 : h;
+    return true;
 }
+DAXQ_HOST_DEVICE bool tile_of_block_banded(int pid, int tiles_m, int tiles_n, int W, int& tm, int& tn) {
+    const BandedGrid g = banded_make(tiles_m, tiles_n, W);
+    const int xcd = pid & 7, local = pid >> 3, slot = local & 31;
+    int row0, col0, h, rows, cols;
+    if (!banded_patch(g, (local >> 5) * 8 + xcd, row0, col0, h, rows, cols)) return false;
+    const int r = slot % h, c = slot / h;
+    tm = row0 + r;
+    tn = col0 + c;
+    return r < rows && c < cols;
+}
+inline int64_t banded_grid(int tiles_m, int tiles_n, int W) { return ((int64_t)banded_make(tiles_m, tiles_n, W).patches + 7) / 8 * 256; }
 // Tile times the slowest XCD needs in the banded order: ceil(its tiles / 32 CUs).  Patches of the full super-rows hold
-// 32 tiles each; only those of the last, partial super-row are counted one by one.
+// 32 tiles each; those of the last, partial super-row are counted one by one.
 inline int64_t banded_xcd_rounds(int tiles_m, int tiles_n, int W) {
-    const int hmain = 32 / W, nb_main = tiles_n / W, rem = tiles_n - nb_main * W;
-    const int64_t full = (int64_t)(tiles_m >> 5) * tiles_n;
+    const BandedGrid g = banded_make(tiles_m, tiles_n, W);
+    const int full = g.full_sr * tiles_n;  // patches of 32 tiles
     int64_t load[8];
-    for (int x = 0; x < 8; ++x) load[x] = (full / 8 + (x < full % 8 ? 1 : 0)) * 32;
-    const int left = tiles_m & 31;
-    int next = (int)(full % 8);
-    for (int s = 0; s * hmain < left; ++s) {
-        const int row = s * hmain, rows_main = left - row < hmain ? left - row : hmain;
-        for (int b = 0; b < nb_main; ++b, next = (next + 1) & 7) load[next] += rows_main * W;
-        for (int wj = 4; wj >= 1; wj >>= 1) {
-            if (!(rem & wj) || row % (32 / wj)) continue;
-            const int hj = 32 / wj;
-            load[next] += (left - row < hj ? left - row : hj) * wj;
-            next = (next + 1) & 7;
-        }
+    for (int x = 0; x < 8; ++x) load[x] = (int64_t)(full / 8 + (x < full % 8 ? 1 : 0)) * 32;
+    for (int patch = full; patch < g.patches; ++patch) {
+        int row0, col0, h, rows, cols;
+        if (banded_patch(g, patch, row0, col0, h, rows, cols)) load[patch & 7] += rows * cols;
     }
     int64_t most = 0;
     for (int x = 0; x < 8; ++x) most = load[x] > most ? load[x] : most;
     return (most + 31) / 32;
-}
-inline int64_t banded_grid(int tiles_m, int tiles_n, int W) {
-    const int hmain = 32 / W, nb_main = tiles_n / W, rem = tiles_n - nb_main * W;
-    const int left = tiles_m & 31;
-    const int64_t patches = (int64_t)(tiles_m >> 5) * tiles_n + banded_before((left + hmain - 1) / hmain, hmain, nb_main, rem);
-    return (patches + 7) / 8 * 256;
 }
 
 }  // namespace daxq

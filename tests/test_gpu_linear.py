@@ -72,10 +72,11 @@ def test_linear_i8_bit_exact(ops, variant, m, n, k):
     np.testing.assert_array_equal(bf16_bits(out2), bf16_bits(ref2))
 
 
-# tile grids (in 256-tiles) whose remainder band is 0 to 7 columns wide, with and without a partial last patch
+# tile grids (in 256-tiles) whose remainder band is 0 to 7 columns wide, with and without a partial last patch; the last
+# two: tile rows under the last whole step of 8 (dense patches of 5 x 6 and 4 x 8 tiles) below whole patches
 PATCH_SHAPES = [(256, 2048, 128), (1100, 2304, 128), (2600, 1024 + 256 * 2, 256), (700, 2048 + 256 * 3, 128), (2100, 256 * 4, 128),
                 (1300, 2048 + 256 * 5, 128), (1500, 256 * 6, 256), (520, 4096 + 256 * 7, 128), (8500, 304, 128), (300, 5120, 384),
-                (9100, 256 * 7, 128)]
+                (9100, 256 * 7, 128), (9450, 5120, 128), (3000, 256 * 7, 128)]
 
 
 @pytest.mark.parametrize("order", [2002])
