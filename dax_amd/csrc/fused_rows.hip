@@ -16,11 +16,43 @@
 // HBM traffic: 2 B read + 1 B written per element (+ 2 B when the bf16 result is wanted), against
 // 2 + 2 + 2 + 1 for producer and quantiser run separately.  The GELU form is VALU-bound on gfx950
 // (one v_exp_f32 and one v_rcp_f32 per element), not HBM-bound.
+#include <type_traits>
+
 #include "quant_rows.h"
 
 namespace daxq {
 
 enum { PRE_LN = 1, PRE_GELU = 2 };
+
+// v_dot2_f32_bf16 d, a, b, c: both products of the bf16 pairs a and b, exact, added to the fp32 value c.  The compiler
+// only selects the form whose destination is the addend (v_dot2c), which costs x - mean a copy per element, so the
+// instruction is written out -- with its hazard: a different VALU instruction that reads a DOT instruction's result
+// needs three wait states behind it, and the compiler keeps those only for instructions it can see (the consumer of a
+// single-instruction asm statement was once scheduled directly behind it and read the register's old value).  Hence
+// whole chunks per statement, closed by the wait states, and results that no input register may share.
+// Row sums of a chunk: sum += x, sq += x * x over its eight values (a DOT reading the previous DOT's result as its
+// addend needs no wait; dot_sums_done() closes the chain before anything else reads the sums).
+__device__ __forceinline__ void dot_sums(const uint4& v, float& sum, float& sq) {
+    asm("v_dot2_f32_bf16 %0, %2, %6, %0\n\tv_dot2_f32_bf16 %1, %2, %2, %1\n\t"
+        "v_dot2_f32_bf16 %0, %3, %6, %0\n\tv_dot2_f32_bf16 %1, %3, %3, %1\n\t"
+        "v_dot2_f32_bf16 %0, %4, %6, %0\n\tv_dot2_f32_bf16 %1, %4, %4, %1\n\t"
+        "v_dot2_f32_bf16 %0, %5, %6, %0\n\tv_dot2_f32_bf16 %1, %5, %5, %1"
+        : "+v"(sum), "+v"(sq)
+        : "v"(v.x), "v"(v.y), "v"(v.z), "v"(v.w), "v"(0x3f803f80u));
+}
+__device__ __forceinline__ void dot_sums_done(float& sum, float& sq) { asm volatile("s_nop 2" : "+v"(sum), "+v"(sq)); }
+// f[e] = x[e] + c for the eight values of a chunk: the pair times (1, 0) or (0, 1) plus c, one instruction per element.
+// (A non-finite neighbour turns the element into NaN through its zero product; the callers' rows are NaN throughout
+// then anyway, their mean being non-finite.)
+__device__ __forceinline__ void dot_add8(const uint4& v, float c, float (&f)[8]) {
+    asm("v_dot2_f32_bf16 %0, %8, %12, %14\n\tv_dot2_f32_bf16 %1, %8, %13, %14\n\t"
+        "v_dot2_f32_bf16 %2, %9, %12, %14\n\tv_dot2_f32_bf16 %3, %9, %13, %14\n\t"
+        "v_dot2_f32_bf16 %4, %10, %12, %14\n\tv_dot2_f32_bf16 %5, %10, %13, %14\n\t"
+        "v_dot2_f32_bf16 %6, %11, %12, %14\n\tv_dot2_f32_bf16 %7, %11, %13, %14\n\t"
+        "s_nop 2"
+        : "=&v"(f[0]), "=&v"(f[1]), "=&v"(f[2]), "=&v"(f[3]), "=&v"(f[4]), "=&v"(f[5]), "=&v"(f[6]), "=&v"(f[7])
+        : "v"(v.x), "v"(v.y), "v"(v.z), "v"(v.w), "v"(0x00003f80u), "v"(0x3f800000u), "v"(c));
+}
 
 __device__ __forceinline__ void unpack8(const uint4& v, float (&f)[8]) {
     const uint32_t w[4] = {v.x, v.y, v.z, v.w};
@@ -62,9 +94,9 @@ __device__ __forceinline__ float gelu_tanh_f32(float x) {
 // PRE_GELU: y = bf16( gelu_tanh(x) ).
 // Requires k % 8 == 0, 16-byte aligned rows of x (and y), 8-byte aligned rows of q, kfill/8 <= NCH*64.
 // The quantise-only LayerNorm form for rows of up to 12 x 64 chunks holds two rows (the current and the requested
-// next one) and is kept at three wavefronts per SIMD (170 registers).
+// next one); rows of whole 512-element columns take ln_rows_exact below instead.
 template <int NCH, int FMT, int PRE, bool WRITE_Y>
-__global__ __launch_bounds__(256, (PRE == PRE_LN && NCH <= 12 && !WRITE_Y) ? 3 : 1) void fused_rows_wave(
+__global__ __launch_bounds__(256, (PRE == PRE_LN && NCH <= 12 && !WRITE_Y) ? 2 : 1) void fused_rows_wave(
     const uint16_t* __restrict__ x, int64_t m, int k, int64_t ld_x, const float* __restrict__ mul,
     const float* __restrict__ add, int64_t rows_per_group, float eps, uint16_t* __restrict__ y, int64_t ld_y,
     uint8_t* __restrict__ q, int64_t ld_q, int kfill, float* __restrict__ scale, float qmax) {
@@ -130,14 +162,8 @@ __global__ __launch_bounds__(256, (PRE == PRE_LN && NCH <= 12 && !WRITE_Y) ? 3 :
             // registers with the mean subtracted first.  The choice is uniform over the wavefront.
             float sum = 0.0f, sq = 0.0f;
 #pragma unroll
-            for (int i = 0; i < NCH; ++i) {  // padding chunks are zero and add nothing
-                const uint32_t w[4] = {v[i].x, v[i].y, v[i].z, v[i].w};
-#pragma unroll
-                for (int h = 0; h < 4; ++h) {
-                    asm("v_dot2_f32_bf16 %0, %1, %2, %0" : "+v"(sum) : "v"(w[h]), "v"(0x3f803f80u));
-                    asm("v_dot2_f32_bf16 %0, %1, %1, %0" : "+v"(sq) : "v"(w[h]));
-                }
-            }
+            for (int i = 0; i < NCH; ++i) dot_sums(v[i], sum, sq);  // padding chunks are zero and add nothing
+            dot_sums_done(sum, sq);
             float mean = wave_sum_f32(sum) / (float)k;
             float var = wave_sum_f32(sq) / (float)k - mean * mean;
             if (!(mean * mean <= 7.0f * var)) {
@@ -165,48 +191,44 @@ __global__ __launch_bounds__(256, (PRE == PRE_LN && NCH <= 12 && !WRITE_Y) ? 3 :
             forget_values(v);
             const float rstd = 1.0f / sqrtf(var + eps);  // IEEE sqrt and division
             const int64_t g = row / rows_per_group;
-            const bool in_lds = g == staged;
+            // The two forms of the pass are separate loops, chosen once per row.  With the choice inside the loop the
+            // registers of the two vectors are written by global loads on one path and by LDS reads on the other, and
+            // the compiler then waits for every load in flight -- the requested next row among them -- before each
+            // chunk's LDS reads.
+            auto modulate = [&](auto IN_LDS) __attribute__((always_inline)) {
 #pragma unroll
-            for (int i = 0; i < NCH; ++i) {
-                const int c = i * 64 + lane;
-                if (c < nch) {
-                    float f[8], a[8], b[8];
-                    {
-                        // x - mean in one instruction per element: the pair times (1, 0) or (0, 1) plus -mean.  (A
-                        // non-finite neighbour turns the element into NaN through its zero product; such a row is
-                        // NaN throughout anyway, its mean being non-finite.)
-                        const uint32_t w[4] = {v[i].x, v[i].y, v[i].z, v[i].w};
-                        const float nm = -mean;
+                for (int i = 0; i < NCH; ++i) {
+                    const int c = i * 64 + lane;
+                    if (c < nch) {
+                        float f[8], a[8], b[8];
+                        dot_add8(v[i], -mean, f);  // x - mean
+                        if constexpr (decltype(IN_LDS)::value) {
+                            const float* sv = s_vec + (i * 128 + lane) * 4;
+                            const float4 a0 = *reinterpret_cast<const float4*>(sv);
+                            const float4 a1 = *reinterpret_cast<const float4*>(sv + 256);
+                            const float4 b0 = *reinterpret_cast<const float4*>(sv + kpad);
+                            const float4 b1 = *reinterpret_cast<const float4*>(sv + kpad + 256);
+                            a[0] = a0.x, a[1] = a0.y, a[2] = a0.z, a[3] = a0.w, a[4] = a1.x, a[5] = a1.y, a[6] = a1.z, a[7] = a1.w;
+                            b[0] = b0.x, b[1] = b0.y, b[2] = b0.z, b[3] = b0.w, b[4] = b1.x, b[5] = b1.y, b[6] = b1.z, b[7] = b1.w;
+                        } else {
 #pragma unroll
-                        for (int h = 0; h < 4; ++h) {
-                            asm("v_dot2_f32_bf16 %0, %1, %2, %3" : "=v"(f[2 * h]) : "v"(w[h]), "v"(0x00003f80u), "v"(nm));
-                            asm("v_dot2_f32_bf16 %0, %1, %2, %3" : "=v"(f[2 * h + 1]) : "v"(w[h]), "v"(0x3f800000u), "v"(nm));
+                            for (int e = 0; e < 8; ++e) {
+                                a[e] = mul ? mul[g * k + c * 8 + e] : 1.0f;
+                                b[e] = add ? add[g * k + c * 8 + e] : 0.0f;
+                            }
                         }
-                    }
-                    if (in_lds) {
-                        const float* sv = s_vec + (i * 128 + lane) * 4;
-                        const float4 a0 = *reinterpret_cast<const float4*>(sv);
-                        const float4 a1 = *reinterpret_cast<const float4*>(sv + 256);
-                        const float4 b0 = *reinterpret_cast<const float4*>(sv + kpad);
-                        const float4 b1 = *reinterpret_cast<const float4*>(sv + kpad + 256);
-                        a[0] = a0.x, a[1] = a0.y, a[2] = a0.z, a[3] = a0.w, a[4] = a1.x, a[5] = a1.y, a[6] = a1.z, a[7] = a1.w;
-                        b[0] = b0.x, b[1] = b0.y, b[2] = b0.z, b[3] = b0.w, b[4] = b1.x, b[5] = b1.y, b[6] = b1.z, b[7] = b1.w;
-                    } else {
 #pragma unroll
                         for (int e = 0; e < 8; ++e) {
-                            a[e] = mul ? mul[g * k + c * 8 + e] : 1.0f;
-                            b[e] = add ? add[g * k + c * 8 + e] : 0.0f;
+                            // the normalised value rounded to fp32, then one fused multiply-add with the two vectors
+                            const float xh = __fmul_rn(f[e], rstd);
+                            f[e] = __builtin_fmaf(xh, a[e], b[e]);
                         }
+                        v[i] = pack8(f);
                     }
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) {
-                        // three separately rounded fp32 operations, like the unfused graph
-                        const float xh = __fmul_rn(f[e], rstd);
-                        f[e] = __fadd_rn(__fmul_rn(xh, a[e]), b[e]);
-                    }
-                    v[i] = pack8(f);
                 }
-            }
+            };
+            if (g == staged) modulate(std::true_type{});
+            else modulate(std::false_type{});
         } else {
 #pragma unroll
             for (int i = 0; i < NCH; ++i) {
@@ -255,6 +277,130 @@ __global__ __launch_bounds__(256, (PRE == PRE_LN && NCH <= 12 && !WRITE_Y) ? 3 :
     }
 }
 
+// The LayerNorm form for rows of exactly NCOL x 512 elements (every lane owns NCOL whole chunks), quantised bytes only,
+// groups of a multiple of four rows (the four rows of a workgroup pass share the staged vectors): the shapes the DiT
+// blocks have.  Against fused_rows_wave it has no lane predicates and no path that reads the vectors from memory, the row
+// number is a scalar (row base in SGPRs, one lane offset for all chunks), and the current and the requested row swap
+// roles from one pass to the next instead of being copied.  Same arithmetic, same bits.
+template <int NCOL, int FMT>
+__global__ __launch_bounds__(256, NCOL <= 10 ? 3 : 2) void ln_rows_exact(const uint16_t* __restrict__ x, int64_t m, int64_t ld_x,
+                                                                          const float* __restrict__ mul, const float* __restrict__ add,
+                                                                          int64_t rows_per_group, float eps, uint8_t* __restrict__ q,
+                                                                          int64_t ld_q, float* __restrict__ scale, float qmax) {
+    constexpr int K = NCOL * 512;
+    extern __shared__ __attribute__((aligned(16))) float s_vec[];  // mul, then add, in the lanes' read order (as above)
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int64_t stride = (int64_t)gridDim.x * 4;
+    int64_t staged = -1;
+    auto load_row = [&](int64_t r, uint4 (&dst)[NCOL]) __attribute__((always_inline)) {
+        const uint4* xr = reinterpret_cast<const uint4*>(x + r * ld_x) + lane;
+#pragma unroll
+        for (int i = 0; i < NCOL; ++i) dst[i] = load_stream_16(xr + i * 64);
+    };
+    // one pass: stage the vectors of the quad's group if they changed, request the row of the next pass, work on `cur`
+    auto pass = [&](int64_t row0, uint4 (&cur)[NCOL], uint4 (&nxt)[NCOL]) __attribute__((always_inline)) {
+        const int64_t g0 = row0 / rows_per_group;
+        if (g0 != staged) {
+            __syncthreads();  // everyone is done with the previous group's vectors
+            for (int e = threadIdx.x; e < K; e += 256) {
+                const int c = e >> 3;
+                const int pos = (((((c >> 6) << 1) + ((e >> 2) & 1)) * 64 + (c & 63)) << 2) | (e & 3);
+                s_vec[pos] = mul ? mul[g0 * K + e] : 1.0f;
+                s_vec[K + pos] = add ? add[g0 * K + e] : 0.0f;
+            }
+            staged = g0;
+            __syncthreads();
+        }
+        const int64_t row = row0 + wave;
+        // always requested, beyond the last row that row again: a load under a condition makes the registers of `nxt` a
+        // merge of two values, which the compiler resolves with copies right behind the loads, i.e. by waiting for them
+        load_row(row + stride < m ? row + stride : m - 1, nxt);
+        if (row >= m) return;
+
+        float sum = 0.0f, sq = 0.0f;  // see fused_rows_wave for the statistics
+#pragma unroll
+        for (int i = 0; i < NCOL; ++i) dot_sums(cur[i], sum, sq);
+        dot_sums_done(sum, sq);
+        float mean = wave_sum_f32(sum) / (float)K;
+        float var = wave_sum_f32(sq) / (float)K - mean * mean;
+        if (!(mean * mean <= 7.0f * var)) {
+            float sd = 0.0f, ssq = 0.0f;
+#pragma unroll
+            for (int i = 0; i < NCOL; ++i) {
+                float f[8];
+                unpack8(cur[i], f);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const float d = f[e] - mean;
+                    sd += d;
+                    ssq += d * d;
+                }
+            }
+            const float dm = wave_sum_f32(sd) / (float)K;
+            var = wave_sum_f32(ssq) / (float)K - dm * dm;
+            mean += dm;
+        }
+        forget_values(cur);
+        const float rstd = 1.0f / sqrtf(var + eps);  // IEEE sqrt and division
+        const float nm = -mean;
+#pragma unroll
+        for (int i = 0; i < NCOL; ++i) {
+            float f[8];
+            dot_add8(cur[i], nm, f);  // x - mean
+            const float* sv = s_vec + (i * 128 + lane) * 4;
+            const float4 a0 = *reinterpret_cast<const float4*>(sv);
+            const float4 a1 = *reinterpret_cast<const float4*>(sv + 256);
+            const float4 b0 = *reinterpret_cast<const float4*>(sv + K);
+            const float4 b1 = *reinterpret_cast<const float4*>(sv + K + 256);
+            const float a[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
+            const float b[8] = {b0.x, b0.y, b0.z, b0.w, b1.x, b1.y, b1.z, b1.w};
+#pragma unroll
+            for (int e = 0; e < 8; ++e) f[e] = __builtin_fmaf(__fmul_rn(f[e], rstd), a[e], b[e]);
+            cur[i] = pack8(f);
+        }
+        uint32_t mx = 0;
+#pragma unroll
+        for (int i = 0; i < NCOL; ++i) mx = chunk_absmax(mx, cur[i]);
+        uint32_t amax = (mx & 0xffffu) > (mx >> 16) ? (mx & 0xffffu) : (mx >> 16);
+        amax = wave_max_u32(amax);
+        const float s = scale_from_amax_bits<true>(amax, qmax);
+        if (lane == 0) scale[row] = s;
+        const float inv = 1.0f / s;
+        uint2* qr = reinterpret_cast<uint2*>(q + row * ld_q) + lane;
+#pragma unroll
+        for (int i = 0; i < NCOL; ++i) store_stream_8(qr + i * 64, quant_chunk<FMT, false, DAXQ_BF16, false>(cur[i], s, inv));
+    };
+    uint4 ra[NCOL], rb[NCOL];
+    int64_t row0 = (int64_t)blockIdx.x * 4;
+    load_row(row0 + wave < m ? row0 + wave : m - 1, ra);
+    while (row0 < m) {
+        pass(row0, ra, rb);
+        row0 += stride;
+        if (row0 >= m) break;
+        pass(row0, rb, ra);
+        row0 += stride;
+    }
+}
+
+template <int NCOL, int FMT>
+static int launch_ln_exact(const char* what, const uint16_t* x, int64_t m, int64_t ld_x, const float* mul, const float* add,
+                           int64_t rows_per_group, float eps, uint8_t* q, int64_t ld_q, float* scale, float qmax, int cus,
+                           hipStream_t st) {
+    constexpr size_t lds = (size_t)NCOL * 512 * 8;
+    static int per_cu = 0;  // asked once per instantiation; a race between two threads stores the same value twice
+    if (per_cu <= 0) {
+        int v = 0;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&v, ln_rows_exact<NCOL, FMT>, 256, lds) != hipSuccess || v <= 0)
+            return fail(DAXQ_ERR_LAUNCH, "%s: occupancy query failed", what);
+        per_cu = v;
+    }
+    const int64_t quads = (m + 3) / 4, want = (int64_t)cus * per_cu;
+    hipLaunchKernelGGL((ln_rows_exact<NCOL, FMT>), dim3((unsigned)(quads < want ? quads : want)), dim3(256), lds, st, x, m, ld_x, mul,
+                       add, rows_per_group, eps, q, ld_q, scale, qmax);
+    return check_launch(what);
+}
+
 template <int FMT, int PRE>
 static int launch_fused_rows(const char* what, const void* x, int64_t m, int64_t k, int64_t ld_x, const float* mul,
                              const float* add, int64_t rows_per_group, float eps, void* y, int64_t ld_y, void* q,
@@ -280,6 +426,24 @@ static int launch_fused_rows(const char* what, const void* x, int64_t m, int64_t
     int dev = 0, cus = 0;
     if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
         return fail(DAXQ_ERR_LAUNCH, "%s: cannot read the CU count", what);
+    if constexpr (PRE == PRE_LN) {
+        // whole 512-element columns, groups of whole row quads, bytes only: the kernel without predicates
+        if (!yp && k % 512 == 0 && kfill == k && rows_per_group % 4 == 0) {
+            switch (k / 512) {
+#define DAXQ_LN_EXACT(N) \
+    case N: return launch_ln_exact<N, FMT>(what, xp, m, ld_x, mul, add, rows_per_group, eps, qp, ld_q, scale, qmax, cus, st);
+                DAXQ_LN_EXACT(3)
+                DAXQ_LN_EXACT(4)
+                DAXQ_LN_EXACT(6)
+                DAXQ_LN_EXACT(8)
+                DAXQ_LN_EXACT(10)
+                DAXQ_LN_EXACT(12)
+                DAXQ_LN_EXACT(16)
+#undef DAXQ_LN_EXACT
+                default: break;
+            }
+        }
+    }
     // PRE_LN keeps its workgroups resident -- exactly as many as fit a CU (measured: 0.340 ms with the exact
     // number against 0.355 / 0.49 ms with twice / half as many) -- so that the staged vectors are reused over
     // many rows; the GELU form has nothing to reuse and takes one quad of rows per workgroup
