@@ -296,6 +296,9 @@ def main():
     ap.add_argument("--tile-group", type=int, default=0, help="tile-order group depth (0 = library default)")
     ap.add_argument("--tile-order", type=int, default=0, help="tile order of the 256x256 kernels: 0 = library default, 1 = row groups, 2 = banded patches")
     ap.add_argument("--m", type=int, default=0, help="tokens (0 = the model's own count)")
+    ap.add_argument("--linear", default=None,
+                    help="comma-separated names of the model's linears to keep (qkv, out, ffn_up, ffn_down): a step of one "
+                         "linear repeats the same weight, i.e. measures it warm")
     ap.add_argument("--cpu-rows", type=int, default=0, help="tokens in the CPU-baseline sample (0 = pick for 10-30 s)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-mfma-ceiling", action="store_true")
@@ -325,7 +328,13 @@ def main():
     dev = torch.device("cuda:0")
     model_name, model_tag, m_model, shapes = MODELS[args.model]
     m = args.m or m_model
-    full = args.model == "14b" and m == M_TOKENS
+    if args.linear:
+        keep = args.linear.split(",")
+        unknown = [nm for nm in keep if nm not in [s_[0] for s_ in shapes]]
+        if unknown:
+            sys.exit(f"bench.py: --linear {unknown}: the {args.model} set has {[s_[0] for s_ in shapes]}")
+        shapes = [s_ for s_ in shapes if s_[0] in keep]
+    full = args.model == "14b" and m == M_TOKENS and not args.linear
     parts = [args.only] if args.only else (["int8", "fp8", "model40"] if full else ["int8"])
     if "model40" in parts and not full:
         sys.exit("bench.py: the 40-layer workload is defined for --model 14b at its own token count")
