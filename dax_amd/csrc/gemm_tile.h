@@ -61,7 +61,11 @@ __device__ __forceinline__ bool tile_origin(const GemmArgs& p, int tile_id, int&
 
 // workgroups of a launch of 256x256 tiles in the tile order a.order
 static inline int64_t grid_of_order(const GemmArgs& a) {
-    return a.order == kOrderBanded ? banded_grid(a.tiles_m, a.tiles_n, 4) : (int64_t)a.tiles_m * a.tiles_n;
+    const int64_t tiles = (int64_t)a.tiles_m * a.tiles_n;
+    if (a.order != kOrderBanded) return tiles;
+    // the patch arithmetic of the banded order is 32-bit: beyond 2^30 tiles none of it runs and the caller's check of the
+    // grid size refuses the launch
+    return tiles <= (1 << 30) ? banded_grid(a.tiles_m, a.tiles_n, 4) : (int64_t)1 << 40;
 }
 
 // accumulators of one 16x16 block: int32 (v_mfma_i32_16x16x64_i8) or fp32 (v_mfma_f32_16x16x128_f8f6f4)
