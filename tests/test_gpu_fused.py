@@ -68,11 +68,12 @@ def test_gelu_tanh_shapes_and_quant_only_form(ops, m, k):
 @pytest.mark.parametrize("fmt", ["i8", "e4m3", "e5m2"])
 @pytest.mark.parametrize("m,k,rpg,vecs", [(300, 1536, 300, "both"), (1001, 5120, 333, "both"), (64, 5120, 64, "none"),
                                           (9, 256, 2, "mul"), (1, 8, 1, "add"), (70, 8192, 35, "both"),
-                                          (9000, 1536, 3000, "both"), (5000, 5120, 2500, "both"), (130, 3072, 4, "mul")])
+                                          (9000, 1536, 3000, "both"), (5000, 5120, 2500, "both"), (130, 3072, 4, "mul"),
+                                          (40, 8192, 8, "both"), (36, 2048, 12, "add"), (20, 4096, 20, "both"), (24, 6144, 24, "mul")])
 def test_layernorm_multiply_add(ops, fmt, m, k, rpg, vecs):
     """Rows of whole 512-element columns in groups of a multiple of four rows take a kernel of their own when only the
-    quantised bytes are asked for (the last three shapes: resident workgroups that make several passes, and a group
-    change at every pass); its bytes and scales must equal those of the general kernel, which writes y as well."""
+    quantised bytes are asked for (from the seventh shape on: every column count it is built for, resident workgroups
+    that make several passes, a group change at every pass); its bytes and scales must equal those of the general kernel, which writes y as well."""
     g = torch.Generator().manual_seed(m * 7 + k)
     x = (torch.randn(m, k, generator=g) * 2 + 0.3).bfloat16()
     x[:, :: max(1, k // 7)] *= 12                                         # outlier channels, as in the DiT
