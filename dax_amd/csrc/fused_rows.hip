@@ -26,10 +26,11 @@ enum { PRE_LN = 1, PRE_GELU = 2 };
 
 // v_dot2_f32_bf16 d, a, b, c: both products of the bf16 pairs a and b, exact, added to the fp32 value c.  The compiler
 // only selects the form whose destination is the addend (v_dot2c), which costs x - mean a copy per element, so the
-// instruction is written out -- with its hazard: a different VALU instruction that reads a DOT instruction's result
-// needs three wait states behind it, and the compiler keeps those only for instructions it can see (the consumer of a
-// single-instruction asm statement was once scheduled directly behind it and read the register's old value).  Hence
-// whole chunks per statement, closed by the wait states, and results that no input register may share.
+// instruction is written out -- with its hazards: a different VALU instruction needs three wait states behind a DOT
+// instruction before it reads the result and four before it overwrites it, and the compiler keeps those only for
+// instructions it can see (the consumer of a single-instruction asm statement was once scheduled directly behind it
+// and read the register's old value).  Hence whole chunks per statement, closed by four wait states, and results that
+// no input register may share.
 // Row sums of a chunk: sum += x, sq += x * x over its eight values (a DOT reading the previous DOT's result as its
 // addend needs no wait; dot_sums_done() closes the chain before anything else reads the sums).
 __device__ __forceinline__ void dot_sums(const uint4& v, float& sum, float& sq) {
@@ -40,7 +41,7 @@ __device__ __forceinline__ void dot_sums(const uint4& v, float& sum, float& sq) 
         : "+v"(sum), "+v"(sq)
         : "v"(v.x), "v"(v.y), "v"(v.z), "v"(v.w), "v"(0x3f803f80u));
 }
-__device__ __forceinline__ void dot_sums_done(float& sum, float& sq) { asm volatile("s_nop 2" : "+v"(sum), "+v"(sq)); }
+__device__ __forceinline__ void dot_sums_done(float& sum, float& sq) { asm volatile("s_nop 3" : "+v"(sum), "+v"(sq)); }
 // f[e] = x[e] + c for the eight values of a chunk: the pair times (1, 0) or (0, 1) plus c, one instruction per element.
 // (A non-finite neighbour turns the element into NaN through its zero product; the callers' rows are NaN throughout
 // then anyway, their mean being non-finite.)
@@ -49,7 +50,7 @@ __device__ __forceinline__ void dot_add8(const uint4& v, float c, float (&f)[8])
         "v_dot2_f32_bf16 %2, %9, %12, %14\n\tv_dot2_f32_bf16 %3, %9, %13, %14\n\t"
         "v_dot2_f32_bf16 %4, %10, %12, %14\n\tv_dot2_f32_bf16 %5, %10, %13, %14\n\t"
         "v_dot2_f32_bf16 %6, %11, %12, %14\n\tv_dot2_f32_bf16 %7, %11, %13, %14\n\t"
-        "s_nop 2"
+        "s_nop 3"
         : "=&v"(f[0]), "=&v"(f[1]), "=&v"(f[2]), "=&v"(f[3]), "=&v"(f[4]), "=&v"(f[5]), "=&v"(f[6]), "=&v"(f[7])
         : "v"(v.x), "v"(v.y), "v"(v.z), "v"(v.w), "v"(0x00003f80u), "v"(0x3f800000u), "v"(c));
 }
