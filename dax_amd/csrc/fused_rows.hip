@@ -384,6 +384,42 @@ __global__ __launch_bounds__(256, NCOL <= 10 ? 3 : 2) void ln_rows_exact(const u
     }
 }
 
+// The GELU form for rows of exactly NCOL x 512 elements, quantised bytes only: no lane predicates (the general kernel
+// keeps one execution mask per chunk alive, 28 of them, which the compiler spills from scalar registers into vector lanes:
+// some 300 v_writelane / v_readlane per row on a kernel that is bound by VALU issue) and a scalar row number.  Same
+// arithmetic, same bits.  One row per wavefront, four per workgroup.
+template <int NCOL, int FMT>
+__global__ __launch_bounds__(256) void gelu_rows_exact(const uint16_t* __restrict__ x, int64_t m, int64_t ld_x, uint8_t* __restrict__ q,
+                                                       int64_t ld_q, float* __restrict__ scale, float qmax) {
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int64_t row = (int64_t)blockIdx.x * 4 + wave;
+    if (row >= m) return;
+    uint4 v[NCOL];
+    const uint4* xr = reinterpret_cast<const uint4*>(x + row * ld_x) + lane;
+#pragma unroll
+    for (int i = 0; i < NCOL; ++i) v[i] = load_stream_16(xr + i * 64);
+#pragma unroll
+    for (int i = 0; i < NCOL; ++i) {
+        float f[8];
+        unpack8(v[i], f);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) f[e] = gelu_tanh_f32(f[e]);
+        v[i] = pack8(f);
+    }
+    uint32_t mx = 0;
+#pragma unroll
+    for (int i = 0; i < NCOL; ++i) mx = chunk_absmax(mx, v[i]);
+    uint32_t amax = (mx & 0xffffu) > (mx >> 16) ? (mx & 0xffffu) : (mx >> 16);
+    amax = wave_max_u32(amax);
+    const float s = scale_from_amax_bits<true>(amax, qmax);
+    if (lane == 0) scale[row] = s;
+    const float inv = 1.0f / s;
+    uint2* qr = reinterpret_cast<uint2*>(q + row * ld_q) + lane;
+#pragma unroll
+    for (int i = 0; i < NCOL; ++i) store_stream_8(qr + i * 64, quant_chunk<FMT, false, DAXQ_BF16, false>(v[i], s, inv));
+}
+
 template <int NCOL, int FMT>
 static int launch_ln_exact(const char* what, const uint16_t* x, int64_t m, int64_t ld_x, const float* mul, const float* add,
                            int64_t rows_per_group, float eps, uint8_t* q, int64_t ld_q, float* scale, float qmax, int cus,
@@ -441,6 +477,23 @@ static int launch_fused_rows(const char* what, const void* x, int64_t m, int64_t
                 DAXQ_LN_EXACT(12)
                 DAXQ_LN_EXACT(16)
 #undef DAXQ_LN_EXACT
+                default: break;
+            }
+        }
+    }
+    if constexpr (PRE == PRE_GELU) {
+        if (!yp && k % 512 == 0 && kfill == k) {
+            const dim3 grid((unsigned)((m + 3) / 4));
+            switch (k / 512) {
+#define DAXQ_GELU_EXACT(N)                                                                                                        \
+    case N:                                                                                                                       \
+        hipLaunchKernelGGL((gelu_rows_exact<N, FMT>), grid, dim3(256), 0, st, xp, m, ld_x, qp, ld_q, scale, qmax);                 \
+        return check_launch(what);
+                DAXQ_GELU_EXACT(12)
+                DAXQ_GELU_EXACT(16)
+                DAXQ_GELU_EXACT(24)
+                DAXQ_GELU_EXACT(27)
+#undef DAXQ_GELU_EXACT
                 default: break;
             }
         }

@@ -54,14 +54,19 @@ def test_gelu_tanh_every_bf16_input(ops, fmt):
     _check_quant_of_own_y(fmt, y, q, s, 1024)
 
 
-@pytest.mark.parametrize("m,k", [(130, 13824), (257, 8960), (33, 1536), (1, 8), (5, 200)])
-def test_gelu_tanh_shapes_and_quant_only_form(ops, m, k):
+@pytest.mark.parametrize("fmt", ["i8", "e4m3", "e5m2"])
+@pytest.mark.parametrize("m,k", [(130, 13824), (257, 8960), (33, 1536), (1, 8), (5, 200), (41, 6144), (9, 8192), (22, 12288)])
+def test_gelu_tanh_shapes_and_quant_only_form(ops, fmt, m, k):
+    """The form that writes only the quantised bytes takes a kernel of its own for rows of 12, 16, 24 or 27 whole
+    512-element columns (K = 13824 and the last three shapes); its bytes and scales must equal those of the general kernel,
+    which writes y as well."""
     g = torch.Generator().manual_seed(m + k)
     x = (torch.randn(m, k, generator=g) * 1.5).bfloat16()
-    q, s, y = ops.gelu_tanh_act_quant_i8(dev(x), True)
+    fn = getattr(ops, "gelu_tanh_act_quant_" + fmt)
+    q, s, y = fn(dev(x), True)
     _check_y(y, O.gelu_tanh_bf16(x), 1e-2)
-    _check_quant_of_own_y("i8", y, q, s, k)
-    q2, s2, y2 = ops.gelu_tanh_act_quant_i8(dev(x), False)                # without writing y
+    _check_quant_of_own_y(fmt, y, q, s, k)
+    q2, s2, y2 = fn(dev(x), False)                                        # without writing y
     assert y2.shape[0] == 0 and torch.equal(q2, q) and torch.equal(s2, s)
 
 
