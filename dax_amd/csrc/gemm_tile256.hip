@@ -659,6 +659,9 @@ static int launch_i8_one(const GemmArgs& a, bool small, hipStream_t st) {
 //   with two quadrants per CU (L up to half the CUs: 4725 x 5120, 1 + 124) -5.3 / -5.9 %: a round of 128x128 tiles
 //   at two per CU takes as long as a round of 256x256 tiles, so those launches stay whole.
 // tail: 0 = cut the last partial round off by shape, 1 = never, 2 = whenever every quadrant gets a CU
+int launch_tile256x128(const GemmArgs& a, int first, int left, hipStream_t st);  // gemm_tile256x128.hip
+int prepare_tile256x128_kernels();
+
 int launch_tile_i8(const GemmArgs& a0, bool small, int tail, hipStream_t st) {
     GemmArgs a = a0;
     const int bt = small ? 128 : 256;
@@ -667,7 +670,14 @@ int launch_tile_i8(const GemmArgs& a0, bool small, int tail, hipStream_t st) {
     a.grid = a.quad_base = 0;
     if (small) a.order = kOrderRowGroups;
     const int left = small ? 0 : tail_tiles(a, tail);
-    if (left == 0) return launch_i8_one(a, small, st);
+    if (left == 0) {
+        const int halves = small ? 0 : tail_half_tiles(a, tail);
+        if (halves == 0) return launch_i8_one(a, small, st);
+        const int whole = a.tiles_m * a.tiles_n - halves;
+        a.grid = whole;
+        if (int rc = launch_i8_one(a, false, st)) return rc;
+        return launch_tile256x128(a, whole, halves, st);
+    }
     const int whole = a.tiles_m * a.tiles_n - left;
     a.grid = whole;
     if (int rc = launch_i8_one(a, false, st)) return rc;
@@ -699,6 +709,7 @@ int prepare_tile256_kernels() {
     DAXQ_PREP(prepare_tile256s5<true, false, 2, false, 128, true>);
     DAXQ_PREP(prepare_tile256s5<true, false, 3, false, 128, true>);
 #undef DAXQ_PREP
+    if (!rc) rc = prepare_tile256x128_kernels();
     return rc;
 }
 

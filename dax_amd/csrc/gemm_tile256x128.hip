@@ -1,0 +1,286 @@
+// INT8 W8A8 GEMM on half tiles of 256 x 128 outputs, bf16: the left-over tiles of a launch of few rounds.
+//
+// A launch of 256x256 tiles that leaves L tiles over after its whole rounds of workgroups pays a whole tile time for
+// them.  Up to a quarter of the CUs' worth of such tiles run as 128x128 quadrants with a CU each (gemm_tile256.hip);
+// between a quarter and a half they run here, as 2 L halves of 256 rows x 128 columns with a CU each: four wavefronts
+// in a 2 x 2 grid with 128 x 64 outputs each (128 accumulator registers), K through five 24 KB LDS stages with the load
+// stream of the large kernel (12 loads per thread and pair of slices: the 8 of the activation rows during the even
+// slice, the 4 of the weight rows during the odd one).  A half tile has 12 fragment reads per 32 MFMAs where the whole
+// tile has 16 per 64, so it runs at about 0.7 of the whole tile's pace: 0.7 of a tile time instead of one.
+// Same arithmetic as the large kernel: int32 accumulators, identical outputs.
+#include "gemm_tile.h"
+
+namespace daxq {
+
+namespace h2 {
+constexpr int BKS = 64, BM = 256, BN = 128, T = 256, NSTG = 5;
+constexpr int A_BYTES = BM * BKS, B_BYTES = BN * BKS, STAGE = A_BYTES + B_BYTES;  // 16 KB + 8 KB per stage
+constexpr int NBI = 8, NBJ = 4;                         // 16-row blocks of a wavefront: activation rows, weight rows
+constexpr int NREG = NBI * NBJ;                         // MFMAs = scheduling regions per slice and wavefront
+constexpr int A_LOADS = 8, B_LOADS = 4;                 // DMA loads per thread and pair of slices: activation rows, weight rows
+constexpr int PAIR_LOADS = A_LOADS + B_LOADS;
+constexpr int SMEM = NSTG * STAGE;
+}  // namespace h2
+
+// Epilogue of a wavefront's 128 x 64 outputs held as acc[j][i]: weight block j (16 output columns), activation block i
+// (16 output rows); in a block a lane owns row l%16 and columns 4*(l/16) + {0..3}.  As tile256_epilogue16 (gemm_tile.h).
+template <bool DUMP>
+__device__ __forceinline__ void h2_epilogue(const GemmArgs& p, v4i (&acc)[h2::NBJ][h2::NBI], uint8_t* smem, int m0, int n0, int t, int wm,
+                                            int wn, int l15, int g4, float pre_sx, float pre_sw, float pre_bias) {
+    using namespace h2;
+    float* s_sx = reinterpret_cast<float*>(smem);
+    float* s_sw = s_sx + BM;
+    float* s_bias = s_sw + BN;
+    s_sx[t] = pre_sx;
+    if (t < BN) {
+        s_sw[t] = pre_sw;
+        s_bias[t] = pre_bias;
+    }
+    __syncthreads();
+    const int mw = wm * 128, nw = wn * 64;
+    if constexpr (DUMP) {
+#pragma unroll
+        for (int j = 0; j < NBJ; ++j)
+#pragma unroll
+            for (int i = 0; i < NBI; ++i) {
+                const int64_t m = m0 + mw + i * 16 + l15;
+#pragma unroll
+                for (int v = 0; v < 4; ++v) static_cast<int32_t*>(p.acc)[m * p.ldacc + n0 + nw + j * 16 + 4 * g4 + v] = acc[j][i][v];
+            }
+    }
+    float sxr[NBI];
+    float4 swr[NBJ], br[NBJ];
+#pragma unroll
+    for (int i = 0; i < NBI; ++i) sxr[i] = s_sx[mw + i * 16 + l15];
+#pragma unroll
+    for (int j = 0; j < NBJ; ++j) {
+        swr[j] = *reinterpret_cast<const float4*>(s_sw + nw + j * 16 + 4 * g4);
+        br[j] = *reinterpret_cast<const float4*>(s_bias + nw + j * 16 + 4 * g4);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 0; i < NBI; ++i) {
+        const float sxv = sxr[i];
+        uint16_t* orow = p.out + (int64_t)(m0 + mw + i * 16 + l15) * p.ldo + n0 + nw + (g4 & 1) * 16 + (g4 >> 1) * 8;
+#pragma unroll
+        for (int jp = 0; jp < NBJ / 2; ++jp) {
+            uint32_t pk[2][2];
+#pragma unroll
+            for (int jj = 0; jj < 2; ++jj) {
+                const int j = 2 * jp + jj;
+                const float sws[4] = {swr[j].x, swr[j].y, swr[j].z, swr[j].w};
+                const float bs[4] = {br[j].x, br[j].y, br[j].z, br[j].w};
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    const int r = 2 * h;
+                    float y0 = (float)acc[j][i][r];  // v_cvt_f32_i32, round to nearest even
+                    float y1 = (float)acc[j][i][r + 1];
+                    y0 = y0 * sxv;
+                    y1 = y1 * sxv;
+                    y0 = y0 * sws[r];
+                    y1 = y1 * sws[r + 1];
+                    const uint32_t o1 = pack_bf16_rne(y0, y1);
+                    // second rounding: the bias is added to the bf16 value
+                    pk[jj][h] = pack_bf16_rne(__uint_as_float(o1 << 16) + bs[r], __uint_as_float(o1 & 0xffff0000u) + bs[r + 1]);
+                }
+            }
+            v2u s0 = __builtin_amdgcn_permlane16_swap(pk[0][0], pk[1][0], false, false);
+            v2u s1 = __builtin_amdgcn_permlane16_swap(pk[0][1], pk[1][1], false, false);
+            *reinterpret_cast<uint4*>(orow + jp * 32) = make_uint4(s0.x, s1.x, s0.y, s1.y);
+        }
+    }
+}
+
+template <bool DUMP>
+__global__ __launch_bounds__(256) void gemm_tile256x128_kernel(const GemmArgs p) {
+    using namespace h2;
+    extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    // half (blockIdx.x & 1) of the 256x256 tile quad_base - 1 + blockIdx.x / 2 of the row-group order
+    int tm, tn;
+    tile_of_block(p.gm, p.quad_base - 1 + ((int)blockIdx.x >> 1), p.tiles_m, p.tiles_n, tm, tn);
+    int m0 = tm * 256, n0 = tn * 256;
+    m0 = m0 + 256 <= p.m ? m0 : p.m - 256;
+    n0 = (n0 + 256 <= p.n ? n0 : p.n - 256) + ((int)blockIdx.x & 1) * 128;
+
+    // ---- HBM side.  One wave instruction fills 1 KB of LDS = 16 rows x 64 B: lane l -> row l/4, stored chunk l%4,
+    //      i.e. global chunk (l%4) ^ ((row>>1)&3).  Instruction j of a thread covers tile rows j*64 + t/4.
+    const uint32_t gsw = (uint32_t)(((t & 3) ^ ((t >> 3) & 3)) << 4);
+    uint32_t voff_a = (uint32_t)(t >> 2) * (uint32_t)p.lda + gsw;
+    uint32_t voff_b = (uint32_t)(t >> 2) * (uint32_t)p.ldb + gsw;
+    uint32_t voff_a1 = voff_a + BKS, voff_b1 = voff_b + BKS;  // second half of the 128-byte line
+    const uint8_t* abase = p.a + (int64_t)m0 * p.lda;
+    const uint8_t* bbase = p.b + (int64_t)n0 * p.ldb;
+    const int64_t a_step = 64 * p.lda, b_step = 64 * p.ldb;
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(DAXQ_LDS uint8_t*)smem;
+    const uint32_t wave_lds = lds0 + (uint32_t)__builtin_amdgcn_readfirstlane(wave * 1024);
+    // load g of a pair (12): 0-7 activation rows, 8-11 weight rows; 64-row block (g/2) % 4, half g%2 -> stage o0 / o1
+    auto issue_one = [&](uint32_t o0, uint32_t o1, int g) {
+        const int opnd = g >= A_LOADS, j = ((opnd ? g - A_LOADS : g) >> 1), half = g & 1;
+        const uint8_t* src = opnd ? bbase + j * b_step : abase + j * a_step;
+        const uint32_t voff = opnd ? (half ? voff_b1 : voff_b) : (half ? voff_a1 : voff_a);
+        const uint32_t dst = wave_lds + (half ? o1 : o0) + opnd * A_BYTES + j * 4096;
+        __builtin_amdgcn_global_load_lds((const DAXQ_GLOBAL void*)(src + voff), (DAXQ_LDS void*)(uintptr_t)dst, 16, 0, 0);
+    };
+    auto advance_a = [&]() {
+        voff_a += 2 * BKS;
+        voff_a1 += 2 * BKS;
+    };
+    auto advance_b = [&]() {
+        voff_b += 2 * BKS;
+        voff_b1 += 2 * BKS;
+    };
+
+    // ---- LDS side: activation row wm*128 + i*16 + l%16, weight row wn*64 + j*16 + l%16; the lane's K chunk is l/16
+    const int lr = lane & 15;
+    const int gq = (lr >> 1) & 3;
+    const uint8_t* a_rd = smem + (wm * 128 + lr) * BKS + (((lane >> 4) ^ gq) << 4);
+    const uint8_t* b_rd = smem + A_BYTES + (wn * 64 + lr) * BKS + (((lane >> 4) ^ gq) << 4);
+    // fragment f of a slice: 0-7 activation block f, 8-11 weight block f-8
+    auto read_frag = [&](uint32_t o, int f, v4i (&af)[NBI], v4i (&bf)[NBJ]) {
+        if (f < NBI) af[f] = *reinterpret_cast<const v4i*>(a_rd + o + f * 16 * BKS);
+        else bf[f - NBI] = *reinterpret_cast<const v4i*>(b_rd + o + (f - NBI) * 16 * BKS);
+    };
+
+    v4i acc[NBJ][NBI];
+    v4i fa0[NBI] = {}, fb0[NBJ] = {}, fa1[NBI] = {}, fb1[NBJ] = {};  // fragment sets by slice parity
+
+    const int S = p.k / BKS;  // slices; even because K is a multiple of 128
+    uint32_t st[NSTG];        // stage offsets of slices s .. s+3 and, last, of slice s-1 (s = the even slice of the pair)
+#pragma unroll
+    for (int i = 0; i < NSTG; ++i) st[i] = i * STAGE;
+
+    // One slice (see gemm_tile256.hip for the scheme).  ODD: slice parity.  ISSUE: start half of pair (s+4, s+5).
+    // NEXT: slice s+1 exists.  YOUNG: tile loads issued behind those of slice s+1 that may stay in flight.  EXTRA:
+    // younger loads that are not tile loads.  FIRST: slice 0, its MFMAs start from zero.
+    auto slice = [&](auto ODD, auto ISSUE, auto NEXT, auto YOUNG, auto EXTRA, auto FIRST, uint32_t o_next, uint32_t o_ld0, uint32_t o_ld1)
+                     __attribute__((always_inline)) {
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm(YOUNG.value + EXTRA.value) & lgkmcnt0_mask());
+        __builtin_amdgcn_s_barrier();
+#pragma unroll
+        for (int g = 0; g < NREG; ++g) {
+            if constexpr (ISSUE.value) {  // even slice: the 8 activation loads, one every 4 regions; odd: the 4 weight loads, every 8
+                if constexpr (ODD.value) {
+                    if (g % (NREG / B_LOADS) == 0) issue_one(o_ld0, o_ld1, A_LOADS + g / (NREG / B_LOADS));
+                } else {
+                    if (g % (NREG / A_LOADS) == 0) issue_one(o_ld0, o_ld1, g / (NREG / A_LOADS));
+                }
+            }
+            if constexpr (NEXT.value) {  // 12 reads, one every second region
+                if (g % 2 == 0 && g / 2 < NBI + NBJ) {
+                    if constexpr (ODD.value) read_frag(o_next, g / 2, fa0, fb0);
+                    else read_frag(o_next, g / 2, fa1, fb1);
+                }
+            }
+            const int j = g / NBI, i = g % NBI;
+            const v4i bfr = ODD.value ? fb1[j] : fb0[j];
+            const v4i afr = ODD.value ? fa1[i] : fa0[i];
+            if constexpr (FIRST.value)
+                asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, 0" : "=a"(acc[j][i]) : "v"(bfr), "v"(afr));
+            else
+                asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+a"(acc[j][i]) : "v"(bfr), "v"(afr));
+            if constexpr (ISSUE.value) {
+                if (g == NREG - 2) {
+                    if constexpr (ODD.value) advance_b();
+                    else advance_a();
+                }
+            }
+            if constexpr (ODD.value) {
+                if (g == NREG - 1) {
+                    const uint32_t r0 = st[0], r1 = st[1];
+#pragma unroll
+                    for (int i2 = 0; i2 + 2 < NSTG; ++i2) st[i2] = st[i2 + 2];
+                    st[NSTG - 2] = r0;
+                    st[NSTG - 1] = r1;
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    auto pair = [&](auto ISSUE, auto YOUNG_E, auto YOUNG_O, auto NEXT_O, auto EXTRA, auto FIRST) __attribute__((always_inline)) {
+        slice(No{}, ISSUE, Yes{}, YOUNG_E, EXTRA, FIRST, st[1], st[NSTG - 1], st[0]);
+        slice(Yes{}, ISSUE, NEXT_O, YOUNG_O, EXTRA, No{}, st[2], st[NSTG - 1], st[0]);
+    };
+    typedef Int<PAIR_LOADS> SteadyE;  // one whole pair younger than the pair of slice s+1
+    typedef Int<A_LOADS> SteadyO;     // the activation half of the newest pair
+
+    // ---- prologue: pairs 0 and 1 in flight, pair 0 landed, fragments of slice 0 in set 0
+#pragma unroll
+    for (int g = 0; g < PAIR_LOADS; ++g) issue_one(0, STAGE, g);
+    advance_a();
+    advance_b();
+    if (S >= 4) {
+#pragma unroll
+        for (int g = 0; g < PAIR_LOADS; ++g) issue_one(2 * STAGE, 3 * STAGE, g);
+        advance_a();
+        advance_b();
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm(PAIR_LOADS));
+    } else {
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+    }
+    __builtin_amdgcn_s_barrier();
+#pragma unroll
+    for (int f = 0; f < NBI + NBJ; ++f) read_frag(0, f, fa0, fb0);
+
+    const int Q = S >> 1;  // pairs
+    if (Q >= 3) {
+        pair(Yes{}, SteadyE{}, SteadyO{}, Yes{}, Int<0>{}, Yes{});
+    } else {  // short K: no pair to peel, clear the accumulators instead
+#pragma unroll
+        for (int j = 0; j < NBJ; ++j)
+#pragma unroll
+            for (int i = 0; i < NBI; ++i) acc[j][i] = v4i{};
+    }
+    for (int q = 1; q + 2 < Q; ++q) pair(Yes{}, SteadyE{}, SteadyO{}, Yes{}, Int<0>{}, No{});
+
+    // the epilogue's scales and bias, requested behind the last tile loads (always three loads per thread: a missing
+    // bias reads a scale instead and is replaced by -0.0)
+    const int tn2 = t & (BN - 1);  // (the upper half of the threads repeats the lower half's weight-side loads: the counts of the waits hold)
+    const float pre_sx = p.sx[m0 + t], pre_sw = p.sw[n0 + tn2];
+    const uint32_t pre_b = (p.bias ? p.bias : reinterpret_cast<const uint16_t*>(p.sw))[n0 + tn2];
+    __builtin_amdgcn_sched_barrier(0);
+
+    if (Q >= 2) pair(No{}, Int<PAIR_LOADS>{}, Int<0>{}, Yes{}, Int<3>{}, No{});
+    pair(No{}, Int<0>{}, Int<0>{}, No{}, Int<3>{}, No{});
+
+    // the MFMAs are inline asm: nothing tells the compiler how long their results take (see gemm_tile256.hip)
+    asm volatile("s_nop 15\n\ts_nop 7");
+#pragma unroll
+    for (int j = 0; j < NBJ; ++j)
+        asm volatile(""
+                     : "+a"(acc[j][0]), "+a"(acc[j][1]), "+a"(acc[j][2]), "+a"(acc[j][3]), "+a"(acc[j][4]), "+a"(acc[j][5]),
+                       "+a"(acc[j][6]), "+a"(acc[j][7]));
+    h2_epilogue<DUMP>(p, acc, smem, m0, n0, t, wm, wn, lr, lane >> 4, pre_sx, pre_sw, p.bias ? bf16_bits_to_f32(pre_b) : -0.0f);
+}
+
+template <bool DUMP>
+static int prepare_h2() {
+    static std::atomic<uint64_t> lds_set{0};
+    return ensure_dynamic_lds(reinterpret_cast<const void*>(gemm_tile256x128_kernel<DUMP>), h2::SMEM, lds_set);
+}
+
+int prepare_tile256x128_kernels() {
+    if (int rc = prepare_h2<false>()) return rc;
+    return prepare_h2<true>();
+}
+
+// The two halves of each of the `left` 256x256 tiles from id `first` on (row-group order; a.tiles_m / a.tiles_n count
+// 256x256 tiles).  INT8, bf16 outputs, m and n of at least 256, K a multiple of 128 (the caller has checked the shape).
+int launch_tile256x128(const GemmArgs& a0, int first, int left, hipStream_t st) {
+    GemmArgs a = a0;
+    if (a.out_kind != DAXQ_BF16) return fail(DAXQ_ERR_ARG, "gemm: the half-tile kernel writes bf16");
+    a.quad_base = first + 1;
+    a.grid = 2 * left;
+    if (a.acc) {
+        if (int rc = prepare_h2<true>()) return rc;
+        hipLaunchKernelGGL(gemm_tile256x128_kernel<true>, dim3((unsigned)a.grid), dim3(h2::T), h2::SMEM, st, a);
+    } else {
+        if (int rc = prepare_h2<false>()) return rc;
+        hipLaunchKernelGGL(gemm_tile256x128_kernel<false>, dim3((unsigned)a.grid), dim3(h2::T), h2::SMEM, st, a);
+    }
+    return check_launch("gemm_tile256x128");
+}
+
+}  // namespace daxq

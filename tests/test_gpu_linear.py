@@ -112,18 +112,25 @@ def test_patch_tile_order_bit_exact(ops, m, n, k, order):
 # (m, n, k): grids of 256-tiles with one to four whole rounds of 256 workgroups and 1 to 64 tiles left over, edge tiles
 # (shifted inwards) among the tiles left over
 TAIL_SHAPES = [(4100, 4352, 128), (8500, 4096, 256), (4725, 13824, 128), (16300, 1024 + 40, 128), (8200, 8192 - 8, 128)]
+# one to four whole rounds and between a quarter and a half of the CUs' worth of tiles left over (they run as halves of
+# 256 x 128): K of one, two, three and many pairs of slices, edge tiles among the tiles left over
+HALF_TAIL_SHAPES = [(4725, 5120, 128), (4725, 15360 - 24, 256), (9000, 2560, 384), (4725 - 3, 5120, 1152)]
 
 
-@pytest.mark.parametrize("m,n,k", TAIL_SHAPES)
+@pytest.mark.parametrize("m,n,k", TAIL_SHAPES + HALF_TAIL_SHAPES)
 def test_last_round_as_a_second_launch_bit_exact(ops, m, n, k):
     """A launch of 256x256 tiles whose last round of workgroups is a few tiles: the whole rounds run as 256x256 tiles,
-    the tiles left over as a second launch of their 128x128 quadrants.  Accumulators and outputs equal the integer
+    the tiles left over as a second launch of their 128x128 quadrants or, INT8 with more than a quarter of the CUs' worth
+    of them, of their 256x128 halves.  Accumulators and outputs equal the integer
     oracle's with the cut forced and by shape; FP8 outputs are the single launch's bits (both tile sizes run the same
     sequence of MFMAs per output element)."""
     from dax_amd import _capi
 
     tiles = -(-m // 256) * -(-n // 256)
-    assert tiles // 256 >= 1 and 0 < tiles % 256 <= 64, "the shape must leave at most a quarter of 256 CUs' worth of tiles"
+    if (m, n, k) in HALF_TAIL_SHAPES:
+        assert tiles // 256 >= 1 and 64 < tiles % 256 <= 128, "the shape must leave a quarter to a half of 256 CUs' worth of tiles"
+    else:
+        assert tiles // 256 >= 1 and 0 < tiles % 256 <= 64, "the shape must leave at most a quarter of 256 CUs' worth of tiles"
     g = torch.Generator().manual_seed(m + n + k)
     xq = torch.randint(-127, 128, (m, k), dtype=torch.int8, generator=g)
     wq = torch.randint(-127, 128, (n, k), dtype=torch.int8, generator=g)
