@@ -246,7 +246,7 @@ static inline int tail_tiles(const GemmArgs& a, int tail) {
     return (tail == 2 || rounds <= kTailMaxRounds) ? (int)left : 0;
 }
 // The same for a last round of more than a quarter and at most half of the CUs' worth of tiles: those run as halves of
-// 256 x 128 with a CU each (gemm_tile256x128.hip: INT8 with bf16 outputs), about 0.7 of a tile time instead of one.
+// 256 x 128 with a CU each (gemm_tile256x128.hip: bf16 outputs), about 0.65 of a tile time instead of one.
 static inline int tail_half_tiles(const GemmArgs& a, int tail) {
     if (tail == 1 || a.order != kOrderRowGroups || a.out_kind != DAXQ_BF16) return 0;
     const int cus = cu_count();

@@ -1,4 +1,4 @@
-// INT8 W8A8 GEMM on half tiles of 256 x 128 outputs, bf16: the left-over tiles of a launch of few rounds.
+// W8A8 GEMM on half tiles of 256 x 128 outputs, bf16: the left-over tiles of a launch of few rounds (INT8 first, FP8 below).
 //
 // A launch of 256x256 tiles that leaves L tiles over after its whole rounds of workgroups pays a whole tile time for
 // them.  Up to a quarter of the CUs' worth of such tiles run as 128x128 quadrants with a CU each (gemm_tile256.hip);
@@ -281,6 +281,281 @@ int launch_tile256x128(const GemmArgs& a0, int first, int left, hipStream_t st) 
         hipLaunchKernelGGL(gemm_tile256x128_kernel<false>, dim3((unsigned)a.grid), dim3(h2::T), h2::SMEM, st, a);
     }
     return check_launch("gemm_tile256x128");
+}
+
+// ---------------------------------------------------------------------------------------------------------------------
+// The same half tile for FP8 operands (v_mfma_f32_16x16x128_f8f6f4).  An output element is the same sequence of MFMAs
+// over the same K bytes in the same register positions as in gemm_tile_fp8.hip -- one MFMA per pair of 64-byte slices,
+// a lane's fragments holding chunk l/16 of the pair's first slice, then of its second -- so its bits do not depend on
+// which of the kernels computed it.  With 128 accumulator registers both operands' fragments fit twice (12 x 8 x 2):
+// the fragments of pair q+1 are read during the MFMAs of pair q, the LDS holds three pairs (48 KB each: pair q+1
+// landed, q+2 in flight, and the slot of pair q, which was read a pair ago, taking the loads of q+3), one barrier per pair.
+namespace h2f {
+constexpr int BKS = 64, BM = 256, BN = 128, T = 256;
+constexpr int A_HALF = BM * BKS, B_HALF = BN * BKS;          // one slice of an operand: 16 KB / 8 KB
+constexpr int A_PART = 2 * A_HALF, SLOT = A_PART + 2 * B_HALF;  // a pair: 32 KB of activation rows, 16 KB of weight rows
+constexpr int NBI = 8, NBJ = 4, NREG = NBI * NBJ;
+constexpr int A_LOADS = 8, B_LOADS = 4, PAIR_LOADS = A_LOADS + B_LOADS;
+constexpr int SMEM = 3 * SLOT;
+}  // namespace h2f
+
+template <int F8>
+__global__ __launch_bounds__(256) void gemm_tile256x128_fp8_kernel(const GemmArgs p) {
+    using namespace h2f;
+    extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    int tm, tn;
+    tile_of_block(p.gm, p.quad_base - 1 + ((int)blockIdx.x >> 1), p.tiles_m, p.tiles_n, tm, tn);
+    int m0 = tm * 256, n0 = tn * 256;
+    m0 = m0 + 256 <= p.m ? m0 : p.m - 256;
+    n0 = (n0 + 256 <= p.n ? n0 : p.n - 256) + ((int)blockIdx.x & 1) * 128;
+
+    const uint32_t gsw = (uint32_t)(((t & 3) ^ ((t >> 3) & 3)) << 4);
+    uint32_t voff_a = (uint32_t)(t >> 2) * (uint32_t)p.lda + gsw;
+    uint32_t voff_b = (uint32_t)(t >> 2) * (uint32_t)p.ldb + gsw;
+    const uint8_t* abase = p.a + (int64_t)m0 * p.lda;
+    const uint8_t* bbase = p.b + (int64_t)n0 * p.ldb;
+    const int64_t a_step = 64 * p.lda, b_step = 64 * p.ldb;
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(DAXQ_LDS uint8_t*)smem;
+    const uint32_t wave_lds = lds0 + (uint32_t)__builtin_amdgcn_readfirstlane(wave * 1024);
+    // load g of a pair (12): 0-7 activation rows, 8-11 weight rows; 64-row block, then slice g%2 of the pair (the two
+    // halves of a 128-byte line by consecutive instructions)
+    auto issue_one = [&](uint32_t slot, int g) {
+        const int opnd = g >= A_LOADS, gg = opnd ? g - A_LOADS : g, j = gg >> 1, half = gg & 1;
+        const uint8_t* src = (opnd ? bbase + j * b_step + voff_b : abase + j * a_step + voff_a) + half * BKS;
+        const uint32_t dst = wave_lds + slot + (opnd ? A_PART + half * B_HALF : half * A_HALF) + j * 4096;
+        __builtin_amdgcn_global_load_lds((const DAXQ_GLOBAL void*)src, (DAXQ_LDS void*)(uintptr_t)dst, 16, 0, 0);
+    };
+    auto advance = [&]() {
+        voff_a += 2 * BKS;
+        voff_b += 2 * BKS;
+    };
+
+    const int lr = lane & 15, kg = lane >> 4;
+    const int xo = (kg ^ ((lr >> 1) & 3)) << 4;
+    const uint8_t* a_rd = smem + (wm * 128 + lr) * BKS + xo;
+    const uint8_t* b_rd = smem + A_PART + (wn * 64 + lr) * BKS + xo;
+    // fragment f of a pair: 0-7 activation block f, 8-11 weight block f-8; registers 0-3 the first slice, 4-7 the second
+    auto read_frag = [&](uint32_t slot, int f, v8i (&af)[NBI], v8i (&bf)[NBJ]) __attribute__((always_inline)) {
+        const bool w = f >= NBI;
+        const uint8_t* pr = (w ? b_rd + (f - NBI) * 16 * BKS : a_rd + f * 16 * BKS) + slot;
+        const v4i lo = *reinterpret_cast<const v4i*>(pr);
+        const v4i up = *reinterpret_cast<const v4i*>(pr + (w ? B_HALF : A_HALF));
+        const v8i v = __builtin_shufflevector(lo, up, 0, 1, 2, 3, 4, 5, 6, 7);
+        if (w) bf[f - NBI] = v;
+        else af[f] = v;
+    };
+
+    v4f acc[NBJ][NBI];
+    v8i fa0[NBI] = {}, fb0[NBJ] = {}, fa1[NBI] = {}, fb1[NBJ] = {};
+    auto mfma = [&](auto PAR, auto FIRST, int g) __attribute__((always_inline)) {
+        const int j = g / NBI, i = g % NBI;
+        const v8i bfr = decltype(PAR)::value ? fb1[j] : fb0[j];
+        const v8i afr = decltype(PAR)::value ? fa1[i] : fa0[i];
+        if constexpr (decltype(FIRST)::value) {
+            if constexpr (F8 == 0) asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, 0" : "=a"(acc[j][i]) : "v"(bfr), "v"(afr));
+            else if constexpr (F8 == kF8XE5) asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, 0 blgp:1" : "=a"(acc[j][i]) : "v"(bfr), "v"(afr));
+            else if constexpr (F8 == kF8WE5) asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, 0 cbsz:1" : "=a"(acc[j][i]) : "v"(bfr), "v"(afr));
+            else asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, 0 cbsz:1 blgp:1" : "=a"(acc[j][i]) : "v"(bfr), "v"(afr));
+        } else {
+            if constexpr (F8 == 0) asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0" : "+a"(acc[j][i]) : "v"(bfr), "v"(afr));
+            else if constexpr (F8 == kF8XE5) asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0 blgp:1" : "+a"(acc[j][i]) : "v"(bfr), "v"(afr));
+            else if constexpr (F8 == kF8WE5) asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0 cbsz:1" : "+a"(acc[j][i]) : "v"(bfr), "v"(afr));
+            else asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0 cbsz:1 blgp:1" : "+a"(acc[j][i]) : "v"(bfr), "v"(afr));
+        }
+    };
+
+    const int Q = p.k / (2 * BKS);  // pairs; K is a multiple of 128
+    uint32_t s0 = 0, s1 = SLOT, s2 = 2 * SLOT;  // slots of pairs q (read a pair ago), q+1, q+2
+    // One pair.  PAR: which register set it consumes.  ISSUE: pair q+3 exists, its loads go into the slot of pair q.
+    // NEXT: pair q+1 exists, its fragments are read into the other set.  YOUNG: tile loads behind those of pair q+1 that
+    // may stay in flight (those of pair q+2).  EXTRA: younger loads that are not tile loads.
+    auto pair = [&](auto PAR, auto ISSUE, auto NEXT, auto YOUNG, auto EXTRA, auto FIRST) __attribute__((always_inline)) {
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm(YOUNG.value + EXTRA.value) & lgkmcnt0_mask());
+        __builtin_amdgcn_s_barrier();  // pair q+1 has landed for everyone, and everyone has read pair q out of its slot
+#pragma unroll
+        for (int g = 0; g < NREG; ++g) {
+            if constexpr (ISSUE.value) {
+                if (g % 4 == 0) issue_one(s0, g / 4);                    // the 8 activation loads
+                else if (g % 8 == 2) issue_one(s0, A_LOADS + g / 8);     // the 4 weight loads
+            }
+            if constexpr (NEXT.value) {
+                if (g % 2 == 1 && g / 2 < NBI + NBJ) {
+                    if constexpr (PAR.value) read_frag(s1, g / 2, fa0, fb0);
+                    else read_frag(s1, g / 2, fa1, fb1);
+                }
+            }
+            mfma(PAR, FIRST, g);
+            if (g == NREG - 1) {
+                if constexpr (ISSUE.value) advance();
+                const uint32_t o = s0;
+                s0 = s1;
+                s1 = s2;
+                s2 = o;
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+
+    const int tn2 = t & (BN - 1);
+    float pre_sx, pre_sw;
+    uint32_t pre_b;
+    auto request_scales = [&]() __attribute__((always_inline)) {
+        pre_sx = p.sx[m0 + t];
+        pre_sw = p.sw[n0 + tn2];
+        pre_b = (p.bias ? p.bias : reinterpret_cast<const uint16_t*>(p.sw))[n0 + tn2];
+        __builtin_amdgcn_sched_barrier(0);
+    };
+
+    if (Q >= 4) {
+        // ---- prologue: pairs 0, 1, 2 in flight (slots s0, s1, s2), pair 0 landed, its fragments in set 0
+#pragma unroll
+        for (int g = 0; g < PAIR_LOADS; ++g) issue_one(s0, g);
+        advance();
+#pragma unroll
+        for (int g = 0; g < PAIR_LOADS; ++g) issue_one(s1, g);
+        advance();
+#pragma unroll
+        for (int g = 0; g < PAIR_LOADS; ++g) issue_one(s2, g);
+        advance();
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm(2 * PAIR_LOADS));
+        __builtin_amdgcn_s_barrier();
+#pragma unroll
+        for (int f = 0; f < NBI + NBJ; ++f) read_frag(s0, f, fa0, fb0);
+        // pair 0, then the steady pairs two at a time; the three pairs of the tail are code paths with fixed sets (odd,
+        // even, odd after an even number of pairs in front of them, else the fragments move over to the other set once)
+        typedef Int<PAIR_LOADS> Y1;
+        pair(No{}, Yes{}, Yes{}, Y1{}, Int<0>{}, Yes{});
+        int q = 1;
+        for (; q + 4 < Q; q += 2) {
+            pair(Yes{}, Yes{}, Yes{}, Y1{}, Int<0>{}, No{});
+            pair(No{}, Yes{}, Yes{}, Y1{}, Int<0>{}, No{});
+        }
+        if (q + 3 < Q) {  // one more steady pair: the tail then starts on an even pair, move its fragments to the odd set
+            pair(Yes{}, Yes{}, Yes{}, Y1{}, Int<0>{}, No{});
+#pragma unroll
+            for (int i = 0; i < NBI; ++i) fa1[i] = fa0[i];
+#pragma unroll
+            for (int j = 0; j < NBJ; ++j) fb1[j] = fb0[j];
+        }
+        request_scales();
+        pair(Yes{}, No{}, Yes{}, Y1{}, Int<3>{}, No{});      // pair Q-3: pairs Q-2 (landing) and Q-1 (in flight)
+        pair(No{}, No{}, Yes{}, Int<0>{}, Int<3>{}, No{});   // pair Q-2
+        pair(Yes{}, No{}, No{}, Int<0>{}, Int<3>{}, No{});   // pair Q-1
+    } else {
+        // ---- short K (one to three pairs): load a pair, wait for it, multiply
+        request_scales();
+        for (int q = 0; q < Q; ++q) {
+            if (q) __builtin_amdgcn_s_barrier();
+#pragma unroll
+            for (int g = 0; g < PAIR_LOADS; ++g) issue_one(0, g);
+            advance();
+            __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+            __builtin_amdgcn_s_barrier();
+#pragma unroll
+            for (int f = 0; f < NBI + NBJ; ++f) read_frag(0, f, fa0, fb0);
+            __builtin_amdgcn_s_waitcnt(lgkmcnt0_mask() & vmcnt_imm(63));
+            __builtin_amdgcn_sched_barrier(0);
+            if (q == 0) {
+#pragma unroll
+                for (int g = 0; g < NREG; ++g) mfma(No{}, Yes{}, g);
+            } else {
+#pragma unroll
+                for (int g = 0; g < NREG; ++g) mfma(No{}, No{}, g);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+    }
+
+    asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 7");
+#pragma unroll
+    for (int j = 0; j < NBJ; ++j)
+        asm volatile(""
+                     : "+a"(acc[j][0]), "+a"(acc[j][1]), "+a"(acc[j][2]), "+a"(acc[j][3]), "+a"(acc[j][4]), "+a"(acc[j][5]),
+                       "+a"(acc[j][6]), "+a"(acc[j][7]));
+
+    // epilogue: bf16(acc * sx * sw + bias), one rounding, as tile256_epilogue16's FP8 form
+    float* s_sx = reinterpret_cast<float*>(smem);
+    float* s_sw = s_sx + BM;
+    float* s_bias = s_sw + BN;
+    __syncthreads();  // (every wavefront is past its last fragment read)
+    s_sx[t] = pre_sx;
+    if (t < BN) {
+        s_sw[t] = pre_sw;
+        s_bias[t] = p.bias ? bf16_bits_to_f32(pre_b) : -0.0f;
+    }
+    __syncthreads();
+    const int mw = wm * 128, nw = wn * 64, g4 = kg;
+    float sxr[NBI];
+    float4 swr[NBJ], br[NBJ];
+#pragma unroll
+    for (int i = 0; i < NBI; ++i) sxr[i] = s_sx[mw + i * 16 + lr];
+#pragma unroll
+    for (int j = 0; j < NBJ; ++j) {
+        swr[j] = *reinterpret_cast<const float4*>(s_sw + nw + j * 16 + 4 * g4);
+        br[j] = *reinterpret_cast<const float4*>(s_bias + nw + j * 16 + 4 * g4);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 0; i < NBI; ++i) {
+        const float sxv = sxr[i];
+        uint16_t* orow = p.out + (int64_t)(m0 + mw + i * 16 + lr) * p.ldo + n0 + nw + (g4 & 1) * 16 + (g4 >> 1) * 8;
+#pragma unroll
+        for (int jp = 0; jp < NBJ / 2; ++jp) {
+            uint32_t pk[2][2];
+#pragma unroll
+            for (int jj = 0; jj < 2; ++jj) {
+                const int j = 2 * jp + jj;
+                const float sws[4] = {swr[j].x, swr[j].y, swr[j].z, swr[j].w};
+                const float bs[4] = {br[j].x, br[j].y, br[j].z, br[j].w};
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    const int r = 2 * h;
+                    const float z0 = acc[j][i][r] * sxv * sws[r] + bs[r], z1 = acc[j][i][r + 1] * sxv * sws[r + 1] + bs[r + 1];
+                    pk[jj][h] = pack_bf16_rne(z0, z1);
+                }
+            }
+            v2u x0 = __builtin_amdgcn_permlane16_swap(pk[0][0], pk[1][0], false, false);
+            v2u x1 = __builtin_amdgcn_permlane16_swap(pk[0][1], pk[1][1], false, false);
+            *reinterpret_cast<uint4*>(orow + jp * 32) = make_uint4(x0.x, x1.x, x0.y, x1.y);
+        }
+    }
+}
+
+template <int F8>
+static int prepare_h2f() {
+    static std::atomic<uint64_t> lds_set{0};
+    return ensure_dynamic_lds(reinterpret_cast<const void*>(gemm_tile256x128_fp8_kernel<F8>), h2f::SMEM, lds_set);
+}
+
+int prepare_tile256x128_fp8_kernels() {
+    if (int rc = prepare_h2f<0>()) return rc;
+    if (int rc = prepare_h2f<1>()) return rc;
+    if (int rc = prepare_h2f<2>()) return rc;
+    return prepare_h2f<3>();
+}
+
+template <int F8>
+static int launch_h2f(const GemmArgs& a, hipStream_t st) {
+    if (int rc = prepare_h2f<F8>()) return rc;
+    hipLaunchKernelGGL(gemm_tile256x128_fp8_kernel<F8>, dim3((unsigned)a.grid), dim3(h2f::T), h2f::SMEM, st, a);
+    return check_launch("gemm_tile256x128_fp8");
+}
+
+// FP8 form of launch_tile256x128: bf16 outputs, no accumulator dump
+int launch_tile256x128_fp8(const GemmArgs& a0, int f8, int first, int left, hipStream_t st) {
+    GemmArgs a = a0;
+    if (a.out_kind != DAXQ_BF16 || a.acc) return fail(DAXQ_ERR_ARG, "gemm: the FP8 half-tile kernel writes bf16 and dumps no accumulators");
+    a.quad_base = first + 1;
+    a.grid = 2 * left;
+    switch (f8) {
+        case 1: return launch_h2f<1>(a, st);
+        case 2: return launch_h2f<2>(a, st);
+        case 3: return launch_h2f<3>(a, st);
+        default: return launch_h2f<0>(a, st);
+    }
 }
 
 }  // namespace daxq

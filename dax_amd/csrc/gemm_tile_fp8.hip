@@ -373,7 +373,11 @@ static int launch_fp8_one(const GemmArgs& a, int f8, hipStream_t st) {
 }
 
 // small: 128x128 tiles (needs m, n >= 128); f8: operand formats (kF8XE5 | kF8WE5); tail: the last, partial round of a
-// launch of 256x256 tiles as a second launch on its 128x128 quadrants (tail_tiles) -- the same bits either way
+// launch of 256x256 tiles as a second launch on its 128x128 quadrants (tail_tiles) or 256x128 halves (tail_half_tiles)
+// -- the same bits either way
+int launch_tile256x128_fp8(const GemmArgs& a, int f8, int first, int left, hipStream_t st);  // gemm_tile256x128.hip
+int prepare_tile256x128_fp8_kernels();
+
 int launch_tile_fp8(const GemmArgs& a0, int f8, bool small, int tail, hipStream_t st) {
     GemmArgs a = a0;
     const int bt = small ? 128 : 256;
@@ -385,7 +389,15 @@ int launch_tile_fp8(const GemmArgs& a0, int f8, bool small, int tail, hipStream_
         return launch_fp8_one<128>(a, f8, st);
     }
     const int left = tail_tiles(a, tail);
-    if (left == 0) return launch_fp8_one<256>(a, f8, st);
+    if (left == 0) {
+        // more than a quarter and at most half of the CUs' worth of tiles left over: their 256x128 halves with a CU each
+        const int halves = a.acc ? 0 : tail_half_tiles(a, tail);
+        if (halves == 0) return launch_fp8_one<256>(a, f8, st);
+        const int whole = a.tiles_m * a.tiles_n - halves;
+        a.grid = whole;
+        if (int rc = launch_fp8_one<256>(a, f8, st)) return rc;
+        return launch_tile256x128_fp8(a, f8, whole, halves, st);
+    }
     const int whole = a.tiles_m * a.tiles_n - left;
     a.grid = whole;
     if (int rc = launch_fp8_one<256>(a, f8, st)) return rc;
@@ -414,6 +426,7 @@ int prepare_tile_fp8_kernels() {
     DAXQ_PREP_F8(3);
 #undef DAXQ_PREP_F8
 #undef DAXQ_PREP
+    if (!rc) rc = prepare_tile256x128_fp8_kernels();
     return rc;
 }
 
