@@ -78,26 +78,28 @@ struct Acc16<true> {
     typedef v4f type;
 };
 
-// The same epilogue for accumulators held as 8 x 8 blocks of 16x16 (v_mfma_i32_16x16x64_i8, v_mfma_f32_16x16x128_f8f6f4).
+// The epilogue of a wavefront's accumulators held as NBJ x NBI blocks of 16x16 (v_mfma_i32_16x16x64_i8,
+// v_mfma_f32_16x16x128_f8f6f4): acc[j][i] is weight block j (16 output columns) and activation block i (16 output rows)
+// of the wavefront's part of a tile of 32 NBI rows x 32 NBJ columns (four wavefronts, 2 x 2).
 // In a block a lane owns output row m = l%16 and the columns n = 4*(l/16) + {0..3}.  One
 // v_permlane16_swap per word over two neighbouring blocks gives each lane 8 consecutive columns of one
 // of them: lanes 0-15 block 2jp columns 0-7, lanes 16-31 block 2jp+1 columns 0-7, lanes 32-47 block
 // 2jp columns 8-15, lanes 48-63 block 2jp+1 columns 8-15.
-// NB: 16x16 blocks per operand and wavefront (8: 256x256 tile, 4: 128x128 tile); the tile edge is 32 * NB.
+// NBJ, NBI: 8, 8 for a 256x256 tile, 4, 4 for a 128x128 tile, 4, 8 for a half tile of 256 rows x 128 columns.
 // OUTK: element type of out and bias, DAXQ_BF16 / DAXQ_F16 / DAXQ_F32.  A template argument, i.e. a kernel
 // of its own per type: with all three forms inside one kernel behind uniform branches its code grew from 27 to 44 KB
 // and the bf16 launches at K = 1536, which change between main loop and epilogue every 24 slices, lost 2.7 %; with
 // the choice inside the loops they lost 2 to 11 % everywhere.
-template <bool DUMP, int NB = 8, bool FP8 = false, int OUTK = DAXQ_BF16>
-__device__ __forceinline__ void tile256_epilogue16(const GemmArgs& p, typename Acc16<FP8>::type (&acc)[NB][NB], uint8_t* smem, int m0, int n0, int t,
-                                                   int wm, int wn, int l15, int g4, float pre_sx, float pre_sw,
-                                                   float pre_bias) {
-    constexpr int BT = 32 * NB, WT = 16 * NB;
+template <bool DUMP, int NBJ, int NBI, bool FP8 = false, int OUTK = DAXQ_BF16>
+__device__ __forceinline__ void tile_epilogue16(const GemmArgs& p, typename Acc16<FP8>::type (&acc)[NBJ][NBI], uint8_t* smem, int m0, int n0, int t,
+                                                int wm, int wn, int l15, int g4, float pre_sx, float pre_sw,
+                                                float pre_bias) {
+    constexpr int BM = 32 * NBI, BN = 32 * NBJ, WTM = 16 * NBI, WTN = 16 * NBJ;
     float* s_sx = reinterpret_cast<float*>(smem);
-    float* s_sw = s_sx + BT;
-    float* s_bias = s_sw + BT;
-    if (BT == 256 || t < BT) {
-        s_sx[t] = pre_sx;
+    float* s_sw = s_sx + BM;
+    float* s_bias = s_sw + BN;
+    if (BM == 256 || t < BM) s_sx[t] = pre_sx;
+    if (BN == 256 || t < BN) {
         s_sw[t] = pre_sw;
         s_bias[t] = pre_bias;
     }
@@ -105,25 +107,25 @@ __device__ __forceinline__ void tile256_epilogue16(const GemmArgs& p, typename A
 
     if constexpr (DUMP) {
 #pragma unroll
-        for (int j = 0; j < NB; ++j)
+        for (int j = 0; j < NBJ; ++j)
 #pragma unroll
-            for (int i = 0; i < NB; ++i) {
-                const int64_t m = m0 + wm * WT + i * 16 + l15;
+            for (int i = 0; i < NBI; ++i) {
+                const int64_t m = m0 + wm * WTM + i * 16 + l15;
 #pragma unroll
                 for (int v = 0; v < 4; ++v) {
-                    if constexpr (FP8) static_cast<float*>(p.acc)[m * p.ldacc + n0 + wn * WT + j * 16 + 4 * g4 + v] = acc[j][i][v];
-                    else static_cast<int32_t*>(p.acc)[m * p.ldacc + n0 + wn * WT + j * 16 + 4 * g4 + v] = acc[j][i][v];
+                    if constexpr (FP8) static_cast<float*>(p.acc)[m * p.ldacc + n0 + wn * WTN + j * 16 + 4 * g4 + v] = acc[j][i][v];
+                    else static_cast<int32_t*>(p.acc)[m * p.ldacc + n0 + wn * WTN + j * 16 + 4 * g4 + v] = acc[j][i][v];
                 }
             }
     }
 
-    float sxr[NB];
-    float4 swr[NB], br[NB];
+    float sxr[NBI];
+    float4 swr[NBJ], br[NBJ];
 #pragma unroll
-    for (int i = 0; i < NB; ++i) sxr[i] = s_sx[wm * WT + i * 16 + l15];
+    for (int i = 0; i < NBI; ++i) sxr[i] = s_sx[wm * WTM + i * 16 + l15];
 #pragma unroll
-    for (int j = 0; j < NB; ++j) {
-        const int nl = wn * WT + j * 16 + 4 * g4;
+    for (int j = 0; j < NBJ; ++j) {
+        const int nl = wn * WTN + j * 16 + 4 * g4;
         swr[j] = *reinterpret_cast<const float4*>(s_sw + nl);
         br[j] = *reinterpret_cast<const float4*>(s_bias + nl);
     }
@@ -133,11 +135,11 @@ __device__ __forceinline__ void tile256_epilogue16(const GemmArgs& p, typename A
     if constexpr (OUTK == DAXQ_F32) {
         {
 #pragma unroll
-            for (int i = 0; i < NB; ++i) {
+            for (int i = 0; i < NBI; ++i) {
                 const float sxv = sxr[i];
-                float* orow = reinterpret_cast<float*>(p.out) + (int64_t)(m0 + wm * WT + i * 16 + l15) * p.ldo + n0 + wn * WT + 4 * g4;
+                float* orow = reinterpret_cast<float*>(p.out) + (int64_t)(m0 + wm * WTM + i * 16 + l15) * p.ldo + n0 + wn * WTN + 4 * g4;
 #pragma unroll
-                for (int j = 0; j < NB; ++j) {
+                for (int j = 0; j < NBJ; ++j) {
                     const float sws[4] = {swr[j].x, swr[j].y, swr[j].z, swr[j].w};
                     const float bs[4] = {br[j].x, br[j].y, br[j].z, br[j].w};
                     float o[4];
@@ -158,12 +160,12 @@ __device__ __forceinline__ void tile256_epilogue16(const GemmArgs& p, typename A
     constexpr bool f16 = OUTK == DAXQ_F16;
     {
 #pragma unroll
-    for (int i = 0; i < NB; ++i) {
-        const int ml = wm * WT + i * 16 + l15;
+    for (int i = 0; i < NBI; ++i) {
+        const int ml = wm * WTM + i * 16 + l15;
         const float sxv = sxr[i];
-        uint16_t* orow = p.out + (int64_t)(m0 + ml) * p.ldo + n0 + wn * WT + (g4 & 1) * 16 + (g4 >> 1) * 8;
+        uint16_t* orow = p.out + (int64_t)(m0 + ml) * p.ldo + n0 + wn * WTN + (g4 & 1) * 16 + (g4 >> 1) * 8;
 #pragma unroll
-        for (int jp = 0; jp < NB / 2; ++jp) {
+        for (int jp = 0; jp < NBJ / 2; ++jp) {
             uint32_t pk[2][2];
 #pragma unroll
             for (int jj = 0; jj < 2; ++jj) {
@@ -246,9 +248,9 @@ static inline int tail_tiles(const GemmArgs& a, int tail) {
     return (tail == 2 || rounds <= kTailMaxRounds) ? (int)left : 0;
 }
 // The same for a last round of more than a quarter and at most half of the CUs' worth of tiles: those run as halves of
-// 256 x 128 with a CU each (gemm_tile256x128.hip: bf16 outputs), about 0.65 of a tile time instead of one.
+// 256 x 128 with a CU each (gemm_tile256x128.hip), about 0.65 of a tile time instead of one.
 static inline int tail_half_tiles(const GemmArgs& a, int tail) {
-    if (tail == 1 || a.order != kOrderRowGroups || a.out_kind != DAXQ_BF16) return 0;
+    if (tail == 1 || a.order != kOrderRowGroups) return 0;
     const int cus = cu_count();
     if (cus < 8) return 0;
     const int64_t tiles = (int64_t)a.tiles_m * a.tiles_n, rounds = tiles / cus, left = tiles - rounds * cus;

@@ -557,7 +557,7 @@ __global__ __launch_bounds__(256) void gemm_tile256s5_kernel(const GemmArgs p) {
         __syncthreads();                      // every thread has read the flag before the epilogue reuses the LDS
     }
     if constexpr (N16)
-        tile256_epilogue16<DUMP, NB, false, OUTK>(p, acc, smem, m0, n0, t, wm, wn, lr, lane >> 4, pre_sx, pre_sw,
+        tile_epilogue16<DUMP, NB, NB, false, OUTK>(p, acc, smem, m0, n0, t, wm, wn, lr, lane >> 4, pre_sx, pre_sw,
                                                   !p.bias ? -0.0f : OUTK == DAXQ_F32 ? __uint_as_float(pre_b) : OUTK == DAXQ_F16 ? f16_bits_to_f32((uint16_t)pre_b) : bf16_bits_to_f32(pre_b));
     else
         tile256_epilogue<FP8, DUMP, NB>(p, acc, smem, m0, n0, t, wm, wn, l31, hi, pre_sx, pre_sw,

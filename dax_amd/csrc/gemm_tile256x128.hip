@@ -1,4 +1,4 @@
-// W8A8 GEMM on half tiles of 256 x 128 outputs, bf16: the left-over tiles of a launch of few rounds (INT8 first, FP8 below).
+// W8A8 GEMM on half tiles of 256 x 128 outputs: the left-over tiles of a launch of few rounds (INT8 first, FP8 below).
 //
 // A launch of 256x256 tiles that leaves L tiles over after its whole rounds of workgroups pays a whole tile time for
 // them.  Up to a quarter of the CUs' worth of such tiles run as 128x128 quadrants with a CU each (gemm_tile256.hip);
@@ -22,77 +22,9 @@ constexpr int PAIR_LOADS = A_LOADS + B_LOADS;
 constexpr int SMEM = NSTG * STAGE;
 }  // namespace h2
 
-// Epilogue of a wavefront's 128 x 64 outputs held as acc[j][i]: weight block j (16 output columns), activation block i
-// (16 output rows); in a block a lane owns row l%16 and columns 4*(l/16) + {0..3}.  As tile256_epilogue16 (gemm_tile.h).
-template <bool DUMP>
-__device__ __forceinline__ void h2_epilogue(const GemmArgs& p, v4i (&acc)[h2::NBJ][h2::NBI], uint8_t* smem, int m0, int n0, int t, int wm,
-                                            int wn, int l15, int g4, float pre_sx, float pre_sw, float pre_bias) {
-    using namespace h2;
-    float* s_sx = reinterpret_cast<float*>(smem);
-    float* s_sw = s_sx + BM;
-    float* s_bias = s_sw + BN;
-    s_sx[t] = pre_sx;
-    if (t < BN) {
-        s_sw[t] = pre_sw;
-        s_bias[t] = pre_bias;
-    }
-    __syncthreads();
-    const int mw = wm * 128, nw = wn * 64;
-    if constexpr (DUMP) {
-#pragma unroll
-        for (int j = 0; j < NBJ; ++j)
-#pragma unroll
-            for (int i = 0; i < NBI; ++i) {
-                const int64_t m = m0 + mw + i * 16 + l15;
-#pragma unroll
-                for (int v = 0; v < 4; ++v) static_cast<int32_t*>(p.acc)[m * p.ldacc + n0 + nw + j * 16 + 4 * g4 + v] = acc[j][i][v];
-            }
-    }
-    float sxr[NBI];
-    float4 swr[NBJ], br[NBJ];
-#pragma unroll
-    for (int i = 0; i < NBI; ++i) sxr[i] = s_sx[mw + i * 16 + l15];
-#pragma unroll
-    for (int j = 0; j < NBJ; ++j) {
-        swr[j] = *reinterpret_cast<const float4*>(s_sw + nw + j * 16 + 4 * g4);
-        br[j] = *reinterpret_cast<const float4*>(s_bias + nw + j * 16 + 4 * g4);
-    }
-    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int i = 0; i < NBI; ++i) {
-        const float sxv = sxr[i];
-        uint16_t* orow = p.out + (int64_t)(m0 + mw + i * 16 + l15) * p.ldo + n0 + nw + (g4 & 1) * 16 + (g4 >> 1) * 8;
-#pragma unroll
-        for (int jp = 0; jp < NBJ / 2; ++jp) {
-            uint32_t pk[2][2];
-#pragma unroll
-            for (int jj = 0; jj < 2; ++jj) {
-                const int j = 2 * jp + jj;
-                const float sws[4] = {swr[j].x, swr[j].y, swr[j].z, swr[j].w};
-                const float bs[4] = {br[j].x, br[j].y, br[j].z, br[j].w};
-#pragma unroll
-                for (int h = 0; h < 2; ++h) {
-                    const int r = 2 * h;
-                    float y0 = (float)acc[j][i][r];  // v_cvt_f32_i32, round to nearest even
-                    float y1 = (float)acc[j][i][r + 1];
-                    y0 = y0 * sxv;
-                    y1 = y1 * sxv;
-                    y0 = y0 * sws[r];
-                    y1 = y1 * sws[r + 1];
-                    const uint32_t o1 = pack_bf16_rne(y0, y1);
-                    // second rounding: the bias is added to the bf16 value
-                    pk[jj][h] = pack_bf16_rne(__uint_as_float(o1 << 16) + bs[r], __uint_as_float(o1 & 0xffff0000u) + bs[r + 1]);
-                }
-            }
-            v2u s0 = __builtin_amdgcn_permlane16_swap(pk[0][0], pk[1][0], false, false);
-            v2u s1 = __builtin_amdgcn_permlane16_swap(pk[0][1], pk[1][1], false, false);
-            *reinterpret_cast<uint4*>(orow + jp * 32) = make_uint4(s0.x, s1.x, s0.y, s1.y);
-        }
-    }
-}
-
-template <bool DUMP>
+template <bool DUMP, int OUTK>
 __global__ __launch_bounds__(256) void gemm_tile256x128_kernel(const GemmArgs p) {
+    static_assert(OUTK == DAXQ_BF16 || !DUMP, "the accumulator dump exists with bf16 outputs");
     using namespace h2;
     extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
 
@@ -239,7 +171,9 @@ __global__ __launch_bounds__(256) void gemm_tile256x128_kernel(const GemmArgs p)
     // bias reads a scale instead and is replaced by -0.0)
     const int tn2 = t & (BN - 1);  // (the upper half of the threads repeats the lower half's weight-side loads: the counts of the waits hold)
     const float pre_sx = p.sx[m0 + t], pre_sw = p.sw[n0 + tn2];
-    const uint32_t pre_b = (p.bias ? p.bias : reinterpret_cast<const uint16_t*>(p.sw))[n0 + tn2];
+    uint32_t pre_b;  // the bias element's bits: bf16 / fp16, or fp32
+    if constexpr (OUTK == DAXQ_F32) pre_b = __float_as_uint((p.bias ? reinterpret_cast<const float*>(p.bias) : p.sw)[n0 + tn2]);
+    else pre_b = (p.bias ? p.bias : reinterpret_cast<const uint16_t*>(p.sw))[n0 + tn2];
     __builtin_amdgcn_sched_barrier(0);
 
     if (Q >= 2) pair(No{}, Int<PAIR_LOADS>{}, Int<0>{}, Yes{}, Int<3>{}, No{});
@@ -252,35 +186,40 @@ __global__ __launch_bounds__(256) void gemm_tile256x128_kernel(const GemmArgs p)
         asm volatile(""
                      : "+a"(acc[j][0]), "+a"(acc[j][1]), "+a"(acc[j][2]), "+a"(acc[j][3]), "+a"(acc[j][4]), "+a"(acc[j][5]),
                        "+a"(acc[j][6]), "+a"(acc[j][7]));
-    h2_epilogue<DUMP>(p, acc, smem, m0, n0, t, wm, wn, lr, lane >> 4, pre_sx, pre_sw, p.bias ? bf16_bits_to_f32(pre_b) : -0.0f);
+    tile_epilogue16<DUMP, NBJ, NBI, false, OUTK>(p, acc, smem, m0, n0, t, wm, wn, lr, lane >> 4, pre_sx, pre_sw,
+                                                 !p.bias ? -0.0f : OUTK == DAXQ_F32 ? __uint_as_float(pre_b) : OUTK == DAXQ_F16 ? f16_bits_to_f32((uint16_t)pre_b) : bf16_bits_to_f32(pre_b));
 }
 
-template <bool DUMP>
+template <bool DUMP, int OUTK>
 static int prepare_h2() {
-    static std::atomic<uint64_t> lds_set{0};
-    return ensure_dynamic_lds(reinterpret_cast<const void*>(gemm_tile256x128_kernel<DUMP>), h2::SMEM, lds_set);
+    static std::atomic<uint64_t> lds_set{0};  // per instantiation
+    return ensure_dynamic_lds(reinterpret_cast<const void*>(gemm_tile256x128_kernel<DUMP, OUTK>), h2::SMEM, lds_set);
+}
+
+template <bool DUMP, int OUTK>
+static int launch_h2(const GemmArgs& a, hipStream_t st) {
+    if (int rc = prepare_h2<DUMP, OUTK>()) return rc;
+    hipLaunchKernelGGL((gemm_tile256x128_kernel<DUMP, OUTK>), dim3((unsigned)a.grid), dim3(h2::T), h2::SMEM, st, a);
+    return check_launch("gemm_tile256x128");
 }
 
 int prepare_tile256x128_kernels() {
-    if (int rc = prepare_h2<false>()) return rc;
-    return prepare_h2<true>();
+    if (int rc = prepare_h2<false, DAXQ_BF16>()) return rc;
+    if (int rc = prepare_h2<true, DAXQ_BF16>()) return rc;
+    if (int rc = prepare_h2<false, DAXQ_F16>()) return rc;
+    return prepare_h2<false, DAXQ_F32>();
 }
 
 // The two halves of each of the `left` 256x256 tiles from id `first` on (row-group order; a.tiles_m / a.tiles_n count
-// 256x256 tiles).  INT8, bf16 outputs, m and n of at least 256, K a multiple of 128 (the caller has checked the shape).
+// 256x256 tiles).  INT8, m and n of at least 256, K a multiple of 128 (the caller has checked the shape).
 int launch_tile256x128(const GemmArgs& a0, int first, int left, hipStream_t st) {
     GemmArgs a = a0;
-    if (a.out_kind != DAXQ_BF16) return fail(DAXQ_ERR_ARG, "gemm: the half-tile kernel writes bf16");
     a.quad_base = first + 1;
     a.grid = 2 * left;
-    if (a.acc) {
-        if (int rc = prepare_h2<true>()) return rc;
-        hipLaunchKernelGGL(gemm_tile256x128_kernel<true>, dim3((unsigned)a.grid), dim3(h2::T), h2::SMEM, st, a);
-    } else {
-        if (int rc = prepare_h2<false>()) return rc;
-        hipLaunchKernelGGL(gemm_tile256x128_kernel<false>, dim3((unsigned)a.grid), dim3(h2::T), h2::SMEM, st, a);
-    }
-    return check_launch("gemm_tile256x128");
+    if (a.acc && a.out_kind != DAXQ_BF16) return fail(DAXQ_ERR_ARG, "gemm: the accumulator dump exists with bf16 outputs");
+    if (a.out_kind == DAXQ_F16) return launch_h2<false, DAXQ_F16>(a, st);
+    if (a.out_kind == DAXQ_F32) return launch_h2<false, DAXQ_F32>(a, st);
+    return a.acc ? launch_h2<true, DAXQ_BF16>(a, st) : launch_h2<false, DAXQ_BF16>(a, st);
 }
 
 // ---------------------------------------------------------------------------------------------------------------------
@@ -299,8 +238,9 @@ constexpr int A_LOADS = 8, B_LOADS = 4, PAIR_LOADS = A_LOADS + B_LOADS;
 constexpr int SMEM = 3 * SLOT;
 }  // namespace h2f
 
-template <int F8>
+template <bool DUMP, int F8, int OUTK>
 __global__ __launch_bounds__(256) void gemm_tile256x128_fp8_kernel(const GemmArgs p) {
+    static_assert(OUTK == DAXQ_BF16 || !DUMP, "the accumulator dump exists with bf16 outputs");
     using namespace h2f;
     extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
@@ -404,7 +344,8 @@ __global__ __launch_bounds__(256) void gemm_tile256x128_fp8_kernel(const GemmArg
     auto request_scales = [&]() __attribute__((always_inline)) {
         pre_sx = p.sx[m0 + t];
         pre_sw = p.sw[n0 + tn2];
-        pre_b = (p.bias ? p.bias : reinterpret_cast<const uint16_t*>(p.sw))[n0 + tn2];
+        if constexpr (OUTK == DAXQ_F32) pre_b = __float_as_uint((p.bias ? reinterpret_cast<const float*>(p.bias) : p.sw)[n0 + tn2]);
+        else pre_b = (p.bias ? p.bias : reinterpret_cast<const uint16_t*>(p.sw))[n0 + tn2];
         __builtin_amdgcn_sched_barrier(0);
     };
 
@@ -476,85 +417,57 @@ __global__ __launch_bounds__(256) void gemm_tile256x128_fp8_kernel(const GemmArg
                      : "+a"(acc[j][0]), "+a"(acc[j][1]), "+a"(acc[j][2]), "+a"(acc[j][3]), "+a"(acc[j][4]), "+a"(acc[j][5]),
                        "+a"(acc[j][6]), "+a"(acc[j][7]));
 
-    // epilogue: bf16(acc * sx * sw + bias), one rounding, as tile256_epilogue16's FP8 form
-    float* s_sx = reinterpret_cast<float*>(smem);
-    float* s_sw = s_sx + BM;
-    float* s_bias = s_sw + BN;
-    __syncthreads();  // (every wavefront is past its last fragment read)
-    s_sx[t] = pre_sx;
-    if (t < BN) {
-        s_sw[t] = pre_sw;
-        s_bias[t] = p.bias ? bf16_bits_to_f32(pre_b) : -0.0f;
-    }
-    __syncthreads();
-    const int mw = wm * 128, nw = wn * 64, g4 = kg;
-    float sxr[NBI];
-    float4 swr[NBJ], br[NBJ];
-#pragma unroll
-    for (int i = 0; i < NBI; ++i) sxr[i] = s_sx[mw + i * 16 + lr];
-#pragma unroll
-    for (int j = 0; j < NBJ; ++j) {
-        swr[j] = *reinterpret_cast<const float4*>(s_sw + nw + j * 16 + 4 * g4);
-        br[j] = *reinterpret_cast<const float4*>(s_bias + nw + j * 16 + 4 * g4);
-    }
-    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int i = 0; i < NBI; ++i) {
-        const float sxv = sxr[i];
-        uint16_t* orow = p.out + (int64_t)(m0 + mw + i * 16 + lr) * p.ldo + n0 + nw + (g4 & 1) * 16 + (g4 >> 1) * 8;
-#pragma unroll
-        for (int jp = 0; jp < NBJ / 2; ++jp) {
-            uint32_t pk[2][2];
-#pragma unroll
-            for (int jj = 0; jj < 2; ++jj) {
-                const int j = 2 * jp + jj;
-                const float sws[4] = {swr[j].x, swr[j].y, swr[j].z, swr[j].w};
-                const float bs[4] = {br[j].x, br[j].y, br[j].z, br[j].w};
-#pragma unroll
-                for (int h = 0; h < 2; ++h) {
-                    const int r = 2 * h;
-                    const float z0 = acc[j][i][r] * sxv * sws[r] + bs[r], z1 = acc[j][i][r + 1] * sxv * sws[r + 1] + bs[r + 1];
-                    pk[jj][h] = pack_bf16_rne(z0, z1);
-                }
-            }
-            v2u x0 = __builtin_amdgcn_permlane16_swap(pk[0][0], pk[1][0], false, false);
-            v2u x1 = __builtin_amdgcn_permlane16_swap(pk[0][1], pk[1][1], false, false);
-            *reinterpret_cast<uint4*>(orow + jp * 32) = make_uint4(x0.x, x1.x, x0.y, x1.y);
-        }
-    }
+    __syncthreads();  // every wavefront is past its last fragment read (the short-K loop has no barrier behind its reads)
+    tile_epilogue16<DUMP, NBJ, NBI, true, OUTK>(p, acc, smem, m0, n0, t, wm, wn, lr, kg, pre_sx, pre_sw,
+                                                !p.bias ? -0.0f : OUTK == DAXQ_F32 ? __uint_as_float(pre_b) : OUTK == DAXQ_F16 ? f16_bits_to_f32((uint16_t)pre_b) : bf16_bits_to_f32(pre_b));
 }
 
-template <int F8>
+template <bool DUMP, int F8, int OUTK>
 static int prepare_h2f() {
-    static std::atomic<uint64_t> lds_set{0};
-    return ensure_dynamic_lds(reinterpret_cast<const void*>(gemm_tile256x128_fp8_kernel<F8>), h2f::SMEM, lds_set);
+    static std::atomic<uint64_t> lds_set{0};  // per instantiation
+    return ensure_dynamic_lds(reinterpret_cast<const void*>(gemm_tile256x128_fp8_kernel<DUMP, F8, OUTK>), h2f::SMEM, lds_set);
 }
 
-int prepare_tile256x128_fp8_kernels() {
-    if (int rc = prepare_h2f<0>()) return rc;
-    if (int rc = prepare_h2f<1>()) return rc;
-    if (int rc = prepare_h2f<2>()) return rc;
-    return prepare_h2f<3>();
-}
-
-template <int F8>
+template <bool DUMP, int F8, int OUTK>
 static int launch_h2f(const GemmArgs& a, hipStream_t st) {
-    if (int rc = prepare_h2f<F8>()) return rc;
-    hipLaunchKernelGGL(gemm_tile256x128_fp8_kernel<F8>, dim3((unsigned)a.grid), dim3(h2f::T), h2f::SMEM, st, a);
+    if (int rc = prepare_h2f<DUMP, F8, OUTK>()) return rc;
+    hipLaunchKernelGGL((gemm_tile256x128_fp8_kernel<DUMP, F8, OUTK>), dim3((unsigned)a.grid), dim3(h2f::T), h2f::SMEM, st, a);
     return check_launch("gemm_tile256x128_fp8");
 }
 
-// FP8 form of launch_tile256x128: bf16 outputs, no accumulator dump
+template <int F8>
+static int prepare_h2f_all() {
+    if (int rc = prepare_h2f<false, F8, DAXQ_BF16>()) return rc;
+    if (int rc = prepare_h2f<true, F8, DAXQ_BF16>()) return rc;
+    if (int rc = prepare_h2f<false, F8, DAXQ_F16>()) return rc;
+    return prepare_h2f<false, F8, DAXQ_F32>();
+}
+
+int prepare_tile256x128_fp8_kernels() {
+    if (int rc = prepare_h2f_all<0>()) return rc;
+    if (int rc = prepare_h2f_all<1>()) return rc;
+    if (int rc = prepare_h2f_all<2>()) return rc;
+    return prepare_h2f_all<3>();
+}
+
+template <int F8>
+static int launch_h2f_out(const GemmArgs& a, hipStream_t st) {
+    if (a.acc && a.out_kind != DAXQ_BF16) return fail(DAXQ_ERR_ARG, "gemm: the accumulator dump exists with bf16 outputs");
+    if (a.out_kind == DAXQ_F16) return launch_h2f<false, F8, DAXQ_F16>(a, st);
+    if (a.out_kind == DAXQ_F32) return launch_h2f<false, F8, DAXQ_F32>(a, st);
+    return a.acc ? launch_h2f<true, F8, DAXQ_BF16>(a, st) : launch_h2f<false, F8, DAXQ_BF16>(a, st);
+}
+
+// FP8 form of launch_tile256x128
 int launch_tile256x128_fp8(const GemmArgs& a0, int f8, int first, int left, hipStream_t st) {
     GemmArgs a = a0;
-    if (a.out_kind != DAXQ_BF16 || a.acc) return fail(DAXQ_ERR_ARG, "gemm: the FP8 half-tile kernel writes bf16 and dumps no accumulators");
     a.quad_base = first + 1;
     a.grid = 2 * left;
     switch (f8) {
-        case 1: return launch_h2f<1>(a, st);
-        case 2: return launch_h2f<2>(a, st);
-        case 3: return launch_h2f<3>(a, st);
-        default: return launch_h2f<0>(a, st);
+        case 1: return launch_h2f_out<1>(a, st);
+        case 2: return launch_h2f_out<2>(a, st);
+        case 3: return launch_h2f_out<3>(a, st);
+        default: return launch_h2f_out<0>(a, st);
     }
 }
 

@@ -336,7 +336,7 @@ __global__ __launch_bounds__(256) void gemm_tile_fp8_kernel(const GemmArgs p) {
                            "+a"(acc[j + 1][1]), "+a"(acc[j + 1][2]), "+a"(acc[j + 1][3]));
         }
     }
-    tile256_epilogue16<DUMP, NB, true, OUTK>(p, acc, smem, m0, n0, t, wm, wn, lr, kg, pre_sx, pre_sw,
+    tile_epilogue16<DUMP, NB, NB, true, OUTK>(p, acc, smem, m0, n0, t, wm, wn, lr, kg, pre_sx, pre_sw,
                                              !p.bias ? -0.0f : OUTK == DAXQ_F32 ? __uint_as_float(pre_b) : OUTK == DAXQ_F16 ? f16_bits_to_f32((uint16_t)pre_b) : bf16_bits_to_f32(pre_b));
 }
 
@@ -391,7 +391,7 @@ int launch_tile_fp8(const GemmArgs& a0, int f8, bool small, int tail, hipStream_
     const int left = tail_tiles(a, tail);
     if (left == 0) {
         // more than a quarter and at most half of the CUs' worth of tiles left over: their 256x128 halves with a CU each
-        const int halves = a.acc ? 0 : tail_half_tiles(a, tail);
+        const int halves = tail_half_tiles(a, tail);
         if (halves == 0) return launch_fp8_one<256>(a, f8, st);
         const int whole = a.tiles_m * a.tiles_n - halves;
         a.grid = whole;

@@ -358,7 +358,7 @@ static int launch_gemm(const void* xq, int64_t ld_xq, const float* sx, const voi
     a.partials = nullptr;
     a.grid = a.quad_base = 0;
     // bits 28-29 of `kernel`: the last partial round of a launch of 256x256 tiles as a second launch on 128x128 tiles (or,
-    // with bf16 outputs, on 256x128 tiles): 0 = by shape, 1 = never, 2 = whenever every such tile gets a CU of its own
+    // when they number more than a quarter of the CUs, on 256x128 tiles): 0 = by shape, 1 = never, 2 = whenever every such tile gets a CU of its own
     const int tail = (kernel >> 28) & 3;
     if (tail > 2) return fail(DAXQ_ERR_ARG, "linear: unknown tail choice %d", tail);
     const int which = kernel & 0xffff;

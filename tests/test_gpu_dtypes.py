@@ -132,11 +132,12 @@ def test_int8_module_fp16_fp32_bit_exact(dtype, m, k, n):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
-@pytest.mark.parametrize("variant,m,n,k", [(8, 700, 520, 256), (11, 300, 392, 384), (8, 4100, 4352, 128), (0, 130, 264, 128)])
+@pytest.mark.parametrize("variant,m,n,k", [(8, 700, 520, 256), (11, 300, 392, 384), (8, 4100, 4352, 128), (0, 130, 264, 128),
+                                           (8, 4725, 5120, 128)])
 def test_int8_fp16_fp32_outputs_of_the_tiled_kernels(variant, m, n, k, dtype):
     """fp16 / fp32 outputs straight from the kernels on 16x16 MFMAs, named by argument, with and without bias, edge
-    tiles included; 289 tiles with the tiles left over after one round forced into a second launch (both write the
-    type).  Values beyond the fp16 range become infinities, as the reference's cast makes them."""
+    tiles included; 289 tiles with the tiles left over after one round forced into a second launch of quadrants, 380
+    tiles with the 124 left over as a second launch of 256x128 halves (all of them write the type).  Values beyond the fp16 range become infinities, as the reference's cast makes them."""
     import dax_amd.ops as ops
     from dax_amd import _capi
 
@@ -164,10 +165,12 @@ def test_int8_fp16_fp32_outputs_of_the_tiled_kernels(variant, m, n, k, dtype):
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
 @pytest.mark.parametrize("x_fmt,w_fmt", [("e4m3", "e4m3"), ("e5m2", "e4m3"), ("e4m3", "e5m2")])
-@pytest.mark.parametrize("variant,m,n,k", [(8, 700, 520, 640), (11, 300, 392, 384), (8, 4100, 4352, 256), (0, 130, 264, 128)])
+@pytest.mark.parametrize("variant,m,n,k", [(8, 700, 520, 640), (11, 300, 392, 384), (8, 4100, 4352, 256), (0, 130, 264, 128),
+                                           (8, 4725, 5120, 256)])
 def test_fp8_fp16_fp32_outputs_of_the_tiled_kernels(variant, m, n, k, dtype, x_fmt, w_fmt):
     """fp16 / fp32 outputs of FP8 operands (what a per-tensor FP8 module that is not bf16 asks for) from the kernel on
-    16x16x128 MFMAs, on both tile sizes, with and without bias, and with the last round cut into a second launch:
+    16x16x128 MFMAs, on both tile sizes, with and without bias, and with the last round cut into a second launch (of
+    quadrants, or of 256x128 halves in the last shape):
     out = T(acc * sx * sw + bias) with one rounding, against the oracle's scaled matmul at 3e-3 relative L2, and
     against the same kernel's bf16 launch (its accumulators are the same, so its fp32 result rounded to bf16 must
     equal the bf16 output bit for bit)."""
