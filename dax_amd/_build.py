@@ -16,7 +16,7 @@ LIBDIR = os.path.join(HERE, "lib")
 LIB = os.path.join(LIBDIR, "libdaxq.so")
 ROOT = os.path.dirname(HERE)
 MFMA_RATE = os.path.join(ROOT, "bench", "mfma_rate")
-SOURCES = ["capi.hip", "quant_rows.hip", "quant_blocks.hip", "fused_rows.hip", "per_tensor.hip", "gemm_w8a8.hip", "gemm_tile256.hip", "gemm_tile_fp8.hip", "gemm_tile256x128.hip"]
+SOURCES = ["capi.hip", "quant_rows.hip", "quant_blocks.hip", "fused_rows.hip", "per_tensor.hip", "gemm_w8a8.hip", "gemm_tile256.hip", "gemm_tile_fp8.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-fast-math",
@@ -30,7 +30,7 @@ FLAGS = [
 # add (INT8 / FP8 epilogues: scale, scale, bias) or by a narrowing convert (fp16 outputs) must round once per
 # operation, as the reference's op sequence does; contraction turns them into an fma or a mixed-precision fma with a
 # single rounding.  fused_rows.hip (LayerNorm / GELU statistics, compared at a stated tolerance) keeps its fmas.
-NO_CONTRACT = {"quant_rows.hip", "quant_blocks.hip", "per_tensor.hip", "gemm_w8a8.hip", "gemm_tile256.hip", "gemm_tile_fp8.hip", "gemm_tile256x128.hip"}
+NO_CONTRACT = {"quant_rows.hip", "quant_blocks.hip", "per_tensor.hip", "gemm_w8a8.hip", "gemm_tile256.hip", "gemm_tile_fp8.hip"}
 
 
 def _compile(src: str, verbose: bool) -> str:

@@ -141,7 +141,7 @@ def debug_select_gemm(v: int) -> None:
     """0 = the library's choice by shape; 2 / 5 / 8 / 11 = one implementation (include/daxq.h: the generic kernel on
     256x256 / 128x128 tiles, the tiled kernel on 256x256 / 128x128 tiles); 1000 + d = depth d of the tile-order groups
     (1000 = default); 2000 + o = tile order of the 256x256 kernels (2000 = by shape, 2001 = groups of tile rows,
-    2002 = banded patches); 3000 + t = the last partial round of a 256x256 launch as a second launch on 128x128 tiles
+    2002 = banded patches); 3000 + t = the last partial round of a 256x256 launch as 128x128 quadrants or 256x128 halves
     (3000 = by shape, 3001 = never, 3002 = whenever every such tile gets a CU)."""
     global _kernel_choice, _tile_group, _tile_order, _tail
     v = int(v)

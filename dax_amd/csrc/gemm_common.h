@@ -48,10 +48,10 @@ struct GemmArgs {
     int32_t* counters;
     void* partials;
     // A launch of 256x256 tiles with few rounds of workgroups leaves most CUs idle during its last, partial round.
-    // Such a launch is cut in two: `grid` > 0 launches only the first `grid` workgroups of the tile order (the whole
-    // rounds), and a second launch on 128x128 tiles with quad_base > 0 computes the four quadrants of each 256x256
-    // tile from id quad_base - 1 on, one workgroup per quadrant (tiles_m / tiles_n count 256x256 tiles in both).
-    // 0 = off.
+    // Such a launch runs the tiles of that round in smaller pieces with a CU each: with `grid` > 0 only the first
+    // `grid` workgroups of the launch compute whole tiles of the row-group order (the whole rounds), and the
+    // workgroups behind them compute the 128x128 quadrants (four workgroups per tile) or the 256x128 halves (two) of
+    // the tiles from id quad_base - 1 on (tiles_m / tiles_n count 256x256 tiles).  0 = off.
     int grid, quad_base;
 };
 

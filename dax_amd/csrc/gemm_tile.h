@@ -36,8 +36,8 @@ constexpr int kOrderRowGroups = 0, kOrderBanded = 1;
 
 // Which BT x BT output tile workgroup `tile_id` computes: its origin (m0, n0), shifted inwards at the M / N edge
 // instead of being predicated (the overlap rows are computed twice with identical results).  False: a padding slot of
-// the banded order, the workgroup exits at once.  A launch with quad_base > 0 (BT = 128) computes the four quadrants
-// of the 256x256 tiles from id quad_base - 1 on, one workgroup per quadrant.
+// the banded order, the workgroup exits at once.  With quad_base > 0, BT = 128 means the four quadrants of the
+// 256x256 tiles from id quad_base - 1 on, one workgroup per quadrant (tile_id counts quadrants).
 template <int BT>
 __device__ __forceinline__ bool tile_origin(const GemmArgs& p, int tile_id, int& m0, int& n0) {
     int tm, tn;
@@ -228,10 +228,12 @@ static inline int cu_count() {
     return cus;
 }
 
-// Tiles of the last, partial round of a 256x256 launch that go to a second launch on 128x128 tiles; 0 = none.
+// Tiles of the last, partial round of a 256x256 launch that run as 128x128 quadrants, in workgroups behind those of
+// the whole tiles; 0 = none.
 // One workgroup of 256x256 tiles fills a CU, so a launch of R whole rounds and L more tiles takes R + 1 tile times
 // however small L is.  As 4 L quadrants with a CU each (L <= a quarter of the CUs) the L tiles take half a tile time
-// or less.  Measured against the single launch (INT8 / e4m3, K = 5120 unless noted):
+// or less.  Measured as a second launch against the launch of whole tiles (INT8 / e4m3, K = 5120 unless noted; in one
+// grid the quadrants start on the first CUs that come free, another +1 to +10 %, most on short launches):
 //   4725 x 13824 (4 rounds + 2 tiles) +5.6 / +6.1 %; 8500 x 4096, K = 2048 (2 + 32) +9.9 / +9.9 %;
 //   4095 x 4608, K = 1536 (1 + 32) +10.7 / +9.8 %, K = 8960 +24 / +26 %;
 //   20000 x 5120 (6 + 44) +3.3 / +2.4 %; 75600 x 5120 in row groups (23 + 32) -0.6 / -0.8 %: over many rounds the CUs
@@ -248,7 +250,7 @@ static inline int tail_tiles(const GemmArgs& a, int tail) {
     return (tail == 2 || rounds <= kTailMaxRounds) ? (int)left : 0;
 }
 // The same for a last round of more than a quarter and at most half of the CUs' worth of tiles: those run as halves of
-// 256 x 128 with a CU each (gemm_tile256x128.hip), about 0.65 of a tile time instead of one.
+// 256 x 128 with a CU each (gemm_tile256x128.h), about 0.65 of a tile time instead of one.
 static inline int tail_half_tiles(const GemmArgs& a, int tail) {
     if (tail == 1 || a.order != kOrderRowGroups) return 0;
     const int cus = cu_count();

@@ -16,6 +16,7 @@
 // rows are computed twice with identical results.  Shapes with M < 128 or N < 128 take the generic kernel in
 // gemm_w8a8.hip.
 #include "gemm_tile.h"
+#include "gemm_tile256x128.h"
 
 namespace daxq {
 
@@ -170,7 +171,7 @@ struct TileAcc<false, true> {
 // in range order (so FP8 sums do not depend on who was last) and runs the epilogue.  No workgroup waits for
 // another.  The last one sets the counter back to zero.
 template <bool FP8, bool DUMP, int F8, bool N16 = false, int BT = 256, bool SPLITK = false, int D = 2, int OUTK = DAXQ_BF16>
-__global__ __launch_bounds__(256) void gemm_tile256s5_kernel(const GemmArgs p) {
+__device__ __forceinline__ void gemm_tile256s5_body(const GemmArgs& p, const int block) {
     static_assert(OUTK == DAXQ_BF16 || (N16 && !SPLITK && !DUMP), "fp16 / fp32 outputs exist in the 16x16 int8 form");
     using namespace t5;
     static_assert(!(FP8 && N16), "the 16x16 form exists for INT8 only");
@@ -193,12 +194,12 @@ __global__ __launch_bounds__(256) void gemm_tile256s5_kernel(const GemmArgs p) {
 
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
     const int wm = wave >> 1, wn = wave & 1;
-    int tile_id = blockIdx.x, split = 0, klen = p.k;  // klen: bytes of K this workgroup covers, a multiple of 128
+    int tile_id = block, split = 0, klen = p.k;  // klen: bytes of K this workgroup covers, a multiple of 128
     int m0, n0;
     if constexpr (SPLITK) {
         static_assert(BT == 128 && !DUMP, "split-K exists on 128 tiles, without the accumulator dump");
-        tile_id = blockIdx.x / p.splits;
-        split = blockIdx.x - tile_id * p.splits;
+        tile_id = block / p.splits;
+        split = block - tile_id * p.splits;
         klen = p.k / p.splits;
         int tm, tn;
         tile_of_block(p.gm, tile_id, p.tiles_m, p.tiles_n, tm, tn);
@@ -489,7 +490,7 @@ __global__ __launch_bounds__(256) void gemm_tile256s5_kernel(const GemmArgs p) {
         constexpr int VPB = N16 ? 1 : 4;           // 16-byte vectors per lane and MFMA block
         constexpr int NV = NB * NB * VPB;          // per lane: 16 of them = 64 registers either way
         typedef uint64_t u64x2 __attribute__((ext_vector_type(2)));
-        uint64_t* mine = static_cast<uint64_t*>(p.partials) + ((int64_t)blockIdx.x * NV * 256 + t) * 2;
+        uint64_t* mine = static_cast<uint64_t*>(p.partials) + ((int64_t)block * NV * 256 + t) * 2;
 #pragma unroll
         for (int j = 0; j < NB; ++j)
 #pragma unroll
@@ -565,6 +566,28 @@ __global__ __launch_bounds__(256) void gemm_tile256s5_kernel(const GemmArgs p) {
 }
 
 template <bool FP8, bool DUMP, int F8, bool N16 = false, int BT = 256, bool SPLITK = false, int D = 2, int OUTK = DAXQ_BF16>
+__global__ __launch_bounds__(256) void gemm_tile256s5_kernel(const GemmArgs p) {
+    gemm_tile256s5_body<FP8, DUMP, F8, N16, BT, SPLITK, D, OUTK>(p, (int)blockIdx.x);
+}
+
+// One grid for a launch of few rounds whose left-over tiles run as halves (tail_half_tiles): workgroups 0 .. p.grid - 1
+// compute whole 256x256 tiles, the rest the 256x128 halves of the tiles from id quad_base - 1 on.  The halves start on
+// the CUs that finish their whole tiles first instead of behind the whole first kernel.
+template <bool DUMP, int OUTK>
+__global__ __launch_bounds__(256) void gemm_tile256_then_halves_kernel(const GemmArgs p) {
+    if ((int)blockIdx.x < p.grid) gemm_tile256s5_body<false, DUMP, 0, true, 256, false, 2, OUTK>(p, (int)blockIdx.x);
+    else gemm_tile256x128_body<DUMP, OUTK>(p, (int)blockIdx.x - p.grid);
+}
+
+// The same for left-over tiles that run as 128x128 quadrants (tail_tiles): workgroups 0 .. p.grid - 1 compute whole
+// tiles, the rest the quadrants of the tiles from id quad_base - 1 on (D: pairs of slices the quadrants keep in flight).
+template <bool DUMP, int OUTK, int D>
+__global__ __launch_bounds__(256) void gemm_tile256_then_quadrants_kernel(const GemmArgs p) {
+    if ((int)blockIdx.x < p.grid) gemm_tile256s5_body<false, DUMP, 0, true, 256, false, 2, OUTK>(p, (int)blockIdx.x);
+    else gemm_tile256s5_body<false, DUMP, 0, true, 128, false, D, OUTK>(p, (int)blockIdx.x - p.grid);
+}
+
+template <bool FP8, bool DUMP, int F8, bool N16 = false, int BT = 256, bool SPLITK = false, int D = 2, int OUTK = DAXQ_BF16>
 static int prepare_tile256s5() {
     static std::atomic<uint64_t> lds_set{0};  // per instantiation
     return ensure_dynamic_lds(reinterpret_cast<const void*>(gemm_tile256s5_kernel<FP8, DUMP, F8, N16, BT, SPLITK, D, OUTK>),
@@ -611,7 +634,7 @@ static int launch_tile256s5_impl(const GemmArgs& a, hipStream_t st) {
     if (a.out_kind != OUTK) return fail(DAXQ_ERR_ARG, "gemm: this kernel writes output type %d, not %d", OUTK, a.out_kind);
     auto kern = gemm_tile256s5_kernel<FP8, DUMP, F8, N16, BT, false, D, OUTK>;
     if (int rc = prepare_tile256s5<FP8, DUMP, F8, N16, BT, false, D, OUTK>()) return rc;
-    const int64_t nt = a.grid > 0 ? a.grid : grid_of_order(a);
+    const int64_t nt = grid_of_order(a);
     if (nt > 0x7fffffff) return fail(DAXQ_ERR_ARG, "gemm: too many tiles");
     hipLaunchKernelGGL(kern, dim3((unsigned)nt), dim3(T), SMEM, st, a);
     return check_launch("gemm_tile256s5");
@@ -628,7 +651,7 @@ static int launch_tile256s5_impl(const GemmArgs& a, hipStream_t st) {
 // one without loads 17 against 22 us.
 template <int OUTK>
 static int launch_i8_128_out(const GemmArgs& a, hipStream_t st) {
-    const bool deep = (a.grid > 0 ? (int64_t)a.grid : (int64_t)a.tiles_m * a.tiles_n) <= 256 && a.k >= 4096;
+    const bool deep = (int64_t)a.tiles_m * a.tiles_n <= 256 && a.k >= 4096;
     if constexpr (OUTK == DAXQ_BF16) {
         if (a.acc) return deep ? launch_tile256s5_impl<false, true, 0, true, 128, 4>(a, st) : launch_tile256s5_impl<false, true, 0, true, 128, 2>(a, st);
     }
@@ -648,19 +671,66 @@ static int launch_i8_one(const GemmArgs& a, bool small, hipStream_t st) {
     return a.acc ? launch_tile256s5_impl<false, true, 0, true>(a, st) : launch_tile256s5_impl<false, false, 0, true>(a, st);
 }
 
-// Tiles of the last, partial round of a 256x256 launch that go to a second launch on 128x128 tiles: tail_tiles
-// (gemm_tile.h).  One workgroup of 256x256 tiles fills a CU, so a launch of R whole rounds and L more tiles takes
-// R + 1 tile times however small L is.  As 4 L quadrants with a CU each (L <= a quarter of the CUs) the L tiles take
-// half a tile time or less.  Measured against the single launch (INT8 / e4m3, K = 5120 unless noted):
-//   4725 x 13824 (4 rounds + 2 tiles) +5.6 / +6.1 %; 8500 x 4096, K = 2048 (2 + 32) +9.9 / +9.9 %;
-//   4095 x 4608, K = 1536 (1 + 32) +10.7 / +9.8 %, K = 8960 +24 / +26 %;
-//   20000 x 5120 (6 + 44) +3.3 / +2.4 %; 75600 x 5120 in row groups (23 + 32) -0.6 / -0.8 %: over many rounds the CUs
-//   drift apart and the early ones pick the last tiles up, so the cut is taken up to kTailMaxRounds whole rounds;
-//   with two quadrants per CU (L up to half the CUs: 4725 x 5120, 1 + 124) -5.3 / -5.9 %: a round of 128x128 tiles
-//   at two per CU takes as long as a round of 256x256 tiles, so those launches stay whole.
-// tail: 0 = cut the last partial round off by shape, 1 = never, 2 = whenever every quadrant gets a CU
-int launch_tile256x128(const GemmArgs& a, int first, int left, hipStream_t st);  // gemm_tile256x128.hip
-int prepare_tile256x128_kernels();
+// The last, partial round of a launch of 256x256 tiles in smaller pieces with a CU each: tail_tiles (quadrants) and
+// tail_half_tiles (halves) in gemm_tile.h say which tiles, the kernels above run them in the same grid, behind the
+// whole tiles.  tail: 0 = by shape, 1 = never, 2 = whenever every piece gets a CU
+template <bool DUMP, int OUTK>
+static int prepare_then_halves() {
+    static std::atomic<uint64_t> lds_set{0};  // per instantiation
+    return ensure_dynamic_lds(reinterpret_cast<const void*>(gemm_tile256_then_halves_kernel<DUMP, OUTK>), 5 * 2 * 256 * t5::BKS, lds_set);
+}
+
+template <bool DUMP, int OUTK>
+static int launch_then_halves_impl(const GemmArgs& a, int64_t nt, hipStream_t st) {
+    if (int rc = prepare_then_halves<DUMP, OUTK>()) return rc;
+    hipLaunchKernelGGL((gemm_tile256_then_halves_kernel<DUMP, OUTK>), dim3((unsigned)nt), dim3(t5::T), 5 * 2 * 256 * t5::BKS, st, a);
+    return check_launch("gemm_tile256_then_halves");
+}
+
+// `whole` 256x256 tiles of the row-group order, then the two halves of each of the `halves` tiles behind them, in one grid
+static int launch_then_halves(const GemmArgs& a0, int whole, int halves, hipStream_t st) {
+    GemmArgs a = a0;
+    a.grid = whole;
+    a.quad_base = whole + 1;
+    const int64_t nt = (int64_t)whole + 2 * (int64_t)halves;
+    if (nt > 0x7fffffff) return fail(DAXQ_ERR_ARG, "gemm: too many tiles");
+    if (a.acc && a.out_kind != DAXQ_BF16) return fail(DAXQ_ERR_ARG, "gemm: the accumulator dump exists with bf16 outputs");
+    if (a.out_kind == DAXQ_F16) return launch_then_halves_impl<false, DAXQ_F16>(a, nt, st);
+    if (a.out_kind == DAXQ_F32) return launch_then_halves_impl<false, DAXQ_F32>(a, nt, st);
+    return a.acc ? launch_then_halves_impl<true, DAXQ_BF16>(a, nt, st) : launch_then_halves_impl<false, DAXQ_BF16>(a, nt, st);
+}
+
+template <bool DUMP, int OUTK, int D>
+static int prepare_then_quadrants() {
+    static std::atomic<uint64_t> lds_set{0};  // per instantiation
+    return ensure_dynamic_lds(reinterpret_cast<const void*>(gemm_tile256_then_quadrants_kernel<DUMP, OUTK, D>), 5 * 2 * 256 * t5::BKS, lds_set);
+}
+
+template <bool DUMP, int OUTK, int D>
+static int launch_then_quadrants_impl(const GemmArgs& a, int64_t nt, hipStream_t st) {
+    if (int rc = prepare_then_quadrants<DUMP, OUTK, D>()) return rc;
+    hipLaunchKernelGGL((gemm_tile256_then_quadrants_kernel<DUMP, OUTK, D>), dim3((unsigned)nt), dim3(t5::T), 5 * 2 * 256 * t5::BKS, st, a);
+    return check_launch("gemm_tile256_then_quadrants");
+}
+
+template <int D>
+static int launch_then_quadrants_out(const GemmArgs& a, int64_t nt, hipStream_t st) {
+    if (a.acc && a.out_kind != DAXQ_BF16) return fail(DAXQ_ERR_ARG, "gemm: the accumulator dump exists with bf16 outputs");
+    if (a.out_kind == DAXQ_F16) return launch_then_quadrants_impl<false, DAXQ_F16, D>(a, nt, st);
+    if (a.out_kind == DAXQ_F32) return launch_then_quadrants_impl<false, DAXQ_F32, D>(a, nt, st);
+    return a.acc ? launch_then_quadrants_impl<true, DAXQ_BF16, D>(a, nt, st) : launch_then_quadrants_impl<false, DAXQ_BF16, D>(a, nt, st);
+}
+
+// `whole` 256x256 tiles of the row-group order, then the four quadrants of each of the `left` tiles behind them, in one
+// grid; the quadrants have a CU each and take the deep ring when K is long (launch_i8_128_out)
+static int launch_then_quadrants(const GemmArgs& a0, int whole, int left, hipStream_t st) {
+    GemmArgs a = a0;
+    a.grid = whole;
+    a.quad_base = whole + 1;
+    const int64_t nt = (int64_t)whole + 4 * (int64_t)left;
+    if (nt > 0x7fffffff) return fail(DAXQ_ERR_ARG, "gemm: too many tiles");
+    return a.k >= 4096 ? launch_then_quadrants_out<4>(a, nt, st) : launch_then_quadrants_out<2>(a, nt, st);
+}
 
 int launch_tile_i8(const GemmArgs& a0, bool small, int tail, hipStream_t st) {
     GemmArgs a = a0;
@@ -673,17 +743,9 @@ int launch_tile_i8(const GemmArgs& a0, bool small, int tail, hipStream_t st) {
     if (left == 0) {
         const int halves = small ? 0 : tail_half_tiles(a, tail);
         if (halves == 0) return launch_i8_one(a, small, st);
-        const int whole = a.tiles_m * a.tiles_n - halves;
-        a.grid = whole;
-        if (int rc = launch_i8_one(a, false, st)) return rc;
-        return launch_tile256x128(a, whole, halves, st);
+        return launch_then_halves(a, a.tiles_m * a.tiles_n - halves, halves, st);
     }
-    const int whole = a.tiles_m * a.tiles_n - left;
-    a.grid = whole;
-    if (int rc = launch_i8_one(a, false, st)) return rc;
-    a.grid = 4 * left;
-    a.quad_base = whole + 1;
-    return launch_i8_one(a, true, st);
+    return launch_then_quadrants(a, a.tiles_m * a.tiles_n - left, left, st);
 }
 
 // Every instantiation the launchers above can pick, prepared on the current device: afterwards no launch changes a
@@ -708,8 +770,19 @@ int prepare_tile256_kernels() {
     DAXQ_PREP(prepare_tile256s5<true, false, 1, false, 128, true>);
     DAXQ_PREP(prepare_tile256s5<true, false, 2, false, 128, true>);
     DAXQ_PREP(prepare_tile256s5<true, false, 3, false, 128, true>);
+    DAXQ_PREP(prepare_then_halves<false, DAXQ_BF16>);
+    DAXQ_PREP(prepare_then_halves<true, DAXQ_BF16>);
+    DAXQ_PREP(prepare_then_halves<false, DAXQ_F16>);
+    DAXQ_PREP(prepare_then_halves<false, DAXQ_F32>);
+    DAXQ_PREP(prepare_then_quadrants<false, DAXQ_BF16, 2>);
+    DAXQ_PREP(prepare_then_quadrants<true, DAXQ_BF16, 2>);
+    DAXQ_PREP(prepare_then_quadrants<false, DAXQ_F16, 2>);
+    DAXQ_PREP(prepare_then_quadrants<false, DAXQ_F32, 2>);
+    DAXQ_PREP(prepare_then_quadrants<false, DAXQ_BF16, 4>);
+    DAXQ_PREP(prepare_then_quadrants<true, DAXQ_BF16, 4>);
+    DAXQ_PREP(prepare_then_quadrants<false, DAXQ_F16, 4>);
+    DAXQ_PREP(prepare_then_quadrants<false, DAXQ_F32, 4>);
 #undef DAXQ_PREP
-    if (!rc) rc = prepare_tile256x128_kernels();
     return rc;
 }
 

@@ -1,4 +1,6 @@
-// W8A8 GEMM on half tiles of 256 x 128 outputs: the left-over tiles of a launch of few rounds (INT8 first, FP8 below).
+// W8A8 GEMM on half tiles of 256 x 128 outputs: the left-over tiles of a launch of few rounds (INT8 first, FP8 below),
+// as device functions that the kernels of gemm_tile256.hip and gemm_tile_fp8.hip run in the workgroups behind those of
+// the whole tiles.
 //
 // A launch of 256x256 tiles that leaves L tiles over after its whole rounds of workgroups pays a whole tile time for
 // them.  Up to a quarter of the CUs' worth of such tiles run as 128x128 quadrants with a CU each (gemm_tile256.hip);
@@ -8,6 +10,8 @@
 // slice, the 4 of the weight rows during the odd one).  A half tile has 12 fragment reads per 32 MFMAs where the whole
 // tile has 16 per 64, so it runs at about 0.7 of the whole tile's pace: 0.7 of a tile time instead of one.
 // Same arithmetic as the large kernel: int32 accumulators, identical outputs.
+#pragma once
+
 #include "gemm_tile.h"
 
 namespace daxq {
@@ -23,19 +27,19 @@ constexpr int SMEM = NSTG * STAGE;
 }  // namespace h2
 
 template <bool DUMP, int OUTK>
-__global__ __launch_bounds__(256) void gemm_tile256x128_kernel(const GemmArgs p) {
+__device__ __forceinline__ void gemm_tile256x128_body(const GemmArgs& p, const int half_id) {
     static_assert(OUTK == DAXQ_BF16 || !DUMP, "the accumulator dump exists with bf16 outputs");
     using namespace h2;
     extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
 
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
     const int wm = wave >> 1, wn = wave & 1;
-    // half (blockIdx.x & 1) of the 256x256 tile quad_base - 1 + blockIdx.x / 2 of the row-group order
+    // half (half_id & 1) of the 256x256 tile quad_base - 1 + half_id / 2 of the row-group order
     int tm, tn;
-    tile_of_block(p.gm, p.quad_base - 1 + ((int)blockIdx.x >> 1), p.tiles_m, p.tiles_n, tm, tn);
+    tile_of_block(p.gm, p.quad_base - 1 + (half_id >> 1), p.tiles_m, p.tiles_n, tm, tn);
     int m0 = tm * 256, n0 = tn * 256;
     m0 = m0 + 256 <= p.m ? m0 : p.m - 256;
-    n0 = (n0 + 256 <= p.n ? n0 : p.n - 256) + ((int)blockIdx.x & 1) * 128;
+    n0 = (n0 + 256 <= p.n ? n0 : p.n - 256) + (half_id & 1) * 128;
 
     // ---- HBM side.  One wave instruction fills 1 KB of LDS = 16 rows x 64 B: lane l -> row l/4, stored chunk l%4,
     //      i.e. global chunk (l%4) ^ ((row>>1)&3).  Instruction j of a thread covers tile rows j*64 + t/4.
@@ -190,38 +194,6 @@ __global__ __launch_bounds__(256) void gemm_tile256x128_kernel(const GemmArgs p)
                                                  !p.bias ? -0.0f : OUTK == DAXQ_F32 ? __uint_as_float(pre_b) : OUTK == DAXQ_F16 ? f16_bits_to_f32((uint16_t)pre_b) : bf16_bits_to_f32(pre_b));
 }
 
-template <bool DUMP, int OUTK>
-static int prepare_h2() {
-    static std::atomic<uint64_t> lds_set{0};  // per instantiation
-    return ensure_dynamic_lds(reinterpret_cast<const void*>(gemm_tile256x128_kernel<DUMP, OUTK>), h2::SMEM, lds_set);
-}
-
-template <bool DUMP, int OUTK>
-static int launch_h2(const GemmArgs& a, hipStream_t st) {
-    if (int rc = prepare_h2<DUMP, OUTK>()) return rc;
-    hipLaunchKernelGGL((gemm_tile256x128_kernel<DUMP, OUTK>), dim3((unsigned)a.grid), dim3(h2::T), h2::SMEM, st, a);
-    return check_launch("gemm_tile256x128");
-}
-
-int prepare_tile256x128_kernels() {
-    if (int rc = prepare_h2<false, DAXQ_BF16>()) return rc;
-    if (int rc = prepare_h2<true, DAXQ_BF16>()) return rc;
-    if (int rc = prepare_h2<false, DAXQ_F16>()) return rc;
-    return prepare_h2<false, DAXQ_F32>();
-}
-
-// The two halves of each of the `left` 256x256 tiles from id `first` on (row-group order; a.tiles_m / a.tiles_n count
-// 256x256 tiles).  INT8, m and n of at least 256, K a multiple of 128 (the caller has checked the shape).
-int launch_tile256x128(const GemmArgs& a0, int first, int left, hipStream_t st) {
-    GemmArgs a = a0;
-    a.quad_base = first + 1;
-    a.grid = 2 * left;
-    if (a.acc && a.out_kind != DAXQ_BF16) return fail(DAXQ_ERR_ARG, "gemm: the accumulator dump exists with bf16 outputs");
-    if (a.out_kind == DAXQ_F16) return launch_h2<false, DAXQ_F16>(a, st);
-    if (a.out_kind == DAXQ_F32) return launch_h2<false, DAXQ_F32>(a, st);
-    return a.acc ? launch_h2<true, DAXQ_BF16>(a, st) : launch_h2<false, DAXQ_BF16>(a, st);
-}
-
 // ---------------------------------------------------------------------------------------------------------------------
 // The same half tile for FP8 operands (v_mfma_f32_16x16x128_f8f6f4).  An output element is the same sequence of MFMAs
 // over the same K bytes in the same register positions as in gemm_tile_fp8.hip -- one MFMA per pair of 64-byte slices,
@@ -239,17 +211,17 @@ constexpr int SMEM = 3 * SLOT;
 }  // namespace h2f
 
 template <bool DUMP, int F8, int OUTK>
-__global__ __launch_bounds__(256) void gemm_tile256x128_fp8_kernel(const GemmArgs p) {
+__device__ __forceinline__ void gemm_tile256x128_fp8_body(const GemmArgs& p, const int half_id) {
     static_assert(OUTK == DAXQ_BF16 || !DUMP, "the accumulator dump exists with bf16 outputs");
     using namespace h2f;
     extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
     const int wm = wave >> 1, wn = wave & 1;
     int tm, tn;
-    tile_of_block(p.gm, p.quad_base - 1 + ((int)blockIdx.x >> 1), p.tiles_m, p.tiles_n, tm, tn);
+    tile_of_block(p.gm, p.quad_base - 1 + (half_id >> 1), p.tiles_m, p.tiles_n, tm, tn);
     int m0 = tm * 256, n0 = tn * 256;
     m0 = m0 + 256 <= p.m ? m0 : p.m - 256;
-    n0 = (n0 + 256 <= p.n ? n0 : p.n - 256) + ((int)blockIdx.x & 1) * 128;
+    n0 = (n0 + 256 <= p.n ? n0 : p.n - 256) + (half_id & 1) * 128;
 
     const uint32_t gsw = (uint32_t)(((t & 3) ^ ((t >> 3) & 3)) << 4);
     uint32_t voff_a = (uint32_t)(t >> 2) * (uint32_t)p.lda + gsw;
@@ -420,55 +392,6 @@ __global__ __launch_bounds__(256) void gemm_tile256x128_fp8_kernel(const GemmArg
     __syncthreads();  // every wavefront is past its last fragment read (the short-K loop has no barrier behind its reads)
     tile_epilogue16<DUMP, NBJ, NBI, true, OUTK>(p, acc, smem, m0, n0, t, wm, wn, lr, kg, pre_sx, pre_sw,
                                                 !p.bias ? -0.0f : OUTK == DAXQ_F32 ? __uint_as_float(pre_b) : OUTK == DAXQ_F16 ? f16_bits_to_f32((uint16_t)pre_b) : bf16_bits_to_f32(pre_b));
-}
-
-template <bool DUMP, int F8, int OUTK>
-static int prepare_h2f() {
-    static std::atomic<uint64_t> lds_set{0};  // per instantiation
-    return ensure_dynamic_lds(reinterpret_cast<const void*>(gemm_tile256x128_fp8_kernel<DUMP, F8, OUTK>), h2f::SMEM, lds_set);
-}
-
-template <bool DUMP, int F8, int OUTK>
-static int launch_h2f(const GemmArgs& a, hipStream_t st) {
-    if (int rc = prepare_h2f<DUMP, F8, OUTK>()) return rc;
-    hipLaunchKernelGGL((gemm_tile256x128_fp8_kernel<DUMP, F8, OUTK>), dim3((unsigned)a.grid), dim3(h2f::T), h2f::SMEM, st, a);
-    return check_launch("gemm_tile256x128_fp8");
-}
-
-template <int F8>
-static int prepare_h2f_all() {
-    if (int rc = prepare_h2f<false, F8, DAXQ_BF16>()) return rc;
-    if (int rc = prepare_h2f<true, F8, DAXQ_BF16>()) return rc;
-    if (int rc = prepare_h2f<false, F8, DAXQ_F16>()) return rc;
-    return prepare_h2f<false, F8, DAXQ_F32>();
-}
-
-int prepare_tile256x128_fp8_kernels() {
-    if (int rc = prepare_h2f_all<0>()) return rc;
-    if (int rc = prepare_h2f_all<1>()) return rc;
-    if (int rc = prepare_h2f_all<2>()) return rc;
-    return prepare_h2f_all<3>();
-}
-
-template <int F8>
-static int launch_h2f_out(const GemmArgs& a, hipStream_t st) {
-    if (a.acc && a.out_kind != DAXQ_BF16) return fail(DAXQ_ERR_ARG, "gemm: the accumulator dump exists with bf16 outputs");
-    if (a.out_kind == DAXQ_F16) return launch_h2f<false, F8, DAXQ_F16>(a, st);
-    if (a.out_kind == DAXQ_F32) return launch_h2f<false, F8, DAXQ_F32>(a, st);
-    return a.acc ? launch_h2f<true, F8, DAXQ_BF16>(a, st) : launch_h2f<false, F8, DAXQ_BF16>(a, st);
-}
-
-// FP8 form of launch_tile256x128
-int launch_tile256x128_fp8(const GemmArgs& a0, int f8, int first, int left, hipStream_t st) {
-    GemmArgs a = a0;
-    a.quad_base = first + 1;
-    a.grid = 2 * left;
-    switch (f8) {
-        case 1: return launch_h2f_out<1>(a, st);
-        case 2: return launch_h2f_out<2>(a, st);
-        case 3: return launch_h2f_out<3>(a, st);
-        default: return launch_h2f_out<0>(a, st);
-    }
 }
 
 }  // namespace daxq

@@ -32,6 +32,7 @@
 // the MFMA needs: the order of K inside an instruction is free as long as both operands agree.
 // K shorter than four pairs (K < 512) takes a plain loop of the same MFMAs: load a pair, wait, multiply.
 #include "gemm_tile.h"
+#include "gemm_tile256x128.h"
 
 namespace daxq {
 
@@ -40,7 +41,7 @@ constexpr int BKS = 64, T = 256, NPART = 5;
 }  // namespace f16
 
 template <bool DUMP, int F8, int BT = 256, int OUTK = DAXQ_BF16>
-__global__ __launch_bounds__(256) void gemm_tile_fp8_kernel(const GemmArgs p) {
+__device__ __forceinline__ void gemm_tile_fp8_body(const GemmArgs& p, const int block) {
     using namespace f16;
     static_assert(BT == 256 || BT == 128, "tile edge");
     static_assert(OUTK == DAXQ_BF16 || !DUMP, "the accumulator dump exists with bf16 outputs");
@@ -57,7 +58,7 @@ __global__ __launch_bounds__(256) void gemm_tile_fp8_kernel(const GemmArgs p) {
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
     const int wm = wave >> 1, wn = wave & 1;
     int m0, n0;
-    if (!tile_origin<BT>(p, blockIdx.x, m0, n0)) return;  // padding slot (before any barrier)
+    if (!tile_origin<BT>(p, block, m0, n0)) return;  // padding slot (before any barrier)
 
     // ---- HBM side: one wave instruction fills 1 KB of LDS = 16 rows x 64 B; lane l -> row l/4, stored chunk l%4,
     //      i.e. global chunk (l%4) ^ ((row >> 1) & 3).  Load g of an operand and pair: row block g/2 (64 rows, of which
@@ -340,6 +341,28 @@ __global__ __launch_bounds__(256) void gemm_tile_fp8_kernel(const GemmArgs p) {
                                              !p.bias ? -0.0f : OUTK == DAXQ_F32 ? __uint_as_float(pre_b) : OUTK == DAXQ_F16 ? f16_bits_to_f32((uint16_t)pre_b) : bf16_bits_to_f32(pre_b));
 }
 
+template <bool DUMP, int F8, int BT = 256, int OUTK = DAXQ_BF16>
+__global__ __launch_bounds__(256) void gemm_tile_fp8_kernel(const GemmArgs p) {
+    gemm_tile_fp8_body<DUMP, F8, BT, OUTK>(p, (int)blockIdx.x);
+}
+
+// One grid for a launch of few rounds whose left-over tiles run as halves (tail_half_tiles): workgroups 0 .. p.grid - 1
+// compute whole 256x256 tiles, the rest the 256x128 halves of the tiles from id quad_base - 1 on.  The halves start on
+// the CUs that finish their whole tiles first instead of behind the whole first kernel.
+template <bool DUMP, int F8, int OUTK>
+__global__ __launch_bounds__(256) void gemm_tile_fp8_then_halves_kernel(const GemmArgs p) {
+    if ((int)blockIdx.x < p.grid) gemm_tile_fp8_body<DUMP, F8, 256, OUTK>(p, (int)blockIdx.x);
+    else gemm_tile256x128_fp8_body<DUMP, F8, OUTK>(p, (int)blockIdx.x - p.grid);
+}
+
+// The same for left-over tiles that run as 128x128 quadrants (tail_tiles): workgroups 0 .. p.grid - 1 compute whole
+// tiles, the rest the quadrants of the tiles from id quad_base - 1 on.
+template <bool DUMP, int F8, int OUTK>
+__global__ __launch_bounds__(256) void gemm_tile_fp8_then_quadrants_kernel(const GemmArgs p) {
+    if ((int)blockIdx.x < p.grid) gemm_tile_fp8_body<DUMP, F8, 256, OUTK>(p, (int)blockIdx.x);
+    else gemm_tile_fp8_body<DUMP, F8, 128, OUTK>(p, (int)blockIdx.x - p.grid);
+}
+
 template <bool DUMP, int F8, int BT, int OUTK>
 static int prepare_fp8() {
     static std::atomic<uint64_t> lds_set{0};  // per instantiation
@@ -349,7 +372,7 @@ static int prepare_fp8() {
 template <bool DUMP, int F8, int BT, int OUTK>
 static int launch_fp8_impl(const GemmArgs& a, hipStream_t st) {
     if (int rc = prepare_fp8<DUMP, F8, BT, OUTK>()) return rc;
-    const int64_t nt = a.grid > 0 ? a.grid : grid_of_order(a);
+    const int64_t nt = grid_of_order(a);
     if (nt > 0x7fffffff) return fail(DAXQ_ERR_ARG, "gemm: too many tiles");
     hipLaunchKernelGGL((gemm_tile_fp8_kernel<DUMP, F8, BT, OUTK>), dim3((unsigned)nt), dim3(f16::T), f16::NPART * 2 * BT * f16::BKS, st, a);
     return check_launch("gemm_tile_fp8");
@@ -372,12 +395,56 @@ static int launch_fp8_one(const GemmArgs& a, int f8, hipStream_t st) {
     }
 }
 
-// small: 128x128 tiles (needs m, n >= 128); f8: operand formats (kF8XE5 | kF8WE5); tail: the last, partial round of a
-// launch of 256x256 tiles as a second launch on its 128x128 quadrants (tail_tiles) or 256x128 halves (tail_half_tiles)
-// -- the same bits either way
-int launch_tile256x128_fp8(const GemmArgs& a, int f8, int first, int left, hipStream_t st);  // gemm_tile256x128.hip
-int prepare_tile256x128_fp8_kernels();
+// QUADS: the second part of the grid is quadrants (else halves)
+template <bool QUADS, bool DUMP, int F8, int OUTK>
+static const void* fp8_then_kernel() {
+    if constexpr (QUADS) return reinterpret_cast<const void*>(gemm_tile_fp8_then_quadrants_kernel<DUMP, F8, OUTK>);
+    else return reinterpret_cast<const void*>(gemm_tile_fp8_then_halves_kernel<DUMP, F8, OUTK>);
+}
 
+template <bool QUADS, bool DUMP, int F8, int OUTK>
+static int prepare_fp8_then() {
+    static std::atomic<uint64_t> lds_set{0};  // per instantiation
+    return ensure_dynamic_lds(fp8_then_kernel<QUADS, DUMP, F8, OUTK>(), f16::NPART * 2 * 256 * f16::BKS, lds_set);
+}
+
+template <bool QUADS, bool DUMP, int F8, int OUTK>
+static int launch_fp8_then_impl(const GemmArgs& a, int64_t nt, hipStream_t st) {
+    if (int rc = prepare_fp8_then<QUADS, DUMP, F8, OUTK>()) return rc;
+    constexpr int SMEM = f16::NPART * 2 * 256 * f16::BKS;
+    if constexpr (QUADS) hipLaunchKernelGGL((gemm_tile_fp8_then_quadrants_kernel<DUMP, F8, OUTK>), dim3((unsigned)nt), dim3(f16::T), SMEM, st, a);
+    else hipLaunchKernelGGL((gemm_tile_fp8_then_halves_kernel<DUMP, F8, OUTK>), dim3((unsigned)nt), dim3(f16::T), SMEM, st, a);
+    return check_launch(QUADS ? "gemm_tile_fp8_then_quadrants" : "gemm_tile_fp8_then_halves");
+}
+
+template <bool QUADS, int F8>
+static int launch_fp8_then_out(const GemmArgs& a, int64_t nt, hipStream_t st) {
+    if (a.acc && a.out_kind != DAXQ_BF16) return fail(DAXQ_ERR_ARG, "gemm: the accumulator dump exists with bf16 outputs");
+    if (a.out_kind == DAXQ_F16) return launch_fp8_then_impl<QUADS, false, F8, DAXQ_F16>(a, nt, st);
+    if (a.out_kind == DAXQ_F32) return launch_fp8_then_impl<QUADS, false, F8, DAXQ_F32>(a, nt, st);
+    return a.acc ? launch_fp8_then_impl<QUADS, true, F8, DAXQ_BF16>(a, nt, st) : launch_fp8_then_impl<QUADS, false, F8, DAXQ_BF16>(a, nt, st);
+}
+
+// `whole` 256x256 tiles of the row-group order, then the pieces of each of the `left` tiles behind them (QUADS: four
+// 128x128 quadrants, else two 256x128 halves), in one grid
+template <bool QUADS>
+static int launch_fp8_then(const GemmArgs& a0, int f8, int whole, int left, hipStream_t st) {
+    GemmArgs a = a0;
+    a.grid = whole;
+    a.quad_base = whole + 1;
+    const int64_t nt = (int64_t)whole + (QUADS ? 4 : 2) * (int64_t)left;
+    if (nt > 0x7fffffff) return fail(DAXQ_ERR_ARG, "gemm: too many tiles");
+    switch (f8) {
+        case 1: return launch_fp8_then_out<QUADS, 1>(a, nt, st);
+        case 2: return launch_fp8_then_out<QUADS, 2>(a, nt, st);
+        case 3: return launch_fp8_then_out<QUADS, 3>(a, nt, st);
+        default: return launch_fp8_then_out<QUADS, 0>(a, nt, st);
+    }
+}
+
+// small: 128x128 tiles (needs m, n >= 128); f8: operand formats (kF8XE5 | kF8WE5); tail: the last, partial round of a
+// launch of 256x256 tiles as 128x128 quadrants (tail_tiles) or 256x128 halves (tail_half_tiles) in the workgroups
+// behind those of the whole tiles -- the same bits either way
 int launch_tile_fp8(const GemmArgs& a0, int f8, bool small, int tail, hipStream_t st) {
     GemmArgs a = a0;
     const int bt = small ? 128 : 256;
@@ -393,17 +460,9 @@ int launch_tile_fp8(const GemmArgs& a0, int f8, bool small, int tail, hipStream_
         // more than a quarter and at most half of the CUs' worth of tiles left over: their 256x128 halves with a CU each
         const int halves = tail_half_tiles(a, tail);
         if (halves == 0) return launch_fp8_one<256>(a, f8, st);
-        const int whole = a.tiles_m * a.tiles_n - halves;
-        a.grid = whole;
-        if (int rc = launch_fp8_one<256>(a, f8, st)) return rc;
-        return launch_tile256x128_fp8(a, f8, whole, halves, st);
+        return launch_fp8_then<false>(a, f8, a.tiles_m * a.tiles_n - halves, halves, st);
     }
-    const int whole = a.tiles_m * a.tiles_n - left;
-    a.grid = whole;
-    if (int rc = launch_fp8_one<256>(a, f8, st)) return rc;
-    a.grid = 4 * left;
-    a.quad_base = whole + 1;
-    return launch_fp8_one<128>(a, f8, st);
+    return launch_fp8_then<true>(a, f8, a.tiles_m * a.tiles_n - left, left, st);
 }
 
 // Every instantiation the launcher can pick, prepared on the current device: afterwards no launch changes a kernel
@@ -419,14 +478,21 @@ int prepare_tile_fp8_kernels() {
     DAXQ_PREP(prepare_fp8<false, F8, 128, DAXQ_BF16>);    \
     DAXQ_PREP(prepare_fp8<true, F8, 128, DAXQ_BF16>);     \
     DAXQ_PREP(prepare_fp8<false, F8, 128, DAXQ_F16>);     \
-    DAXQ_PREP(prepare_fp8<false, F8, 128, DAXQ_F32>)
+    DAXQ_PREP(prepare_fp8<false, F8, 128, DAXQ_F32>);     \
+    DAXQ_PREP(prepare_fp8_then<false, false, F8, DAXQ_BF16>); \
+    DAXQ_PREP(prepare_fp8_then<false, true, F8, DAXQ_BF16>);  \
+    DAXQ_PREP(prepare_fp8_then<false, false, F8, DAXQ_F16>);  \
+    DAXQ_PREP(prepare_fp8_then<false, false, F8, DAXQ_F32>);  \
+    DAXQ_PREP(prepare_fp8_then<true, false, F8, DAXQ_BF16>);  \
+    DAXQ_PREP(prepare_fp8_then<true, true, F8, DAXQ_BF16>);   \
+    DAXQ_PREP(prepare_fp8_then<true, false, F8, DAXQ_F16>);   \
+    DAXQ_PREP(prepare_fp8_then<true, false, F8, DAXQ_F32>)
     DAXQ_PREP_F8(0);
     DAXQ_PREP_F8(1);
     DAXQ_PREP_F8(2);
     DAXQ_PREP_F8(3);
 #undef DAXQ_PREP_F8
 #undef DAXQ_PREP
-    if (!rc) rc = prepare_tile256x128_fp8_kernels();
     return rc;
 }
 

@@ -305,7 +305,7 @@ enum { K_DEFAULT = 0, K_GENERIC256 = 2, K_GENERIC128 = 5, K_TILED_256 = 8, K_TIL
 // five bands (N < 5120), K below 2048 or few rounds the row groups were as fast or faster (K = 1536: -2 %; N = K = 4096:
 // -2 %; M = 9450, a 1/8 share of the rows, 3 to 9 rounds: -0.8 to +2 % per linear and +0.2 / +1.0 % INT8 / FP8 over the
 // four, now that the rows under the last whole step form dense patches, -3 to -16 % before; M = 4725: -4 to -5 %; M =
-// 20000: +3 % at N >= 13824, -3 % at N = 5120, where the row groups run their last tiles as a second launch).
+// 20000: +3 % at N >= 13824, -3 % at N = 5120, where the row groups run their last tiles as quadrants).
 static int order_by_shape(int64_t m, int64_t n, int64_t k) {
     const int64_t tm = (m + 255) / 256, tn = (n + 255) / 256, tiles = tm * tn;
     // (tm >= 64: at least two super-rows of whole 8 x 4 patches; tm <= 100000 and tn <= 4096: the range the host-side
@@ -357,8 +357,8 @@ static int launch_gemm(const void* xq, int64_t ld_xq, const float* sx, const voi
     a.counters = nullptr;
     a.partials = nullptr;
     a.grid = a.quad_base = 0;
-    // bits 28-29 of `kernel`: the last partial round of a launch of 256x256 tiles as a second launch on 128x128 tiles (or,
-    // when they number more than a quarter of the CUs, on 256x128 tiles): 0 = by shape, 1 = never, 2 = whenever every such tile gets a CU of its own
+    // bits 28-29 of `kernel`: the last partial round of a launch of 256x256 tiles as 128x128 quadrants (or, when its tiles
+    // number more than a quarter of the CUs, as 256x128 halves): 0 = by shape, 1 = never, 2 = whenever every piece gets a CU of its own
     const int tail = (kernel >> 28) & 3;
     if (tail > 2) return fail(DAXQ_ERR_ARG, "linear: unknown tail choice %d", tail);
     const int which = kernel & 0xffff;

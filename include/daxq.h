@@ -290,8 +290,9 @@ int daxq_linear_e5m2_e4m3(const uint8_t* xq, int64_t ld_xq, const float* sx,
  * (0 = by shape, 1 = groups of tile rows, 2 = banded patches of 8 x 4 tiles per XCD; every order computes every tile
  * once, the results are the same bits); bits 28-29 the treatment of the last, partial round of workgroups of a launch
  * of 256x256 tiles in row groups (0 = by shape: when the launch has one to eight whole rounds and the tiles left over
- * number at most a quarter of the CUs, they run as a second launch of 128x128 tiles with a CU each, and when they
- * number at most half of the CUs, as a second launch of 256x128 tiles with a CU each (every output type);
+ * number at most a quarter of the CUs, they run as their 128x128 quadrants with a CU each, and when they
+ * number at most half of the CUs, as their 256x128 halves with a CU each, in workgroups of the same grid behind
+ * those of the whole tiles;
  * 1 = never; 2 = whenever they number at most a quarter / half of the CUs).
  * int8 results are the same bits for every choice.  fp8 results are the same bits for every choice of tile size, tile
  * order and cut of the tiled kernel (one sequence of MFMAs per output element), so an output row does not depend on

@@ -136,8 +136,8 @@ def test_int8_module_fp16_fp32_bit_exact(dtype, m, k, n):
                                            (8, 4725, 5120, 128)])
 def test_int8_fp16_fp32_outputs_of_the_tiled_kernels(variant, m, n, k, dtype):
     """fp16 / fp32 outputs straight from the kernels on 16x16 MFMAs, named by argument, with and without bias, edge
-    tiles included; 289 tiles with the tiles left over after one round forced into a second launch of quadrants, 380
-    tiles with the 124 left over as a second launch of 256x128 halves (all of them write the type).  Values beyond the fp16 range become infinities, as the reference's cast makes them."""
+    tiles included; 289 tiles with the tiles left over after one round forced into quadrants, 380
+    tiles with the 124 left over as 256x128 halves (all of them write the type).  Values beyond the fp16 range become infinities, as the reference's cast makes them."""
     import dax_amd.ops as ops
     from dax_amd import _capi
 
@@ -169,8 +169,8 @@ def test_int8_fp16_fp32_outputs_of_the_tiled_kernels(variant, m, n, k, dtype):
                                            (8, 4725, 5120, 256)])
 def test_fp8_fp16_fp32_outputs_of_the_tiled_kernels(variant, m, n, k, dtype, x_fmt, w_fmt):
     """fp16 / fp32 outputs of FP8 operands (what a per-tensor FP8 module that is not bf16 asks for) from the kernel on
-    16x16x128 MFMAs, on both tile sizes, with and without bias, and with the last round cut into a second launch (of
-    quadrants, or of 256x128 halves in the last shape):
+    16x16x128 MFMAs, on both tile sizes, with and without bias, and with the last round cut into smaller pieces
+    (quadrants, or 256x128 halves in the last shape):
     out = T(acc * sx * sw + bias) with one rounding, against the oracle's scaled matmul at 3e-3 relative L2, and
     against the same kernel's bf16 launch (its accumulators are the same, so its fp32 result rounded to bf16 must
     equal the bf16 output bit for bit)."""

@@ -118,12 +118,12 @@ HALF_TAIL_SHAPES = [(4725, 5120, 128), (4725, 15360 - 24, 256), (9000, 2560, 384
 
 
 @pytest.mark.parametrize("m,n,k", TAIL_SHAPES + HALF_TAIL_SHAPES)
-def test_last_round_as_a_second_launch_bit_exact(ops, m, n, k):
+def test_last_round_in_smaller_pieces_bit_exact(ops, m, n, k):
     """A launch of 256x256 tiles whose last round of workgroups is a few tiles: the whole rounds run as 256x256 tiles,
-    the tiles left over as a second launch of their 128x128 quadrants or, INT8 with more than a quarter of the CUs' worth
-    of them, of their 256x128 halves.  Accumulators and outputs equal the integer
-    oracle's with the cut forced and by shape; FP8 outputs are the single launch's bits (both tile sizes run the same
-    sequence of MFMAs per output element)."""
+    the tiles left over, in the workgroups behind them in the same grid, as their 128x128 quadrants or, with more than a
+    quarter of the CUs' worth of them, as their 256x128 halves.  Accumulators and outputs equal the integer
+    oracle's with the cut forced and by shape; FP8 outputs are the bits of the launch of whole tiles (every tile size
+    runs the same sequence of MFMAs per output element)."""
     from dax_amd import _capi
 
     tiles = -(-m // 256) * -(-n // 256)

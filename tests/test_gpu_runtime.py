@@ -231,7 +231,7 @@ def test_split_k_shape_captured_on_a_stream_that_already_has_a_workspace():
 def test_captured_graph_of_the_256_tile_kernels_replays_match_eager(fp8, m, n, k, order, tail):
     """The kernels the large shapes run on (INT8 16x16x64, FP8 16x16x128; chosen by argument here because the shape
     is small), captured and replayed with new operand contents: in the banded tile order with its padding workgroups,
-    and as the two launches of a grid whose last round of workgroups is cut off (289 tiles: 256 + 33 as quadrants)."""
+    and as the grid whose last round of workgroups runs in smaller pieces (289 tiles: 256 + 33 as quadrants)."""
     import dax_amd.ops as ops
     from dax_amd import _capi
 
