@@ -226,12 +226,13 @@ def test_split_k_shape_captured_on_a_stream_that_already_has_a_workspace():
         assert _same(static_out, want), f"replay with seed {seed} differs from eager"
 
 
-@pytest.mark.parametrize("m,n,k,order,tail", [(700, 2304, 1024, 2002, 3000), (4100, 4352, 256, 2001, 3002)])
+@pytest.mark.parametrize("m,n,k,order,tail", [(700, 2304, 1024, 2002, 3000), (4100, 4352, 256, 2001, 3002), (4725, 5120, 256, 2001, 3000)])
 @pytest.mark.parametrize("fp8", [False, True])
 def test_captured_graph_of_the_256_tile_kernels_replays_match_eager(fp8, m, n, k, order, tail):
     """The kernels the large shapes run on (INT8 16x16x64, FP8 16x16x128; chosen by argument here because the shape
     is small), captured and replayed with new operand contents: in the banded tile order with its padding workgroups,
-    and as the grid whose last round of workgroups runs in smaller pieces (289 tiles: 256 + 33 as quadrants)."""
+    and as the grids whose last round of workgroups runs in smaller pieces (289 tiles: 256 + 33 as quadrants; 380 tiles:
+    256 + 124 as halves)."""
     import dax_amd.ops as ops
     from dax_amd import _capi
 
