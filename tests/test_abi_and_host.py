@@ -31,6 +31,36 @@ def test_library_exports_every_declared_symbol():
     assert "undefined symbol" not in _capi.last_error()
 
 
+def test_header_is_plain_c_and_a_c_program_links(tmp_path):
+    """include/daxq.h is the boundary a cgo / JNI / FFI binding would consume: it must compile as C99 and as C++11
+    without extensions, and a C program that includes it must link against the library and run (only entry points that
+    need no device are called)."""
+    import shutil
+    import subprocess
+
+    from dax_amd import _capi
+
+    gcc, gxx = shutil.which("gcc"), shutil.which("g++")
+    if not gcc or not gxx:
+        pytest.skip("no host compiler")
+    src = tmp_path / "abi.c"
+    src.write_text('#include <stdio.h>\n#include "daxq.h"\n'
+                   "int main(void) {\n"
+                   "    int (*f)(int, int, int, const void*, int64_t, const float*, const void*, int64_t, const float*, const void*,\n"
+                   "             void*, int64_t, void*, int64_t, int64_t, int64_t, int64_t, int, daxq_stream_t) = daxq_linear_w8a8;\n"
+                   '    printf("%d %d %s\\n", daxq_abi_version(), DAXQ_ABI_VERSION, f ? "ok" : "null");\n'
+                   "    return daxq_abi_version() == DAXQ_ABI_VERSION ? 0 : 1;\n}\n")
+    inc = os.path.join(ROOT, "include")
+    subprocess.run([gcc, "-std=c99", "-pedantic", "-Wall", "-Wextra", "-Werror", "-fsyntax-only", "-I", inc, str(src)], check=True)
+    subprocess.run([gxx, "-std=c++11", "-pedantic", "-Wall", "-Wextra", "-Werror", "-fsyntax-only", "-x", "c++", "-I", inc, str(src)], check=True)
+    exe = tmp_path / "abi"
+    libdir = os.path.dirname(_capi.LIB_PATH)
+    subprocess.run([gcc, "-std=c99", "-I", inc, str(src), "-o", str(exe), "-L", libdir, "-ldaxq", f"-Wl,-rpath,{libdir}",
+                    "-Wl,--allow-shlib-undefined"], check=True)
+    out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.split()
+    assert out == [str(_capi.ABI_VERSION), str(_capi.ABI_VERSION), "ok"]
+
+
 def test_patch_tile_order_covers_every_tile_once():
     """tests/host/tile_order_check (built by __graft_entry__.build() from the header the kernels include): every tile
     grid up to 320 x 72 and sampled grids up to 100003 tile rows and 4096 tile columns (the range the library's choice
