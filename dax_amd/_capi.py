@@ -138,8 +138,8 @@ _tail = 0
 
 
 def debug_select_gemm(v: int) -> None:
-    """0 = the library's choice by shape; 2 / 5 / 8 / 11 = one implementation (include/daxq.h: the generic kernel on
-    256x256 / 128x128 tiles, the tiled kernel on 256x256 / 128x128 tiles); 1000 + d = depth d of the tile-order groups
+    """0 = the library's choice by shape; 2 / 5 / 8 / 11 / 14 = one implementation (include/daxq.h: the generic kernel on
+    256x256 / 128x128 tiles, the tiled kernel on 256x256 / 128x128 / 256x128 tiles); 1000 + d = depth d of the tile-order groups
     (1000 = default); 2000 + o = tile order of the 256x256 kernels (2000 = by shape, 2001 = groups of tile rows,
     2002 = banded patches); 3000 + t = the last partial round of a 256x256 launch as 128x128 quadrants or 256x128 halves
     (3000 = by shape, 3001 = never, 3002 = whenever every such tile gets a CU)."""
@@ -151,7 +151,7 @@ def debug_select_gemm(v: int) -> None:
         _tile_order = v - 2000
     elif 3000 <= v < 3003:
         _tail = v - 3000
-    elif v in (0, 2, 5, 8, 11):
+    elif v in (0, 2, 5, 8, 11, 14):
         _kernel_choice = v
     else:
         raise DaxqError(f"unknown gemm kernel choice {v}")

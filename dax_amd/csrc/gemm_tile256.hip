@@ -732,6 +732,17 @@ static int launch_then_quadrants(const GemmArgs& a0, int whole, int left, hipStr
     return a.k >= 4096 ? launch_then_quadrants_out<4>(a, nt, st) : launch_then_quadrants_out<2>(a, nt, st);
 }
 
+// Every 256x256 tile as its two 256x128 halves (needs m, n >= 256): the grid of launch_then_halves without whole tiles
+int launch_halves_i8(const GemmArgs& a0, hipStream_t st) {
+    GemmArgs a = a0;
+    a.tiles_m = (a.m + 255) / 256;
+    a.tiles_n = (a.n + 255) / 256;
+    a.order = kOrderRowGroups;
+    const int64_t tiles = (int64_t)a.tiles_m * a.tiles_n;
+    if (tiles > 0x3fffffff) return fail(DAXQ_ERR_ARG, "gemm: too many tiles");
+    return launch_then_halves(a, 0, (int)tiles, st);
+}
+
 int launch_tile_i8(const GemmArgs& a0, bool small, int tail, hipStream_t st) {
     GemmArgs a = a0;
     const int bt = small ? 128 : 256;

@@ -442,6 +442,17 @@ static int launch_fp8_then(const GemmArgs& a0, int f8, int whole, int left, hipS
     }
 }
 
+// Every 256x256 tile as its two 256x128 halves (needs m, n >= 256): the grid of launch_fp8_then without whole tiles
+int launch_halves_fp8(const GemmArgs& a0, int f8, hipStream_t st) {
+    GemmArgs a = a0;
+    a.tiles_m = (a.m + 255) / 256;
+    a.tiles_n = (a.n + 255) / 256;
+    a.order = kOrderRowGroups;
+    const int64_t tiles = (int64_t)a.tiles_m * a.tiles_n;
+    if (tiles > 0x3fffffff) return fail(DAXQ_ERR_ARG, "gemm: too many tiles");
+    return launch_fp8_then<false>(a, f8, 0, (int)tiles, st);
+}
+
 // small: 128x128 tiles (needs m, n >= 128); f8: operand formats (kF8XE5 | kF8WE5); tail: the last, partial round of a
 // launch of 256x256 tiles as 128x128 quadrants (tail_tiles) or 256x128 halves (tail_half_tiles) in the workgroups
 // behind those of the whole tiles -- the same bits either way

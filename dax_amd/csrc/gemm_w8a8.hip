@@ -243,6 +243,8 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_w8a8_kernel(const GemmArgs p
 bool tile256_applies(const GemmArgs& a);
 int launch_tile_i8(const GemmArgs& a, bool small, int tail, hipStream_t st);           // gemm_tile256.hip
 int launch_tile_fp8(const GemmArgs& a, int f8, bool small, int tail, hipStream_t st);  // gemm_tile_fp8.hip
+int launch_halves_i8(const GemmArgs& a, hipStream_t st);                                // gemm_tile256.hip
+int launch_halves_fp8(const GemmArgs& a, int f8, hipStream_t st);                       // gemm_tile_fp8.hip
 template <bool FP8>
 int launch_tile128_splitk(const GemmArgs& a, int f8, hipStream_t st);
 
@@ -250,6 +252,12 @@ template <bool FP8>
 static int launch_tiled(const GemmArgs& a, int f8, bool small, int tail, hipStream_t st) {
     if constexpr (FP8) return launch_tile_fp8(a, f8, small, tail, st);
     else return launch_tile_i8(a, small, tail, st);
+}
+
+template <bool FP8>
+static int launch_halves(const GemmArgs& a, int f8, hipStream_t st) {
+    if constexpr (FP8) return launch_halves_fp8(a, f8, st);
+    else return launch_halves_i8(a, st);
 }
 
 int prepare_tile_fp8_kernels();
@@ -293,7 +301,7 @@ static int launch_generic(const GemmArgs& a, int f8, hipStream_t st) {
 
 // Kernel choices of the `kernel` argument (daxq_linear_w8a8): low 16 bits pick the implementation, bits 16-23 the
 // depth of the tile-order groups (0 = 4 tile rows).
-enum { K_DEFAULT = 0, K_GENERIC256 = 2, K_GENERIC128 = 5, K_TILED_256 = 8, K_TILED_128 = 11 };
+enum { K_DEFAULT = 0, K_GENERIC256 = 2, K_GENERIC128 = 5, K_TILED_256 = 8, K_TILED_128 = 11, K_TILED_HALVES = 14 };
 
 // Tile order a launch of 256x256 tiles takes when the caller names none.  The banded order (tile_order.h: patches of
 // 8 x 4 tiles per XCD, the eight XCDs of a round on the same activation rows and on different weight bands) reads the
@@ -375,7 +383,16 @@ static int launch_gemm(const void* xq, int64_t ld_xq, const float* sx, const voi
             // one such tile.  Measured at N = K = 5120 (INT8, T-op/s, 128 / 256 tiles):
             // M = 512 -> 1127 / 551, M = 1024 (80 large tiles) -> 1275 / 1055, M = 2048 (160) -> 1542 / 1817;
             // 4096 x 1536 x 1536 (96) -> 1182 / 895, 8192 x 1536 x 1536 (192) -> 1517 / 1587.
+            // Between a quarter and a half of the CUs' worth of large tiles, every tile runs as its two 256x128 halves with
+            // a CU each (K >= 2048).  Measured against what these launches took before (128x128 tiles up to 127 large
+            // tiles, whole 256x256 tiles at 128), INT8 / e4m3, us: 1024 x 5120 x 5120 (80 tiles) 38.7 -> 31.0 / 37.7 -> 34.7,
+            // 1536 x 5120 x 5120 (120) 41.1 -> 35.0 / 40.3 -> 37.9, 1100 x 4352 x 5120 (85) 42.4 -> 31.6 / 41.1 -> 35.6,
+            // 2048 x 4096 x 4096 (128) 39.6 -> 30.7 / 38.7 -> 31.4, 1024 x 5120, K = 13824 95.9 -> 69.3 / 93.1 -> 80.6,
+            // 4096 x 1536, K = 8960 62.3 -> 50.7 / 60.5 -> 55.6, K = 3072 +9 to +15 % / +4 to +5 %, K = 2048 0 to +10 % / +2 %;
+            // at K = 1536 -2 / -5 %, and with 60 tiles (768 x 5120 x 5120) the quadrants' 23.8 us become 30.5.
             const int64_t tiles256 = ((m + 255) / 256) * ((n + 255) / 256);
+            const int cus = cu_count();
+            if (tile256_applies(a) && k >= 2048 && cus >= 8 && 4 * tiles256 > cus && 2 * tiles256 <= cus) return launch_halves<FP8>(a, f8, st);
             if (tile256_applies(a) && tiles256 >= 128) return launch_tiled<FP8>(a, f8, false, tail, st);
             if (m >= 128 && n >= 128 && fits32) return launch_tiled<FP8>(a, f8, true, 1, st);
             return launch_generic<FP8, 128>(a, f8, st);
@@ -388,6 +405,9 @@ static int launch_gemm(const void* xq, int64_t ld_xq, const float* sx, const voi
         case K_TILED_128:
             if (m < 128 || n < 128 || !fits32) return fail(DAXQ_ERR_ARG, "linear: the 128x128 kernel needs m, n >= 128");
             return launch_tiled<FP8>(a, f8, true, 1, st);
+        case K_TILED_HALVES:
+            if (!tile256_applies(a)) return fail(DAXQ_ERR_ARG, "linear: the 256x128 kernel needs m, n >= 256");
+            return launch_halves<FP8>(a, f8, st);
         default: return fail(DAXQ_ERR_ARG, "linear: unknown kernel choice %d", which);
     }
 }

@@ -284,8 +284,9 @@ int daxq_linear_e5m2_e4m3(const uint8_t* xq, int64_t ld_xq, const float* sx,
  *   fp8:  out = T( acc * sx[i] * sw[j] + f32(bias[j]) )                        (torch._scaled_mm, :155-173)
  * acc: optional int32 (int8) / fp32 (fp8) dump of the raw accumulators.
  * kernel: 0 = the library's choice by shape.  Other values pick one implementation, for tests and comparisons: low 16
- * bits 2 / 5 = the generic kernel on 256x256 / 128x128 tiles (an implementation of its own, any shape), 8 / 11 = the
- * tiled kernel on 256x256 / 128x128 tiles (int8: 16x16x64 MFMAs; fp8: 16x16x128 MFMAs; needs m, n >= the tile edge);
+ * bits 2 / 5 = the generic kernel on 256x256 / 128x128 tiles (an implementation of its own, any shape), 8 / 11 / 14 =
+ * the tiled kernel on 256x256 / 128x128 / 256x128 tiles (int8: 16x16x64 MFMAs; fp8: 16x16x128 MFMAs; needs m, n >= the
+ * tile edge, 256 for the 256x128 tiles);
  * bits 16-23, when not zero, set the depth of the tile-order groups; bits 24-27 the tile order of the 256x256 kernels
  * (0 = by shape, 1 = groups of tile rows, 2 = banded patches of 8 x 4 tiles per XCD; every order computes every tile
  * once, the results are the same bits); bits 28-29 the treatment of the last, partial round of workgroups of a launch

@@ -87,6 +87,17 @@ def test_config2_3_wan_14b_720p_shapes(k, n, fp8):
     _check(75600, k, n, seed=2, fp8=fp8)
 
 
+@pytest.mark.parametrize("fp8", [False, True])
+@pytest.mark.parametrize("m,k,n", [(1100, 2048, 4352), (1024, 5120, 5120)])
+def test_mid_size_launches_on_half_tiles(m, k, n, fp8):
+    """Between a quarter and a half of 256 CUs' worth of 256x256 tiles (85 and 80 here, K >= 2048) the library runs every
+    tile as its two 256x128 halves: outputs against the oracle, and the same bits as the launch of a row sample, which
+    takes the 128x128 tiles."""
+    tiles = -(-m // 256) * -(-n // 256)
+    assert 64 < tiles <= 128 and k >= 2048
+    _check(m, k, n, seed=5, fp8=fp8)
+
+
 def test_config4_cross_attention_small_m():
     # K / V projections of the 512-token text context (skinny M), and M = 1 / 17 leftovers
     for m in (512, 17, 1):

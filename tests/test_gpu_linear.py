@@ -14,12 +14,12 @@ from tests.util import bf16_bits, rel_l2
 
 pytestmark = pytest.mark.gpu
 
-VARIANTS = [0, 2, 5, 8, 11]  # 0 = library default, 2 / 5 = generic kernel on 256x256 / 128x128 tiles, 8 / 11 = tiled kernel on 256x256 / 128x128 tiles
+VARIANTS = [0, 2, 5, 8, 11, 14]  # 0 = library default, 2 / 5 = generic kernel on 256x256 / 128x128 tiles, 8 / 11 / 14 = tiled kernel on 256x256 / 128x128 / 256x128 tiles
 
 
 def _skip_if_too_small(variant, m, n):
-    if variant == 8 and (m < 256 or n < 256):
-        pytest.skip("the 256x256 kernel needs m, n >= 256")
+    if variant in (8, 14) and (m < 256 or n < 256):
+        pytest.skip("the 256x256 and 256x128 kernels need m, n >= 256")
     if variant == 11 and (m < 128 or n < 128):
         pytest.skip("the 128x128 kernel needs m, n >= 128")
 FP8_TOL = 2e-2
@@ -178,7 +178,7 @@ def _random_shapes(count, seed):
     return shapes
 
 
-@pytest.mark.parametrize("variant", [8, 11, 2, 8 | (2 << 24), 8 | (1 << 24)])
+@pytest.mark.parametrize("variant", [8, 11, 14, 2, 8 | (2 << 24), 8 | (1 << 24)])
 @pytest.mark.parametrize("m,n,k,pad_k,pad_n", _random_shapes(14, seed=2024))
 def test_linear_i8_random_shapes_and_strides_bit_exact(ops, variant, m, n, k, pad_k, pad_n):
     """Seeded random M, N, K (edge tiles shifted inwards in both directions, short and long K) with padded leading
@@ -233,7 +233,7 @@ def test_linear_i8_adversarial_extremes(ops, variant):
     np.testing.assert_array_equal(bf16_bits(out), bf16_bits(O.epilogue_int8(want, sx.view(-1, 1), sw.view(1, -1), None)))
 
 
-@pytest.mark.parametrize("variant", [0, 2, 8, 11])
+@pytest.mark.parametrize("variant", [0, 2, 8, 11, 14])
 def test_linear_i8_one_hot_layout(ops, variant):
     # a single non-zero in each operand lands in exactly one accumulator: catches any
     # row/column or operand transposition inside the MFMA tiling
@@ -275,7 +275,7 @@ def test_linear_e4m3_within_tolerance(ops, variant, m, n, k):
     assert r < 3e-3, r                          # what fp32 accumulation actually delivers
 
 
-@pytest.mark.parametrize("variant", [8, 11, 2])
+@pytest.mark.parametrize("variant", [8, 11, 14, 2])
 @pytest.mark.parametrize("e5m2", [False, True])
 @pytest.mark.parametrize("m,n,k,pad_k,pad_n", _random_shapes(8, seed=77))
 def test_linear_fp8_random_shapes_accumulators(ops, variant, e5m2, m, n, k, pad_k, pad_n):
@@ -316,13 +316,13 @@ def test_linear_fp8_random_shapes_accumulators(ops, variant, e5m2, m, n, k, pad_
     assert torch.equal(out_wide[:, :n].cpu(), acc_wide[:, :n].cpu().bfloat16())   # unit scales, no bias: out = bf16(acc)
 
 
-@pytest.mark.parametrize("variant", [8, 11])
+@pytest.mark.parametrize("variant", [8, 11, 14])
 @pytest.mark.parametrize("k", [128, 256, 384, 512, 640, 768, 896, 1024, 1152, 1280, 1408, 1536])
 def test_fp8_16x16x128_form_every_count_of_slice_pairs(ops, k, variant):
-    """Every number of 128-byte pairs of K slices from 1 to 12 on both tile sizes: the plain loop below four pairs, then
-    first pair, steady pairs in twos, the odd one and the register moves in front of the three tail pairs all occur.
-    Accumulators against exact float64 sums, element by element, on a grid of tiles with ragged edges; both tile sizes
-    give the same bits."""
+    """Every number of 128-byte pairs of K slices from 1 to 12 on the three tile sizes: the plain loop below four pairs,
+    then first pair, steady pairs in twos, the odd one and the register moves in front of the three tail pairs all occur.
+    Accumulators against exact float64 sums, element by element, on a grid of tiles with ragged edges; every tile size
+    gives the same bits."""
     from dax_amd import _capi
 
     m, n = 300, 700
@@ -343,7 +343,7 @@ def test_fp8_16x16x128_form_every_count_of_slice_pairs(ops, k, variant):
     np.testing.assert_array_equal(bf16_bits(out), bf16_bits(ref))
     _capi.debug_select_gemm(8 if variant == 11 else 11)
     out2, acc2 = ops.linear_e4m3_acc(dev(xf.view(torch.uint8)), dev(sx), dev(wf.view(torch.uint8)), dev(sw), dev(b))
-    assert torch.equal(acc, acc2) and torch.equal(out, out2), "256x256 and 128x128 tiles must give the same FP8 bits"
+    assert torch.equal(acc, acc2) and torch.equal(out, out2), "every tile size must give the same FP8 bits"
 
 
 @pytest.mark.parametrize("k", [3968, 4096, 4224, 4352, 4480, 5120, 13824])
@@ -440,7 +440,7 @@ def test_linear_rejects_unaligned_k(ops):
         ops.linear_i8(xq, torch.ones(8, device="cuda"), wq, torch.ones(8, device="cuda"), None)
 
 
-@pytest.mark.parametrize("variant", [0, 5, 2, 8, 11])
+@pytest.mark.parametrize("variant", [0, 5, 2, 8, 11, 14])
 def test_linear_leading_dimensions_through_the_c_abi(ops, variant):
     """Operands and output as column slices of wider buffers (ld > logical width), straight through the C ABI:
     what a caller does that writes q | k | v into one [M, 3N] tensor with three launches."""
