@@ -226,22 +226,27 @@ __device__ __forceinline__ void gemm_tile256x128_fp8_body(const GemmArgs& p, con
     const uint32_t gsw = (uint32_t)(((t & 3) ^ ((t >> 3) & 3)) << 4);
     uint32_t voff_a = (uint32_t)(t >> 2) * (uint32_t)p.lda + gsw;
     uint32_t voff_b = (uint32_t)(t >> 2) * (uint32_t)p.ldb + gsw;
+    uint32_t voff_a1 = voff_a + BKS, voff_b1 = voff_b + BKS;  // second half of the 128-byte line
     const uint8_t* abase = p.a + (int64_t)m0 * p.lda;
     const uint8_t* bbase = p.b + (int64_t)n0 * p.ldb;
     const int64_t a_step = 64 * p.lda, b_step = 64 * p.ldb;
     const uint32_t lds0 = (uint32_t)(uintptr_t)(DAXQ_LDS uint8_t*)smem;
     const uint32_t wave_lds = lds0 + (uint32_t)__builtin_amdgcn_readfirstlane(wave * 1024);
     // load g of a pair (12): 0-7 activation rows, 8-11 weight rows; 64-row block, then slice g%2 of the pair (the two
-    // halves of a 128-byte line by consecutive instructions)
+    // halves of a 128-byte line by consecutive instructions).  Address = uniform row-block base (SGPR pair) + per-lane
+    // 32-bit offset: no VALU work per load.
     auto issue_one = [&](uint32_t slot, int g) {
         const int opnd = g >= A_LOADS, gg = opnd ? g - A_LOADS : g, j = gg >> 1, half = gg & 1;
-        const uint8_t* src = (opnd ? bbase + j * b_step + voff_b : abase + j * a_step + voff_a) + half * BKS;
+        const uint8_t* src = opnd ? bbase + j * b_step : abase + j * a_step;
+        const uint32_t voff = opnd ? (half ? voff_b1 : voff_b) : (half ? voff_a1 : voff_a);
         const uint32_t dst = wave_lds + slot + (opnd ? A_PART + half * B_HALF : half * A_HALF) + j * 4096;
-        __builtin_amdgcn_global_load_lds((const DAXQ_GLOBAL void*)src, (DAXQ_LDS void*)(uintptr_t)dst, 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((const DAXQ_GLOBAL void*)(src + voff), (DAXQ_LDS void*)(uintptr_t)dst, 16, 0, 0);
     };
     auto advance = [&]() {
         voff_a += 2 * BKS;
         voff_b += 2 * BKS;
+        voff_a1 += 2 * BKS;
+        voff_b1 += 2 * BKS;
     };
 
     const int lr = lane & 15, kg = lane >> 4;
