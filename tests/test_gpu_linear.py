@@ -117,6 +117,46 @@ TAIL_SHAPES = [(4100, 4352, 128), (8500, 4096, 256), (4725, 13824, 128), (16300,
 HALF_TAIL_SHAPES = [(4725, 5120, 128), (4725, 15360 - 24, 256), (9000, 2560, 384), (4725 - 3, 5120, 1152)]
 
 
+# 256-tile rows of a grid of 20 tile columns, one per way the library cuts a launch by its tile count on 256 CUs: 60 tiles
+# (128x128 tiles), 80 and 120 (every tile as two halves), 140 (whole tiles, part of a round), 260 and 320 (a round, the
+# rest as quadrants), 340 and 380 (the rest as halves), 400 (two rounds of whole tiles)
+CUT_ROWS = [3, 4, 6, 7, 13, 16, 17, 19, 20]
+
+
+@pytest.mark.parametrize("tile_rows", CUT_ROWS)
+def test_every_cut_of_a_launch_by_tile_count(ops, tile_rows):
+    """The library's own choice (kernel argument 0) on either side of every tile count at which it changes the way a
+    launch is cut into workgroups, ragged in both dimensions, K = 2048.  INT8: sampled rows (both edges of every tile
+    row among them) against the integer oracle, and the whole output against the launch forced onto whole 256x256 tiles.
+    FP8: the whole output is the bits of the launch forced onto whole 256x256 tiles."""
+    from dax_amd import _capi
+
+    m, n, k = 256 * tile_rows - 37, 5120 - 8, 2048
+    g = torch.Generator().manual_seed(tile_rows)
+    xq = torch.randint(-127, 128, (m, k), dtype=torch.int8, generator=g)
+    wq = torch.randint(-127, 128, (n, k), dtype=torch.int8, generator=g)
+    sx = torch.rand(m, generator=g) * 0.02 + 1e-3
+    sw = torch.rand(n, generator=g) * 0.002 + 1e-4
+    b = (torch.randn(n, generator=g) * 0.5).bfloat16()
+    xd, wd, sxd, swd, bd = dev(xq), dev(wq), dev(sx), dev(sw), dev(b)
+    out = ops.linear_i8(xd, sxd, wd, swd, bd)
+    edges = [r for t in range(tile_rows) for r in (256 * t, 256 * t + 255) if r < m] + [m - 256, m - 1]
+    rows = torch.tensor(sorted(set(edges)) + torch.randint(0, m, (64,), generator=g).tolist())
+    want = O.epilogue_int8(O.int_mm(xq[rows], wq), sx[rows].view(-1, 1), sw.view(1, -1), b)
+    np.testing.assert_array_equal(bf16_bits(out[rows.to("cuda")]), bf16_bits(want))
+    # any finite e4m3fn bytes
+    x8 = torch.where((xq.view(torch.uint8) & 0x7f) == 0x7f, torch.zeros((), dtype=torch.uint8), xq.view(torch.uint8)).cuda()
+    w8 = torch.where((wq.view(torch.uint8) & 0x7f) == 0x7f, torch.zeros((), dtype=torch.uint8), wq.view(torch.uint8)).cuda()
+    swf = swd * 1e-3
+    out8 = ops.linear_e4m3(x8, sxd, w8, swf, bd)
+    _capi.debug_select_gemm(8)
+    _capi.debug_select_gemm(3001)
+    assert torch.equal(out.view(torch.int16), ops.linear_i8(xd, sxd, wd, swd, bd).view(torch.int16))
+    whole8 = ops.linear_e4m3(x8, sxd, w8, swf, bd)
+    assert bool(torch.isfinite(whole8.float()).all())
+    assert torch.equal(out8.view(torch.int16), whole8.view(torch.int16)), "FP8 bits depend on how the launch is cut"
+
+
 @pytest.mark.parametrize("m,n,k", TAIL_SHAPES + HALF_TAIL_SHAPES)
 def test_last_round_in_smaller_pieces_bit_exact(ops, m, n, k):
     """A launch of 256x256 tiles whose last round of workgroups is a few tiles: the whole rounds run as 256x256 tiles,
