@@ -293,9 +293,19 @@ __device__ __forceinline__ void gemm_tile256x128_fp8_body(const GemmArgs& p, con
         __builtin_amdgcn_s_barrier();  // pair q+1 has landed for everyone, and everyone has read pair q out of its slot
 #pragma unroll
         for (int g = 0; g < NREG; ++g) {
+            // Two loads per region, the two halves of a 128-byte line: the activation rows' four lines in regions 0, 8,
+            // 16, 24, the weight rows' two in regions 4 and 20.  (One load per region in twelve regions, between the
+            // regions that read fragments, ran the pair in 0.70 us instead of 0.56: 80.3 against 65.3 us at 1024 x 5120,
+            // K = 13824; three or four loads per region 67 to 68 us, all twelve at once 92.7.  The other tiled kernels
+            // were tried with their loads in twos as well and are as fast or 1 to 2 % faster with single ones.)
             if constexpr (ISSUE.value) {
-                if (g % 4 == 0) issue_one(s0, g / 4);                    // the 8 activation loads
-                else if (g % 8 == 2) issue_one(s0, A_LOADS + g / 8);     // the 4 weight loads
+                if (g % 8 == 0) {
+                    issue_one(s0, g / 4);
+                    issue_one(s0, g / 4 + 1);
+                } else if (g % 16 == 4) {
+                    issue_one(s0, A_LOADS + g / 8);
+                    issue_one(s0, A_LOADS + g / 8 + 1);
+                }
             }
             if constexpr (NEXT.value) {
                 if (g % 2 == 1 && g / 2 < NBI + NBJ) {

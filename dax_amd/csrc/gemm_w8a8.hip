@@ -385,10 +385,10 @@ static int launch_gemm(const void* xq, int64_t ld_xq, const float* sx, const voi
             // 4096 x 1536 x 1536 (96) -> 1182 / 895, 8192 x 1536 x 1536 (192) -> 1517 / 1587.
             // Between a quarter and a half of the CUs' worth of large tiles, every tile runs as its two 256x128 halves with
             // a CU each (K >= 2048).  Measured against what these launches took before (128x128 tiles up to 127 large
-            // tiles, whole 256x256 tiles at 128), INT8 / e4m3, us: 1024 x 5120 x 5120 (80 tiles) 38.7 -> 31.0 / 37.7 -> 34.7,
-            // 1536 x 5120 x 5120 (120) 41.1 -> 35.0 / 40.3 -> 37.9, 1100 x 4352 x 5120 (85) 42.4 -> 31.6 / 41.1 -> 35.6,
-            // 2048 x 4096 x 4096 (128) 39.6 -> 30.7 / 38.7 -> 31.4, 1024 x 5120, K = 13824 95.9 -> 69.3 / 93.1 -> 80.6,
-            // 4096 x 1536, K = 8960 62.3 -> 50.7 / 60.5 -> 55.6, K = 3072 +9 to +15 % / +4 to +5 %, K = 2048 0 to +10 % / +2 %;
+            // tiles, whole 256x256 tiles at 128), INT8 / e4m3, us: 1024 x 5120 x 5120 (80 tiles) 38.7 -> 31.0 / 37.7 -> 29.6,
+            // 1536 x 5120 x 5120 (120) 41.1 -> 35.0 / 40.3 -> 35.3, 1100 x 4352 x 5120 (85) 42.4 -> 31.6 / 41.1 -> 31.1,
+            // 2048 x 4096 x 4096 (128) 39.6 -> 30.7 / 38.7 -> 31.2, 1024 x 5120, K = 13824 95.9 -> 69.3 / 93.1 -> 66.8,
+            // 4096 x 1536, K = 8960 62.3 -> 50.7 / 60.5 -> 50.3, K = 3072 +9 to +15 % / +16 %, K = 2048 0 to +10 % / +2 %;
             // at K = 1536 -2 / -5 %, and with 60 tiles (768 x 5120 x 5120) the quadrants' 23.8 us become 30.5.
             const int64_t tiles256 = ((m + 255) / 256) * ((n + 255) / 256);
             const int cus = cu_count();
