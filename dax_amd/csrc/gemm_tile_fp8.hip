@@ -169,11 +169,30 @@ __device__ __forceinline__ void gemm_tile_fp8_body(const GemmArgs& p, const int 
                 __builtin_amdgcn_s_waitcnt(vmcnt_imm((ISSUE_A.value ? 2 * LPO : 0) + EXTRA.value));
                 __builtin_amdgcn_s_barrier();
             }
+            // 128 tiles issue their loads in twos (both halves of a 128-byte line in one region): with a load in every other
+            // region of so short a pair nearly every MFMA has a memory instruction in front of it; +2.5 % on launches with
+            // a CU per workgroup and long K (512 x 5120 x 5120: 21.0 -> 20.5 us), nothing elsewhere.  The 256 tiles, a
+            // load every fourth region, lose 1 % that way.
+            constexpr bool twos = BT == 128;
             if constexpr (ISSUE_A.value) {
-                if (g < HREG && g % DMA_EVERY == 0) issue_a(r0, g / DMA_EVERY);
+                if constexpr (twos) {
+                    if (g < HREG && g % (2 * DMA_EVERY) == 0) {
+                        issue_a(r0, g / DMA_EVERY);
+                        issue_a(r0, g / DMA_EVERY + 1);
+                    }
+                } else {
+                    if (g < HREG && g % DMA_EVERY == 0) issue_a(r0, g / DMA_EVERY);
+                }
             }
             if constexpr (ISSUE_B.value) {
-                if (g >= HREG && (g - HREG) % DMA_EVERY == 0) issue_b(r1, (g - HREG) / DMA_EVERY);
+                if constexpr (twos) {
+                    if (g >= HREG && (g - HREG) % (2 * DMA_EVERY) == 0) {
+                        issue_b(r1, (g - HREG) / DMA_EVERY);
+                        issue_b(r1, (g - HREG) / DMA_EVERY + 1);
+                    }
+                } else {
+                    if (g >= HREG && (g - HREG) % DMA_EVERY == 0) issue_b(r1, (g - HREG) / DMA_EVERY);
+                }
             }
             if constexpr (nxt) {
                 // the last B block of the next pair into the set this pair does not use
